@@ -1,0 +1,229 @@
+/* knhip.h - C ABI of libknhip, the MI355X (gfx950) executor for Kyanite graphs.
+ *
+ * This is what a `kn-hip-sys` crate binds in place of `kn-cuda-sys`. Every function returns 0 on success and a
+ * non-zero status otherwise; `knhip_last_error()` then describes the failure (thread local). No exception or
+ * panic crosses this boundary: where the reference panics (kn-cuda-sys/src/wrapper/status.rs:9-33 and the asserts
+ * of kn-cuda-eval/src/executor.rs:118-127) these functions report an error, and a binding can turn it back into
+ * a panic to keep the reference's behaviour.
+ *
+ * Handles are not thread safe (the reference's executor is Send but takes &mut self, executor.rs:41, :117);
+ * every entry point selects its device itself (handle.rs:60-64).
+ *
+ * File/line citations name the reference interface each group replaces, relative to the Kyanite repository.
+ */
+#ifndef KNHIP_H
+#define KNHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status ------------------------------------------------------------------------------------------------ */
+#define KNHIP_OK 0
+#define KNHIP_ERROR 1          /* contract violation or runtime failure, see knhip_last_error() */
+#define KNHIP_BUFFER_TOO_SMALL 2
+
+const char *knhip_last_error(void);
+
+/* ---- element types (kn-graph/src/dtype.rs:24-37, plus F16) --------------------------------------------------- */
+enum {
+    KNHIP_F32 = 0, KNHIP_F64 = 1, KNHIP_I8 = 2, KNHIP_I16 = 3, KNHIP_I32 = 4, KNHIP_I64 = 5,
+    KNHIP_U8 = 6, KNHIP_U16 = 7, KNHIP_U32 = 8, KNHIP_U64 = 9, KNHIP_BOOL = 10, KNHIP_F16 = 11
+};
+
+/* one dimension `fixed_factor * batch_size^batch_exp` (kn-graph/src/shape.rs:31-38) */
+typedef struct {
+    uint64_t fixed_factor;
+    uint32_t batch_exp;
+} knhip_size_t;
+
+/* operation codes as stored in value infos and in the serialised graph (kn-graph/src/graph.rs:106-162) */
+enum {
+    KNHIP_OP_INPUT = 0, KNHIP_OP_CONSTANT = 1, KNHIP_OP_VIEW = 2, KNHIP_OP_BROADCAST = 3, KNHIP_OP_PERMUTE = 4,
+    KNHIP_OP_SLICE = 5, KNHIP_OP_FLIP = 6, KNHIP_OP_GATHER = 7, KNHIP_OP_CONCAT = 8, KNHIP_OP_CONV = 9,
+    KNHIP_OP_MATMUL = 10, KNHIP_OP_UNARY = 11, KNHIP_OP_BINARY = 12, KNHIP_OP_SOFTMAX = 13, KNHIP_OP_LAYERNORM = 14,
+    KNHIP_OP_REDUCE = 15
+};
+/* graph.rs:173-195 */
+enum {
+    KNHIP_UNARY_ABS = 0, KNHIP_UNARY_NEG = 1, KNHIP_UNARY_SIN = 2, KNHIP_UNARY_COS = 3, KNHIP_UNARY_EXP = 4,
+    KNHIP_UNARY_LOG = 5, KNHIP_UNARY_SQRT = 6, KNHIP_UNARY_SIGMOID = 7, KNHIP_UNARY_TANH = 8, KNHIP_UNARY_ERF = 9,
+    KNHIP_UNARY_MISH = 10, KNHIP_UNARY_SOFTPLUS = 11, KNHIP_UNARY_VALUE_CAST = 12, KNHIP_UNARY_BIT_CAST = 13
+};
+/* graph.rs:197-206 */
+enum { KNHIP_BINARY_ADD = 0, KNHIP_BINARY_SUB = 1, KNHIP_BINARY_MUL = 2, KNHIP_BINARY_DIV = 3, KNHIP_BINARY_MIN = 4,
+       KNHIP_BINARY_MAX = 5, KNHIP_BINARY_POW = 6 };
+/* graph.rs:208-217 */
+enum { KNHIP_REDUCE_SUM = 0, KNHIP_REDUCE_MEAN = 1, KNHIP_REDUCE_PROD = 2, KNHIP_REDUCE_MAX = 3, KNHIP_REDUCE_MIN = 4 };
+
+/* ---- device and memory shim (replaces kn-cuda-sys/src/wrapper/handle.rs:37-103 and mem/{device,pinned}.rs) ---- */
+int knhip_device_count(int *count);
+int knhip_device_name(int device, char *buf, size_t cap, size_t *needed);
+int knhip_malloc(int device, size_t bytes, void **ptr);
+int knhip_free(int device, void *ptr);
+int knhip_memcpy_h2d(int device, void *dst, const void *src, size_t bytes);
+int knhip_memcpy_d2h(int device, void *dst, const void *src, size_t bytes);
+int knhip_memcpy_d2d(int device, void *dst, const void *src, size_t bytes);
+int knhip_host_alloc(size_t bytes, void **ptr);
+int knhip_host_free(void *ptr);
+int knhip_device_synchronize(int device);
+
+/* ---- graph (kn-graph/src/graph.rs) ------------------------------------------------------------------------- */
+typedef struct knhip_graph knhip_graph;
+typedef uint32_t knhip_value; /* index of a value inside its graph; values are append-only (graph.rs:86-91) */
+
+int knhip_graph_new(knhip_graph **out);                                   /* graph.rs:364-373 */
+int knhip_graph_clone(const knhip_graph *graph, knhip_graph **out);
+void knhip_graph_free(knhip_graph *graph);
+/* flat binary form, the way a host language hands over a graph built with its own kn-graph */
+int knhip_graph_deserialize(const uint8_t *blob, size_t len, knhip_graph **out);
+int knhip_graph_serialize(const knhip_graph *graph, uint8_t *buf, size_t cap, size_t *needed);
+int knhip_graph_str(const knhip_graph *graph, char *buf, size_t cap, size_t *needed); /* graph.rs:1473-1512 */
+
+/* builder, one entry per public builder method (graph.rs:583-1363) */
+int knhip_graph_input(knhip_graph *g, const knhip_size_t *dims, size_t rank, int dtype, knhip_value *out);
+int knhip_graph_constant(knhip_graph *g, const knhip_size_t *dims, size_t rank, int dtype, const void *data,
+                         size_t data_bytes, knhip_value *out);
+int knhip_graph_view(knhip_graph *g, knhip_value input, const knhip_size_t *dims, size_t rank, knhip_value *out);
+int knhip_graph_broadcast(knhip_graph *g, knhip_value input, const knhip_size_t *dims, size_t rank, knhip_value *out);
+int knhip_graph_repeat_unary(knhip_graph *g, knhip_value input, size_t axis, knhip_size_t count, knhip_value *out);
+int knhip_graph_flatten(knhip_graph *g, knhip_value input, size_t start_axis, knhip_value *out);
+int knhip_graph_permute(knhip_graph *g, knhip_value input, const size_t *permutation, size_t rank, knhip_value *out);
+int knhip_graph_slice(knhip_graph *g, knhip_value input, size_t axis, size_t start, size_t end, size_t step,
+                      knhip_value *out);
+int knhip_graph_index(knhip_graph *g, knhip_value input, size_t axis, size_t index, knhip_value *out);
+int knhip_graph_flip(knhip_graph *g, knhip_value input, size_t axis, knhip_value *out);
+int knhip_graph_repeat(knhip_graph *g, knhip_value input, size_t axis, knhip_size_t count, int interleave,
+                       knhip_value *out);
+int knhip_graph_gather(knhip_graph *g, knhip_value input, size_t axis, knhip_value indices, knhip_value *out);
+/* base_dims may be NULL (infer from the first input); dtype may be -1 (infer) */
+int knhip_graph_concat(knhip_graph *g, const knhip_value *inputs, size_t count, size_t axis,
+                       const knhip_size_t *base_dims, size_t base_rank, int dtype, knhip_value *out);
+/* pad_amount holds rank (before, after) pairs */
+int knhip_graph_pad(knhip_graph *g, knhip_value input, const size_t *pad_amount, size_t rank, knhip_value pad_value,
+                    knhip_value *out);
+int knhip_graph_conv(knhip_graph *g, knhip_value input, knhip_value filter, size_t stride_y, size_t stride_x,
+                     size_t padding_y, size_t padding_x, knhip_value *out);
+int knhip_graph_linear(knhip_graph *g, knhip_value input, knhip_value weight, knhip_value *out);
+int knhip_graph_mat_mul(knhip_graph *g, knhip_value left, knhip_value right, knhip_value *out);
+int knhip_graph_batched_mat_mul(knhip_graph *g, knhip_value left, knhip_value right, knhip_value *out);
+int knhip_graph_softmax(knhip_graph *g, knhip_value input, size_t axis, knhip_value *out);
+int knhip_graph_layernorm(knhip_graph *g, knhip_value input, size_t axis, float eps, knhip_value *out);
+int knhip_graph_reduce(knhip_graph *g, knhip_value input, const size_t *axes, size_t count, int op, knhip_value *out);
+/* min and max point at one element of the value's dtype */
+int knhip_graph_clamp(knhip_graph *g, knhip_value input, const void *min, const void *max, knhip_value *out);
+int knhip_graph_relu(knhip_graph *g, knhip_value input, knhip_value *out);
+int knhip_graph_unary(knhip_graph *g, int op, int cast_dtype, knhip_value input, knhip_value *out);
+int knhip_graph_binary(knhip_graph *g, int op, knhip_value left, knhip_value right, knhip_value *out);
+/* graph.rs:1319-1351: inline `callee` into `g`; `outputs` receives callee's output count values */
+int knhip_graph_call(knhip_graph *g, const knhip_graph *callee, const knhip_value *inputs, size_t input_count,
+                     knhip_value *outputs, size_t output_cap, size_t *output_count);
+int knhip_graph_output(knhip_graph *g, knhip_value value);
+int knhip_graph_set_debug_id(knhip_graph *g, knhip_value value, const char *id);
+
+/* queries */
+int knhip_graph_value_count(const knhip_graph *g, size_t *count);
+int knhip_graph_inputs(const knhip_graph *g, knhip_value *buf, size_t cap, size_t *count);
+int knhip_graph_outputs(const knhip_graph *g, knhip_value *buf, size_t cap, size_t *count);
+typedef struct {
+    int dtype;
+    int op;           /* KNHIP_OP_* */
+    int sub_op;       /* unary / binary / reduce code, else -1 */
+    int cast_dtype;   /* for casts, else -1 */
+    size_t rank;
+    size_t operand_count;
+    size_t axis_count; /* permutation / axis / axes */
+    size_t non_output_uses;
+    size_t slice_start, slice_end, slice_step;
+    float eps;
+    int is_hidden;
+} knhip_value_info;
+int knhip_graph_value_info(const knhip_graph *g, knhip_value value, knhip_value_info *info);
+int knhip_graph_value_shape(const knhip_graph *g, knhip_value value, knhip_size_t *dims, size_t cap);
+int knhip_graph_value_operands(const knhip_graph *g, knhip_value value, knhip_value *buf, size_t cap);
+int knhip_graph_value_axes(const knhip_graph *g, knhip_value value, size_t *buf, size_t cap);
+/* data of a Constant value: pointer stays valid as long as the graph lives */
+int knhip_graph_value_constant(const knhip_graph *g, knhip_value value, const void **data, size_t *bytes);
+/* graph.rs:490-527: 1 in *is_single and the element in `element` (8 bytes of room) when every element is equal */
+int knhip_graph_as_single_const(const knhip_graph *g, knhip_value value, int *is_single, void *element);
+
+/* kn-graph/src/shape.rs:353-365. `actual` holds the concatenated dims of all inputs. *status: 0 ok, 1 different
+ * length, 2 constant mismatch, 3 batch conflict, 4 impossible batch value; *has_batch 0 when any batch size fits */
+int knhip_graph_infer_batch_size(const knhip_graph *g, const size_t *actual, const size_t *ranks, size_t input_count,
+                                 int *status, int *has_batch, uint64_t *batch);
+
+/* kn-graph/src/optimizer/mod.rs:11-46 */
+typedef struct {
+    int optimize;
+    int force_bias_through_conv;
+    int fuse_layernorm;
+    int div_to_mul;
+} knhip_optimizer_settings;
+int knhip_optimizer_settings_default(knhip_optimizer_settings *settings);
+int knhip_graph_optimize(const knhip_graph *g, const knhip_optimizer_settings *settings, knhip_graph **out);
+
+/* ---- executor (kn-cuda-eval/src/executor.rs:60-258, kn-runtime/src/lib.rs:85-126) ------------------------------ */
+typedef struct knhip_executor knhip_executor;
+
+/* CudaExecutor::new(device, &graph, batch_size) (executor.rs:61). With plan_only != 0 nothing touches a device:
+ * the graph is planned and its kernels are compiled, which works on a machine without a GPU. */
+int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int plan_only, knhip_executor **out);
+int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int plan_only,
+                                 knhip_executor **out);
+void knhip_executor_free(knhip_executor *ex);
+
+int knhip_executor_io_count(const knhip_executor *ex, size_t *inputs, size_t *outputs);
+/* dtype, rank and concrete dims (cap entries of room) of input / output `index` */
+int knhip_executor_io_info(const knhip_executor *ex, int is_output, size_t index, int *dtype, size_t *rank,
+                           size_t *dims, size_t cap);
+
+/* CudaExecutor::evaluate (executor.rs:117-195): dense row-major host buffers in, dense row-major host buffers out.
+ * Byte counts are checked against the planned shapes. */
+int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const size_t *input_bytes, size_t input_count,
+                            void *const *outputs, const size_t *output_bytes, size_t output_count);
+/* run_async (executor.rs:199-258): launch all steps on the executor's stream, no synchronisation */
+int knhip_executor_run_async(knhip_executor *ex);
+int knhip_executor_synchronize(knhip_executor *ex);
+/* device addresses of the dense input / output tensors inside the arena (pub device_inputs / device_outputs) */
+int knhip_executor_input_ptr(const knhip_executor *ex, size_t index, void **ptr);
+int knhip_executor_output_ptr(const knhip_executor *ex, size_t index, void **ptr);
+/* the HIP stream (hipStream_t) every step is launched on (CudaExecutor::stream, executor.rs:112-114) */
+int knhip_executor_stream(const knhip_executor *ex, void **stream);
+
+/* set_profile / last_profile (executor.rs:260-266). Seconds per step kind in the order
+ * conv, mat_mul, scalar_op, reduce_op, softmax_op, layernorm_op, gather_op. */
+typedef struct {
+    float per_kind[7];
+    float total_cpu, total_gpu, timing_overhead;
+    size_t step_count;
+} knhip_profile;
+int knhip_executor_set_profile(knhip_executor *ex, int enabled);
+int knhip_executor_last_profile(const knhip_executor *ex, int *available, knhip_profile *profile);
+int knhip_executor_profile_step_seconds(const knhip_executor *ex, float *buf, size_t cap);
+int knhip_executor_profile_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed);
+
+/* MemoryUsage (kn-cuda-eval/src/planner.rs:67-81) */
+typedef struct {
+    size_t dedicated_bytes, shared_bytes, zero_bytes, hypo_shared_bytes_peak, hypo_shared_bytes_total, arena_bytes;
+} knhip_mem_usage;
+int knhip_executor_mem_usage(const knhip_executor *ex, knhip_mem_usage *usage);
+
+/* the planned launch list (Debug output of the executor, executor.rs:269-289) */
+int knhip_executor_step_count(const knhip_executor *ex, size_t *count);
+/* kind: 0 conv, 1 mat_mul, 2 scalar_op, 3 reduce_op, 4 softmax_op, 5 layernorm_op, 6 gather_op */
+int knhip_executor_step_kind(const knhip_executor *ex, size_t index, int *kind);
+int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed);
+int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed);
+int knhip_executor_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed);
+
+/* kernel compile cache counters (autokernel/common.rs:14-46) */
+int knhip_compile_stats(size_t *compiled, size_t *memory_hits, size_t *disk_hits);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* KNHIP_H */

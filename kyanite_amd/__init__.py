@@ -1,0 +1,15 @@
+"""kyanite_amd: an MI355X (gfx950) executor for Kyanite graphs.
+
+The work is done by libknhip.so (C++ host runtime + HIP kernels); this package is the ctypes face of its C ABI,
+shaped like the reference's `kn-graph` builder and `CudaExecutor`.
+"""
+from ._lib import KnError, LIB_PATH
+from .executor import Device, HipDevice, HipExecutor, PreparedGraph, Profile, compile_stats
+from .graph import (BATCH, BINARY_ALL, REDUCE_ALL, UNARY_ALL, BinaryOp, DType, Graph, OpKind, OptimizerSettings,
+                    ReduceOp, Size, UnaryOp, Value, optimize_graph, shape)
+
+__all__ = [
+    "KnError", "LIB_PATH", "Device", "HipDevice", "HipExecutor", "PreparedGraph", "Profile", "compile_stats",
+    "BATCH", "BINARY_ALL", "REDUCE_ALL", "UNARY_ALL", "BinaryOp", "DType", "Graph", "OpKind", "OptimizerSettings",
+    "ReduceOp", "Size", "UnaryOp", "Value", "optimize_graph", "shape",
+]

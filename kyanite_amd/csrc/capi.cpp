@@ -1,0 +1,712 @@
+// The extern "C" surface declared in include/knhip.h. Every entry point catches all exceptions and converts
+// them into a status code plus a thread-local message.
+#include "../../include/knhip.h"
+
+#include <cstring>
+#include <new>
+
+#include "executor.h"
+#include "optimizer.h"
+
+using namespace kn;
+
+struct knhip_graph {
+    Graph graph;
+};
+struct knhip_executor {
+    HipExecutor ex;
+    knhip_executor(int device, const Graph &g, size_t batch, bool plan_only) : ex(device, g, batch, plan_only) {}
+};
+
+namespace {
+
+thread_local std::string g_last_error;
+
+template <typename F>
+int guarded(F f) {
+    try {
+        return f();
+    } catch (const std::exception &e) {
+        g_last_error = e.what();
+        return KNHIP_ERROR;
+    } catch (...) {
+        g_last_error = "unknown failure";
+        return KNHIP_ERROR;
+    }
+}
+
+#define KN_REQUIRE(cond)                                       \
+    do {                                                       \
+        if (!(cond)) fail("invalid argument: " #cond " does not hold"); \
+    } while (0)
+
+Shape to_shape(const knhip_size_t *dims, size_t rank) {
+    KN_REQUIRE(dims != nullptr || rank == 0);
+    Shape s;
+    for (size_t i = 0; i < rank; i++) s.dims.push_back(Size(dims[i].batch_exp, dims[i].fixed_factor));
+    return s;
+}
+
+DType to_dtype(int code) {
+    if (!dtype_valid(code)) fail("invalid dtype code ", code);
+    return (DType) code;
+}
+
+int copy_out(const std::string &s, char *buf, size_t cap, size_t *needed) {
+    if (needed) *needed = s.size() + 1;
+    if (buf == nullptr || cap < s.size() + 1) {
+        if (buf == nullptr && cap == 0) return KNHIP_OK;  // size query
+        g_last_error = "buffer too small";
+        return KNHIP_BUFFER_TOO_SMALL;
+    }
+    std::memcpy(buf, s.c_str(), s.size() + 1);
+    return KNHIP_OK;
+}
+
+template <typename T, typename U>
+int copy_list(const std::vector<T> &v, U *buf, size_t cap, size_t *count) {
+    if (count) *count = v.size();
+    if (buf == nullptr && cap == 0) return KNHIP_OK;
+    if (cap < v.size()) {
+        g_last_error = "buffer too small";
+        return KNHIP_BUFFER_TOO_SMALL;
+    }
+    for (size_t i = 0; i < v.size(); i++) buf[i] = (U) v[i];
+    return KNHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *knhip_last_error(void) { return g_last_error.c_str(); }
+
+// ---------------------------------------------------------------------------------------------- device shim
+
+int knhip_device_count(int *count) {
+    return guarded([&] {
+        KN_REQUIRE(count != nullptr);
+        *count = HipDevice::count();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_device_name(int device, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] { return copy_out(HipDevice::name(device), buf, cap, needed); });
+}
+
+int knhip_malloc(int device, size_t bytes, void **ptr) {
+    return guarded([&] {
+        KN_REQUIRE(ptr != nullptr);
+        HipDevice::check(device);
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        hip_check(hipMalloc(ptr, std::max<size_t>(bytes, 1)), "hipMalloc");
+        return KNHIP_OK;
+    });
+}
+
+int knhip_free(int device, void *ptr) {
+    return guarded([&] {
+        HipDevice::check(device);
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        hip_check(hipFree(ptr), "hipFree");
+        return KNHIP_OK;
+    });
+}
+
+static int do_memcpy(int device, void *dst, const void *src, size_t bytes, hipMemcpyKind kind) {
+    return guarded([&] {
+        HipDevice::check(device);
+        KN_REQUIRE(bytes == 0 || (dst != nullptr && src != nullptr));
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        if (bytes) hip_check(hipMemcpy(dst, src, bytes, kind), "hipMemcpy");
+        return KNHIP_OK;
+    });
+}
+int knhip_memcpy_h2d(int device, void *dst, const void *src, size_t bytes) { return do_memcpy(device, dst, src, bytes, hipMemcpyHostToDevice); }
+int knhip_memcpy_d2h(int device, void *dst, const void *src, size_t bytes) { return do_memcpy(device, dst, src, bytes, hipMemcpyDeviceToHost); }
+int knhip_memcpy_d2d(int device, void *dst, const void *src, size_t bytes) { return do_memcpy(device, dst, src, bytes, hipMemcpyDeviceToDevice); }
+
+int knhip_host_alloc(size_t bytes, void **ptr) {
+    return guarded([&] {
+        KN_REQUIRE(ptr != nullptr);
+        hip_check(hipHostMalloc(ptr, std::max<size_t>(bytes, 1), hipHostMallocDefault), "hipHostMalloc");
+        return KNHIP_OK;
+    });
+}
+
+int knhip_host_free(void *ptr) {
+    return guarded([&] {
+        hip_check(hipHostFree(ptr), "hipHostFree");
+        return KNHIP_OK;
+    });
+}
+
+int knhip_device_synchronize(int device) {
+    return guarded([&] {
+        HipDevice::check(device);
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        hip_check(hipDeviceSynchronize(), "hipDeviceSynchronize");
+        return KNHIP_OK;
+    });
+}
+
+// ---------------------------------------------------------------------------------------------- graph
+
+int knhip_graph_new(knhip_graph **out) {
+    return guarded([&] {
+        KN_REQUIRE(out != nullptr);
+        *out = new knhip_graph();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_clone(const knhip_graph *graph, knhip_graph **out) {
+    return guarded([&] {
+        KN_REQUIRE(graph != nullptr && out != nullptr);
+        *out = new knhip_graph{graph->graph};
+        return KNHIP_OK;
+    });
+}
+
+void knhip_graph_free(knhip_graph *graph) { delete graph; }
+
+int knhip_graph_deserialize(const uint8_t *blob, size_t len, knhip_graph **out) {
+    return guarded([&] {
+        KN_REQUIRE(blob != nullptr && out != nullptr);
+        *out = new knhip_graph{Graph::deserialize(blob, len)};
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_serialize(const knhip_graph *graph, uint8_t *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(graph != nullptr);
+        std::vector<uint8_t> blob = graph->graph.serialize();
+        if (needed) *needed = blob.size();
+        if (buf == nullptr && cap == 0) return KNHIP_OK;
+        if (cap < blob.size()) {
+            g_last_error = "buffer too small";
+            return KNHIP_BUFFER_TOO_SMALL;
+        }
+        std::memcpy(buf, blob.data(), blob.size());
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_str(const knhip_graph *graph, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(graph != nullptr);
+        return copy_out(graph->graph.str(), buf, cap, needed);
+    });
+}
+
+#define KN_BUILD(expr)                          \
+    return guarded([&] {                        \
+        KN_REQUIRE(g != nullptr && out != nullptr); \
+        *out = (expr);                          \
+        return KNHIP_OK;                        \
+    })
+
+int knhip_graph_input(knhip_graph *g, const knhip_size_t *dims, size_t rank, int dtype, knhip_value *out) {
+    KN_BUILD(g->graph.input(to_shape(dims, rank), to_dtype(dtype)));
+}
+
+int knhip_graph_constant(knhip_graph *g, const knhip_size_t *dims, size_t rank, int dtype, const void *data,
+                         size_t data_bytes, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr);
+        Shape shape = to_shape(dims, rank);
+        DType dt = to_dtype(dtype);
+        ConcreteShape cs = shape.unwrap_fixed("constant shape");
+        if (data_bytes != concrete_size(cs) * dtype_bytes(dt))
+            fail("constant data has ", data_bytes, " bytes, shape ", shape.str(), " of ", dtype_name(dt), " needs ",
+                 concrete_size(cs) * dtype_bytes(dt));
+        KN_REQUIRE(data != nullptr || data_bytes == 0);
+        *out = g->graph.constant(shape, dt, data);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_view(knhip_graph *g, knhip_value input, const knhip_size_t *dims, size_t rank, knhip_value *out) {
+    KN_BUILD(g->graph.view(input, to_shape(dims, rank)));
+}
+int knhip_graph_broadcast(knhip_graph *g, knhip_value input, const knhip_size_t *dims, size_t rank, knhip_value *out) {
+    KN_BUILD(g->graph.broadcast(input, to_shape(dims, rank)));
+}
+int knhip_graph_repeat_unary(knhip_graph *g, knhip_value input, size_t axis, knhip_size_t count, knhip_value *out) {
+    KN_BUILD(g->graph.repeat_unary(input, axis, Size(count.batch_exp, count.fixed_factor)));
+}
+int knhip_graph_flatten(knhip_graph *g, knhip_value input, size_t start_axis, knhip_value *out) {
+    KN_BUILD(g->graph.flatten(input, start_axis));
+}
+int knhip_graph_permute(knhip_graph *g, knhip_value input, const size_t *permutation, size_t rank, knhip_value *out) {
+    KN_BUILD(g->graph.permute(input, std::vector<size_t>(permutation, permutation + rank)));
+}
+int knhip_graph_slice(knhip_graph *g, knhip_value input, size_t axis, size_t start, size_t end, size_t step, knhip_value *out) {
+    KN_BUILD(g->graph.slice(input, axis, SliceRange::make(start, end, step)));
+}
+int knhip_graph_index(knhip_graph *g, knhip_value input, size_t axis, size_t index, knhip_value *out) {
+    KN_BUILD(g->graph.index(input, axis, index));
+}
+int knhip_graph_flip(knhip_graph *g, knhip_value input, size_t axis, knhip_value *out) { KN_BUILD(g->graph.flip(input, axis)); }
+int knhip_graph_repeat(knhip_graph *g, knhip_value input, size_t axis, knhip_size_t count, int interleave, knhip_value *out) {
+    KN_BUILD(interleave ? g->graph.repeat_interleave(input, axis, Size(count.batch_exp, count.fixed_factor))
+                        : g->graph.repeat(input, axis, Size(count.batch_exp, count.fixed_factor)));
+}
+int knhip_graph_gather(knhip_graph *g, knhip_value input, size_t axis, knhip_value indices, knhip_value *out) {
+    KN_BUILD(g->graph.gather(input, axis, indices));
+}
+int knhip_graph_concat(knhip_graph *g, const knhip_value *inputs, size_t count, size_t axis, const knhip_size_t *base_dims,
+                       size_t base_rank, int dtype, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr && (inputs != nullptr || count == 0));
+        std::optional<Shape> base;
+        if (base_dims != nullptr) base = to_shape(base_dims, base_rank);
+        std::optional<DType> dt;
+        if (dtype >= 0) dt = to_dtype(dtype);
+        *out = g->graph.concat(std::vector<Value>(inputs, inputs + count), axis, base, dt);
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_pad(knhip_graph *g, knhip_value input, const size_t *pad_amount, size_t rank, knhip_value pad_value, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr && (pad_amount != nullptr || rank == 0));
+        std::vector<std::pair<size_t, size_t>> pads;
+        for (size_t i = 0; i < rank; i++) pads.push_back({pad_amount[2 * i], pad_amount[2 * i + 1]});
+        *out = g->graph.pad(input, pads, pad_value);
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_conv(knhip_graph *g, knhip_value input, knhip_value filter, size_t stride_y, size_t stride_x, size_t padding_y,
+                     size_t padding_x, knhip_value *out) {
+    KN_BUILD(g->graph.conv(input, filter, stride_y, stride_x, padding_y, padding_x));
+}
+int knhip_graph_linear(knhip_graph *g, knhip_value input, knhip_value weight, knhip_value *out) { KN_BUILD(g->graph.linear(input, weight)); }
+int knhip_graph_mat_mul(knhip_graph *g, knhip_value left, knhip_value right, knhip_value *out) { KN_BUILD(g->graph.mat_mul(left, right)); }
+int knhip_graph_batched_mat_mul(knhip_graph *g, knhip_value left, knhip_value right, knhip_value *out) {
+    KN_BUILD(g->graph.batched_mat_mul(left, right));
+}
+int knhip_graph_softmax(knhip_graph *g, knhip_value input, size_t axis, knhip_value *out) { KN_BUILD(g->graph.softmax(input, axis)); }
+int knhip_graph_layernorm(knhip_graph *g, knhip_value input, size_t axis, float eps, knhip_value *out) {
+    KN_BUILD(g->graph.layernorm(input, axis, eps));
+}
+int knhip_graph_reduce(knhip_graph *g, knhip_value input, const size_t *axes, size_t count, int op, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr && (axes != nullptr || count == 0));
+        if (op < 0 || op >= REDUCE_OP_COUNT) fail("invalid reduce op ", op);
+        *out = g->graph.reduce(input, std::vector<size_t>(axes, axes + count), (ReduceOp) op);
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_clamp(knhip_graph *g, knhip_value input, const void *min, const void *max, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr && min != nullptr && max != nullptr);
+        DType dt = g->graph[input].dtype;
+        *out = g->graph.clamp_dyn(input, DScalar::load(dt, min), DScalar::load(dt, max));
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_relu(knhip_graph *g, knhip_value input, knhip_value *out) { KN_BUILD(g->graph.relu(input)); }
+int knhip_graph_unary(knhip_graph *g, int op, int cast_dtype, knhip_value input, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr);
+        if (op < 0 || op >= UNARY_OP_COUNT) fail("invalid unary op ", op);
+        bool is_cast = op == KNHIP_UNARY_VALUE_CAST || op == KNHIP_UNARY_BIT_CAST;
+        DType to = is_cast ? to_dtype(cast_dtype) : DType::F32;
+        *out = g->graph.unary((UnaryOp) op, input, to);
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_binary(knhip_graph *g, int op, knhip_value left, knhip_value right, knhip_value *out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr);
+        if (op < 0 || op >= BINARY_OP_COUNT) fail("invalid binary op ", op);
+        *out = g->graph.binary((BinaryOp) op, left, right);
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_call(knhip_graph *g, const knhip_graph *callee, const knhip_value *inputs, size_t input_count,
+                     knhip_value *outputs, size_t output_cap, size_t *output_count) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && callee != nullptr && (inputs != nullptr || input_count == 0));
+        if (callee->graph.outputs.size() > output_cap) {
+            if (output_count) *output_count = callee->graph.outputs.size();
+            g_last_error = "buffer too small";
+            return KNHIP_BUFFER_TOO_SMALL;
+        }
+        std::vector<Value> r = g->graph.call(callee->graph, std::vector<Value>(inputs, inputs + input_count));
+        return copy_list(r, outputs, output_cap, output_count);
+    });
+}
+int knhip_graph_output(knhip_graph *g, knhip_value value) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr);
+        g->graph.output(value);
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_set_debug_id(knhip_graph *g, knhip_value value, const char *id) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && id != nullptr);
+        g->graph.set_debug_id(value, id);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_value_count(const knhip_graph *g, size_t *count) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && count != nullptr);
+        *count = g->graph.len();
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_inputs(const knhip_graph *g, knhip_value *buf, size_t cap, size_t *count) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr);
+        return copy_list(g->graph.inputs, buf, cap, count);
+    });
+}
+int knhip_graph_outputs(const knhip_graph *g, knhip_value *buf, size_t cap, size_t *count) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr);
+        return copy_list(g->graph.outputs, buf, cap, count);
+    });
+}
+int knhip_graph_value_info(const knhip_graph *g, knhip_value value, knhip_value_info *info) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && info != nullptr);
+        const ValueInfo &vi = g->graph[value];
+        const Operation &op = vi.operation;
+        std::memset(info, 0, sizeof *info);
+        info->dtype = (int) vi.dtype;
+        info->op = (int) op.kind;
+        info->sub_op = op.kind == OpKind::Unary ? (int) op.unary : op.kind == OpKind::Binary ? (int) op.binary
+                       : op.kind == OpKind::Reduce ? (int) op.reduce : -1;
+        bool is_cast = op.kind == OpKind::Unary && (op.unary == UnaryOp::ValueCast || op.unary == UnaryOp::BitCast);
+        info->cast_dtype = is_cast ? (int) op.cast_to : -1;
+        info->rank = vi.shape.rank();
+        info->operand_count = op.inputs.size();
+        info->axis_count = op.axes.size();
+        info->non_output_uses = vi.non_output_uses;
+        info->slice_start = op.range.start;
+        info->slice_end = op.range.end;
+        info->slice_step = op.range.step;
+        info->eps = op.eps;
+        info->is_hidden = g->graph.is_hidden(value) ? 1 : 0;
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_value_shape(const knhip_graph *g, knhip_value value, knhip_size_t *dims, size_t cap) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr);
+        const Shape &s = g->graph[value].shape;
+        if (cap < s.rank()) {
+            g_last_error = "buffer too small";
+            return KNHIP_BUFFER_TOO_SMALL;
+        }
+        for (size_t i = 0; i < s.rank(); i++) dims[i] = knhip_size_t{s.dims[i].fixed_factor, s.dims[i].batch_exp};
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_value_operands(const knhip_graph *g, knhip_value value, knhip_value *buf, size_t cap) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr);
+        return copy_list(g->graph[value].operation.inputs, buf, cap, (size_t *) nullptr);
+    });
+}
+int knhip_graph_value_axes(const knhip_graph *g, knhip_value value, size_t *buf, size_t cap) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr);
+        return copy_list(g->graph[value].operation.axes, buf, cap, (size_t *) nullptr);
+    });
+}
+int knhip_graph_value_constant(const knhip_graph *g, knhip_value value, const void **data, size_t *bytes) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && data != nullptr && bytes != nullptr);
+        const Operation &op = g->graph[value].operation;
+        if (op.kind != OpKind::Constant) fail("value ", value, " is not a constant");
+        *data = op.tensor.bytes();
+        *bytes = op.tensor.nbytes();
+        return KNHIP_OK;
+    });
+}
+int knhip_graph_as_single_const(const knhip_graph *g, knhip_value value, int *is_single, void *element) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && is_single != nullptr && element != nullptr);
+        auto c = g->graph.as_single_const(value);
+        *is_single = c.has_value() ? 1 : 0;
+        if (c) c->store(element);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_infer_batch_size(const knhip_graph *g, const size_t *actual, const size_t *ranks, size_t input_count,
+                                 int *status, int *has_batch, uint64_t *batch) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && status != nullptr && has_batch != nullptr && batch != nullptr);
+        KN_REQUIRE(input_count == 0 || (actual != nullptr && ranks != nullptr));
+        std::vector<ConcreteShape> shapes;
+        size_t pos = 0;
+        for (size_t i = 0; i < input_count; i++) {
+            shapes.push_back(ConcreteShape(actual + pos, actual + pos + ranks[i]));
+            pos += ranks[i];
+        }
+        std::optional<uint64_t> b;
+        *status = (int) infer_batch_size(g->graph.input_shapes(), shapes, &b);
+        *has_batch = b.has_value() ? 1 : 0;
+        *batch = b.value_or(0);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_optimizer_settings_default(knhip_optimizer_settings *settings) {
+    return guarded([&] {
+        KN_REQUIRE(settings != nullptr);
+        OptimizerSettings d;
+        *settings = knhip_optimizer_settings{d.optimize, d.force_bias_through_conv, d.fuse_layernorm, d.div_to_mul};
+        return KNHIP_OK;
+    });
+}
+
+int knhip_graph_optimize(const knhip_graph *g, const knhip_optimizer_settings *settings, knhip_graph **out) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && out != nullptr);
+        OptimizerSettings s;
+        if (settings) {
+            s.optimize = settings->optimize != 0;
+            s.force_bias_through_conv = settings->force_bias_through_conv != 0;
+            s.fuse_layernorm = settings->fuse_layernorm != 0;
+            s.div_to_mul = settings->div_to_mul != 0;
+        }
+        *out = new knhip_graph{optimize_graph(g->graph, s)};
+        return KNHIP_OK;
+    });
+}
+
+// ---------------------------------------------------------------------------------------------- executor
+
+int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int plan_only, knhip_executor **out) {
+    return guarded([&] {
+        KN_REQUIRE(graph != nullptr && out != nullptr);
+        *out = new knhip_executor(device, graph->graph, batch_size, plan_only != 0);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int plan_only,
+                                 knhip_executor **out) {
+    return guarded([&] {
+        KN_REQUIRE(blob != nullptr && out != nullptr);
+        Graph g = Graph::deserialize(blob, len);
+        *out = new knhip_executor(device, g, batch_size, plan_only != 0);
+        return KNHIP_OK;
+    });
+}
+
+void knhip_executor_free(knhip_executor *ex) {
+    try {
+        delete ex;
+    } catch (...) {
+    }
+}
+
+int knhip_executor_io_count(const knhip_executor *ex, size_t *inputs, size_t *outputs) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && inputs != nullptr && outputs != nullptr);
+        *inputs = ex->ex.plan().inputs.size();
+        *outputs = ex->ex.plan().outputs.size();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_io_info(const knhip_executor *ex, int is_output, size_t index, int *dtype, size_t *rank, size_t *dims, size_t cap) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && dtype != nullptr && rank != nullptr);
+        const auto &list = is_output ? ex->ex.plan().outputs : ex->ex.plan().inputs;
+        if (index >= list.size()) fail("index ", index, " out of range");
+        const PlanTensor &t = list[index];
+        *dtype = (int) t.dtype;
+        *rank = t.shape.rank();
+        if (dims == nullptr && cap == 0) return KNHIP_OK;
+        if (cap < t.shape.rank()) {
+            g_last_error = "buffer too small";
+            return KNHIP_BUFFER_TOO_SMALL;
+        }
+        for (size_t i = 0; i < t.shape.rank(); i++) dims[i] = t.shape.shape()[i];
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const size_t *input_bytes, size_t input_count,
+                            void *const *outputs, const size_t *output_bytes, size_t output_count) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        const Plan &plan = ex->ex.plan();
+        if (input_count != plan.inputs.size()) fail("Wrong input count: expected ", plan.inputs.size(), ", got ", input_count);
+        if (output_count != plan.outputs.size()) fail("Wrong output count: expected ", plan.outputs.size(), ", got ", output_count);
+        KN_REQUIRE(input_count == 0 || (inputs != nullptr && input_bytes != nullptr));
+        KN_REQUIRE(output_count == 0 || (outputs != nullptr && output_bytes != nullptr));
+        std::vector<HostTensor> in;
+        for (size_t i = 0; i < input_count; i++) {
+            const PlanTensor &t = plan.inputs[i];
+            size_t expected = t.shape.size() * dtype_bytes(t.dtype);
+            if (input_bytes[i] != expected) fail("Wrong size for input ", i, ": expected ", expected, " bytes, got ", input_bytes[i]);
+            KN_REQUIRE(inputs[i] != nullptr || expected == 0);
+            in.push_back(HostTensor(t.dtype, t.shape.shape(), inputs[i]));
+        }
+        for (size_t i = 0; i < output_count; i++) {
+            const PlanTensor &t = plan.outputs[i];
+            size_t expected = t.shape.size() * dtype_bytes(t.dtype);
+            if (output_bytes[i] != expected) fail("Wrong size for output ", i, ": expected ", expected, " bytes, got ", output_bytes[i]);
+            KN_REQUIRE(outputs[i] != nullptr || expected == 0);
+        }
+        const std::vector<HostTensor> &out = ex->ex.evaluate(in);
+        for (size_t i = 0; i < output_count; i++)
+            if (out[i].nbytes()) std::memcpy(outputs[i], out[i].bytes(), out[i].nbytes());
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_run_async(knhip_executor *ex) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        ex->ex.run_async();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_synchronize(knhip_executor *ex) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        ex->ex.synchronize();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_input_ptr(const knhip_executor *ex, size_t index, void **ptr) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && ptr != nullptr);
+        *ptr = ex->ex.input_ptr(index);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_output_ptr(const knhip_executor *ex, size_t index, void **ptr) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && ptr != nullptr);
+        *ptr = ex->ex.output_ptr(index);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_stream(const knhip_executor *ex, void **stream) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && stream != nullptr);
+        *stream = (void *) ex->ex.stream();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_set_profile(knhip_executor *ex, int enabled) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        ex->ex.set_profile(enabled != 0);
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_last_profile(const knhip_executor *ex, int *available, knhip_profile *profile) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && available != nullptr && profile != nullptr);
+        const auto &p = ex->ex.last_profile();
+        *available = p.has_value() ? 1 : 0;
+        std::memset(profile, 0, sizeof *profile);
+        if (p) {
+            for (int k = 0; k < STEP_KIND_COUNT; k++) profile->per_kind[k] = p->per_kind[k];
+            profile->total_cpu = p->total_cpu;
+            profile->total_gpu = p->total_gpu;
+            profile->timing_overhead = p->timing_overhead;
+            profile->step_count = p->step_seconds.size();
+        }
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_profile_step_seconds(const knhip_executor *ex, float *buf, size_t cap) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        const auto &p = ex->ex.last_profile();
+        if (!p) fail("no profile available");
+        return copy_list(p->step_seconds, buf, cap, (size_t *) nullptr);
+    });
+}
+
+int knhip_executor_profile_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        const auto &p = ex->ex.last_profile();
+        if (!p) fail("no profile available");
+        return copy_out(p->str(), buf, cap, needed);
+    });
+}
+
+int knhip_executor_mem_usage(const knhip_executor *ex, knhip_mem_usage *usage) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && usage != nullptr);
+        const Plan &p = ex->ex.plan();
+        *usage = knhip_mem_usage{p.mem_usage.dedicated_bytes, p.mem_usage.shared_bytes, p.mem_usage.zero_bytes,
+                                 p.mem_usage.hypo_shared_bytes_peak, p.mem_usage.hypo_shared_bytes_total, p.arena_bytes};
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_step_count(const knhip_executor *ex, size_t *count) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && count != nullptr);
+        *count = ex->ex.plan().steps.size();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_step_kind(const knhip_executor *ex, size_t index, int *kind) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && kind != nullptr);
+        *kind = (int) ex->ex.plan().steps.at(index).kind;
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        return copy_out(ex->ex.plan().steps.at(index).str(), buf, cap, needed);
+    });
+}
+
+int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        return copy_out(ex->ex.plan().steps.at(index).kernel.source, buf, cap, needed);
+    });
+}
+
+int knhip_executor_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        return copy_out(ex->ex.str(), buf, cap, needed);
+    });
+}
+
+int knhip_compile_stats(size_t *compiled, size_t *memory_hits, size_t *disk_hits) {
+    return guarded([&] {
+        KN_REQUIRE(compiled != nullptr && memory_hits != nullptr && disk_hits != nullptr);
+        CompileStats s = compile_stats();
+        *compiled = s.compiled;
+        *memory_hits = s.memory_hits;
+        *disk_hits = s.disk_hits;
+        return KNHIP_OK;
+    });
+}
+
+}  // extern "C"

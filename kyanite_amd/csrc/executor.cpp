@@ -1,0 +1,247 @@
+#include "executor.h"
+
+#include <chrono>
+#include <map>
+
+namespace kn {
+
+void hip_check(hipError_t e, const char *what) {
+    if (e != hipSuccess) fail("HIP failure in ", what, ": ", hipGetErrorName(e), " (", hipGetErrorString(e), ")");
+}
+
+int HipDevice::count() {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) return 0;
+    return n;
+}
+
+void HipDevice::check(int device) {
+    int n = count();
+    if (device < 0 || device >= n) fail("HIP device ", device, " is not available (", n, " device(s) visible)");
+}
+
+std::string HipDevice::name(int device) {
+    check(device);
+    hipDeviceProp_t prop;
+    hip_check(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties");
+    return std::string(prop.name) + " (" + prop.gcnArchName + ")";
+}
+
+std::string Profile::str() const {
+    std::ostringstream ss;
+    ss << "Profile {\n  steps: [\n";
+    for (auto &s : steps) ss << "    " << s << "\n";
+    ss << "  ]\n";
+    for (int k = 0; k < STEP_KIND_COUNT; k++) ss << "  " << step_kind_name((StepKind) k) << ": " << per_kind[k] << " s\n";
+    ss << "  total_cpu: " << total_cpu << " s\n  total_gpu: " << total_gpu << " s\n  timing_overhead: " << timing_overhead << " s\n}\n";
+    return ss.str();
+}
+
+HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only)
+    : device_(device), batch_size_(batch_size), plan_only_(plan_only) {
+    if (!plan_only) HipDevice::check(device);
+    PlannerOptions options;
+    plan_ = plan_graph(graph, batch_size, options);
+    for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
+    if (plan_only) return;
+
+    hip_check(hipSetDevice(device_), "hipSetDevice");
+    hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+    hip_check(hipMalloc((void **) &arena_, plan_.arena_bytes), "hipMalloc(arena)");
+    // constants are uploaded once; the shared region needs no initialisation
+    for (auto &up : plan_.uploads) {
+        if (up.tensor.nbytes() == 0) continue;
+        hip_check(hipMemcpy(arena_ + up.arena_offset, up.tensor.bytes(), up.tensor.nbytes(), hipMemcpyHostToDevice),
+                  "hipMemcpy(constant)");
+    }
+    // plan-time copies of the constants are not needed any more
+    plan_.uploads.clear();
+    plan_.uploads.shrink_to_fit();
+
+    // load every distinct code object once and resolve the launch arguments
+    std::map<uint64_t, hipModule_t> loaded;
+    launches_.resize(plan_.steps.size());
+    for (size_t si = 0; si < plan_.steps.size(); si++) {
+        Step &step = plan_.steps[si];
+        Launch &l = launches_[si];
+        for (auto &op : step.operands) l.ptrs.push_back(arena_ + plan_.resolve(op.tensor.ptr));
+        if (step.kind == StepKind::MatMul) {
+            step.gemm.a = (const float *) l.ptrs[0];
+            step.gemm.b = (const float *) l.ptrs[1];
+            step.gemm.c = (float *) l.ptrs[2];
+        } else if (step.kind == StepKind::Conv) {
+            size_t k = 0;
+            step.conv.input = (const float *) l.ptrs[k++];
+            step.conv.filter = (const float *) l.ptrs[k++];
+            step.conv.bias = step.conv_has_bias ? (const float *) l.ptrs[k++] : nullptr;
+            step.conv.res = step.conv_has_res ? (const float *) l.ptrs[k++] : nullptr;
+            step.conv.output = (float *) l.ptrs[k++];
+        } else {
+            KN_ASSERT(step.code != nullptr, "kernel was not compiled");
+            KN_ASSERT(l.ptrs.size() == step.kernel.n_ptrs);
+            auto it = loaded.find(step.code->key);
+            if (it == loaded.end()) {
+                hipModule_t module;
+                hip_check(hipModuleLoadData(&module, step.code->binary.data()), "hipModuleLoadData");
+                modules_.push_back(module);
+                it = loaded.emplace(step.code->key, module).first;
+            }
+            hip_check(hipModuleGetFunction(&l.function, it->second, step.kernel.name.c_str()), "hipModuleGetFunction");
+        }
+    }
+
+    for (auto &t : plan_.inputs) {
+        void *p = nullptr;
+        hip_check(hipHostMalloc(&p, std::max<size_t>(t.shape.size() * dtype_bytes(t.dtype), 1), hipHostMallocDefault), "hipHostMalloc");
+        pinned_inputs_.push_back(p);
+    }
+    for (auto &t : plan_.outputs) {
+        void *p = nullptr;
+        hip_check(hipHostMalloc(&p, std::max<size_t>(t.shape.size() * dtype_bytes(t.dtype), 1), hipHostMallocDefault), "hipHostMalloc");
+        pinned_outputs_.push_back(p);
+    }
+}
+
+HipExecutor::~HipExecutor() {
+    if (plan_only_) return;
+    hipSetDevice(device_);
+    if (stream_) hipStreamSynchronize(stream_);
+    for (void *p : pinned_inputs_) hipHostFree(p);
+    for (void *p : pinned_outputs_) hipHostFree(p);
+    for (hipModule_t m : modules_) hipModuleUnload(m);
+    if (arena_) hipFree(arena_);
+    if (stream_) hipStreamDestroy(stream_);
+}
+
+void *HipExecutor::input_ptr(size_t i) const {
+    KN_ASSERT(!plan_only_ && i < plan_.inputs.size());
+    return arena_ + plan_.resolve(plan_.inputs[i].ptr);
+}
+
+void *HipExecutor::output_ptr(size_t i) const {
+    KN_ASSERT(!plan_only_ && i < plan_.outputs.size());
+    return arena_ + plan_.resolve(plan_.outputs[i].ptr);
+}
+
+void HipExecutor::synchronize() {
+    KN_ASSERT(!plan_only_);
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+}
+
+void HipExecutor::launch_step(size_t index) {
+    Step &step = plan_.steps[index];
+    Launch &l = launches_[index];
+    switch (step.kind) {
+        case StepKind::MatMul: hip_check((hipError_t) launch_gemm_f32(step.gemm, stream_), "matmul launch"); break;
+        case StepKind::Conv: hip_check((hipError_t) launch_conv_f32(step.conv, stream_), "conv launch"); break;
+        default: {
+            void *args[] = {l.ptrs.data()};
+            hip_check(hipModuleLaunchKernel(l.function, step.kernel.grid, 1, 1, step.kernel.block, 1, 1, 0, stream_, args, nullptr),
+                      "hipModuleLaunchKernel");
+            break;
+        }
+    }
+}
+
+void HipExecutor::run_async() {
+    if (plan_only_) fail("this executor was created without a device and cannot run");
+    int current = -1;
+    hip_check(hipGetDevice(&current), "hipGetDevice");
+    if (current != device_) hip_check(hipSetDevice(device_), "hipSetDevice");
+
+    if (!profile_) {
+        for (size_t si = 0; si < plan_.steps.size(); si++) launch_step(si);
+        last_profile_ = std::nullopt;
+        return;
+    }
+
+    // executor.rs:208-257: one event pair per step
+    using clock = std::chrono::steady_clock;
+    size_t n = plan_.steps.size();
+    std::vector<hipEvent_t> events(2 * n + 2);
+    for (auto &e : events) hip_check(hipEventCreate(&e), "hipEventCreate");
+    hip_check(hipEventRecord(events[2 * n], stream_), "hipEventRecord");
+    hip_check(hipEventSynchronize(events[2 * n]), "hipEventSynchronize");
+    auto start_cpu = clock::now();
+    for (size_t si = 0; si < n; si++) {
+        hip_check(hipEventRecord(events[2 * si], stream_), "hipEventRecord");
+        launch_step(si);
+        hip_check(hipEventRecord(events[2 * si + 1], stream_), "hipEventRecord");
+    }
+    hip_check(hipEventRecord(events[2 * n + 1], stream_), "hipEventRecord");
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    auto end_cpu = clock::now();
+
+    Profile profile;
+    for (size_t si = 0; si < n; si++) {
+        float ms = 0;
+        hip_check(hipEventElapsedTime(&ms, events[2 * si], events[2 * si + 1]), "hipEventElapsedTime");
+        profile.per_kind[(int) plan_.steps[si].kind] += ms * 1e-3f;
+        profile.step_seconds.push_back(ms * 1e-3f);
+        char buf[64];
+        snprintf(buf, sizeof buf, "%4zu time %10.4f ms, step ", si, ms);
+        profile.steps.push_back(buf + plan_.steps[si].str());
+    }
+    float total_ms = 0;
+    hip_check(hipEventElapsedTime(&total_ms, events[2 * n], events[2 * n + 1]), "hipEventElapsedTime");
+    profile.total_gpu = total_ms * 1e-3f;
+    profile.total_cpu = std::chrono::duration<float>(end_cpu - start_cpu).count();
+    for (auto &e : events) hipEventDestroy(e);
+    profile.timing_overhead = std::chrono::duration<float>(clock::now() - end_cpu).count();
+    last_profile_ = std::move(profile);
+}
+
+const std::vector<HostTensor> &HipExecutor::evaluate(const std::vector<HostTensor> &inputs) {
+    if (plan_only_) fail("this executor was created without a device and cannot run");
+    if (inputs.size() != plan_.inputs.size()) fail("Wrong input count: expected ", plan_.inputs.size(), ", got ", inputs.size());
+    for (size_t i = 0; i < inputs.size(); i++) {
+        if (inputs[i].shape != plan_.inputs[i].shape.shape())
+            fail("Wrong shape for input ", i, ": expected ", vec_str(plan_.inputs[i].shape.shape()), ", got ", vec_str(inputs[i].shape));
+        if (inputs[i].dtype != plan_.inputs[i].dtype)
+            fail("Wrong dtype for input ", i, ": expected ", dtype_name(plan_.inputs[i].dtype), ", got ", dtype_name(inputs[i].dtype));
+    }
+    hip_check(hipSetDevice(device_), "hipSetDevice");
+    // make sure nothing else is still using the staging buffers
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    for (size_t i = 0; i < inputs.size(); i++) {
+        size_t bytes = inputs[i].nbytes();
+        if (bytes == 0) continue;
+        std::memcpy(pinned_inputs_[i], inputs[i].bytes(), bytes);
+        KN_ASSERT(plan_.inputs[i].shape.has_simple_strides());
+        hip_check(hipMemcpyAsync(input_ptr(i), pinned_inputs_[i], bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync(H2D)");
+    }
+    run_async();
+    for (size_t i = 0; i < plan_.outputs.size(); i++) {
+        size_t bytes = tensor_outputs_[i].nbytes();
+        if (bytes == 0) continue;
+        hip_check(hipMemcpyAsync(pinned_outputs_[i], output_ptr(i), bytes, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync(D2H)");
+    }
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    for (size_t i = 0; i < plan_.outputs.size(); i++) {
+        HostTensor &t = tensor_outputs_[i];
+        size_t bytes = t.nbytes();
+        if (bytes == 0) continue;
+        // outputs are handed out as shared tensors: never write into storage a caller may still hold
+        if (t.data.use_count() > 1) t = HostTensor(t.dtype, t.shape);
+        std::memcpy(t.bytes_mut(), pinned_outputs_[i], bytes);
+        if (t.dtype == DType::Bool) {
+            for (size_t k = 0; k < bytes; k++)
+                if (t.bytes()[k] > 1) fail("bool output ", i, " holds a value other than 0 or 1");
+        }
+    }
+    return tensor_outputs_;
+}
+
+std::string HipExecutor::str() const {
+    std::ostringstream ss;
+    ss << "HipExecutor {\n  device: " << device_ << ",\n  batch_size: " << batch_size_ << ",\n  arena_bytes: " << plan_.arena_bytes
+       << ",\n  mem_usage: { dedicated: " << plan_.mem_usage.dedicated_bytes << ", shared: " << plan_.mem_usage.shared_bytes
+       << ", zero: " << plan_.mem_usage.zero_bytes << ", hypo_peak: " << plan_.mem_usage.hypo_shared_bytes_peak
+       << ", hypo_total: " << plan_.mem_usage.hypo_shared_bytes_total << " },\n  steps: [\n";
+    for (auto &s : plan_.steps) ss << "    " << s.str() << "\n";
+    ss << "  ]\n}\n";
+    return ss.str();
+}
+
+}  // namespace kn

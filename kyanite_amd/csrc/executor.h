@@ -1,0 +1,76 @@
+// HipExecutor: the MI355X counterpart of CudaExecutor (kn-cuda-eval/src/executor.rs:20-37, :60-258).
+// new(device, graph, batch_size) plans the graph into one device arena; evaluate(inputs) copies the inputs in,
+// launches the planned steps in order on one stream and copies the outputs back.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include "planner.h"
+
+namespace kn {
+
+struct Profile {  // executor.rs:43-58
+    std::vector<std::string> steps;
+    std::vector<float> step_seconds;
+    float per_kind[STEP_KIND_COUNT] = {0};
+    float total_cpu = 0, total_gpu = 0, timing_overhead = 0;
+    std::string str() const;
+};
+
+class HipDevice {  // kn-cuda-sys/src/wrapper/handle.rs:37-103
+public:
+    static int count();
+    static void check(int device);  // fails when the device does not exist
+    static std::string name(int device);
+};
+
+class HipExecutor {
+public:
+    // `plan_only` builds and compiles the plan without touching a device (no allocation, no launches)
+    HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only = false);
+    ~HipExecutor();
+    HipExecutor(const HipExecutor &) = delete;
+    HipExecutor &operator=(const HipExecutor &) = delete;
+
+    // host tensors in, host tensors out; the returned tensors stay valid until the next call
+    const std::vector<HostTensor> &evaluate(const std::vector<HostTensor> &inputs);
+    // launch the steps on the executor's stream without any synchronisation (executor.rs:197-258)
+    void run_async();
+    void synchronize();
+
+    void set_profile(bool on) { profile_ = on; }
+    const std::optional<Profile> &last_profile() const { return last_profile_; }
+
+    int device() const { return device_; }
+    size_t batch_size() const { return batch_size_; }
+    const Plan &plan() const { return plan_; }
+    hipStream_t stream() const { return stream_; }
+    // device addresses of the (dense, row-major) input and output tensors
+    void *input_ptr(size_t i) const;
+    void *output_ptr(size_t i) const;
+    std::string str() const;
+
+private:
+    struct Launch {
+        hipFunction_t function = nullptr;
+        std::vector<void *> ptrs;
+    };
+    void launch_step(size_t index);
+
+    int device_;
+    size_t batch_size_;
+    bool plan_only_;
+    Plan plan_;
+    uint8_t *arena_ = nullptr;
+    hipStream_t stream_ = nullptr;
+    std::vector<hipModule_t> modules_;
+    std::vector<Launch> launches_;
+    std::vector<void *> pinned_inputs_, pinned_outputs_;
+    std::vector<HostTensor> tensor_outputs_;
+    bool profile_ = false;
+    std::optional<Profile> last_profile_;
+};
+
+void hip_check(hipError_t e, const char *what);
+
+}  // namespace kn

@@ -1,0 +1,958 @@
+#include "kernels.h"
+
+#include <cinttypes>
+
+namespace kn {
+
+// ------------------------------------------------------------------------------------------------ prelude
+
+const char *kernel_prelude() {
+    return R"KN(
+typedef signed char kn_i8; typedef short kn_i16; typedef int kn_i32; typedef long long kn_i64;
+typedef unsigned char kn_u8; typedef unsigned short kn_u16; typedef unsigned int kn_u32; typedef unsigned long long kn_u64;
+#define int8_t kn_i8
+#define int16_t kn_i16
+#define int32_t kn_i32
+#define int64_t kn_i64
+#define uint8_t kn_u8
+#define uint16_t kn_u16
+#define uint32_t kn_u32
+#define uint64_t kn_u64
+#define KN_DEV __device__ __forceinline__
+#define KN_INF (__builtin_inff())
+
+template<typename T, typename U> KN_DEV T kn_bit_cast(U v) {
+    static_assert(sizeof(T) == sizeof(U), "bit cast needs equal sizes");
+    T r; __builtin_memcpy(&r, &v, sizeof(T)); return r;
+}
+
+// round an f32 value to the nearest f16 value (ties to even) and back
+KN_DEV float kn_r16(float x) { return (float) (_Float16) x; }
+
+// Abramowitz-Stegun erf, evaluated in f64 exactly like the host reference does
+KN_DEV double kn_erf(double x) {
+    double s = (x != x) ? x : (__builtin_signbit(x) ? -1.0 : 1.0);
+    double a = __builtin_fabs(x);
+    double d = 1.0, p = a;
+    d += 0.0705230784 * p; p *= a;
+    d += 0.0422820123 * p; p *= a;
+    d += 0.0092705272 * p; p *= a;
+    d += 0.0001520143 * p; p *= a;
+    d += 0.0002765672 * p; p *= a;
+    d += 0.0000430638 * p;
+    double d2 = d * d, d4 = d2 * d2, d8 = d4 * d4, d16 = d8 * d8;
+    return s * (1.0 - 1.0 / d16);
+}
+
+// low 64 bits of the value converted to a 128 bit signed integer: truncation toward zero, saturation at the
+// 128 bit bounds, NaN gives 0. Narrower integer targets wrap from here.
+KN_DEV kn_u64 kn_f2i(double x) {
+    kn_u64 bits = kn_bit_cast<kn_u64>(x);
+    bool neg = (bits >> 63) != 0;
+    int exp = (int) ((bits >> 52) & 0x7ff);
+    kn_u64 mant = bits & 0xfffffffffffffull;
+    if (exp == 0x7ff) return (mant != 0) ? 0ull : (neg ? 0ull : ~0ull);
+    if (exp == 0) return 0ull;
+    mant |= 1ull << 52;
+    int e = exp - 1075;
+    kn_u64 low;
+    if (e >= 0) {
+        if (exp - 1023 >= 127) return neg ? 0ull : ~0ull;
+        low = e >= 64 ? 0ull : (mant << e);
+    } else {
+        low = (-e) >= 64 ? 0ull : (mant >> (-e));
+    }
+    return neg ? (0ull - low) : low;
+}
+
+template<typename T> KN_DEV T kn_shfl_xor(T v, int mask) {
+    if constexpr (sizeof(T) <= 4) {
+        int w = 0; __builtin_memcpy(&w, &v, sizeof(T));
+        w = __shfl_xor(w, mask, 64);
+        __builtin_memcpy(&v, &w, sizeof(T));
+        return v;
+    } else {
+        int w[2]; __builtin_memcpy(w, &v, 8);
+        w[0] = __shfl_xor(w[0], mask, 64);
+        w[1] = __shfl_xor(w[1], mask, 64);
+        __builtin_memcpy(&v, w, 8);
+        return v;
+    }
+}
+
+// butterfly reduction over aligned groups of G consecutive lanes (G a power of two, at most 64); every lane of
+// the group ends up with the result
+template<int G, typename T, typename F> KN_DEV T kn_group_reduce(T v, F f) {
+#pragma unroll
+    for (int m = G / 2; m > 0; m >>= 1) v = f(v, kn_shfl_xor(v, m));
+    return v;
+}
+
+// reduction over a whole workgroup of NW waves through LDS; every thread gets the result
+template<int NW, typename T, typename F> KN_DEV T kn_block_reduce(T v, F f, T *lds) {
+    v = kn_group_reduce<64>(v, f);
+    if constexpr (NW > 1) {
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+        __syncthreads();
+        v = lds[0];
+#pragma unroll
+        for (int w = 1; w < NW; w++) v = f(v, lds[w]);
+    }
+    return v;
+}
+)KN";
+}
+
+// ------------------------------------------------------------------------------------------------ small helpers
+
+namespace {
+
+// the type a value of this dtype has while it sits in registers
+const char *compute_type(DType t) {
+    switch (t) {
+        case DType::F16: return "float";
+        case DType::Bool: return "bool";
+        default: return dtype_c_name(t);
+    }
+}
+
+// the type used for loads and stores
+const char *storage_type(DType t) {
+    switch (t) {
+        case DType::Bool: return "uint8_t";
+        default: return dtype_c_name(t);
+    }
+}
+
+std::string from_storage(DType t, const std::string &e) {
+    if (t == DType::Bool) return "((" + e + ") != 0)";
+    if (t == DType::F16) return "((float) (" + e + "))";
+    return e;
+}
+
+std::string to_storage(DType t, const std::string &e) {
+    if (t == DType::Bool) return "((uint8_t) ((" + e + ") ? 1 : 0))";
+    if (t == DType::F16) return "((_Float16) (" + e + "))";
+    return e;
+}
+
+std::string i64_str(int64_t v) {
+    char buf[32];
+    snprintf(buf, sizeof buf, "%" PRId64, v);
+    return buf;
+}
+
+std::string int_array(const std::vector<int64_t> &v) {
+    std::string r = "{";
+    for (size_t i = 0; i < v.size(); i++) {
+        if (i) r += ", ";
+        r += i64_str(v[i]);
+    }
+    if (v.empty()) r += "0";
+    return r + "}";
+}
+
+std::string fn(bool is_f64, const char *name) { return is_f64 ? std::string(name) : std::string(name) + "f"; }
+
+std::string unary_expr(const ScalarNode &n, DType in, const std::string &x) {
+    bool d = in == DType::F64;
+    switch (n.unary) {
+        case UnaryOp::Abs:
+            if (dtype_is_float(in)) return fn(d, "__builtin_fabs") + "(" + x + ")";
+            // wrapping two's complement abs
+            return std::string("((") + dtype_c_name(in) + ") ((" + x + ") < 0 ? (0 - (uint64_t) (" + x + ")) : (uint64_t) (" + x + ")))";
+        case UnaryOp::Neg:
+            if (dtype_is_float(in)) return "(-(" + x + "))";
+            return std::string("((") + dtype_c_name(in) + ") (0 - (uint64_t) (" + x + ")))";
+        case UnaryOp::Sin: return fn(d, "sin") + "(" + x + ")";
+        case UnaryOp::Cos: return fn(d, "cos") + "(" + x + ")";
+        case UnaryOp::Exp: return fn(d, "exp") + "(" + x + ")";
+        case UnaryOp::Log: return fn(d, "log") + "(" + x + ")";
+        case UnaryOp::Sqrt: return fn(d, "sqrt") + "(" + x + ")";
+        case UnaryOp::Sigmoid:
+            return d ? "(1.0 / (1.0 + exp(-(" + x + "))))" : "(1.0f / (1.0f + expf(-(" + x + "))))";
+        case UnaryOp::Tanh: return fn(d, "tanh") + "(" + x + ")";
+        case UnaryOp::Erf: return d ? "kn_erf(" + x + ")" : "((float) kn_erf((double) (" + x + ")))";
+        case UnaryOp::Mish: return "((" + x + ") * " + fn(d, "tanh") + "(" + fn(d, "log1p") + "(" + fn(d, "exp") + "(" + x + "))))";
+        case UnaryOp::Softplus:
+            return "(" + fn(d, "log1p") + "(" + fn(d, "exp") + "(-" + fn(d, "__builtin_fabs") + "(" + x + "))) + " + fn(d, "fmax") + "(" + x + ", " + (d ? "0.0" : "0.0f") + "))";
+        case UnaryOp::ValueCast: {
+            DType to = n.cast_to;
+            if (to == DType::Bool) return "((" + x + ") != 0)";
+            if (in == DType::Bool) return std::string("((") + compute_type(to) + ") ((" + x + ") ? 1 : 0))";
+            if (dtype_is_float(in)) {
+                if (dtype_is_float(to)) return std::string("((") + compute_type(to) + ") (" + x + "))";
+                return std::string("((") + dtype_c_name(to) + ") kn_f2i((double) (" + x + ")))";
+            }
+            // integer source: floats go through f64 first, integers wrap
+            if (to == DType::F64) return "((double) (" + x + "))";
+            if (dtype_is_float(to)) return "((float) (double) (" + x + "))";
+            return std::string("((") + dtype_c_name(to) + ") (" + x + "))";
+        }
+        case UnaryOp::BitCast: {
+            // f16 values live in registers as float: go through the storage type
+            std::string src = in == DType::F16 ? "((_Float16) (" + x + "))" : x;
+            std::string r = std::string("kn_bit_cast<") + storage_type(n.cast_to) + ">(" + src + ")";
+            return n.cast_to == DType::F16 ? "((float) " + r + ")" : r;
+        }
+    }
+    fail("invalid unary op");
+}
+
+std::string binary_expr(BinaryOp op, DType t, const std::string &a, const std::string &b) {
+    if (t == DType::Bool) {
+        switch (op) {
+            case BinaryOp::Add: case BinaryOp::Max: return "((" + a + ") || (" + b + "))";
+            case BinaryOp::Mul: case BinaryOp::Min: return "((" + a + ") && (" + b + "))";
+            case BinaryOp::Sub: case BinaryOp::Div: return "((" + a + ") && !(" + b + "))";
+            default: fail("unsupported bool operation");
+        }
+    }
+    bool fl = dtype_is_float(t), d = t == DType::F64;
+    std::string T = dtype_c_name(t);
+    switch (op) {
+        case BinaryOp::Add: case BinaryOp::Sub: case BinaryOp::Mul: {
+            const char *sym = op == BinaryOp::Add ? "+" : op == BinaryOp::Sub ? "-" : "*";
+            if (fl) return "((" + a + ") " + sym + " (" + b + "))";
+            // wrap in unsigned arithmetic so that signed overflow is defined
+            return "((" + T + ") ((uint64_t) (" + a + ") " + sym + " (uint64_t) (" + b + ")))";
+        }
+        case BinaryOp::Div:
+            if (fl) return "((" + a + ") / (" + b + "))";
+            if (dtype_is_signed(t)) return "((" + b + ") == -1 ? (" + T + ") (0 - (uint64_t) (" + a + ")) : (" + T + ") ((" + a + ") / (" + b + ")))";
+            return "((" + T + ") ((" + a + ") / (" + b + ")))";
+        case BinaryOp::Min:
+            if (fl) return fn(d, "fmin") + "(" + a + ", " + b + ")";
+            return "((" + a + ") < (" + b + ") ? (" + a + ") : (" + b + "))";
+        case BinaryOp::Max:
+            if (fl) return fn(d, "fmax") + "(" + a + ", " + b + ")";
+            return "((" + a + ") > (" + b + ") ? (" + a + ") : (" + b + "))";
+        case BinaryOp::Pow:
+            if (!fl) fail("Pow is only supported for floats");
+            return fn(d, "pow") + "(" + a + ", " + b + ")";
+    }
+    fail("invalid binary op");
+}
+
+// Emit the statements of an expression. `load` names the already loaded register value for an operand.
+// Returns the name of the result variable.
+template <typename LoadName>
+std::string emit_expr(std::ostringstream &ss, const ScalarExpr &expr, const std::string &prefix, LoadName load,
+                      const char *indent = "    ") {
+    KN_ASSERT(!expr.nodes.empty());
+    for (size_t i = 0; i < expr.nodes.size(); i++) {
+        const ScalarNode &n = expr.nodes[i];
+        std::string name = prefix + std::to_string(i);
+        std::string rhs;
+        switch (n.kind) {
+            case ScalarNode::Load: rhs = load(n.operand); break;
+            case ScalarNode::Const: rhs = n.constant.to_c_str(); break;
+            case ScalarNode::Unary: rhs = unary_expr(n, expr.nodes[n.a].dtype, prefix + std::to_string(n.a)); break;
+            case ScalarNode::Binary:
+                rhs = binary_expr(n.binary, expr.nodes[n.a].dtype, prefix + std::to_string(n.a), prefix + std::to_string(n.b));
+                break;
+        }
+        // values of type f16 are kept as floats that are exactly representable in f16
+        if (n.dtype == DType::F16 && (n.kind == ScalarNode::Unary || n.kind == ScalarNode::Binary)) rhs = "kn_r16(" + rhs + ")";
+        ss << indent << "const " << compute_type(n.dtype) << " " << name << " = " << rhs << ";\n";
+    }
+    return prefix + std::to_string(expr.result());
+}
+
+// Axis bookkeeping shared by all kernels: drop unit axes, optionally order by the first operand's strides and
+// merge neighbours that are contiguous for every operand.
+struct Collapsed {
+    std::vector<size_t> shape;
+    std::vector<std::vector<int64_t>> strides;  // [operand][axis]
+    size_t rank() const { return shape.size(); }
+    size_t size() const { return concrete_size(shape); }
+};
+
+Collapsed collapse_axes(const std::vector<size_t> &shape, const std::vector<std::vector<int64_t>> &strides, bool reorder) {
+    size_t n_ops = strides.size();
+    std::vector<size_t> axes;
+    for (size_t a = 0; a < shape.size(); a++)
+        if (shape[a] != 1) axes.push_back(a);
+    if (reorder) {
+        std::stable_sort(axes.begin(), axes.end(),
+                         [&](size_t x, size_t y) { return std::llabs(strides[0][x]) > std::llabs(strides[0][y]); });
+    }
+    Collapsed c;
+    c.strides.resize(n_ops);
+    for (size_t a : axes) {
+        bool merged = false;
+        if (!c.shape.empty()) {
+            merged = true;
+            for (size_t k = 0; k < n_ops; k++)
+                merged &= c.strides[k].back() == strides[k][a] * (int64_t) shape[a];
+            if (merged) {
+                c.shape.back() *= shape[a];
+                for (size_t k = 0; k < n_ops; k++) c.strides[k].back() = strides[k][a];
+            }
+        }
+        if (!merged) {
+            c.shape.push_back(shape[a]);
+            for (size_t k = 0; k < n_ops; k++) c.strides[k].push_back(strides[k][a]);
+        }
+    }
+    return c;
+}
+
+bool fits_i32(const std::vector<KernelOperand> &ops, size_t total) {
+    if (total >= (1ull << 31)) return false;
+    for (auto &op : ops) {
+        auto [lo, hi] = op.shape.offset_bounds();
+        if (lo <= -(1ll << 31) || hi >= (1ll << 31)) return false;
+    }
+    return true;
+}
+
+// Emit code that splits `var` (a flat index over `dims`, last axis fastest) into per-operand offsets.
+// `offs[k]` are the names of the accumulators, which must already be declared.
+void emit_decompose(std::ostringstream &ss, const std::string &indent, const std::string &var,
+                    const std::vector<size_t> &dims, const std::vector<std::vector<int64_t>> &strides,
+                    const std::vector<std::string> &offs) {
+    size_t rank = dims.size();
+    if (rank == 0) return;
+    ss << indent << "{ idx_t kn_left = " << var << ";\n";
+    for (size_t a = rank; a-- > 0;) {
+        std::string c = "kn_c" + std::to_string(a);
+        if (a == 0) ss << indent << "  const idx_t " << c << " = kn_left;\n";
+        else {
+            ss << indent << "  const idx_t " << c << " = kn_left % (idx_t) " << dims[a] << "; kn_left /= (idx_t) " << dims[a] << ";\n";
+        }
+        for (size_t k = 0; k < offs.size(); k++)
+            if (strides[k][a] != 0) ss << indent << "  " << offs[k] << " += " << c << " * (idx_t) " << strides[k][a] << ";\n";
+    }
+    ss << indent << "}\n";
+}
+
+uint32_t ceil_div_u32(size_t a, size_t b) {
+    size_t r = (a + b - 1) / b;
+    if (r > 0x7fffffffull) fail("kernel grid too large: ", r);
+    return (uint32_t) r;
+}
+
+void emit_header(std::ostringstream &ss, bool idx64, size_t n_ptrs) {
+    ss << kernel_prelude();
+    ss << "typedef " << (idx64 ? "long long" : "int") << " idx_t;\n";
+    ss << "struct KnPtrs { void *p[" << std::max<size_t>(n_ptrs, 1) << "]; };\n";
+}
+
+std::string vec_type_decl(const std::string &name, DType t, size_t vec) {
+    return std::string("typedef ") + storage_type(t) + " " + name + " __attribute__((ext_vector_type(" + std::to_string(vec) + ")));\n";
+}
+
+// Largest power-of-two vector width (in elements) such that every operand can be accessed with aligned vectors
+// along the last collapsed axis. `inner_strides[k]` must be 0 or 1 for a width above one.
+size_t pick_vec(const std::vector<KernelOperand> &ops, const Collapsed &c, size_t inner_size) {
+    if (c.rank() == 0) return 1;
+    size_t max_bytes = 1;
+    for (auto &op : ops) max_bytes = std::max(max_bytes, dtype_bytes(op.dtype));
+    size_t vec = 16 / max_bytes;
+    size_t last = c.rank() - 1;
+    for (; vec > 1; vec /= 2) {
+        bool ok = inner_size % vec == 0;
+        for (size_t k = 0; k < ops.size() && ok; k++) {
+            int64_t is = c.strides[k][last];
+            if (is != 0 && is != 1) ok = false;
+            size_t es = dtype_bytes(ops[k].dtype);
+            if (is == 1) {
+                ok &= ops[k].offset_bytes % (int64_t) (vec * es) == 0;
+                for (size_t a = 0; a < last; a++) ok &= c.strides[k][a] % (int64_t) vec == 0;
+            }
+        }
+        if (ok) break;
+    }
+    return vec;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------ scalar kernel
+
+KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const ScalarExpr &expr) {
+    KN_ASSERT(!operands.empty());
+    const std::vector<size_t> &shape = operands[0].shape.shape();
+    std::vector<std::vector<int64_t>> strides;
+    for (auto &op : operands) {
+        KN_ASSERT(op.shape.shape() == shape, "all operands of an elementwise kernel must have the same shape");
+        strides.push_back(op.shape.strides());
+    }
+    KN_ASSERT(expr.nodes.back().dtype == operands[0].dtype);
+
+    KernelSpec spec;
+    spec.name = "kn_scalar";
+    spec.n_ptrs = operands.size();
+    spec.block = 256;
+    size_t total = concrete_size(shape);
+    if (total == 0) return spec;
+
+    Collapsed c = collapse_axes(shape, strides, true);
+    if (c.rank() == 0) {
+        c.shape = {1};
+        for (auto &s : c.strides) s = {1};
+    }
+    size_t rank = c.rank();
+    size_t inner = c.shape[rank - 1];
+    size_t vec = pick_vec(operands, c, inner);
+    size_t total_vecs = total / vec;
+    size_t unroll = total_vecs >= 256 * 4 * 1024 ? 4 : (total_vecs >= 256 * 2 * 512 ? 2 : 1);
+    bool idx64 = !fits_i32(operands, total + 256 * unroll);
+
+    std::ostringstream ss;
+    emit_header(ss, idx64, operands.size());
+    for (size_t k = 0; k < operands.size(); k++) {
+        ss << "typedef " << storage_type(operands[k].dtype) << " S" << k << ";\n";
+        if (vec > 1) ss << vec_type_decl("V" + std::to_string(k), operands[k].dtype, vec);
+    }
+    // the fused expression
+    ss << "KN_DEV " << compute_type(operands[0].dtype) << " kn_op(";
+    for (size_t k = 1; k < operands.size(); k++) ss << (k > 1 ? ", " : "") << compute_type(operands[k].dtype) << " x" << k;
+    ss << ") {\n";
+    std::string res = emit_expr(ss, expr, "y", [&](size_t operand) { return "x" + std::to_string(operand); });
+    ss << "    return " << res << ";\n}\n";
+
+    // dims in vector units along the last axis
+    std::vector<size_t> dims = c.shape;
+    dims[rank - 1] = inner / vec;
+    std::vector<std::vector<int64_t>> vstrides = c.strides;
+    for (auto &s : vstrides) s[rank - 1] *= (int64_t) vec;
+
+    ss << "#define UNROLL " << unroll << "\n#define VEC " << vec << "\n";
+    ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_scalar(KnPtrs ptrs) {\n";
+    for (size_t k = 0; k < operands.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
+    ss << "    const idx_t total = (idx_t) " << total_vecs << ";\n";
+    ss << "    const idx_t base = (idx_t) blockIdx.x * (idx_t) (256 * UNROLL) + (idx_t) threadIdx.x;\n";
+    ss << "    idx_t off[UNROLL][" << operands.size() << "];\n    bool ok[UNROLL];\n";
+    for (size_t k = 1; k < operands.size(); k++) {
+        bool vload = vec > 1 && c.strides[k][rank - 1] == 1;
+        ss << "    " << (vload ? "V" : "S") << k << " r" << k << "[UNROLL];\n";
+    }
+    // phase 1: addresses and loads, all issued before any arithmetic
+    ss << "#pragma unroll\n    for (int u = 0; u < UNROLL; u++) {\n";
+    ss << "        const idx_t v = base + (idx_t) (u * 256);\n        ok[u] = v < total;\n";
+    ss << "        for (int k = 0; k < " << operands.size() << "; k++) off[u][k] = 0;\n";
+    ss << "        if (ok[u]) {\n";
+    {
+        std::vector<std::string> offs;
+        for (size_t k = 0; k < operands.size(); k++) offs.push_back("off[u][" + std::to_string(k) + "]");
+        emit_decompose(ss, "            ", "v", dims, vstrides, offs);
+    }
+    for (size_t k = 1; k < operands.size(); k++) {
+        bool vload = vec > 1 && c.strides[k][rank - 1] == 1;
+        if (vload) ss << "            r" << k << "[u] = *(const V" << k << " *) (p" << k << " + off[u][" << k << "]);\n";
+        else ss << "            r" << k << "[u] = p" << k << "[off[u][" << k << "]];\n";
+    }
+    ss << "        }\n    }\n";
+    // phase 2: arithmetic and stores
+    ss << "#pragma unroll\n    for (int u = 0; u < UNROLL; u++) {\n        if (ok[u]) {\n";
+    if (vec > 1) {
+        ss << "            V0 out;\n#pragma unroll\n            for (int j = 0; j < VEC; j++) {\n";
+        ss << "                out[j] = " << to_storage(operands[0].dtype, [&] {
+            std::string call = "kn_op(";
+            for (size_t k = 1; k < operands.size(); k++) {
+                bool vload = c.strides[k][rank - 1] == 1;
+                std::string e = vload ? "r" + std::to_string(k) + "[u][j]" : "r" + std::to_string(k) + "[u]";
+                call += (k > 1 ? ", " : "") + from_storage(operands[k].dtype, e);
+            }
+            return call + ")";
+        }()) << ";\n            }\n";
+        int64_t os = c.strides[0][rank - 1];
+        if (os == 1) ss << "            *(V0 *) (p0 + off[u][0]) = out;\n";
+        else {
+            // output is not contiguous along the vector axis (never picked by pick_vec, kept for completeness)
+            ss << "#pragma unroll\n            for (int j = 0; j < VEC; j++) p0[off[u][0] + (idx_t) j * (idx_t) " << os << "] = out[j];\n";
+        }
+    } else {
+        std::string call = "kn_op(";
+        for (size_t k = 1; k < operands.size(); k++)
+            call += (k > 1 ? ", " : "") + from_storage(operands[k].dtype, "r" + std::to_string(k) + "[u]");
+        call += ")";
+        ss << "            p0[off[u][0]] = " << to_storage(operands[0].dtype, call) << ";\n";
+    }
+    ss << "        }\n    }\n}\n";
+
+    spec.source = ss.str();
+    spec.grid = ceil_div_u32(total_vecs, 256 * unroll);
+    std::ostringstream note;
+    note << "rank=" << rank << " vec=" << vec << " unroll=" << unroll << " idx=" << (idx64 ? 64 : 32);
+    spec.strategy = note.str();
+    return spec;
+}
+
+// ------------------------------------------------------------------------------------------------ reduce kernel
+
+KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
+                              ReduceOp rop) {
+    const auto &ishape = input.shape.shape();
+    DType dtype = input.dtype;
+    KN_ASSERT(output.dtype == dtype);
+
+    // split axes into kept and reduced
+    std::vector<size_t> kept_shape, red_shape;
+    std::vector<int64_t> kept_in, kept_out, red_in;
+    size_t out_axis = 0;
+    for (size_t a = 0; a < ishape.size(); a++) {
+        bool reduced = std::find(axes.begin(), axes.end(), a) != axes.end();
+        if (reduced) {
+            red_shape.push_back(ishape[a]);
+            red_in.push_back(input.shape.strides()[a]);
+        } else {
+            KN_ASSERT(out_axis < output.shape.rank() && output.shape.shape()[out_axis] == ishape[a]);
+            kept_shape.push_back(ishape[a]);
+            kept_in.push_back(input.shape.strides()[a]);
+            kept_out.push_back(output.shape.strides()[out_axis]);
+            out_axis++;
+        }
+    }
+    KN_ASSERT(out_axis == output.shape.rank());
+
+    KernelSpec spec;
+    spec.name = "kn_reduce";
+    spec.n_ptrs = 2;
+    size_t kept_size = concrete_size(kept_shape), red_size = concrete_size(red_shape);
+    if (kept_size == 0) return spec;
+
+    Collapsed kc = collapse_axes(kept_shape, {kept_out, kept_in}, true);
+    // the reduction order is free: iterate with the smallest stride innermost
+    Collapsed rc = collapse_axes(red_shape, {red_in}, true);
+
+    int64_t min_kept = INT64_MAX, min_red = INT64_MAX;
+    for (size_t a = 0; a < kc.rank(); a++) min_kept = std::min<int64_t>(min_kept, std::llabs(kc.strides[1][a]));
+    for (size_t a = 0; a < rc.rank(); a++) min_red = std::min<int64_t>(min_red, std::llabs(rc.strides[0][a]));
+    bool row = kc.rank() == 0 || rc.rank() == 0 || min_red <= min_kept;
+
+    std::vector<KernelOperand> both{input, output};
+    bool idx64 = !fits_i32(both, std::max(kept_size, red_size) + 4096);
+    size_t es = dtype_bytes(dtype);
+
+    const char *T = compute_type(dtype);
+    DScalar identity = reduce_identity(rop, dtype);
+    BinaryOp bop = rop == ReduceOp::Prod ? BinaryOp::Mul : rop == ReduceOp::Min ? BinaryOp::Min
+                   : rop == ReduceOp::Max ? BinaryOp::Max : BinaryOp::Add;
+
+    std::ostringstream ss;
+    emit_header(ss, idx64, 2);
+    ss << "typedef " << storage_type(dtype) << " S;\ntypedef " << T << " T;\n";
+    ss << "KN_DEV T kn_f(T a, T b) { return " << binary_expr(bop, dtype, "a", "b") << "; }\n";
+    ss << "KN_DEV T kn_identity() { return " << identity.to_c_str() << "; }\n";
+    ss << "KN_DEV T kn_post(T v) { return "
+       << (rop == ReduceOp::Mean ? "v / (float) " + std::to_string(red_size) + ".0f" : std::string("v")) << "; }\n";
+
+    std::ostringstream note;
+    if (row) {
+        // ---- a group of G lanes folds one output element, lanes stride over the (contiguous) reduced index
+        size_t vec = 1;
+        if (rc.rank() > 0 && rc.strides[0].back() == 1) {
+            for (vec = 16 / es; vec > 1; vec /= 2) {
+                bool ok = rc.shape.back() % vec == 0 && input.offset_bytes % (int64_t) (vec * es) == 0;
+                for (size_t a = 0; a + 1 < rc.rank(); a++) ok &= rc.strides[0][a] % (int64_t) vec == 0;
+                for (size_t a = 0; a < kc.rank(); a++) ok &= kc.strides[1][a] % (int64_t) vec == 0;
+                if (ok) break;
+            }
+        }
+        size_t red_vecs = red_size / vec;
+        size_t G = red_vecs >= 2048 ? 256 : red_vecs >= 128 ? 64 : red_vecs >= 16 ? 16 : 1;
+        size_t block = 256, rows_per_block = block / G;
+        size_t iters = (red_vecs + G - 1) / G;
+        std::vector<size_t> rdims = rc.shape;
+        std::vector<std::vector<int64_t>> rstrides = rc.strides;
+        if (rc.rank() > 0) {
+            rdims.back() /= vec;
+            rstrides[0].back() *= (int64_t) vec;
+        }
+        if (vec > 1) ss << vec_type_decl("V", dtype, vec);
+        ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_reduce(KnPtrs ptrs) {\n";
+        ss << "    const S *in = (const S *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
+        if (G == 256) ss << "    __shared__ T lds[4];\n";
+        ss << "    const idx_t row = (idx_t) blockIdx.x * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / " << G << ");\n";
+        ss << "    const idx_t lane = (idx_t) (threadIdx.x % " << G << ");\n";
+        if (G != 256) ss << "    if (row >= (idx_t) " << kept_size << ") return;\n";
+        ss << "    idx_t o_out = 0, o_in = 0;\n";
+        emit_decompose(ss, "    ", "row", kc.shape, kc.strides, {"o_out", "o_in"});
+        ss << "    T acc[4] = {kn_identity(), kn_identity(), kn_identity(), kn_identity()};\n";
+        ss << (iters <= 32 ? "#pragma unroll\n" : "#pragma unroll 8\n");
+        ss << "    for (idx_t i = 0; i < (idx_t) " << iters << "; i++) {\n";
+        ss << "        const idx_t r = lane + i * (idx_t) " << G << ";\n";
+        ss << "        if (r < (idx_t) " << red_vecs << ") {\n            idx_t o = o_in;\n";
+        emit_decompose(ss, "            ", "r", rdims, rstrides, {"o"});
+        if (vec > 1) {
+            ss << "            const V v = *(const V *) (in + o);\n#pragma unroll\n";
+            ss << "            for (int j = 0; j < " << vec << "; j++) acc[(i + j) & 3] = kn_f(acc[(i + j) & 3], " << from_storage(dtype, "v[j]") << ");\n";
+        } else {
+            ss << "            acc[i & 3] = kn_f(acc[i & 3], " << from_storage(dtype, "in[o]") << ");\n";
+        }
+        ss << "        }\n    }\n";
+        ss << "    T total = kn_f(kn_f(acc[0], acc[1]), kn_f(acc[2], acc[3]));\n";
+        if (G == 256) ss << "    total = kn_block_reduce<4>(total, kn_f, lds);\n";
+        else if (G > 1) ss << "    total = kn_group_reduce<" << G << ">(total, kn_f);\n";
+        ss << "    if (lane == 0) out[o_out] = " << to_storage(dtype, "kn_post(total)") << ";\n}\n";
+        spec.block = (uint32_t) block;
+        spec.grid = ceil_div_u32(kept_size, rows_per_block);
+        note << "row G=" << G << " vec=" << vec << " iters=" << iters;
+    } else {
+        // ---- every thread owns VEC neighbouring kept elements and walks the reduced index; TY slices of the
+        // reduction run side by side and are combined through LDS
+        size_t vec = 1;
+        if (kc.strides[1].back() == 1 && kc.strides[0].back() == 1) {
+            for (vec = 16 / es; vec > 1; vec /= 2) {
+                bool ok = kc.shape.back() % vec == 0 && input.offset_bytes % (int64_t) (vec * es) == 0 &&
+                          output.offset_bytes % (int64_t) (vec * es) == 0;
+                for (size_t a = 0; a + 1 < kc.rank(); a++)
+                    ok &= kc.strides[0][a] % (int64_t) vec == 0 && kc.strides[1][a] % (int64_t) vec == 0;
+                for (size_t a = 0; a < rc.rank(); a++) ok &= rc.strides[0][a] % (int64_t) vec == 0;
+                if (ok) break;
+            }
+        }
+        size_t kept_vecs = kept_size / vec;
+        size_t TX = 64;
+        while (TX > 1 && TX / 2 >= kept_vecs) TX /= 2;
+        size_t TY = 256 / TX;
+        while (TY > 1 && TY > red_size) TY /= 2;
+        // with plenty of independent outputs there is no need to split the reduction
+        if (kept_vecs >= 256 * 1024) { TX = 256; TY = 1; }
+        size_t block = TX * TY;
+        std::vector<size_t> kdims = kc.shape;
+        std::vector<std::vector<int64_t>> kstrides = kc.strides;
+        kdims.back() /= vec;
+        kstrides[0].back() *= (int64_t) vec;
+        kstrides[1].back() *= (int64_t) vec;
+        if (vec > 1) ss << vec_type_decl("V", dtype, vec);
+        ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void kn_reduce(KnPtrs ptrs) {\n";
+        ss << "    const S *in = (const S *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
+        if (TY > 1) ss << "    __shared__ T lds[" << TY << "][" << vec << "][" << TX << "];\n";
+        ss << "    const idx_t tx = (idx_t) (threadIdx.x % " << TX << "), ty = (idx_t) (threadIdx.x / " << TX << ");\n";
+        ss << "    const idx_t kv = (idx_t) blockIdx.x * (idx_t) " << TX << " + tx;\n";
+        ss << "    const bool valid = kv < (idx_t) " << kept_vecs << ";\n";
+        ss << "    idx_t o_out = 0, o_in = 0;\n";
+        ss << "    T acc[" << vec << "];\n    for (int j = 0; j < " << vec << "; j++) acc[j] = kn_identity();\n";
+        ss << "    if (valid) {\n";
+        emit_decompose(ss, "        ", "kv", kdims, kstrides, {"o_out", "o_in"});
+        ss << "#pragma unroll 4\n        for (idx_t r = ty; r < (idx_t) " << red_size << "; r += (idx_t) " << TY << ") {\n            idx_t o = o_in;\n";
+        emit_decompose(ss, "            ", "r", rc.shape, rc.strides, {"o"});
+        if (vec > 1) {
+            ss << "            const V v = *(const V *) (in + o);\n#pragma unroll\n";
+            ss << "            for (int j = 0; j < " << vec << "; j++) acc[j] = kn_f(acc[j], " << from_storage(dtype, "v[j]") << ");\n";
+        } else {
+            ss << "            acc[0] = kn_f(acc[0], " << from_storage(dtype, "in[o]") << ");\n";
+        }
+        ss << "        }\n    }\n";
+        if (TY > 1) {
+            ss << "    for (int j = 0; j < " << vec << "; j++) lds[ty][j][tx] = acc[j];\n    __syncthreads();\n";
+            ss << "    if (ty == 0 && valid) {\n        for (int j = 0; j < " << vec << "; j++) {\n            T t = lds[0][j][tx];\n";
+            ss << "            for (int s = 1; s < " << TY << "; s++) t = kn_f(t, lds[s][j][tx]);\n            acc[j] = t;\n        }\n";
+        } else {
+            ss << "    if (valid) {\n";
+        }
+        if (vec > 1) {
+            ss << "        V o;\n        for (int j = 0; j < " << vec << "; j++) o[j] = " << to_storage(dtype, "kn_post(acc[j])") << ";\n";
+            ss << "        *(V *) (out + o_out) = o;\n";
+        } else {
+            ss << "        out[o_out] = " << to_storage(dtype, "kn_post(acc[0])") << ";\n";
+        }
+        ss << "    }\n}\n";
+        spec.block = (uint32_t) block;
+        spec.grid = ceil_div_u32(kept_vecs, TX);
+        note << "col TX=" << TX << " TY=" << TY << " vec=" << vec;
+    }
+    spec.source = ss.str();
+    spec.strategy = note.str();
+    return spec;
+}
+
+// ------------------------------------------------------------------------------------------------ row kernels
+
+KernelSpec make_row_kernel(const RowKernelDesc &desc) {
+    const auto &ops = desc.operands;
+    KN_ASSERT(ops.size() >= 2);
+    const auto &shape = ops[0].shape.shape();
+    size_t axis = desc.axis;
+    KN_ASSERT(axis < shape.size());
+    size_t size = shape[axis];
+
+    std::vector<size_t> static_shape;
+    std::vector<std::vector<int64_t>> static_strides(ops.size());
+    std::vector<int64_t> axis_strides;
+    for (size_t k = 0; k < ops.size(); k++) {
+        KN_ASSERT(ops[k].shape.shape() == shape, "all operands of a row kernel must have the same shape");
+        axis_strides.push_back(ops[k].shape.strides()[axis]);
+    }
+    for (size_t a = 0; a < shape.size(); a++) {
+        if (a == axis) continue;
+        static_shape.push_back(shape[a]);
+        for (size_t k = 0; k < ops.size(); k++) static_strides[k].push_back(ops[k].shape.strides()[a]);
+    }
+
+    bool softmax = desc.kind == RowKernelDesc::Softmax;
+    KernelSpec spec;
+    spec.name = "kn_row";
+    spec.n_ptrs = ops.size();
+    size_t static_size = concrete_size(static_shape);
+    if (static_size == 0 || size == 0) return spec;
+
+    Collapsed sc = collapse_axes(static_shape, static_strides, true);
+
+    // vector width along the normalised axis
+    size_t max_bytes = 1;
+    for (auto &op : ops) max_bytes = std::max(max_bytes, dtype_bytes(op.dtype));
+    size_t vec = 16 / max_bytes;
+    for (; vec > 1; vec /= 2) {
+        bool ok = size % vec == 0;
+        for (size_t k = 0; k < ops.size() && ok; k++) {
+            int64_t as = axis_strides[k];
+            if (as != 0 && as != 1) ok = false;
+            if (k == 0 && as != 1) ok = false;
+            if (as == 1) {
+                size_t es = dtype_bytes(ops[k].dtype);
+                ok &= ops[k].offset_bytes % (int64_t) (vec * es) == 0;
+                for (size_t a = 0; a < sc.rank(); a++) ok &= sc.strides[k][a] % (int64_t) vec == 0;
+            }
+        }
+        if (ok) break;
+    }
+    size_t nv = size / vec;
+    // G lanes share a row; the row stays in registers when every lane holds at most MAX_ITEMS vectors
+    const size_t MAX_ITEMS = 16;
+    size_t G = 1024;
+    for (size_t g : {1, 4, 16, 64, 256, 1024}) {
+        size_t per_lane = (nv + g - 1) / g;
+        if (per_lane <= (g >= 256 ? (g == 1024 ? MAX_ITEMS : 8) : (g == 1 ? 2 : 4))) {
+            G = g;
+            break;
+        }
+    }
+    size_t items = (nv + G - 1) / G;
+    bool cached = items <= MAX_ITEMS;
+    size_t block = std::max<size_t>(G, 256);
+    size_t rows_per_block = block / G;
+    size_t nw = G / 64;  // waves per row when a row spans several waves
+    bool idx64 = !fits_i32(ops, std::max(static_size, size) + 4096);
+
+    std::ostringstream ss;
+    emit_header(ss, idx64, ops.size());
+    for (size_t k = 0; k < ops.size(); k++) {
+        ss << "typedef " << storage_type(ops[k].dtype) << " S" << k << ";\n";
+        if (vec > 1) ss << vec_type_decl("V" + std::to_string(k), ops[k].dtype, vec);
+    }
+    // which operands feed the prologue / epilogue
+    std::vector<bool> in_pre(ops.size(), false), in_post(ops.size(), false);
+    for (auto &n : desc.pre.nodes)
+        if (n.kind == ScalarNode::Load) in_pre.at(n.operand) = true;
+    for (auto &n : desc.post.nodes)
+        if (n.kind == ScalarNode::Load && n.operand != SIZE_MAX) in_post.at(n.operand) = true;
+
+    auto emit_fn = [&](const char *name, const ScalarExpr &expr, const std::vector<bool> &used, bool with_norm, DType result) {
+        ss << "KN_DEV " << compute_type(result) << " " << name << "(";
+        bool first = true;
+        if (with_norm) {
+            ss << "float xn";
+            first = false;
+        }
+        for (size_t k = 1; k < ops.size(); k++) {
+            if (!used[k]) continue;
+            ss << (first ? "" : ", ") << compute_type(ops[k].dtype) << " x" << k;
+            first = false;
+        }
+        ss << ") {\n";
+        std::string res = emit_expr(ss, expr, "y", [&](size_t operand) {
+            return operand == SIZE_MAX ? std::string("xn") : "x" + std::to_string(operand);
+        });
+        ss << "    return " << res << ";\n}\n";
+    };
+    KN_ASSERT(desc.pre.nodes.back().dtype == DType::F32);
+    KN_ASSERT(desc.post.nodes.back().dtype == ops[0].dtype);
+    emit_fn("kn_pre", desc.pre, in_pre, false, DType::F32);
+    emit_fn("kn_post", desc.post, in_post, true, ops[0].dtype);
+
+    ss << "#define VEC " << vec << "\n#define ITEMS " << items << "\n#define G " << G << "\n";
+    ss << "KN_DEV float kn_max(float a, float b) { return fmaxf(a, b); }\nKN_DEV float kn_add(float a, float b) { return a + b; }\n";
+    ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void kn_row(KnPtrs ptrs) {\n";
+    for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
+    if (nw > 1) ss << "    __shared__ float lds[" << nw << "];\n";
+    ss << "    const idx_t row = (idx_t) blockIdx.x * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / G);\n";
+    ss << "    const idx_t lane = (idx_t) (threadIdx.x % G);\n";
+    if (nw <= 1) ss << "    if (row >= (idx_t) " << static_size << ") return;\n";
+    ss << "    idx_t base[" << ops.size() << "];\n    for (int k = 0; k < " << ops.size() << "; k++) base[k] = 0;\n";
+    {
+        std::vector<std::string> offs;
+        for (size_t k = 0; k < ops.size(); k++) offs.push_back("base[" + std::to_string(k) + "]");
+        emit_decompose(ss, "    ", "row", sc.shape, sc.strides, offs);
+    }
+    // the reduction helper: over G lanes of a wave, or over the waves of the workgroup
+    auto reduce = [&](const std::string &var, const char *f) {
+        if (G == 1) return;
+        if (nw > 1) ss << "    " << var << " = kn_block_reduce<" << nw << ">(" << var << ", " << f << ", lds);\n";
+        else ss << "    " << var << " = kn_group_reduce<G>(" << var << ", " << f << ");\n";
+    };
+    // load one vector position `i` (in vector units along the axis) and run the prologue on it
+    auto emit_load_pre = [&](const std::string &indent, const std::string &i, const std::string &dst) {
+        for (size_t k = 1; k < ops.size(); k++) {
+            if (!in_pre[k]) continue;
+            std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
+            if (vec > 1 && axis_strides[k] == 1) ss << indent << "const V" << k << " a" << k << " = *(const V" << k << " *) (p" << k << " + " << o << ");\n";
+            else ss << indent << "const S" << k << " a" << k << " = p" << k << "[" << o << "];\n";
+        }
+        ss << indent << "for (int j = 0; j < VEC; j++) " << dst << "[j] = kn_pre(";
+        bool first = true;
+        for (size_t k = 1; k < ops.size(); k++) {
+            if (!in_pre[k]) continue;
+            std::string e = (vec > 1 && axis_strides[k] == 1) ? "a" + std::to_string(k) + "[j]" : "a" + std::to_string(k);
+            ss << (first ? "" : ", ") << from_storage(ops[k].dtype, e);
+            first = false;
+        }
+        ss << ");\n";
+    };
+    // run the epilogue on normalised values `src[j]` of vector position `i` and store
+    auto emit_post_store = [&](const std::string &indent, const std::string &i, const std::string &src) {
+        for (size_t k = 1; k < ops.size(); k++) {
+            if (!in_post[k]) continue;
+            std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
+            if (vec > 1 && axis_strides[k] == 1) ss << indent << "const V" << k << " b" << k << " = *(const V" << k << " *) (p" << k << " + " << o << ");\n";
+            else ss << indent << "const S" << k << " b" << k << " = p" << k << "[" << o << "];\n";
+        }
+        std::string o0 = "(base[0] + " + i + " * (idx_t) " + i64_str(axis_strides[0] * (int64_t) vec) + ")";
+        auto call = [&](const std::string &j) {
+            std::string c = "kn_post(" + src + "[" + j + "]";
+            for (size_t k = 1; k < ops.size(); k++) {
+                if (!in_post[k]) continue;
+                std::string e = (vec > 1 && axis_strides[k] == 1) ? "b" + std::to_string(k) + "[" + j + "]" : "b" + std::to_string(k);
+                c += ", " + from_storage(ops[k].dtype, e);
+            }
+            return to_storage(ops[0].dtype, c + ")");
+        };
+        if (vec > 1) {
+            ss << indent << "V0 o;\n" << indent << "for (int j = 0; j < VEC; j++) o[j] = " << call("j") << ";\n";
+            ss << indent << "*(V0 *) (p0 + " << o0 << ") = o;\n";
+        } else {
+            ss << indent << "p0[" << o0 << "] = " << call("0") << ";\n";
+        }
+    };
+
+    const std::string valid = nw > 1 ? std::string("(row < (idx_t) ") + std::to_string(static_size) + ")" : std::string("true");
+    if (cached) {
+        ss << "    float x[ITEMS][VEC];\n";
+        ss << "    float m = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
+        ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
+        ss << "        if (i < (idx_t) " << nv << " && " << valid << ") {\n";
+        emit_load_pre("            ", "i", "x[it]");
+        if (softmax) ss << "            for (int j = 0; j < VEC; j++) m = fmaxf(m, x[it][j]);\n";
+        else ss << "            for (int j = 0; j < VEC; j++) m += x[it][j];\n";
+        ss << "        } else {\n            for (int j = 0; j < VEC; j++) x[it][j] = " << (softmax ? "-KN_INF" : "0.0f") << ";\n        }\n    }\n";
+        reduce("m", softmax ? "kn_max" : "kn_add");
+        ss << "    float s = 0.0f;\n";
+        if (softmax) {
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
+            ss << "        for (int j = 0; j < VEC; j++) {\n            const float e = (i < (idx_t) " << nv << ") ? expf(x[it][j] - m) : 0.0f;\n";
+            ss << "            x[it][j] = e;\n            s += e;\n        }\n    }\n";
+            reduce("s", "kn_add");
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / s;\n    }\n";
+        } else {
+            ss << "    const float mean = m / (float) " << size << ".0f;\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
+            ss << "        for (int j = 0; j < VEC; j++) {\n            const float d = (i < (idx_t) " << nv << ") ? (x[it][j] - mean) : 0.0f;\n";
+            ss << "            x[it][j] = d;\n            s += d * d;\n        }\n    }\n";
+            reduce("s", "kn_add");
+            ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / denom;\n    }\n";
+        }
+        ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
+        ss << "        if (i < (idx_t) " << nv << " && " << valid << ") {\n";
+        emit_post_store("            ", "i", "x[it]");
+        ss << "        }\n    }\n}\n";
+    } else {
+        // rows too long for registers: stream the row three times (the re-reads come from cache)
+        ss << "    float t[VEC];\n";
+        ss << "    float m = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
+        ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
+        emit_load_pre("        ", "i", "t");
+        if (softmax) ss << "        for (int j = 0; j < VEC; j++) m = fmaxf(m, t[j]);\n";
+        else ss << "        for (int j = 0; j < VEC; j++) m += t[j];\n";
+        ss << "    }\n";
+        reduce("m", softmax ? "kn_max" : "kn_add");
+        if (!softmax) ss << "    const float mean = m / (float) " << size << ".0f;\n";
+        ss << "    float s = 0.0f;\n";
+        ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
+        emit_load_pre("        ", "i", "t");
+        if (softmax) ss << "        for (int j = 0; j < VEC; j++) s += expf(t[j] - m);\n";
+        else ss << "        for (int j = 0; j < VEC; j++) { const float d = t[j] - mean; s += d * d; }\n";
+        ss << "    }\n";
+        reduce("s", "kn_add");
+        if (!softmax) ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
+        ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
+        emit_load_pre("        ", "i", "t");
+        if (softmax) ss << "        for (int j = 0; j < VEC; j++) t[j] = expf(t[j] - m) / s;\n";
+        else ss << "        for (int j = 0; j < VEC; j++) t[j] = (t[j] - mean) / denom;\n";
+        emit_post_store("        ", "i", "t");
+        ss << "    }\n}\n";
+    }
+
+    spec.source = ss.str();
+    spec.block = (uint32_t) block;
+    spec.grid = ceil_div_u32(static_size, rows_per_block);
+    std::ostringstream note;
+    note << (softmax ? "softmax" : "layernorm") << " G=" << G << " vec=" << vec << " items=" << items << (cached ? " cached" : " streamed");
+    spec.strategy = note.str();
+    return spec;
+}
+
+// ------------------------------------------------------------------------------------------------ gather kernel
+
+KernelSpec make_gather_kernel(const KernelOperand &input, const KernelOperand &indices, const KernelOperand &output,
+                              size_t axis) {
+    KN_ASSERT(indices.shape.rank() == 1);
+    KN_ASSERT(input.dtype == output.dtype);
+    const auto &ishape = input.shape.shape();
+    const auto &oshape = output.shape.shape();
+    KN_ASSERT(ishape.size() == oshape.size() && axis < ishape.size());
+    size_t n_idx = indices.shape.shape()[0];
+    KN_ASSERT(oshape[axis] == n_idx);
+
+    KernelSpec spec;
+    spec.name = "kn_gather";
+    spec.n_ptrs = 3;
+    spec.block = 256;
+    size_t total = concrete_size(oshape);
+    if (total == 0) return spec;
+
+    // iterate in output order: all output axes, the gathered one included
+    std::vector<std::vector<int64_t>> strides(3);
+    for (size_t a = 0; a < oshape.size(); a++) {
+        strides[0].push_back(output.shape.strides()[a]);
+        strides[1].push_back(a == axis ? 0 : input.shape.strides()[a]);
+        strides[2].push_back(a == axis ? indices.shape.strides()[0] : 0);
+    }
+    Collapsed c = collapse_axes(oshape, strides, true);
+    if (c.rank() == 0) {
+        c.shape = {1};
+        for (auto &s : c.strides) s = {0};
+    }
+    std::vector<KernelOperand> all{input, indices, output};
+    bool idx64 = !fits_i32(all, total + 4096);
+
+    std::ostringstream ss;
+    emit_header(ss, idx64, 3);
+    ss << "typedef " << storage_type(input.dtype) << " S;\ntypedef " << dtype_c_name(indices.dtype) << " I;\n";
+    ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_gather(KnPtrs ptrs) {\n";
+    ss << "    const S *in = (const S *) ptrs.p[0];\n    const I *indices = (const I *) ptrs.p[1];\n    S *out = (S *) ptrs.p[2];\n";
+    ss << "    const idx_t flat = (idx_t) blockIdx.x * 256 + (idx_t) threadIdx.x;\n";
+    ss << "    if (flat >= (idx_t) " << total << ") return;\n";
+    ss << "    idx_t o_out = 0, o_in = 0, o_idx = 0;\n";
+    emit_decompose(ss, "    ", "flat", c.shape, c.strides, {"o_out", "o_in", "o_idx"});
+    ss << "    const I index = indices[o_idx];\n";
+    ss << "    S value = 0;\n";
+    if (dtype_is_signed(indices.dtype))
+        ss << "    if (index >= 0 && (unsigned long long) index < " << ishape[axis] << "ull)";
+    else
+        ss << "    if ((unsigned long long) index < " << ishape[axis] << "ull)";
+    ss << " value = in[o_in + (idx_t) index * (idx_t) " << input.shape.strides()[axis] << "];\n";
+    ss << "    out[o_out] = value;\n}\n";
+
+    spec.source = ss.str();
+    spec.grid = ceil_div_u32(total, 256);
+    spec.strategy = "rank=" + std::to_string(c.rank());
+    return spec;
+}
+
+}  // namespace kn

@@ -1,0 +1,76 @@
+// Generators for the run-time compiled gfx950 kernels ("autokernels"): fused elementwise chains / strided copy,
+// reduce, softmax, layernorm and gather. They take the role of kn-cuda-eval/src/autokernel/{scalar,reduce,softmax,
+// layernorm,gather}.rs + the matching .cu templates, but the device code is new and written for CDNA4:
+// wave64 shuffles, 128-bit accesses on the contiguous axis, rows held in registers so HBM is touched once per
+// element, and all index arithmetic against compile-time constants.
+#pragma once
+
+#include "strided_shape.h"
+
+namespace kn {
+
+// A kernel ready to be compiled: every shape, stride and expression is baked into `source`; the only launch
+// arguments are the operand base addresses, in `operands` order.
+struct KernelSpec {
+    std::string name;    // entry point
+    std::string source;  // complete translation unit
+    uint32_t grid = 0;   // number of workgroups; 0 means nothing to do
+    uint32_t block = 0;  // threads per workgroup
+    size_t n_ptrs = 0;
+    std::string strategy;  // human readable note on the specialisation that was picked
+};
+
+// One node of a fused elementwise expression: operands are loaded (`Load`), single-valued constants are inlined
+// (`Const`), everything else refers to earlier nodes.
+struct ScalarNode {
+    enum Kind { Load, Const, Unary, Binary } kind = Load;
+    DType dtype = DType::F32;  // type of the produced value
+    size_t operand = 0;        // Load: index into the operand list
+    DScalar constant;          // Const
+    UnaryOp unary = UnaryOp::Abs;
+    DType cast_to = DType::F32;
+    BinaryOp binary = BinaryOp::Add;
+    size_t a = 0, b = 0;  // argument node indices
+};
+
+// An expression DAG in evaluation order, the last node being the result.
+struct ScalarExpr {
+    std::vector<ScalarNode> nodes;
+    size_t result() const { return nodes.size() - 1; }
+};
+
+struct KernelOperand {
+    DType dtype;
+    StridedShape shape;
+    int64_t offset_bytes;  // offset of the view origin inside its buffer, known at plan time (for alignment)
+};
+
+// out = expr(loads...). operands[0] is the output; the rest are the loaded operands, all of the same shape.
+KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const ScalarExpr &expr);
+
+// output[kept] = post(fold(op, input[kept, reduced...])) (reduce.rs:35-153)
+KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
+                              ReduceOp op);
+
+// Row kernels. The value that gets normalised is `pre(load operands...)`, the value stored is
+// `post(normalised, load operands...)`: this is how a preceding scale / residual add and a following affine
+// (gamma, beta) or activation are fused into the single pass over the row.
+struct RowKernelDesc {
+    enum Kind { Softmax, Layernorm } kind = Softmax;
+    size_t axis = 0;
+    float eps = 0;
+    // operands[0] is the output, operands[1..] are inputs; every operand has the full (output) shape
+    std::vector<KernelOperand> operands;
+    ScalarExpr pre;   // over Load nodes only; result f32
+    ScalarExpr post;  // Load nodes refer to operands; the node with kind Load and operand == SIZE_MAX is the normalised value
+};
+KernelSpec make_row_kernel(const RowKernelDesc &desc);
+
+// output[kept.., i, kept..] = input[kept.., indices[i], kept..], zero when the index is out of range (gather.rs:30-129)
+KernelSpec make_gather_kernel(const KernelOperand &input, const KernelOperand &indices, const KernelOperand &output,
+                              size_t axis);
+
+// Common device-side helpers prepended to every generated kernel.
+const char *kernel_prelude();
+
+}  // namespace kn

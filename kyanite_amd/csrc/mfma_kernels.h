@@ -1,0 +1,43 @@
+// Host-side interface of the ahead-of-time compiled MFMA kernels (batched matrix multiply and fused convolution).
+// They replace the library calls of the reference: cublasSgemm[StridedBatched] (kn-cuda-sys/src/wrapper/group.rs:107-171)
+// and cudnnConvolutionBiasActivationForward (kn-cuda-sys/src/wrapper/operation.rs:157-240).
+#pragma once
+
+#include <cstdint>
+
+struct ihipStream_t;
+
+namespace kn {
+
+// C[b, i, j] = sum_k A[b, i, k] * B[b, k, j]; element strides are arbitrary (zero batch stride = broadcast operand).
+struct GemmParams {
+    const float *a;
+    const float *b;
+    float *c;
+    int batch, m, n, k;
+    long long a_sb, a_sm, a_sk;
+    long long b_sb, b_sk, b_sn;
+    long long c_sb, c_sm, c_sn;
+};
+
+// out[n, ko, oy, ox] = act(sum_{c, fy, fx} in[n, c, oy*sy + fy - py, ox*sx + fx - px] * filter[ko, c, fy, fx]
+//                          + bias[ko] + res[n, ko, oy, ox])
+// Input, residual and output are dense NCHW, the filter is dense [K, C, kh, kw]; bias may be null (zero) and has
+// element stride `bias_stride` between channels; res may be null.
+struct ConvParams {
+    const float *input;
+    const float *filter;
+    const float *bias;
+    const float *res;
+    float *output;
+    int batch, in_c, in_h, in_w, out_c, out_h, out_w;
+    int kernel_h, kernel_w, stride_y, stride_x, pad_y, pad_x;
+    long long bias_stride;
+    int relu;
+};
+
+// Both return a hipError_t value (0 = success).
+int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
+int launch_conv_f32(const ConvParams &p, ihipStream_t *stream);
+
+}  // namespace kn

@@ -1,0 +1,765 @@
+#include "planner.h"
+
+#include <map>
+
+namespace kn {
+
+const char *step_kind_name(StepKind k) {
+    static const char *names[] = {"Conv", "MatMul", "ScalarOp", "ReduceOp", "SoftmaxOp", "LayernormOp", "GatherOp"};
+    return names[(int) k];
+}
+
+std::string Step::str() const {
+    std::ostringstream ss;
+    ss << step_kind_name(kind) << " value=" << debug_value;
+    if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
+    if (kind == StepKind::MatMul) ss << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k;
+    else if (kind == StepKind::Conv)
+        ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="
+           << conv.kernel_h << "x" << conv.kernel_w << (conv_has_bias ? " +bias" : "") << (conv_has_res ? " +res" : "")
+           << (conv.relu ? " relu" : "");
+    else ss << " [" << kernel.strategy << "] grid=" << kernel.grid << "x" << kernel.block;
+    ss << " operands:";
+    for (auto &op : operands) ss << " " << dtype_name(op.tensor.dtype) << vec_str(op.tensor.shape.shape());
+    return ss.str();
+}
+
+size_t Plan::resolve(const PlanPtr &ptr) const {
+    size_t base;
+    switch (ptr.kind) {
+        case BufferKind::Constant: base = constant_offsets.at(ptr.index); break;
+        case BufferKind::Zero: base = zero_offset; break;
+        default:
+            base = shared_offsets.at(ptr.index);
+            if (base == SIZE_MAX) fail("Unused shared buffer ", ptr.index, " is actually used");
+            break;
+    }
+    int64_t r = (int64_t) base + ptr.offset_bytes;
+    KN_ASSERT(r >= 0);
+    return (size_t) r;
+}
+
+namespace {
+
+template <typename T>
+struct Visit {
+    bool ok;
+    Value need;
+    T value;
+    static Visit done(T v) { return {true, 0, std::move(v)}; }
+    static Visit missing(Value v) { return {false, v, T()}; }
+};
+
+#define KN_TRY(name, expr)                                          \
+    auto name##_visit = (expr);                                     \
+    if (!name##_visit.ok) return {false, name##_visit.need, {}};    \
+    auto &name = name##_visit.value
+
+// The expression under construction for one fused elementwise kernel (planner.rs:994-1060), with common
+// sub-expressions computed once.
+struct ScalarBlock {
+    std::vector<PlanTensor> operands;  // operands[0] is reserved for the result
+    ScalarExpr expr;
+    std::map<Value, size_t> value_nodes;
+    std::vector<std::optional<size_t>> loaded;  // per operand: the node that holds its loaded value
+    std::optional<Value> row_value;             // the layernorm / softmax whose result this block post-processes
+    size_t row_node = 0;
+
+    size_t load_operand(const PlanTensor &t) {
+        for (size_t x = 1; x < operands.size(); x++) {
+            if (operands[x] == t) return *loaded[x];
+        }
+        operands.push_back(t);
+        ScalarNode n;
+        n.kind = ScalarNode::Load;
+        n.dtype = t.dtype;
+        n.operand = operands.size() - 1;
+        expr.nodes.push_back(n);
+        loaded.push_back(expr.nodes.size() - 1);
+        return expr.nodes.size() - 1;
+    }
+};
+
+struct FusedRow {
+    RowKernelDesc::Kind kind;
+    size_t axis;
+    float eps;
+    std::vector<PlanTensor> inputs;  // 1 or 2 tensors
+    ScalarExpr pre;                  // Load operand indices are 1-based positions into `inputs`
+};
+
+class Planner {
+public:
+    Planner(const Graph &g, size_t batch, const PlannerOptions &o) : graph(g), batch_size(batch), options(o) {}
+
+    const Graph &graph;
+    size_t batch_size;
+    PlannerOptions options;
+
+    std::vector<size_t> shared_sizes;
+    std::vector<HostTensor> constants;
+    std::unordered_map<Value, PlanTensor> map;
+    std::vector<Step> steps;
+
+    using VT = Visit<PlanTensor>;
+
+    PlanTensor visit_completely(Value value) {
+        std::vector<Value> stack{value};
+        while (true) {
+            VT r = visit_single_cached(stack.back());
+            if (r.ok) {
+                stack.pop_back();
+                if (stack.empty()) return r.value;
+            } else {
+                stack.push_back(r.need);
+            }
+        }
+    }
+
+    PlanTensor visit_completely_ensure_simple_strides(Value value) {
+        visit_completely(value);
+        VT r = visit_ensure_simple_strides(value);
+        KN_ASSERT(r.ok);
+        return r.value;
+    }
+
+private:
+    VT visit(Value value) {
+        auto it = map.find(value);
+        if (it != map.end()) return VT::done(it->second);
+        return VT::missing(value);
+    }
+
+    void insert_mapping(Value value, const PlanTensor &t) {
+        if (t.shape.shape() != graph[value].shape.eval(batch_size)) fail("Got wrong result shape for value ", value);
+        bool inserted = map.emplace(value, t).second;
+        KN_ASSERT(inserted);
+    }
+
+    VT visit_single_cached(Value value) {
+        auto it = map.find(value);
+        if (it != map.end()) return VT::done(it->second);
+        KN_TRY(result, visit_single_new(value));
+        const ValueInfo &info = graph[value];
+        KN_ASSERT(result.dtype == info.dtype);
+        // a fused conv or row kernel may already have registered this value
+        if (!map.count(value)) insert_mapping(value, result);
+        return VT::done(result);
+    }
+
+    bool can_fuse(Value v) const { return graph.is_hidden_with_uses(v, 1); }
+
+    PlanPtr alloc_buffer_shared(size_t bytes) {
+        shared_sizes.push_back(bytes);
+        return PlanPtr{BufferKind::Shared, shared_sizes.size() - 1, 0};
+    }
+
+    PlanTensor alloc_tensor_shared(const ConcreteShape &shape, DType dtype) {
+        PlanTensor t;
+        t.ptr = alloc_buffer_shared(dtype_bytes(dtype) * concrete_size(shape));
+        t.dtype = dtype;
+        t.shape = StridedShape::simple(shape);
+        return t;
+    }
+
+    void push(Step step, Value debug_value) {
+        step.debug_value = debug_value;
+        step.debug_id = graph[debug_value].debug_id;
+        if (step.kind != StepKind::Conv && step.kind != StepKind::MatMul) {
+            if (step.kernel.grid == 0) return;  // nothing to compute (empty tensors)
+            if (options.compile) step.code = compile_kernel(step.kernel.source);
+        }
+        steps.push_back(std::move(step));
+    }
+
+    static KernelOperand kop(const PlanTensor &t) { return KernelOperand{t.dtype, t.shape, t.ptr.offset_bytes}; }
+
+    VT visit_single_new(Value value) {
+        {
+            auto fused = try_visit_fused_conv(value);
+            if (!fused.ok) return VT::missing(fused.need);
+            if (fused.value) return VT::done(*fused.value);
+        }
+        const ValueInfo &info = graph[value];
+        ConcreteShape result_shape = info.shape.eval(batch_size);
+        DType result_dtype = info.dtype;
+        const Operation &op = info.operation;
+
+        switch (op.kind) {
+            case OpKind::Input: return VT::done(alloc_tensor_shared(result_shape, result_dtype));
+            case OpKind::Constant: {
+                PlanTensor t;
+                constants.push_back(op.tensor);
+                t.ptr = PlanPtr{BufferKind::Constant, constants.size() - 1, 0};
+                t.dtype = op.tensor.dtype;
+                t.shape = StridedShape::simple(result_shape);
+                return VT::done(t);
+            }
+            case OpKind::View: {
+                KN_TRY(input, visit(op.inputs[0]));
+                // try a pure stride edit, otherwise restride into a dense copy first
+                if (auto v = input.view(result_shape)) return VT::done(*v);
+                PlanTensor dense = alloc_tensor_shared(input.shape.shape(), input.dtype);
+                plan_copy_tensor(input, dense, value);
+                auto v = dense.view(result_shape);
+                KN_ASSERT(v.has_value());
+                return VT::done(*v);
+            }
+            case OpKind::Broadcast: {
+                KN_TRY(input, visit(op.inputs[0]));
+                return VT::done(input.broadcast(result_shape));
+            }
+            case OpKind::Permute: return visit_permute(op.inputs[0], op.axes);
+            case OpKind::Slice: {
+                KN_TRY(input, visit(op.inputs[0]));
+                return VT::done(input.slice(op.axis(), op.range));
+            }
+            case OpKind::Flip: {
+                KN_TRY(input, visit(op.inputs[0]));
+                return VT::done(input.flip(op.axis()));
+            }
+            case OpKind::Gather: {
+                KN_TRY(input, visit(op.inputs[0]));
+                KN_TRY(indices, visit(op.inputs[1]));
+                PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
+                Step step;
+                step.kind = StepKind::GatherOp;
+                step.kernel = make_gather_kernel(kop(input), kop(indices), kop(output), op.axis());
+                step.operands = {{input, OperandKind::In}, {indices, OperandKind::In}, {output, OperandKind::Out}};
+                push(std::move(step), value);
+                return VT::done(output);
+            }
+            case OpKind::Concat: {
+                std::vector<PlanTensor> ins;
+                for (Value x : op.inputs) {
+                    KN_TRY(t, visit(x));
+                    ins.push_back(t);
+                }
+                PlanTensor result = alloc_tensor_shared(result_shape, result_dtype);
+                size_t axis = op.axis(), start = 0;
+                for (auto &in : ins) {
+                    size_t len = in.shape.shape()[axis];
+                    plan_copy_tensor(in, result.slice(axis, SliceRange{start, start + len, 1}), value);
+                    start += len;
+                }
+                return VT::done(result);
+            }
+            case OpKind::Conv: fail("Conv should have been handled by the conv fuser (only rank-4 f32 convolutions are supported)");
+            case OpKind::MatMul: return visit_matmul(value, op.inputs[0], op.inputs[1], true);
+            case OpKind::Unary: case OpKind::Binary: return visit_fused_scalar(value);
+            case OpKind::Softmax: case OpKind::Layernorm: {
+                KN_ASSERT(result_dtype == DType::F32);
+                auto row = visit_row_inputs(value);
+                if (!row.ok) return VT::missing(row.need);
+                // no elementwise consumer was fused: the epilogue is the identity
+                ScalarExpr post;
+                ScalarNode n;
+                n.kind = ScalarNode::Load;
+                n.dtype = DType::F32;
+                n.operand = SIZE_MAX;
+                post.nodes.push_back(n);
+                return VT::done(push_row_kernel(value, value, row.value, post, {}));
+            }
+            case OpKind::Reduce: {
+                KN_TRY(input, visit(op.inputs[0]));
+                PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
+                if (op.reduce == ReduceOp::Mean) KN_ASSERT(result_dtype == DType::F32);
+                Step step;
+                step.kind = StepKind::ReduceOp;
+                step.kernel = make_reduce_kernel(kop(input), kop(output), op.axes, op.reduce);
+                step.operands = {{input, OperandKind::In}, {output, OperandKind::Out}};
+                push(std::move(step), value);
+                return VT::done(output);
+            }
+        }
+        fail("unreachable");
+    }
+
+    // planner.rs:554-567
+    VT visit_permute(Value input, const std::vector<size_t> &permutation) {
+        if (can_fuse(input) && permutation == std::vector<size_t>{1, 0, 2} && !map.count(input)) {
+            const Operation &iop = graph[input].operation;
+            if (iop.kind == OpKind::MatMul) {
+                // avoid a non-dense result for the typical attention matmul: write directly in [m, b, n] order
+                KN_TRY(mm, visit_matmul(input, iop.inputs[0], iop.inputs[1], false));
+                insert_mapping(input, mm);
+                return VT::done(mm.permute(permutation));
+            }
+        }
+        KN_TRY(t, visit(input));
+        return VT::done(t.permute(permutation));
+    }
+
+    // planner.rs:569-582
+    VT visit_ensure_simple_strides(Value value) {
+        KN_TRY(inner, visit(value));
+        if (inner.shape.has_simple_strides()) return VT::done(inner);
+        PlanTensor dense = alloc_tensor_shared(inner.shape.shape(), inner.dtype);
+        plan_copy_tensor(inner, dense, value);
+        return VT::done(dense);
+    }
+
+    // planner.rs:584-604: `alpha * x` with a single-valued constant alpha
+    Visit<std::pair<std::optional<DScalar>, PlanTensor>> visit_scalable_value(Value value) {
+        using R = Visit<std::pair<std::optional<DScalar>, PlanTensor>>;
+        const Operation &op = graph[value].operation;
+        if (op.kind == OpKind::Binary && op.binary == BinaryOp::Mul && !map.count(value)) {
+            if (auto alpha = graph.as_single_const(op.inputs[0])) {
+                auto t = visit(op.inputs[1]);
+                if (!t.ok) return R::missing(t.need);
+                return R::done({alpha, t.value});
+            }
+            if (auto alpha = graph.as_single_const(op.inputs[1])) {
+                auto t = visit(op.inputs[0]);
+                if (!t.ok) return R::missing(t.need);
+                return R::done({alpha, t.value});
+            }
+        }
+        auto t = visit(value);
+        if (!t.ok) return R::missing(t.need);
+        return R::done({std::nullopt, t.value});
+    }
+
+    // The operands and prologue of a softmax (planner.rs:418-441) or layernorm (:443-476, :522-552) value.
+    Visit<FusedRow> visit_row_inputs(Value value) {
+        using R = Visit<FusedRow>;
+        const Operation &op = graph[value].operation;
+        FusedRow row;
+        row.axis = op.axis();
+        row.eps = op.eps;
+        auto load = [&](size_t operand) {
+            ScalarNode n;
+            n.kind = ScalarNode::Load;
+            n.dtype = DType::F32;
+            n.operand = operand;
+            row.pre.nodes.push_back(n);
+            return row.pre.nodes.size() - 1;
+        };
+        auto scaled = [&](const std::optional<DScalar> &alpha, size_t x) {
+            if (!alpha) return x;
+            ScalarNode c;
+            c.kind = ScalarNode::Const;
+            c.dtype = DType::F32;
+            c.constant = *alpha;
+            row.pre.nodes.push_back(c);
+            ScalarNode m;
+            m.kind = ScalarNode::Binary;
+            m.dtype = DType::F32;
+            m.binary = BinaryOp::Mul;
+            m.a = x;
+            m.b = row.pre.nodes.size() - 1;
+            row.pre.nodes.push_back(m);
+            return row.pre.nodes.size() - 1;
+        };
+        Value input = op.inputs[0];
+        if (op.kind == OpKind::Softmax) {
+            row.kind = RowKernelDesc::Softmax;
+            auto sv = visit_scalable_value(input);
+            if (!sv.ok) return R::missing(sv.need);
+            row.inputs = {sv.value.second};
+            scaled(sv.value.first, load(1));
+            return R::done(row);
+        }
+        row.kind = RowKernelDesc::Layernorm;
+        const Operation &iop = graph[input].operation;
+        if (iop.kind == OpKind::Binary && iop.binary == BinaryOp::Add && !map.count(input)) {
+            auto l = visit_scalable_value(iop.inputs[0]);
+            if (!l.ok) return R::missing(l.need);
+            auto r = visit_scalable_value(iop.inputs[1]);
+            if (!r.ok) return R::missing(r.need);
+            if (l.value.second.shape == r.value.second.shape) {
+                row.inputs = {l.value.second, r.value.second};
+                size_t a = scaled(l.value.first, load(1));
+                size_t b = scaled(r.value.first, load(2));
+                ScalarNode add;
+                add.kind = ScalarNode::Binary;
+                add.dtype = DType::F32;
+                add.binary = BinaryOp::Add;
+                add.a = a;
+                add.b = b;
+                row.pre.nodes.push_back(add);
+                return R::done(row);
+            }
+            // differently laid out operands: fall back to materialising the sum
+            auto total = visit(input);
+            if (!total.ok) return R::missing(total.need);
+            row.inputs = {total.value};
+            load(1);
+            return R::done(row);
+        }
+        auto sv = visit_scalable_value(input);
+        if (!sv.ok) return R::missing(sv.need);
+        row.inputs = {sv.value.second};
+        scaled(sv.value.first, load(1));
+        return R::done(row);
+    }
+
+    // Emit the row kernel for `row_value`, storing `post(normalised, extra...)` as the result of `result_value`.
+    // Load nodes of `post` index into `extra` (1-based, 0 is unused); SIZE_MAX is the normalised value.
+    PlanTensor push_row_kernel(Value row_value, Value result_value, const FusedRow &row, const ScalarExpr &post_in,
+                               const std::vector<PlanTensor> &extra) {
+        const ValueInfo &info = graph[result_value];
+        PlanTensor output = alloc_tensor_shared(info.shape.eval(batch_size), info.dtype);
+        RowKernelDesc desc;
+        desc.kind = row.kind;
+        desc.axis = row.axis;
+        desc.eps = row.eps;
+        // operand order: output, row inputs, epilogue operands
+        std::vector<PlanTensor> all{output};
+        for (auto &t : row.inputs) all.push_back(t);
+        size_t extra_base = all.size();
+        for (size_t k = 1; k < extra.size(); k++) all.push_back(extra[k]);
+        for (auto &t : all) desc.operands.push_back(kop(t));
+        desc.pre = row.pre;
+        desc.post = post_in;
+        for (auto &n : desc.post.nodes)
+            if (n.kind == ScalarNode::Load && n.operand != SIZE_MAX) n.operand = extra_base + n.operand - 1;
+
+        Step step;
+        step.kind = row.kind == RowKernelDesc::Softmax ? StepKind::SoftmaxOp : StepKind::LayernormOp;
+        step.kernel = make_row_kernel(desc);
+        step.operands.push_back({output, OperandKind::Out});
+        for (size_t k = 1; k < all.size(); k++) step.operands.push_back({all[k], OperandKind::In});
+        push(std::move(step), row_value);
+        return output;
+    }
+
+    // planner.rs:606-648
+    VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first) {
+        if (graph[value].dtype != DType::F32) fail("GPU matmul only supports f32, got ", dtype_name(graph[value].dtype));
+        KN_TRY(left, visit(left_v));
+        KN_TRY(right, visit(right_v));
+        KN_ASSERT(left.shape.rank() == 3 && right.shape.rank() == 3);
+        size_t b = left.shape.shape()[0], m = left.shape.shape()[1], k = left.shape.shape()[2], n = right.shape.shape()[2];
+        PlanTensor result = batch_first ? alloc_tensor_shared({b, m, n}, DType::F32)
+                                        : alloc_tensor_shared({m, b, n}, DType::F32).permute({1, 0, 2});
+        if (b * m * n != 0) {
+            KN_ASSERT(b <= INT32_MAX && m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX);
+            Step step;
+            step.kind = StepKind::MatMul;
+            GemmParams &g = step.gemm;
+            g.batch = (int) b; g.m = (int) m; g.n = (int) n; g.k = (int) k;
+            g.a_sb = left.shape.strides()[0]; g.a_sm = left.shape.strides()[1]; g.a_sk = left.shape.strides()[2];
+            g.b_sb = right.shape.strides()[0]; g.b_sk = right.shape.strides()[1]; g.b_sn = right.shape.strides()[2];
+            g.c_sb = result.shape.strides()[0]; g.c_sm = result.shape.strides()[1]; g.c_sn = result.shape.strides()[2];
+            step.operands = {{left, OperandKind::In}, {right, OperandKind::In}, {result, OperandKind::Out}};
+            push(std::move(step), value);
+        }
+        return VT::done(result);
+    }
+
+    // planner.rs:669-833: relu?( conv(x, w) [+ bias] [+ res] )
+    Visit<std::optional<PlanTensor>> try_visit_fused_conv(Value value) {
+        using R = Visit<std::optional<PlanTensor>>;
+        if (graph[value].dtype != DType::F32 || graph[value].shape.rank() != 4) return R::done(std::nullopt);
+        Value curr = value;
+        bool relu = false;
+        {
+            const Operation &op = graph[curr].operation;
+            if (op.kind == OpKind::Binary && op.binary == BinaryOp::Max) {
+                Value l = op.inputs[0], r = op.inputs[1];
+                if (!(can_fuse(l) && can_fuse(r))) return R::done(std::nullopt);
+                if (graph.is_const_zero(l)) curr = r;
+                else if (graph.is_const_zero(r)) curr = l;
+                else return R::done(std::nullopt);
+                relu = true;
+            }
+        }
+        std::optional<Value> bias, res;
+        while (true) {
+            const Operation &op = graph[curr].operation;
+            if (!(op.kind == OpKind::Binary && op.binary == BinaryOp::Add)) break;
+            Value l = op.inputs[0], r = op.inputs[1];
+            if (!can_fuse(l)) return R::done(std::nullopt);
+            bool is_res = graph[l].shape == graph[r].shape;
+            std::optional<Value> bias_inner;
+            const Operation &rop = graph[r].operation;
+            if (rop.kind == OpKind::Broadcast) {
+                Value ri = rop.inputs[0];
+                if (graph[l].shape.keep(1, Size::one()) == graph[ri].shape) bias_inner = ri;
+            }
+            if (bias_inner) {
+                if (bias) return R::done(std::nullopt);
+                bias = bias_inner;
+            } else if (is_res) {
+                if (res) return R::done(std::nullopt);
+                res = r;
+            } else {
+                return R::done(std::nullopt);
+            }
+            curr = l;
+        }
+        const Operation &cop = graph[curr].operation;
+        if (cop.kind != OpKind::Conv) return R::done(std::nullopt);
+        Value input_v = cop.inputs[0], filter_v = cop.inputs[1];
+        const ConvDetails &d = cop.conv;
+        KN_ASSERT(d.dtype == DType::F32);
+        // the residual has to be shaped like the input; otherwise the conv is retried later without it
+        if (res && graph[input_v].shape != graph[*res].shape) return R::done(std::nullopt);
+
+        auto input = visit_ensure_simple_strides(input_v);
+        if (!input.ok) return R::missing(input.need);
+        auto filter = visit_ensure_simple_strides(filter_v);
+        if (!filter.ok) return R::missing(filter.need);
+        std::optional<PlanTensor> bias_t, res_t;
+        if (bias) {
+            auto bt = visit(*bias);
+            if (!bt.ok) return R::missing(bt.need);
+            bias_t = bt.value;
+        }
+        if (res) {
+            auto rt = visit_ensure_simple_strides(*res);
+            if (!rt.ok) return R::missing(rt.need);
+            res_t = rt.value;
+        }
+        ConcreteShape out_shape = graph[curr].shape.eval(batch_size);
+        PlanTensor output = alloc_tensor_shared(out_shape, DType::F32);
+        if (res_t) KN_ASSERT(res_t->shape.shape() == out_shape, "conv residual must match the output shape");
+
+        if (concrete_size(out_shape) != 0) {
+            Step step;
+            step.kind = StepKind::Conv;
+            ConvParams &p = step.conv;
+            KN_ASSERT(out_shape[0] <= INT32_MAX);
+            p.batch = (int) out_shape[0];
+            p.in_c = (int) d.input_channels; p.in_h = (int) d.input_h; p.in_w = (int) d.input_w;
+            p.out_c = (int) d.output_channels; p.out_h = (int) d.output_h; p.out_w = (int) d.output_w;
+            p.kernel_h = (int) d.kernel_h; p.kernel_w = (int) d.kernel_w;
+            p.stride_y = (int) d.stride_y; p.stride_x = (int) d.stride_x;
+            p.pad_y = (int) d.padding_y; p.pad_x = (int) d.padding_x;
+            p.relu = relu ? 1 : 0;
+            p.bias_stride = bias_t ? bias_t->shape.strides()[1] : 0;
+            step.conv_has_bias = bias_t.has_value();
+            step.conv_has_res = res_t.has_value();
+            step.operands = {{input.value, OperandKind::In}, {filter.value, OperandKind::In}};
+            if (bias_t) step.operands.push_back({*bias_t, OperandKind::In});
+            if (res_t) step.operands.push_back({*res_t, OperandKind::In});
+            step.operands.push_back({output, OperandKind::Out});
+            push(std::move(step), value);
+        }
+        return R::done(output);
+    }
+
+    // planner.rs:835-871
+    VT visit_fused_scalar(Value value) {
+        const ValueInfo &info = graph[value];
+        ScalarBlock block;
+        block.operands.push_back(PlanTensor());  // placeholder for the result
+        block.loaded.push_back(std::nullopt);
+        auto root = visit_fused_scalar_recurse(value, block, true);
+        if (!root.ok) return VT::missing(root.need);
+        KN_ASSERT(root.value == block.expr.result());
+
+        if (block.row_value) {
+            // the chain hangs off a layernorm / softmax: it becomes the epilogue of that row kernel
+            auto row = visit_row_inputs(*block.row_value);
+            if (!row.ok) return VT::missing(row.need);
+            return VT::done(push_row_kernel(*block.row_value, value, row.value, block.expr, block.operands));
+        }
+
+        PlanTensor result = alloc_tensor_shared(info.shape.eval(batch_size), info.dtype);
+        block.operands[0] = result;
+        plan_scalar_op(block.expr, block.operands, value);
+        return VT::done(result);
+    }
+
+    // planner.rs:873-923; returns the node index that holds `value`
+    Visit<size_t> visit_fused_scalar_recurse(Value value, ScalarBlock &block, bool is_root) {
+        using R = Visit<size_t>;
+        auto known = block.value_nodes.find(value);
+        if (known != block.value_nodes.end()) return R::done(known->second);
+
+        size_t node;
+        auto mapped = map.find(value);
+        if (mapped != map.end()) {
+            node = block.load_operand(mapped->second);
+        } else {
+            // give the conv fuser the first shot, so that this chain does not steal its relu, add or bias
+            auto fused = try_visit_fused_conv(value);
+            if (!fused.ok) return R::missing(fused.need);
+            if (fused.value) {
+                if (!map.count(value)) insert_mapping(value, *fused.value);
+                node = block.load_operand(*fused.value);
+            } else {
+                const ValueInfo &info = graph[value];
+                const Operation &op = info.operation;
+                ScalarNode n;
+                n.dtype = info.dtype;
+                if (op.kind == OpKind::Unary) {
+                    auto a = visit_fused_scalar_recurse(op.inputs[0], block, false);
+                    if (!a.ok) return a;
+                    n.kind = ScalarNode::Unary;
+                    n.unary = op.unary;
+                    n.cast_to = op.cast_to;
+                    n.a = a.value;
+                } else if (op.kind == OpKind::Binary) {
+                    auto a = visit_fused_scalar_recurse(op.inputs[0], block, false);
+                    if (!a.ok) return a;
+                    auto b = visit_fused_scalar_recurse(op.inputs[1], block, false);
+                    if (!b.ok) return b;
+                    n.kind = ScalarNode::Binary;
+                    n.binary = op.binary;
+                    n.a = a.value;
+                    n.b = b.value;
+                } else {
+                    KN_ASSERT(!is_root);
+                    if (auto c = graph.as_single_const(value)) {
+                        n.kind = ScalarNode::Const;
+                        n.constant = *c;
+                    } else if (options.fuse_row_epilogue && !block.row_value && can_fuse(value) &&
+                               (op.kind == OpKind::Layernorm || op.kind == OpKind::Softmax)) {
+                        block.row_value = value;
+                        n.kind = ScalarNode::Load;
+                        n.operand = SIZE_MAX;
+                    } else {
+                        auto t = visit(value);
+                        if (!t.ok) return R::missing(t.need);
+                        node = block.load_operand(t.value);
+                        block.value_nodes[value] = node;
+                        return R::done(node);
+                    }
+                }
+                block.expr.nodes.push_back(n);
+                node = block.expr.nodes.size() - 1;
+            }
+        }
+        block.value_nodes[value] = node;
+        return R::done(node);
+    }
+
+    // planner.rs:926-931
+    void plan_copy_tensor(const PlanTensor &old_t, const PlanTensor &new_t, Value debug_value) {
+        KN_ASSERT(old_t.shape.shape() == new_t.shape.shape() && old_t.dtype == new_t.dtype);
+        ScalarExpr expr;
+        ScalarNode n;
+        n.kind = ScalarNode::Load;
+        n.dtype = old_t.dtype;
+        n.operand = 1;
+        expr.nodes.push_back(n);
+        plan_scalar_op(expr, {new_t, old_t}, debug_value);
+    }
+
+    // planner.rs:933-954
+    void plan_scalar_op(const ScalarExpr &expr, const std::vector<PlanTensor> &operands, Value debug_value) {
+        std::vector<KernelOperand> kops;
+        for (auto &t : operands) kops.push_back(kop(t));
+        Step step;
+        step.kind = StepKind::ScalarOp;
+        step.kernel = make_scalar_kernel(kops, expr);
+        step.operands.push_back({operands[0], OperandKind::Out});
+        for (size_t k = 1; k < operands.size(); k++) step.operands.push_back({operands[k], OperandKind::In});
+        push(std::move(step), debug_value);
+    }
+};
+
+size_t align_up(size_t v) { return (v + ARENA_ALIGN - 1) / ARENA_ALIGN * ARENA_ALIGN; }
+
+}  // namespace
+
+Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &options) {
+    Planner planner(graph, batch_size, options);
+    Plan plan;
+
+    // allocate inputs (even if they are not actually used), then plan everything the outputs need
+    for (Value in : graph.inputs) plan.inputs.push_back(planner.visit_completely(in));
+    for (Value out : graph.outputs) plan.outputs.push_back(planner.visit_completely_ensure_simple_strides(out));
+
+    size_t buffer_count = planner.shared_sizes.size();
+    size_t step_count = planner.steps.size();
+
+    // live ranges of the shared buffers over step indices (planner.rs:134-164)
+    std::vector<std::pair<size_t, size_t>> live(buffer_count, {step_count, 0});
+    auto touch = [&](const PlanPtr &p, size_t si) {
+        if (p.kind != BufferKind::Shared) return;
+        live[p.index].first = std::min(live[p.index].first, si);
+        live[p.index].second = std::max(live[p.index].second, si);
+    };
+    for (size_t si = 0; si < step_count; si++)
+        for (auto &op : planner.steps[si].operands) touch(op.tensor.ptr, si);
+    for (auto &t : plan.outputs)
+        if (t.ptr.kind == BufferKind::Shared) live[t.ptr.index].second = step_count;
+    for (auto &t : plan.inputs)
+        if (t.ptr.kind == BufferKind::Shared) live[t.ptr.index].first = 0;
+
+    // ---- arena layout: constants first
+    size_t cursor = 0;
+    for (auto &c : planner.constants) {
+        plan.constant_offsets.push_back(cursor);
+        plan.uploads.push_back({cursor, c});
+        plan.mem_usage.dedicated_bytes += c.nbytes();
+        cursor = align_up(cursor + c.nbytes());
+    }
+    plan.zero_offset = cursor;
+    size_t shared_base = cursor;
+
+    // ---- shared region: first-fit placement of live intervals. A buffer whose last use is step s may share
+    // memory with one whose first use is step s + 1, never with one that is touched by step s itself.
+    plan.shared_offsets.assign(buffer_count, SIZE_MAX);
+    plan.shared_sizes = planner.shared_sizes;
+    std::vector<size_t> order;
+    for (size_t b = 0; b < buffer_count; b++)
+        if (live[b].first <= live[b].second) order.push_back(b);
+    std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) {
+        if (live[x].first != live[y].first) return live[x].first < live[y].first;
+        return planner.shared_sizes[x] > planner.shared_sizes[y];
+    });
+    struct Active {
+        size_t offset, size, end;
+    };
+    std::vector<Active> active;
+    size_t shared_extent = 0;
+    for (size_t b : order) {
+        size_t start = live[b].first, end = live[b].second;
+        size_t size = align_up(std::max<size_t>(planner.shared_sizes[b], 1));
+        active.erase(std::remove_if(active.begin(), active.end(), [&](const Active &a) { return a.end < start; }), active.end());
+        std::sort(active.begin(), active.end(), [](const Active &x, const Active &y) { return x.offset < y.offset; });
+        size_t offset = 0;
+        for (auto &a : active) {
+            if (offset + size <= a.offset) break;
+            offset = std::max(offset, a.offset + a.size);
+        }
+        active.push_back({offset, size, end});
+        plan.shared_offsets[b] = shared_base + offset;
+        shared_extent = std::max(shared_extent, offset + size);
+        plan.mem_usage.hypo_shared_bytes_total += planner.shared_sizes[b];
+    }
+    plan.mem_usage.shared_bytes = shared_extent;
+    plan.arena_bytes = std::max<size_t>(shared_base + shared_extent, ARENA_ALIGN);
+
+    // the amount of memory that is live at the same time, as a lower bound for the shared region
+    {
+        std::vector<int64_t> delta(step_count + 2, 0);
+        for (size_t b : order) {
+            delta[live[b].first] += (int64_t) planner.shared_sizes[b];
+            delta[live[b].second + 1] -= (int64_t) planner.shared_sizes[b];
+        }
+        int64_t curr = 0;
+        for (int64_t d : delta) {
+            curr += d;
+            plan.mem_usage.hypo_shared_bytes_peak = std::max<size_t>(plan.mem_usage.hypo_shared_bytes_peak, (size_t) curr);
+        }
+    }
+
+    // ---- every access of every step has to stay inside its buffer: checked here, on the host, so that a planning
+    // mistake is reported as an error instead of faulting on the device
+    auto buffer_bytes = [&](const PlanPtr &p) {
+        return p.kind == BufferKind::Constant ? planner.constants[p.index].nbytes() : planner.shared_sizes[p.index];
+    };
+    for (auto &step : planner.steps) {
+        for (auto &op : step.operands) {
+            const PlanTensor &t = op.tensor;
+            if (t.shape.size() == 0) continue;
+            auto [lo, hi] = t.shape.offset_bounds();
+            int64_t es = (int64_t) dtype_bytes(t.dtype);
+            int64_t first = t.ptr.offset_bytes + lo * es, last = t.ptr.offset_bytes + (hi + 1) * es;
+            if (first < 0 || last > (int64_t) buffer_bytes(t.ptr))
+                fail("planned operand of ", step.str(), " reaches outside its buffer: bytes [", first, ", ", last, ") of ",
+                     buffer_bytes(t.ptr));
+        }
+    }
+
+    plan.steps = std::move(planner.steps);
+    return plan;
+}
+
+}  // namespace kn

@@ -1,0 +1,82 @@
+// Planner: turns a Graph plus a concrete batch size into a launch list over one device arena.
+// Keeps the planning semantics of kn-cuda-eval/src/planner.rs (layout propagation :345-364, fused convolution
+// matcher :669-833, scalar chain fusion :835-954, softmax / layernorm operand folding :418-476, :522-604, matmul
+// :606-648, live ranges :134-164), but plans into byte offsets of a single arena instead of separate allocations,
+// and fuses elementwise work that follows a layernorm or softmax into that kernel's single pass over the row.
+#pragma once
+
+#include <memory>
+
+#include "kernels.h"
+#include "mfma_kernels.h"
+#include "rtc.h"
+
+namespace kn {
+
+enum class StepKind : uint8_t { Conv = 0, MatMul = 1, ScalarOp = 2, ReduceOp = 3, SoftmaxOp = 4, LayernormOp = 5, GatherOp = 6 };
+constexpr int STEP_KIND_COUNT = 7;
+const char *step_kind_name(StepKind k);
+
+enum class OperandKind : uint8_t { In, Out, InOut, Scratch };  // step.rs:82-94
+
+struct StepOperand {
+    PlanTensor tensor;
+    OperandKind kind;
+};
+
+struct Step {
+    StepKind kind = StepKind::ScalarOp;
+    Value debug_value = 0;
+    std::string debug_id;
+    // every tensor the step touches, in kernel argument order
+    std::vector<StepOperand> operands;
+    // run-time compiled kernels
+    KernelSpec kernel;
+    std::shared_ptr<const CodeObject> code;
+    // matrix-core kernels; the pointers are filled in when the plan is realised
+    GemmParams gemm{};
+    ConvParams conv{};
+    bool conv_has_bias = false, conv_has_res = false;
+
+    std::string str() const;
+};
+
+struct MemoryUsage {  // planner.rs:67-81
+    size_t dedicated_bytes = 0;  // constants
+    size_t shared_bytes = 0;     // inputs, outputs, hidden values
+    size_t zero_bytes = 0;
+    size_t hypo_shared_bytes_peak = 0;   // lower bound: what is live at the same time
+    size_t hypo_shared_bytes_total = 0;  // without any reuse
+};
+
+struct ConstantUpload {
+    size_t arena_offset;
+    HostTensor tensor;
+};
+
+struct Plan {
+    std::vector<PlanTensor> inputs, outputs;
+    std::vector<Step> steps;
+    MemoryUsage mem_usage;
+    // arena layout: [constants | zeros | shared], every buffer aligned to ARENA_ALIGN
+    size_t arena_bytes = 0;
+    std::vector<size_t> constant_offsets;  // per constant slot
+    size_t zero_offset = 0;
+    std::vector<size_t> shared_offsets;  // per shared buffer; SIZE_MAX for buffers that are never used
+    std::vector<size_t> shared_sizes;
+    std::vector<ConstantUpload> uploads;
+
+    // resolve a planned pointer to a byte offset inside the arena
+    size_t resolve(const PlanPtr &ptr) const;
+};
+
+constexpr size_t ARENA_ALIGN = 256;
+
+struct PlannerOptions {
+    bool compile = true;          // compile the generated kernels (can be switched off to inspect the plan only)
+    bool fuse_row_epilogue = true;  // fold elementwise consumers of a layernorm / softmax into the row kernel
+};
+
+Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &options);
+
+}  // namespace kn

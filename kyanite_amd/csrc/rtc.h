@@ -1,0 +1,31 @@
+// Run-time compilation of generated kernels for gfx950 through hipRTC, with an in-memory and an on-disk cache.
+// Takes the role of kn-cuda-sys/src/wrapper/rtc/core.rs (compile, module load, launch) and of the process-wide
+// kernel cache in kn-cuda-eval/src/autokernel/common.rs:14-46.
+#pragma once
+
+#include <memory>
+#include <mutex>
+
+#include "kernels.h"
+
+namespace kn {
+
+struct CodeObject {
+    std::vector<char> binary;
+    uint64_t key = 0;
+};
+
+// Compile (or fetch from cache) the code object for a kernel source. Works without a GPU.
+// The disk cache lives in $KNHIP_CACHE_DIR, or next to the library in `_kcache/` when that is unset;
+// set KNHIP_CACHE_DIR to an empty string to disable it.
+std::shared_ptr<const CodeObject> compile_kernel(const std::string &source);
+
+struct CompileStats {
+    size_t compiled = 0, memory_hits = 0, disk_hits = 0;
+};
+CompileStats compile_stats();
+
+// The directory of the shared library that contains this code.
+std::string library_dir();
+
+}  // namespace kn

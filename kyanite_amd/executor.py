@@ -1,0 +1,206 @@
+"""HipExecutor and the runtime device selector, mirroring kn-cuda-eval's CudaExecutor
+(executor.rs:60-266) and kn-runtime's Device / PreparedGraph (kn-runtime/src/lib.rs:68-126)."""
+import ctypes
+from ctypes import byref, c_float, c_int, c_size_t, c_void_p
+
+import numpy as np
+
+from ._lib import KnError, MemUsageT, ProfileT, check, get_string, lib
+from .graph import DType, Graph
+
+STEP_KINDS = ["conv", "mat_mul", "scalar_op", "reduce_op", "softmax_op", "layernorm_op", "gather_op"]
+
+
+class HipDevice:
+    """kn-cuda-sys/src/wrapper/handle.rs:37-103"""
+
+    def __init__(self, index=0):
+        n = HipDevice.count()
+        if not 0 <= index < n:
+            raise KnError(f"HIP device {index} is not available ({n} device(s) visible)")
+        self.index = index
+
+    @staticmethod
+    def count():
+        n = c_int()
+        check(lib.knhip_device_count(byref(n)))
+        return n.value
+
+    @staticmethod
+    def all():
+        return [HipDevice(i) for i in range(HipDevice.count())]
+
+    def name(self):
+        return get_string(lib.knhip_device_name, self.index)
+
+    def __repr__(self):
+        return f"HipDevice({self.index})"
+
+
+class Profile:
+    def __init__(self, raw, step_seconds, text):
+        for i, k in enumerate(STEP_KINDS):
+            setattr(self, k, raw.per_kind[i])
+        self.total_cpu = raw.total_cpu
+        self.total_gpu = raw.total_gpu
+        self.timing_overhead = raw.timing_overhead
+        self.step_seconds = step_seconds
+        self.text = text
+
+    def __str__(self):
+        return self.text
+
+
+class HipExecutor:
+    """`HipExecutor(device, graph, batch_size)` / `evaluate(inputs) -> outputs`."""
+
+    def __init__(self, device, graph, batch_size, plan_only=False):
+        index = device.index if isinstance(device, HipDevice) else int(device)
+        h = c_void_p()
+        check(lib.knhip_executor_new(index, graph._h, batch_size, int(plan_only), byref(h)))
+        self._h = h
+        self.device = index
+        self.batch_size = batch_size
+        self.plan_only = plan_only
+        n_in, n_out = c_size_t(), c_size_t()
+        check(lib.knhip_executor_io_count(h, byref(n_in), byref(n_out)))
+        self.input_info = [self._io_info(0, i) for i in range(n_in.value)]
+        self.output_info = [self._io_info(1, i) for i in range(n_out.value)]
+
+    def __del__(self):
+        h = getattr(self, "_h", None)
+        if h is not None and lib is not None:
+            lib.knhip_executor_free(h)
+            self._h = None
+
+    def _io_info(self, is_output, i):
+        dtype, rank = c_int(), c_size_t()
+        check(lib.knhip_executor_io_info(self._h, is_output, i, byref(dtype), byref(rank), None, 0))
+        dims = (c_size_t * max(rank.value, 1))()
+        check(lib.knhip_executor_io_info(self._h, is_output, i, byref(dtype), byref(rank), dims, rank.value))
+        return DType(dtype.value), [dims[k] for k in range(rank.value)]
+
+    def evaluate(self, inputs):
+        """Dense numpy arrays in, freshly allocated numpy arrays out. Shapes and dtypes are checked like
+        executor.rs:118-127 does."""
+        if len(inputs) != len(self.input_info):
+            raise KnError(f"Wrong input count: expected {len(self.input_info)}, got {len(inputs)}")
+        arrays = []
+        for i, (x, (dtype, dims)) in enumerate(zip(inputs, self.input_info)):
+            x = np.asarray(x)
+            if list(x.shape) != dims:
+                raise KnError(f"Wrong shape for input {i}: expected {dims}, got {list(x.shape)}")
+            if x.dtype != dtype.numpy:
+                raise KnError(f"Wrong dtype for input {i}: expected {dtype.name}, got {x.dtype}")
+            arrays.append(np.ascontiguousarray(x))
+        outputs = [np.empty(dims, dtype.numpy) for dtype, dims in self.output_info]
+        n_in, n_out = len(arrays), len(outputs)
+        in_ptrs = (c_void_p * max(n_in, 1))(*[a.ctypes.data for a in arrays])
+        in_bytes = (c_size_t * max(n_in, 1))(*[a.nbytes for a in arrays])
+        out_ptrs = (c_void_p * max(n_out, 1))(*[a.ctypes.data for a in outputs])
+        out_bytes = (c_size_t * max(n_out, 1))(*[a.nbytes for a in outputs])
+        check(lib.knhip_executor_evaluate(self._h, in_ptrs, in_bytes, n_in, out_ptrs, out_bytes, n_out))
+        return outputs
+
+    def run_async(self):
+        check(lib.knhip_executor_run_async(self._h))
+
+    def synchronize(self):
+        check(lib.knhip_executor_synchronize(self._h))
+
+    def input_ptr(self, i):
+        p = c_void_p()
+        check(lib.knhip_executor_input_ptr(self._h, i, byref(p)))
+        return p.value
+
+    def output_ptr(self, i):
+        p = c_void_p()
+        check(lib.knhip_executor_output_ptr(self._h, i, byref(p)))
+        return p.value
+
+    def stream(self):
+        p = c_void_p()
+        check(lib.knhip_executor_stream(self._h, byref(p)))
+        return p.value or 0
+
+    def set_profile(self, enabled):
+        check(lib.knhip_executor_set_profile(self._h, int(enabled)))
+
+    def last_profile(self):
+        available, raw = c_int(), ProfileT()
+        check(lib.knhip_executor_last_profile(self._h, byref(available), byref(raw)))
+        if not available.value:
+            return None
+        buf = (c_float * max(raw.step_count, 1))()
+        check(lib.knhip_executor_profile_step_seconds(self._h, buf, raw.step_count))
+        text = get_string(lib.knhip_executor_profile_str, self._h)
+        return Profile(raw, [buf[i] for i in range(raw.step_count)], text)
+
+    @property
+    def mem_usage(self):
+        u = MemUsageT()
+        check(lib.knhip_executor_mem_usage(self._h, byref(u)))
+        return {name: getattr(u, name) for name, _ in MemUsageT._fields_}
+
+    def step_count(self):
+        n = c_size_t()
+        check(lib.knhip_executor_step_count(self._h, byref(n)))
+        return n.value
+
+    def step_kinds(self):
+        kinds = []
+        for i in range(self.step_count()):
+            k = c_int()
+            check(lib.knhip_executor_step_kind(self._h, i, byref(k)))
+            kinds.append(STEP_KINDS[k.value])
+        return kinds
+
+    def step_str(self, i):
+        return get_string(lib.knhip_executor_step_str, self._h, i)
+
+    def step_source(self, i):
+        return get_string(lib.knhip_executor_step_source, self._h, i)
+
+    def __str__(self):
+        return get_string(lib.knhip_executor_str, self._h)
+
+
+def compile_stats():
+    a, b, c = c_size_t(), c_size_t(), c_size_t()
+    check(lib.knhip_compile_stats(byref(a), byref(b), byref(c)))
+    return {"compiled": a.value, "memory_hits": b.value, "disk_hits": c.value}
+
+
+class PreparedGraph:
+    """kn-runtime/src/lib.rs:104-126 for the `Hip` arm."""
+
+    def __init__(self, executor):
+        self.executor = executor
+
+    def eval(self, inputs):
+        return self.executor.evaluate(inputs)
+
+
+class Device:
+    """kn-runtime/src/lib.rs:68-102; only the GPU arm exists in this package: there is no CPU execution path."""
+
+    def __init__(self, hip_device):
+        self.hip = hip_device
+
+    @staticmethod
+    def best():
+        if HipDevice.count() == 0:
+            raise KnError("no HIP device available and this package has no CPU executor")
+        return Device(HipDevice(0))
+
+    @staticmethod
+    def parse(text):
+        """Device strings as kn-python accepts them (kn-python/src/lib.rs:139-162), with `hip` for `cuda`."""
+        if text in ("best", "hip"):
+            return Device.best()
+        if text.startswith("hip:"):
+            return Device(HipDevice(int(text[4:])))
+        raise KnError(f"Invalid device string '{text}', expected 'best', 'hip' or 'hip:N'")
+
+    def prepare(self, graph, batch_size):
+        return PreparedGraph(HipExecutor(self.hip, graph, batch_size))

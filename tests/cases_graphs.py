@@ -1,0 +1,830 @@
+"""Graph test cases mirroring kn-cuda-eval/tests/root/graphs.rs (line numbers in each docstring).
+
+Every case returns `(graph, batch_size, inputs, expected_or_None)`. Expected values are the ones the reference's
+test holds; where the reference passes `None` the CPU path is the oracle, so any seeded input keeps the intent.
+"""
+import itertools
+
+import numpy as np
+
+from kyanite_amd import BATCH, BinaryOp, DType, Graph, OpKind, REDUCE_ALL, ReduceOp, Size, UnaryOp, optimize_graph
+from runner import linspace_tensor, linspace_vec, range_vec, rng_tensor
+
+CASES = {}
+
+
+def case(fn):
+    CASES[fn.__name__] = fn
+    return fn
+
+
+def f32(shape, data):
+    return np.asarray(data, dtype=np.float32).reshape(shape)
+
+
+@case
+def empty():
+    """graphs.rs:17-19"""
+    return Graph(), 8, [], []
+
+
+@case
+def copy():
+    """graphs.rs:22-41"""
+    g = Graph()
+    fixed = g.input([10])
+    batch = g.input([BATCH])
+    g.output_all([fixed, batch])
+    a, b = linspace_tensor(10), linspace_tensor(8)
+    return g, 8, [a, b], [a, b]
+
+
+@case
+def slice_():
+    """graphs.rs:44-61"""
+    g = Graph()
+    x = g.input([10, 4])
+    indexed = g.index(x, 1, 0)
+    g.output_all([indexed, g.slice(x, 0, 0, 2), g.slice(indexed, 0, 0, 2)])
+    return g, 0, [linspace_tensor(10, 4)], None
+
+
+@case
+def flip():
+    """graphs.rs:64-90, expected values from the reference"""
+    g = Graph()
+    x = g.constant([2, 3], [0.0, 1.0, 2.0, 3.0, 4.0, 5.0])
+    first_once = g.flip(x, 0)
+    first_twice = g.flip(first_once, 0)
+    other_once = g.flip(x, 1)
+    other_twice = g.flip(other_once, 1)
+    combined = g.flip(first_once, 1)
+    g.output_all([first_once, first_twice, other_once, other_twice, combined])
+    expected = [
+        f32((2, 3), [3, 4, 5, 0, 1, 2]), f32((2, 3), [0, 1, 2, 3, 4, 5]), f32((2, 3), [2, 1, 0, 5, 4, 3]),
+        f32((2, 3), [0, 1, 2, 3, 4, 5]), f32((2, 3), [5, 4, 3, 2, 1, 0]),
+    ]
+    return g, 0, [], expected
+
+
+@case
+def flip_conv():
+    """graphs.rs:93-104"""
+    g = Graph()
+    x = g.input([2, 4, 8, 8])
+    flipped = g.flip(x, 3)
+    w = g.constant([4, 4, 3, 3], linspace_vec(4 * 4 * 3 * 3))
+    g.output(g.conv(flipped, w, 1, 1, 1, 1))
+    return g, 0, [linspace_tensor(2, 4, 8, 8)], None
+
+
+@case
+def repeat():
+    """graphs.rs:107-122"""
+    g = Graph()
+    x = g.input([2, 3])
+    g.output_all([g.repeat(x, 0, 0), g.repeat(x, 0, 2), g.repeat(x, 1, 0), g.repeat(x, 1, 2)])
+    return g, 0, [rng_tensor(np.random.default_rng(0), 2, 3)], None
+
+
+@case
+def repeat_interleave():
+    """graphs.rs:125-138"""
+    g = Graph()
+    x = g.input([2, 3])
+    g.output_all([g.repeat_interleave(x, 0, 0), g.repeat_interleave(x, 0, 2), g.repeat_interleave(x, 1, 0),
+                  g.repeat_interleave(x, 1, 2)])
+    return g, 0, [rng_tensor(np.random.default_rng(0), 2, 3)], None
+
+
+@case
+def repeat_manual():
+    """graphs.rs:141-158, expected values from the reference"""
+    g = Graph()
+    x = g.input([3])
+    g.output_all([g.repeat(x, 0, 2), g.repeat_interleave(x, 0, 2)])
+    return g, 0, [f32((3,), [1, 2, 3])], [f32((6,), [1, 2, 3, 1, 2, 3]), f32((6,), [1, 1, 2, 2, 3, 3])]
+
+
+@case
+def gather_simple_axis_0():
+    """graphs.rs:161-172"""
+    g = Graph()
+    x = g.constant([2, 3], [7.0, 7.1, 7.2, 7.3, 7.4, 7.5])
+    index = g.constant([4], np.array([0, 1, 1, 0], np.uint32))
+    g.output(g.gather(x, 0, index))
+    return g, 0, [], [f32((4, 3), [7.0, 7.1, 7.2, 7.3, 7.4, 7.5, 7.3, 7.4, 7.5, 7.0, 7.1, 7.2])]
+
+
+@case
+def gather_simple_axis_1():
+    """graphs.rs:175-185"""
+    g = Graph()
+    x = g.constant([2, 3], [7.0, 7.1, 7.2, 7.3, 7.4, 7.5])
+    index = g.constant([4], np.array([0, 2, 1, 0], np.uint32))
+    g.output(g.gather(x, 1, index))
+    return g, 0, [], [f32((2, 4), [7.0, 7.2, 7.1, 7.0, 7.3, 7.5, 7.4, 7.3])]
+
+
+@case
+def gather_complex_axis_0():
+    """graphs.rs:188-199"""
+    g = Graph()
+    x = g.input([3, 2])
+    indices = g.constant([2, 2], np.array([0, 1, 1, 2], np.uint32))
+    g.output(g.gather(x, 0, indices))
+    return (g, 0, [f32((3, 2), [1.0, 1.2, 2.3, 3.4, 4.5, 5.7])],
+            [f32((2, 2, 2), [1.0, 1.2, 2.3, 3.4, 2.3, 3.4, 4.5, 5.7])])
+
+
+@case
+def gather_complex_axis_1():
+    """graphs.rs:202-213"""
+    g = Graph()
+    x = g.input([3, 3])
+    indices = g.constant([1, 2], np.array([0, 2], np.uint32))
+    g.output(g.gather(x, 1, indices))
+    return (g, 0, [f32((3, 3), [1.0, 1.2, 1.9, 2.3, 3.4, 3.9, 4.5, 5.7, 5.9])],
+            [f32((3, 1, 2), [1.0, 1.9, 2.3, 3.9, 4.5, 5.9])])
+
+
+@case
+def gather_size_0():
+    """graphs.rs:216-233"""
+    g = Graph()
+    x = g.input([8, 4])
+    indices = g.constant([0], np.array([], np.uint32))
+    o0 = g.gather(x, 0, indices)
+    o1 = g.gather(x, 1, indices)
+    g.output_all([o0, o1])
+    assert g[o0].shape == [0, 4] and g[o1].shape == [8, 0]
+    return g, 0, [linspace_tensor(8, 4)], None
+
+
+@case
+def gather_as_index():
+    """graphs.rs:236-259: a gather with a single constant index has to become a slice"""
+    g = Graph()
+    x = g.input([16, 8, 4])
+    index = g.scalar(4, DType.U32)
+    indices = g.view(index, [1])
+    indices_repeat = g.broadcast(indices, [3])
+    g.output_all([g.gather(x, 1, indices), g.gather(x, 1, indices_repeat)])
+    for v in g.values():
+        assert g[v].op != OpKind.GATHER, "gather should have been replaced by an index operation"
+    return g, 0, [rng_tensor(np.random.default_rng(0), 16, 8, 4)], None
+
+
+@case
+def gather_real():
+    """gather with non constant indices, several index dtypes (not in the reference; its kernel is generic in the
+    index type, gather.rs:30-129)"""
+    g = Graph()
+    x = g.input([5, 7, 3])
+    i8 = g.input([4], DType.I8)
+    u64 = g.input([6], DType.U64)
+    g.output_all([g.gather(x, 0, i8), g.gather(x, 1, u64), g.gather(x, 2, i8)])
+    rng = np.random.default_rng(1)
+    return (g, 0, [rng_tensor(rng, 5, 7, 3), np.array([0, 2, 1, 2], np.int8), np.array([6, 0, 3, 3, 1, 5], np.uint64)], None)
+
+
+@case
+def linear():
+    """graphs.rs:262-283, expected values from the reference"""
+    g = Graph()
+    x = g.input([1, 4])
+    w = g.constant([2, 4], range_vec(8))
+    b = g.constant([1, 2], [-10.0, 10.0])
+    lin = g.linear(x, w)
+    g.output_all([lin, g.add(lin, b)])
+    return g, 0, [f32((1, 4), [0, 1, 2, 3])], [f32((1, 2), [14, 38]), f32((1, 2), [4, 48])]
+
+
+@case
+def linear_sliced():
+    """graphs.rs:286-297"""
+    g = Graph()
+    left = g.input([8, 4])
+    left_sliced = g.slice(left, 0, 0, 8, 2)
+    right = g.input([4, 3])
+    g.output(g.mat_mul(left_sliced, right))
+    return g, 0, [linspace_tensor(8, 4), linspace_tensor(4, 3)], None
+
+
+@case
+def mat_mul_broadcast():
+    """graphs.rs:300-335"""
+    shapes = [([4, 2], [2, 3], [4, 3]), ([8, 4, 2], [2, 3], [8, 4, 3]), ([4, 2], [8, 2, 3], [8, 4, 3]),
+              ([8, 4, 2], [8, 2, 3], [8, 4, 3]), ([1, 1, 1, 4, 2], [8, 1, 2, 3], [1, 8, 1, 4, 3])]
+    rng = np.random.default_rng(0)
+    g = Graph()
+    inputs = []
+    for ls, rs, os_ in shapes:
+        inputs += [rng_tensor(rng, *ls), rng_tensor(rng, *rs)]
+        result = g.mat_mul(g.input(ls), g.input(rs))
+        assert g[result].shape == os_
+        g.output(result)
+    return g, 0, inputs, None
+
+
+def _mat_mul_transpose(ta, tb):
+    g = Graph()
+    sa, sb = [4, 5, 6], [4, 6, 3]
+    if ta:
+        sa = [4, 6, 5]
+    if tb:
+        sb = [4, 3, 6]
+    a = g.constant(sa, linspace_vec(4 * 5 * 6))
+    b = g.constant(sb, linspace_vec(4 * 6 * 3))
+    if ta:
+        a = g.permute(a, [0, 2, 1])
+    if tb:
+        b = g.permute(b, [0, 2, 1])
+    result = g.batched_mat_mul(a, b)
+    assert g[result].shape == [4, 5, 3]
+    g.output(result)
+    return g, 0, [], None
+
+
+for _ta, _tb in itertools.product([True, False], repeat=2):
+    CASES[f"mat_mul_transpose_{int(_ta)}{int(_tb)}"] = (lambda ta=_ta, tb=_tb: _mat_mul_transpose(ta, tb))  # graphs.rs:338-376
+
+
+@case
+def horizontal_1x1_conv():
+    """graphs.rs:379-390"""
+    g = Graph()
+    x = g.constant([2, 4, 1, 8], linspace_vec(2 * 4 * 8))
+    f = g.constant([3, 4, 1, 1], linspace_vec(3 * 4))
+    out = g.conv(x, f, 1, 1, 0, 0)
+    assert g[out].shape == [2, 3, 1, 8]
+    g.output(out)
+    return g, 0, [], None
+
+
+@case
+def vertical_1x1_conv():
+    """graphs.rs:393-404"""
+    g = Graph()
+    x = g.constant([2, 4, 8, 1], linspace_vec(2 * 4 * 8))
+    f = g.constant([3, 4, 1, 1], linspace_vec(3 * 4))
+    out = g.conv(x, f, 1, 1, 0, 0)
+    assert g[out].shape == [2, 3, 8, 1]
+    g.output(out)
+    return g, 0, [], None
+
+
+@case
+def fuse_clamp():
+    """graphs.rs:407-425, expected values from the reference"""
+    g = Graph()
+    curr = g.input([BATCH])
+    inf = float("inf")
+    curr = g.clamp(curr, -5.0, inf)
+    curr = g.clamp(curr, -inf, 2.0)
+    curr = g.clamp(curr, 0.0, 1.0)
+    curr = g.clamp(curr, -1.0, 2.0)
+    g.output(curr)
+    return g, 5, [f32((5,), [-2.0, 0.0, 0.5, 1.0, 2.0])], [f32((5,), [0.0, 0.0, 0.5, 1.0, 1.0])]
+
+
+def _ele_broadcast(op):
+    g = Graph()
+    left = g.constant([2, 3, 4], linspace_vec(24))
+    for shp in ([], [1, 1, 1], [2, 3, 4], [2, 1, 4]):
+        size = int(np.prod(shp)) if shp else 1
+        right = g.constant(shp, linspace_vec(size))
+        g.output(g.binary(op, left, right))
+    return g, 0, [], None
+
+
+for _op in (BinaryOp.ADD, BinaryOp.SUB, BinaryOp.MUL, BinaryOp.MIN, BinaryOp.MAX, BinaryOp.DIV):
+    CASES[f"ele_broadcast_{_op.name.lower()}"] = (lambda op=_op: _ele_broadcast(op))  # graphs.rs:428-452 (+ div)
+
+
+@case
+def add_broadcast():
+    """graphs.rs:455-473, expected values from the reference"""
+    g = Graph()
+    left = g.constant([2, 2, 2], [0.0, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0])
+    right = g.constant([1, 2, 2], [0.0, 1.0, 2.0, 3.0])
+    scalar = g.constant([], [10.0])
+    g.output_all([g.add(left, right), g.add(right, left), g.add(right, scalar)])
+    e01 = f32((2, 2, 2), [0, 2, 4, 6, 4, 6, 8, 10])
+    return g, 0, [], [e01, e01, f32((1, 2, 2), [10, 11, 12, 13])]
+
+
+@case
+def affine_single_element():
+    """graphs.rs:476-502, closed form from the reference"""
+    x = f32((8, 1, 1, 1), range_vec(8))
+    expected = ((x + 1.0) * 2.0 * 10.0 + 3.0) * 4.0
+    g = Graph()
+    cs = [1, 1, 1, 1]
+    bias_0, scale_0, filt = g.constant(cs, [1.0]), g.constant(cs, [2.0]), g.constant(cs, [10.0])
+    bias_1, scale_1 = g.constant(cs, [3.0]), g.constant(cs, [4.0])
+    curr = g.input([8, 1, 1, 1])
+    curr = g.mul(g.add(curr, bias_0), scale_0)
+    curr = g.conv(curr, filt, 1, 1, 0, 0)
+    curr = g.mul(g.add(curr, bias_1), scale_1)
+    g.output(curr)
+    return g, 0, [x], [expected.astype(np.float32)]
+
+
+@case
+def affine_add_twice():
+    """graphs.rs:505-523"""
+    g = Graph()
+    x = g.input([BATCH, 1, 1, 1])
+    w1, w2 = g.constant([1, 1, 1, 1], [1.0]), g.constant([1, 1, 1, 1], [2.0])
+    g.output(g.add(g.add(x, w1), w2))
+    return g, 2, [f32((2, 1, 1, 1), [0, 1])], [f32((2, 1, 1, 1), [3, 4])]
+
+
+@case
+def affine_single_div():
+    """graphs.rs:526-536"""
+    g = Graph()
+    left = g.constant([2, 3], range_vec(6))
+    right = g.scalar(2.0)
+    g.output(g.binary(BinaryOp.DIV, left, right))
+    return g, 0, [], [f32((2, 3), [0.0, 0.5, 1.0, 1.5, 2.0, 2.5])]
+
+
+@case
+def affine_multiple_channels():
+    """graphs.rs:539-564"""
+    x = f32((8, 3, 1, 1), range_vec(24))
+    g = Graph()
+    bias_0 = g.constant([1, 3, 1, 1], [1.0, 2.0, 3.0])
+    scale_0 = g.constant([1, 3, 1, 1], [2.0, 3.0, 4.0])
+    filt = g.constant([2, 3, 1, 1], [10.0, 20.0, 30.0, 40.0, 50.0, 60.0])
+    bias_1 = g.constant([1, 2, 1, 1], [3.0, 4.0])
+    scale_1 = g.constant([1, 2, 1, 1], [4.0, 5.0])
+    curr = g.input([8, 3, 1, 1])
+    curr = g.mul(g.add(curr, bias_0), scale_0)
+    curr = g.conv(curr, filt, 1, 1, 0, 0)
+    curr = g.mul(g.add(curr, bias_1), scale_1)
+    g.output(curr)
+    # independent closed form (numpy, f64)
+    xb = (x.astype(np.float64)[:, :, 0, 0] + [1, 2, 3]) * [2, 3, 4]
+    w = np.array([[10, 20, 30], [40, 50, 60]], np.float64)
+    expected = ((xb @ w.T + [3, 4]) * [4, 5]).astype(np.float32).reshape(8, 2, 1, 1)
+    return g, 0, [x], [expected]
+
+
+@case
+def conv_padding():
+    """graphs.rs:567-592"""
+    g = Graph()
+    i0 = g.input([1, 1, 1, 1])
+    i1 = g.input([1, 1, 8, 8])
+    filt = g.constant([1, 1, 3, 3], range_vec(9))
+    g.output_all([g.conv(i0, filt, 1, 1, 1, 1), g.conv(i0, filt, 1, 1, 4, 4), g.conv(i1, filt, 1, 1, 1, 1),
+                  g.conv(i1, filt, 1, 1, 4, 1)])
+    return g, 0, [f32((1, 1, 1, 1), [1.0]), linspace_tensor(1, 1, 8, 8)], None
+
+
+@case
+def affine_padding():
+    """graphs.rs:595-613"""
+    g = Graph()
+    filt = g.constant([5, 3, 3, 3], linspace_vec(5 * 27))
+    bias_0 = g.constant([1, 3, 1, 1], linspace_vec(3))
+    bias_1 = g.constant([1, 5, 1, 1], linspace_vec(5))
+    curr = g.input([8, 3, 8, 8])
+    curr = g.add(curr, bias_0)
+    curr = g.conv(curr, filt, 1, 1, 1, 1)
+    curr = g.add(curr, bias_1)
+    g.output(curr)
+    return g, 0, [linspace_tensor(8, 3, 8, 8)], None
+
+
+def _channel_batchnorm(g, x):
+    """graphs.rs:645-661"""
+    c = g[x].shape[1].fixed_factor
+    cs = [1, c, 1, 1]
+    mean, var, scale, bias = (g.constant(cs, linspace_vec(c)) for _ in range(4))
+    curr = g.add(x, mean)
+    curr = g.mul(curr, var)
+    curr = g.mul(curr, scale)
+    return g.add(curr, bias)
+
+
+@case
+def pre_act_resnet():
+    """graphs.rs:616-643"""
+    g = Graph()
+    x = g.input([8, 3, 8, 8])
+    f_init = g.constant([5, 3, 3, 3], linspace_vec(5 * 27))
+    f_tower = g.constant([5, 5, 3, 3], linspace_vec(5 * 45))
+    f_policy = g.constant([2, 5, 1, 1], linspace_vec(10))
+    tower = g.conv(x, f_init, 1, 1, 1, 1)
+    for _ in range(2):
+        curr = _channel_batchnorm(g, tower)
+        curr = g.clamp(curr, 0.0, 6.0)
+        curr = g.conv(curr, f_tower, 1, 1, 1, 1)
+        curr = g.clamp(curr, 0.0, 6.0)
+        curr = g.conv(curr, f_tower, 1, 1, 1, 1)
+        tower = g.add(curr, tower)
+    policy = g.conv(tower, f_policy, 1, 1, 0, 0)
+    g.output_all([tower, policy])
+    return g, 0, [linspace_tensor(8, 3, 8, 8)], None
+
+
+@case
+def fuse_res():
+    """graphs.rs:664-687"""
+    g = Graph()
+    rng = np.random.default_rng(0)
+    x = g.input([10, 4, 8, 8])
+    other = g.input([10, 4, 8, 8])
+    filt = g.constant([4, 4, 3, 3], linspace_vec(4 * 36))
+    curr = g.conv(x, filt, 1, 1, 1, 1)
+    curr = g.add(curr, other)
+    curr = g.clamp(curr, 0.0, float("inf"))
+    g.output(curr)
+    return g, 0, [rng_tensor(rng, 10, 4, 8, 8), rng_tensor(rng, 10, 4, 8, 8)], None
+
+
+@case
+def concat():
+    """graphs.rs:690-701"""
+    g = Graph()
+    a = g.constant([2, 3, 4], linspace_vec(24))
+    b = g.constant([2, 1, 4], linspace_vec(8))
+    c = g.constant([2, 8, 4], linspace_vec(64))
+    g.output(g.concat([a, b, c], 1))
+    return g, 0, [], None
+
+
+@case
+def pad():
+    """graphs.rs:704-714"""
+    g = Graph()
+    a = g.constant([2, 3, 4], linspace_vec(24))
+    zero = g.scalar(0.0)
+    g.output(g.pad(a, [(0, 0), (1, 2), (2, 0)], zero))
+    expected = np.pad(linspace_vec(24).reshape(2, 3, 4), [(0, 0), (1, 2), (2, 0)])
+    return g, 0, [], [expected]
+
+
+@case
+def permute():
+    """graphs.rs:719-731: all 24 permutations of a rank-4 tensor; expected from numpy.transpose"""
+    g = Graph()
+    data = range_vec(120).reshape(2, 3, 4, 5)
+    a = g.constant([2, 3, 4, 5], data)
+    expected = []
+    for p in itertools.permutations(range(4)):
+        g.output(g.permute(a, list(p)))
+        expected.append(np.ascontiguousarray(data.transpose(p)))
+    return g, 0, [], expected
+
+
+@case
+def chain():
+    """graphs.rs:734-760, expected values from the reference"""
+    child = Graph()
+    cx = child.input([2])
+    cw = child.constant([1], [2.0])
+    child.output(child.mul(cx, cw))
+    parent = Graph()
+    px = parent.input([2])
+    pw = parent.constant([1], [3.0])
+    pz = parent.add(px, pw)
+    py = parent.call(child, [pz])
+    assert len(py) == 1
+    parent.output(py[0])
+    return parent, 0, [f32((2,), [1, 2])], [f32((2,), [8, 10])]
+
+
+@case
+def repeated_conv():
+    """graphs.rs:763-785"""
+    g = Graph()
+    w0 = g.constant([4, 4, 3, 3], np.linspace(-1, 1, 144).astype(np.float32))
+    w1 = g.constant([4, 4, 3, 3], np.linspace(-2, 2, 144).astype(np.float32))
+    x = g.input([BATCH, 4, 8, 8])
+    a = x
+    for _ in range(4):
+        a = g.conv(a, w0, 1, 1, 1, 1)
+    b = x
+    for _ in range(4):
+        b = g.conv(b, w1, 1, 1, 1, 1)
+    g.output_all([a, b])
+    return g, 2, [linspace_tensor(2, 4, 8, 8)], None
+
+
+@case
+def strided_conv():
+    """graphs.rs:788-800"""
+    g = Graph()
+    rng = np.random.default_rng(0)
+    x = g.input([BATCH, 3, 8, 8])
+    filt = g.constant([16, 3, 3, 3], rng_tensor(rng, 16 * 27))
+    out = g.conv(x, filt, 2, 4, 1, 1)
+    assert g[out].shape == [BATCH, 16, 4, 2]
+    g.output(out)
+    return g, 4, [rng_tensor(rng, 4, 3, 8, 8)], None
+
+
+@case
+def softmax():
+    """graphs.rs:803-819, includes -inf and a scaled input"""
+    g = Graph()
+    x = g.input([3, 3])
+    r0 = g.softmax(x, 0)
+    r1 = g.softmax(x, 1)
+    scaled = g.mul(x, g.scalar(2.0))
+    r2 = g.softmax(scaled, 0)
+    g.output_all([r0, r1, r2])
+    return g, 0, [f32((3, 3), [0.0, 0.0, 0.0, 1.0, 2.0, 3.0, 1.0, -1.0, -np.inf])], None
+
+
+@case
+def reduce_easy():
+    """graphs.rs:822-836: all reduce ops on both axes, -inf included"""
+    g = Graph()
+    x = g.input([4, 3])
+    for axis in (0, 1):
+        for op in REDUCE_ALL:
+            g.output(g.reduce(x, [axis], op))
+    return g, 0, [f32((4, 3), [0.0, 0.0, 0.0, 1.0, 2.0, 3.0, 1.0, -1.0, -np.inf, 0.0, 1.0, 2.0])], None
+
+
+@case
+def reduce_mixed():
+    """graphs.rs:839-848"""
+    g = Graph()
+    x = g.input([12, 3, 7, 9, 13])
+    mixed = g.permute(x, [0, 3, 2, 1, 4])
+    g.output(g.reduce(mixed, [1, 2, 4], ReduceOp.SUM))
+    return g, 0, [linspace_tensor(12, 3, 7, 9, 13)], None
+
+
+@case
+def reduce_single():
+    """graphs.rs:851-859"""
+    g = Graph()
+    x = g.input([4])
+    g.output(g.reduce(x, [0], ReduceOp.SUM))
+    return g, 0, [linspace_tensor(4)], None
+
+
+@case
+def softmax_single():
+    """graphs.rs:862-870"""
+    g = Graph()
+    x = g.input([4])
+    g.output(g.softmax(x, 0))
+    return g, 0, [linspace_tensor(4)], None
+
+
+def layernorm_pattern_graph():
+    """graphs.rs:873-905: the mean / variance / sqrt / div pattern the optimizer has to recognise"""
+    g = Graph()
+    eps, axis = 1e-5, 2
+    x = g.input([BATCH, 8, 32])
+    reduced = [BATCH, 8, 1]
+    const_2 = g.scalar(2.0)
+    const_eps = g.scalar(eps)
+    mean = g.view(g.reduce(x, [axis], ReduceOp.MEAN), reduced)
+    zeroed = g.sub(x, mean)
+    pw = g.pow(zeroed, const_2)
+    var = g.view(g.reduce(pw, [axis], ReduceOp.MEAN), reduced)
+    var = g.add(var, const_eps)
+    std = g.unary(UnaryOp.SQRT, var)
+    g.output(g.binary(BinaryOp.DIV, zeroed, std))
+    return g
+
+
+@case
+def layernorm_fused():
+    """graphs.rs:873-929: optimized graph must be exactly [Input, Layernorm{axis 2, eps 1e-5}]"""
+    g = layernorm_pattern_graph()
+    opt = optimize_graph(g)
+    values = opt.values()
+    assert len(values) == 2, str(opt)
+    assert opt[values[0]].op == OpKind.INPUT
+    info = opt[values[1]]
+    assert info.op == OpKind.LAYERNORM and info.operands == [values[0]] and info.axes == [2]
+    assert info.eps == np.float32(1e-5)
+    return g, 2, [linspace_tensor(2, 8, 32)], None
+
+
+@case
+def scalar_scalar():
+    """graphs.rs:932-940"""
+    g = Graph()
+    x = g.input([])
+    g.output(g.unary(UnaryOp.EXP, x))
+    return g, 0, [f32((), [2.0])], None
+
+
+@case
+def split_stride():
+    """graphs.rs:943-959"""
+    g = Graph()
+    n = 4
+    x = g.input([2 * n])
+    g.output(g.slice(x, 0, 1, 2 * n + 1, 2))
+    data = rng_tensor(np.random.default_rng(0), 2 * n)
+    return g, 0, [data], [data[1::2].copy()]
+
+
+def _complex_multiply(new_axis):
+    """graphs.rs:971-1065, expected from the reference's closed form"""
+    batch, n, axis = 8, 32, 1
+    g = Graph()
+    a = g.input([batch, n * 2])
+    b = g.input([batch, n * 2])
+    if new_axis:
+        a_split, b_split = g.view(a, [batch, n, 2]), g.view(b, [batch, n, 2])
+        ar = g.view(g.slice(a_split, axis + 1, 0, 1), [batch, n])
+        ai = g.view(g.slice(a_split, axis + 1, 1, 2), [batch, n])
+        br = g.view(g.slice(b_split, axis + 1, 0, 1), [batch, n])
+        bi = g.view(g.slice(b_split, axis + 1, 1, 2), [batch, n])
+    else:
+        ar = g.slice(a, axis, 0, n * 2, 2)
+        ai = g.slice(a, axis, 1, n * 2 + 1, 2)
+        br = g.slice(b, axis, 0, n * 2, 2)
+        bi = g.slice(b, axis, 1, n * 2 + 1, 2)
+    r = g.sub(g.mul(ar, br), g.mul(ai, bi))
+    i = g.add(g.mul(ar, bi), g.mul(ai, br))
+    extra = g.concat([g.view(r, [batch, n, 1]), g.view(i, [batch, n, 1])], axis + 1)
+    g.output(g.view(extra, [batch, n * 2]))
+    rng = np.random.default_rng(0)
+    ia, ib = rng_tensor(rng, batch, n * 2), rng_tensor(rng, batch, n * 2)
+    out = np.empty((batch, n * 2), np.float32)
+    out[:, 0::2] = ia[:, 0::2] * ib[:, 0::2] - ia[:, 1::2] * ib[:, 1::2]
+    out[:, 1::2] = ia[:, 0::2] * ib[:, 1::2] + ia[:, 1::2] * ib[:, 0::2]
+    return g, 0, [ia, ib], [out]
+
+
+CASES["complex_multiply_stride"] = lambda: _complex_multiply(False)
+CASES["complex_multiply_new_axis"] = lambda: _complex_multiply(True)
+
+
+# ---- cases beyond the reference's list: shapes that exercise the other kernel specialisations
+
+@case
+def layernorm_affine():
+    """layernorm followed by gamma / beta on the normalised axis: planned as ONE row kernel"""
+    g = Graph()
+    rng = np.random.default_rng(3)
+    x = g.input([BATCH, 96])
+    gamma = g.constant([96], (1 + 0.1 * rng.standard_normal(96)).astype(np.float32))
+    beta = g.constant([96], (0.1 * rng.standard_normal(96)).astype(np.float32))
+    y = g.add(g.mul(g.layernorm(x, 1, 1e-5), gamma), beta)
+    g.output(y)
+    return g, 5, [rng.standard_normal((5, 96)).astype(np.float32)], None
+
+
+@case
+def layernorm_residual():
+    """planner.rs:522-552: layernorm(alpha0 * a + alpha1 * b) with equally laid out operands"""
+    g = Graph()
+    rng = np.random.default_rng(4)
+    a = g.input([4, 6, 40])
+    b = g.input([4, 6, 40])
+    s = g.add(g.mul(a, g.scalar(0.5)), b)
+    g.output(g.layernorm(s, 2, 1e-3))
+    g.output(g.layernorm(g.permute(a, [0, 2, 1]), 1, 1e-3))
+    return g, 0, [rng.standard_normal((4, 6, 40)).astype(np.float32), rng.standard_normal((4, 6, 40)).astype(np.float32)], None
+
+
+@case
+def softmax_shapes():
+    """rows shorter than a wave, rows spanning a workgroup, a strided (non innermost) softmax axis, odd lengths"""
+    g = Graph()
+    rng = np.random.default_rng(5)
+    a = g.input([6, 1000])
+    b = g.input([3, 37, 5])
+    c = g.input([2, 4672])
+    g.output_all([g.softmax(a, 1), g.softmax(b, 1), g.softmax(b, 2), g.softmax(c, 1), g.softmax(a, 0)])
+    return g, 0, [rng.standard_normal((6, 1000)).astype(np.float32) * 3, rng.standard_normal((3, 37, 5)).astype(np.float32),
+                  rng.standard_normal((2, 4672)).astype(np.float32)], None
+
+
+@case
+def row_kernel_long():
+    """rows too long to sit in registers: the streaming variant"""
+    g = Graph()
+    rng = np.random.default_rng(6)
+    a = g.input([3, 70001])
+    g.output_all([g.softmax(a, 1), g.layernorm(a, 1, 1e-5)])
+    return g, 0, [rng.standard_normal((3, 70001)).astype(np.float32)], None
+
+
+@case
+def reduce_shapes():
+    """row and column strategies, vector and scalar tails, several dtypes"""
+    g = Graph()
+    rng = np.random.default_rng(7)
+    a = g.input([33, 4096])
+    b = g.input([1000, 7])
+    c = g.input([5, 6, 64], DType.I32)
+    d = g.input([300, 50], DType.F64)
+    outs = [g.reduce(a, [1], ReduceOp.SUM), g.reduce(a, [0], ReduceOp.MAX), g.reduce(a, [0, 1], ReduceOp.MEAN),
+            g.reduce(b, [0], ReduceOp.SUM), g.reduce(b, [1], ReduceOp.MIN), g.reduce(c, [1], ReduceOp.SUM),
+            g.reduce(c, [0, 2], ReduceOp.MAX), g.reduce(c, [2], ReduceOp.PROD), g.reduce(d, [0], ReduceOp.SUM)]
+    g.output_all(outs)
+    return g, 0, [rng.standard_normal((33, 4096)).astype(np.float32), rng.standard_normal((1000, 7)).astype(np.float32),
+                  rng.integers(-3, 4, (5, 6, 64)).astype(np.int32), rng.standard_normal((300, 50))], None
+
+
+@case
+def scalar_dtypes():
+    """integer and bool arithmetic is bit exact: wrapping add / mul, min / max, value and bit casts"""
+    g = Graph()
+    rng = np.random.default_rng(8)
+    a = g.input([257], DType.I8)
+    b = g.input([257], DType.I8)
+    u = g.input([64], DType.U32)
+    f = g.input([64], DType.F32)
+    p = g.input([33], DType.BOOL)
+    q = g.input([33], DType.BOOL)
+    outs = [g.add(a, b), g.mul(a, b), g.binary(BinaryOp.MIN, a, b), g.unary(UnaryOp.NEG, a), g.unary(UnaryOp.ABS, a),
+            g.value_cast(a, DType.U16), g.value_cast(u, DType.F32), g.value_cast(f, DType.I32), g.value_cast(f, DType.U8),
+            g.value_cast(f, DType.I64), g.bit_cast(f, DType.U32), g.bit_cast(u, DType.F32), g.value_cast(f, DType.BOOL),
+            g.add(p, q), g.mul(p, q), g.sub(p, q), g.value_cast(p, DType.F32), g.value_cast(a, DType.F64),
+            g.value_cast(f, DType.F16), g.value_cast(u, DType.I8)]
+    g.output_all(outs)
+    fv = (rng.standard_normal(64) * 1000).astype(np.float32)
+    fv[:6] = [np.nan, np.inf, -np.inf, 3e9, -3e9, 1e20]
+    uv = rng.integers(0, 2 ** 32, 64, dtype=np.uint64).astype(np.uint32)
+    uv[:2] = [0x7fc00000, 0x3f800000]
+    return g, 0, [rng.integers(-128, 128, 257).astype(np.int8), rng.integers(-128, 128, 257).astype(np.int8), uv, fv,
+                  rng.integers(0, 2, 33).astype(np.bool_), rng.integers(0, 2, 33).astype(np.bool_)], None
+
+
+@case
+def strided_scalar():
+    """elementwise work on permuted, flipped, sliced and broadcast operands, and a view that needs a copy"""
+    g = Graph()
+    rng = np.random.default_rng(9)
+    a = g.input([6, 10, 8])
+    b = g.input([8, 10])
+    c = g.input([10, 1])
+    t = g.permute(a, [0, 2, 1])                        # [6, 8, 10]
+    s = g.add(t, g.flip(b, 1))                         # broadcast over the first axis, flipped last axis
+    s = g.mul(s, g.permute(c, [1, 0]))                 # [1, 10] broadcast
+    v = g.view(g.slice(s, 2, 0, 10, 2), [6, 40])       # strided slice, then a view that cannot be a stride edit
+    g.output_all([s, v, g.unary(UnaryOp.TANH, v)])
+    return g, 0, [rng.standard_normal((6, 10, 8)).astype(np.float32), rng.standard_normal((8, 10)).astype(np.float32),
+                  rng.standard_normal((10, 1)).astype(np.float32)], None
+
+
+@case
+def tiny_mlp():
+    """the smallest benchmark configuration: Linear 16->32 + bias, ReLU, Linear 32->10 + bias, softmax"""
+    from kyanite_amd.configs import build_tiny_mlp
+    g, inputs = build_tiny_mlp(seed=0)
+    return g, 8, inputs, None
+
+
+@case
+def attention_block():
+    """matmul -> scaled softmax -> matmul with the [1, 0, 2] permute after the last product (planner.rs:554-567)"""
+    g = Graph()
+    rng = np.random.default_rng(10)
+    heads, seq, dim = 3, 20, 8
+    q = g.input([seq, heads, dim])
+    k = g.input([seq, heads, dim])
+    v = g.input([seq, heads, dim])
+    qh = g.permute(q, [1, 0, 2])
+    kh = g.permute(k, [1, 2, 0])
+    vh = g.permute(v, [1, 0, 2])
+    scores = g.batched_mat_mul(qh, kh)
+    probs = g.softmax(g.mul(scores, g.scalar(1.0 / np.sqrt(dim))), 2)
+    out = g.permute(g.batched_mat_mul(probs, vh), [1, 0, 2])
+    g.output(g.view(out, [seq, heads * dim]))
+    return g, 0, [rng.standard_normal((seq, heads, dim)).astype(np.float32) for _ in range(3)], None
+
+
+@case
+def matmul_sizes():
+    """products that do not line up with the 128 x 128 x 16 tiles, and a broadcast (zero stride) batch operand"""
+    g = Graph()
+    rng = np.random.default_rng(11)
+    a = g.input([2, 130, 70])
+    b = g.input([70, 257])
+    c = g.input([2, 257, 3])
+    ab = g.mat_mul(a, b)
+    g.output_all([ab, g.mat_mul(ab, c)])
+    return g, 0, [rng.standard_normal((2, 130, 70)).astype(np.float32), rng.standard_normal((70, 257)).astype(np.float32),
+                  rng.standard_normal((2, 257, 3)).astype(np.float32)], None
+
+
+@case
+def conv_fused_all():
+    """relu(conv + bias + res) with 130 output channels and 200 positions: partial tiles on both axes"""
+    g = Graph()
+    rng = np.random.default_rng(12)
+    x = g.input([BATCH, 130, 5, 8])
+    w = g.constant([130, 130, 3, 3], (rng.standard_normal((130, 130, 3, 3)) * 0.05).astype(np.float32))
+    bias = g.constant([1, 130, 1, 1], rng.standard_normal(130).astype(np.float32))
+    y = g.relu(g.add(g.add(g.conv(x, w, 1, 1, 1, 1), bias), x))
+    g.output(y)
+    return g, 5, [rng.standard_normal((5, 130, 5, 8)).astype(np.float32)], None
