@@ -13,10 +13,13 @@ from oracle import cpu_eval_graph
 TOLERANCE_ABS_DIFF = 0.001
 TOLERANCE_REL_DIFF = 0.001
 
-# The tighter bar this project states for its own GPU path against the oracle: max relative error with an
-# absolute floor of FLOOR_FRACTION * rms(expected) (needed where sums cross zero).
+# The tighter bar this project states for its own GPU path against the oracle:
+#   max over elements of |actual - expected| / max(|expected|, FLOOR_FRACTION * rms(expected)) <= F32_MAX_REL.
+# The floor is needed because sums that cancel to (almost) zero carry the rounding of their large terms: an f32
+# contraction over K terms is only reproducible to about eps * sqrt(K) of the tensor's scale under reordering,
+# i.e. ~6e-6 * rms for K = 11008, so the floor sits at a tenth of the tensor's rms.
 F32_MAX_REL = 1e-4
-FLOOR_FRACTION = 1e-3
+FLOOR_FRACTION = 0.1
 
 
 def assert_tensors_match(expected, actual, what=""):
