@@ -187,6 +187,10 @@ int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const
 /* run_async (executor.rs:199-258): launch all steps on the executor's stream, no synchronisation */
 int knhip_executor_run_async(knhip_executor *ex);
 int knhip_executor_synchronize(knhip_executor *ex);
+/* The timing loop of the reference's profile_net (kn-cuda-eval/src/bin/profile_net.rs:146-180, `--skip-io`):
+ * `iterations` back-to-back run_async calls bracketed by two HIP events recorded on the executor's stream;
+ * returns the elapsed device time in milliseconds for all iterations together. */
+int knhip_executor_time_runs(knhip_executor *ex, size_t iterations, float *elapsed_ms);
 /* device addresses of the dense input / output tensors inside the arena (pub device_inputs / device_outputs) */
 int knhip_executor_input_ptr(const knhip_executor *ex, size_t index, void **ptr);
 int knhip_executor_output_ptr(const knhip_executor *ex, size_t index, void **ptr);

@@ -1,6 +1,6 @@
 """Loads libknhip.so and declares the C ABI of include/knhip.h for ctypes.
 
-There is no fallback: if the library is missing (run `python -m kyanite_amd.build`) importing fails loudly.
+There is no fallback: if the library is missing (run `python kyanite_amd/build.py`) importing fails loudly.
 """
 import ctypes
 import os
@@ -112,6 +112,7 @@ SIGNATURES = {
     "knhip_executor_evaluate": [E, POINTER(c_void_p), PZ, c_size_t, POINTER(c_void_p), PZ, c_size_t],
     "knhip_executor_run_async": [E],
     "knhip_executor_synchronize": [E],
+    "knhip_executor_time_runs": [E, c_size_t, POINTER(c_float)],
     "knhip_executor_input_ptr": [E, c_size_t, POINTER(c_void_p)],
     "knhip_executor_output_ptr": [E, c_size_t, POINTER(c_void_p)],
     "knhip_executor_stream": [E, POINTER(c_void_p)],
@@ -137,7 +138,7 @@ SPECIAL = {
 
 def _load():
     if not os.path.exists(LIB_PATH):
-        raise ImportError(f"{LIB_PATH} is missing: build it with `python -m kyanite_amd.build` "
+        raise ImportError(f"{LIB_PATH} is missing: build it with `python kyanite_amd/build.py` "
                           "(there is no fallback implementation)")
     lib = ctypes.CDLL(LIB_PATH)
     for name, argtypes in SIGNATURES.items():

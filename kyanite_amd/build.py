@@ -1,6 +1,6 @@
 """Build libknhip.so (host runtime + ahead-of-time gfx950 kernels) in-tree with hipcc.
 
-Usage: python -m kyanite_amd.build [--force]
+Usage: python kyanite_amd/build.py [--force]  (run as a script: importing the package needs the built library)
 """
 import hashlib
 import os

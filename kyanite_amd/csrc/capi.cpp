@@ -584,6 +584,14 @@ int knhip_executor_synchronize(knhip_executor *ex) {
     });
 }
 
+int knhip_executor_time_runs(knhip_executor *ex, size_t iterations, float *elapsed_ms) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && elapsed_ms != nullptr);
+        *elapsed_ms = ex->ex.time_runs(iterations);
+        return KNHIP_OK;
+    });
+}
+
 int knhip_executor_input_ptr(const knhip_executor *ex, size_t index, void **ptr) {
     return guarded([&] {
         KN_REQUIRE(ex != nullptr && ptr != nullptr);

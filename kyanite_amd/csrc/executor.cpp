@@ -129,6 +129,26 @@ void HipExecutor::synchronize() {
     hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
 }
 
+float HipExecutor::time_runs(size_t iterations) {
+    KN_ASSERT(!plan_only_);
+    bool was_profiling = profile_;
+    profile_ = false;
+    hip_check(hipSetDevice(device_), "hipSetDevice");
+    hipEvent_t start, stop;
+    hip_check(hipEventCreate(&start), "hipEventCreate");
+    hip_check(hipEventCreate(&stop), "hipEventCreate");
+    hip_check(hipEventRecord(start, stream_), "hipEventRecord");
+    for (size_t i = 0; i < iterations; i++) run_async();
+    hip_check(hipEventRecord(stop, stream_), "hipEventRecord");
+    hip_check(hipEventSynchronize(stop), "hipEventSynchronize");
+    float ms = 0;
+    hip_check(hipEventElapsedTime(&ms, start, stop), "hipEventElapsedTime");
+    hipEventDestroy(start);
+    hipEventDestroy(stop);
+    profile_ = was_profiling;
+    return ms;
+}
+
 void HipExecutor::launch_step(size_t index) {
     Step &step = plan_.steps[index];
     Launch &l = launches_[index];

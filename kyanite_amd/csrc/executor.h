@@ -37,6 +37,8 @@ public:
     // launch the steps on the executor's stream without any synchronisation (executor.rs:197-258)
     void run_async();
     void synchronize();
+    // `iterations` back-to-back runs timed with events on the executor's stream; elapsed milliseconds in total
+    float time_runs(size_t iterations);
 
     void set_profile(bool on) { profile_ = on; }
     const std::optional<Profile> &last_profile() const { return last_profile_; }

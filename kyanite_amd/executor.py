@@ -108,6 +108,31 @@ class HipExecutor:
     def synchronize(self):
         check(lib.knhip_executor_synchronize(self._h))
 
+    def time_runs(self, iterations):
+        """Device milliseconds for `iterations` back-to-back runs (events on the executor's stream)."""
+        ms = c_float()
+        check(lib.knhip_executor_time_runs(self._h, iterations, byref(ms)))
+        return ms.value
+
+    def upload_input(self, i, array):
+        """Copy a host array into input `i` on the device (for callers that drive `run_async` themselves)."""
+        dtype, dims = self.input_info[i]
+        array = np.ascontiguousarray(array)
+        if list(array.shape) != dims or array.dtype != dtype.numpy:
+            raise KnError(f"Wrong shape or dtype for input {i}")
+        if array.nbytes:
+            check(lib.knhip_memcpy_h2d(self.device, self.input_ptr(i), array.ctypes.data, array.nbytes))
+
+    def download_output(self, i, rows=None):
+        """Copy output `i` (or its first `rows` entries along axis 0) back to the host."""
+        dtype, dims = self.output_info[i]
+        if rows is not None:
+            dims = [min(rows, dims[0])] + dims[1:]
+        out = np.empty(dims, dtype.numpy)
+        if out.nbytes:
+            check(lib.knhip_memcpy_d2h(self.device, out.ctypes.data, self.output_ptr(i), out.nbytes))
+        return out
+
     def input_ptr(self, i):
         p = c_void_p()
         check(lib.knhip_executor_input_ptr(self._h, i, byref(p)))
