@@ -168,10 +168,14 @@ int knhip_graph_optimize(const knhip_graph *g, const knhip_optimizer_settings *s
 /* ---- executor (kn-cuda-eval/src/executor.rs:60-258, kn-runtime/src/lib.rs:85-126) ------------------------------ */
 typedef struct knhip_executor knhip_executor;
 
-/* CudaExecutor::new(device, &graph, batch_size) (executor.rs:61). With plan_only != 0 nothing touches a device:
- * the graph is planned and its kernels are compiled, which works on a machine without a GPU. */
-int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int plan_only, knhip_executor **out);
-int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int plan_only,
+/* CudaExecutor::new(device, &graph, batch_size) (executor.rs:61); `flags` is 0 for the reference's behaviour.
+ * KNHIP_PLAN_ONLY: nothing touches a device, the graph is planned and its kernels are compiled (works on a machine
+ * without a GPU). KNHIP_PRESERVE_INPUTS: input buffers are never reused for later values, for callers that write
+ * the inputs on the device once and then call run_async many times (the reference re-uploads them per evaluate). */
+#define KNHIP_PLAN_ONLY 1
+#define KNHIP_PRESERVE_INPUTS 2
+int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int flags, knhip_executor **out);
+int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int flags,
                                  knhip_executor **out);
 void knhip_executor_free(knhip_executor *ex);
 

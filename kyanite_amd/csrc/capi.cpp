@@ -15,7 +15,8 @@ struct knhip_graph {
 };
 struct knhip_executor {
     HipExecutor ex;
-    knhip_executor(int device, const Graph &g, size_t batch, bool plan_only) : ex(device, g, batch, plan_only) {}
+    knhip_executor(int device, const Graph &g, size_t batch, int flags)
+        : ex(device, g, batch, (flags & KNHIP_PLAN_ONLY) != 0, (flags & KNHIP_PRESERVE_INPUTS) != 0) {}
 };
 
 namespace {
@@ -486,20 +487,20 @@ int knhip_graph_optimize(const knhip_graph *g, const knhip_optimizer_settings *s
 
 // ---------------------------------------------------------------------------------------------- executor
 
-int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int plan_only, knhip_executor **out) {
+int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int flags, knhip_executor **out) {
     return guarded([&] {
         KN_REQUIRE(graph != nullptr && out != nullptr);
-        *out = new knhip_executor(device, graph->graph, batch_size, plan_only != 0);
+        *out = new knhip_executor(device, graph->graph, batch_size, flags);
         return KNHIP_OK;
     });
 }
 
-int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int plan_only,
+int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int flags,
                                  knhip_executor **out) {
     return guarded([&] {
         KN_REQUIRE(blob != nullptr && out != nullptr);
         Graph g = Graph::deserialize(blob, len);
-        *out = new knhip_executor(device, g, batch_size, plan_only != 0);
+        *out = new knhip_executor(device, g, batch_size, flags);
         return KNHIP_OK;
     });
 }

@@ -1,5 +1,12 @@
 #include "executor.h"
 
+// declared here instead of including <hip/hip_ext.h>, whose templates need the HIP compiler
+extern "C" hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalWorkSizeX, uint32_t globalWorkSizeY,
+                                               uint32_t globalWorkSizeZ, uint32_t localWorkSizeX, uint32_t localWorkSizeY,
+                                               uint32_t localWorkSizeZ, size_t sharedMemBytes, hipStream_t hStream,
+                                               void **kernelParams, void **extra, hipEvent_t startEvent, hipEvent_t stopEvent,
+                                               uint32_t flags);
+
 #include <chrono>
 #include <map>
 
@@ -38,10 +45,11 @@ std::string Profile::str() const {
     return ss.str();
 }
 
-HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only)
+HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only, bool preserve_inputs)
     : device_(device), batch_size_(batch_size), plan_only_(plan_only) {
     if (!plan_only) HipDevice::check(device);
     PlannerOptions options;
+    options.preserve_inputs = preserve_inputs;
     plan_ = plan_graph(graph, batch_size, options);
     for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
     if (plan_only) return;
@@ -105,13 +113,14 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
 
 HipExecutor::~HipExecutor() {
     if (plan_only_) return;
-    hipSetDevice(device_);
-    if (stream_) hipStreamSynchronize(stream_);
-    for (void *p : pinned_inputs_) hipHostFree(p);
-    for (void *p : pinned_outputs_) hipHostFree(p);
-    for (hipModule_t m : modules_) hipModuleUnload(m);
-    if (arena_) hipFree(arena_);
-    if (stream_) hipStreamDestroy(stream_);
+    // failures while tearing down are ignored on purpose (the reference does the same in its drop handlers)
+    (void) hipSetDevice(device_);
+    if (stream_) (void) hipStreamSynchronize(stream_);
+    for (void *p : pinned_inputs_) (void) hipHostFree(p);
+    for (void *p : pinned_outputs_) (void) hipHostFree(p);
+    for (hipModule_t m : modules_) (void) hipModuleUnload(m);
+    if (arena_) (void) hipFree(arena_);
+    if (stream_) (void) hipStreamDestroy(stream_);
 }
 
 void *HipExecutor::input_ptr(size_t i) const {
@@ -143,15 +152,25 @@ float HipExecutor::time_runs(size_t iterations) {
     hip_check(hipEventSynchronize(stop), "hipEventSynchronize");
     float ms = 0;
     hip_check(hipEventElapsedTime(&ms, start, stop), "hipEventElapsedTime");
-    hipEventDestroy(start);
-    hipEventDestroy(stop);
+    (void) hipEventDestroy(start);
+    (void) hipEventDestroy(stop);
     profile_ = was_profiling;
     return ms;
 }
 
-void HipExecutor::launch_step(size_t index) {
+void HipExecutor::launch_step(size_t index, hipEvent_t start, hipEvent_t stop) {
     Step &step = plan_.steps[index];
     Launch &l = launches_[index];
+    bool jit = step.kind != StepKind::MatMul && step.kind != StepKind::Conv;
+    if (start && jit && (uint64_t) step.kernel.grid * step.kernel.block <= 0xffffffffull) {
+        // the events are attached to the dispatch itself, so they time the kernel without any launch gaps
+        void *args[] = {l.ptrs.data()};
+        hip_check(hipExtModuleLaunchKernel(l.function, step.kernel.grid * step.kernel.block, 1, 1, step.kernel.block, 1, 1, 0,
+                                           stream_, args, nullptr, start, stop, 0),
+                  "hipExtModuleLaunchKernel");
+        return;
+    }
+    if (start) hip_check(hipEventRecord(start, stream_), "hipEventRecord");
     switch (step.kind) {
         case StepKind::MatMul: hip_check((hipError_t) launch_gemm_f32(step.gemm, stream_), "matmul launch"); break;
         case StepKind::Conv: hip_check((hipError_t) launch_conv_f32(step.conv, stream_), "conv launch"); break;
@@ -162,6 +181,7 @@ void HipExecutor::launch_step(size_t index) {
             break;
         }
     }
+    if (stop) hip_check(hipEventRecord(stop, stream_), "hipEventRecord");
 }
 
 void HipExecutor::run_async() {
@@ -185,9 +205,7 @@ void HipExecutor::run_async() {
     hip_check(hipEventSynchronize(events[2 * n]), "hipEventSynchronize");
     auto start_cpu = clock::now();
     for (size_t si = 0; si < n; si++) {
-        hip_check(hipEventRecord(events[2 * si], stream_), "hipEventRecord");
-        launch_step(si);
-        hip_check(hipEventRecord(events[2 * si + 1], stream_), "hipEventRecord");
+        launch_step(si, events[2 * si], events[2 * si + 1]);
     }
     hip_check(hipEventRecord(events[2 * n + 1], stream_), "hipEventRecord");
     hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
@@ -207,7 +225,7 @@ void HipExecutor::run_async() {
     hip_check(hipEventElapsedTime(&total_ms, events[2 * n], events[2 * n + 1]), "hipEventElapsedTime");
     profile.total_gpu = total_ms * 1e-3f;
     profile.total_cpu = std::chrono::duration<float>(end_cpu - start_cpu).count();
-    for (auto &e : events) hipEventDestroy(e);
+    for (auto &e : events) (void) hipEventDestroy(e);
     profile.timing_overhead = std::chrono::duration<float>(clock::now() - end_cpu).count();
     last_profile_ = std::move(profile);
 }

@@ -27,7 +27,9 @@ public:
 class HipExecutor {
 public:
     // `plan_only` builds and compiles the plan without touching a device (no allocation, no launches)
-    HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only = false);
+    // `preserve_inputs` keeps the input buffers from being reused for later values, for callers that write the
+    // inputs on the device once and then call run_async many times
+    HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only = false, bool preserve_inputs = false);
     ~HipExecutor();
     HipExecutor(const HipExecutor &) = delete;
     HipExecutor &operator=(const HipExecutor &) = delete;
@@ -57,7 +59,7 @@ private:
         hipFunction_t function = nullptr;
         std::vector<void *> ptrs;
     };
-    void launch_step(size_t index);
+    void launch_step(size_t index, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 
     int device_;
     size_t batch_size_;

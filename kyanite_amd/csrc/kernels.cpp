@@ -1,6 +1,7 @@
 #include "kernels.h"
 
 #include <cinttypes>
+#include <cstdlib>
 
 namespace kn {
 
@@ -88,11 +89,11 @@ template<int G, typename T, typename F> KN_DEV T kn_group_reduce(T v, F f) {
     return v;
 }
 
-// reduction over a whole workgroup of NW waves through LDS; every thread gets the result
+// reduction over a whole workgroup of NW waves through LDS; every thread gets the result. Each call site owns
+// its `lds` slots and uses them once, so a single barrier between the partial writes and the reads is enough.
 template<int NW, typename T, typename F> KN_DEV T kn_block_reduce(T v, F f, T *lds) {
     v = kn_group_reduce<64>(v, f);
     if constexpr (NW > 1) {
-        __syncthreads();
         if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
         __syncthreads();
         v = lds[0];
@@ -328,6 +329,38 @@ void emit_decompose(std::ostringstream &ss, const std::string &indent, const std
     ss << indent << "}\n";
 }
 
+// Streaming heuristics: a big tensor that is touched exactly once per element gains nothing from the caches, and
+// its dirty lines would only delay whatever runs next. Such operands are read and written with non-temporal
+// accesses. The threshold can be overridden with KNHIP_NT_BYTES (0 switches the hint off).
+size_t nt_threshold_bytes() {
+    static const size_t value = [] {
+        const char *env = getenv("KNHIP_NT_BYTES");
+        if (env && *env) {
+            unsigned long long v = strtoull(env, nullptr, 10);
+            return v == 0 ? SIZE_MAX : (size_t) v;
+        }
+        return (size_t) 64 << 20;
+    }();
+    return value;
+}
+
+bool is_streaming(const KernelOperand &op) {
+    if (op.shape.size() * dtype_bytes(op.dtype) < nt_threshold_bytes()) return false;
+    for (size_t a = 0; a < op.shape.rank(); a++)
+        if (op.shape.shape()[a] > 1 && op.shape.strides()[a] == 0) return false;
+    return true;
+}
+
+std::string load_expr(const std::string &type, const std::string &ptr, bool nt) {
+    if (nt) return "__builtin_nontemporal_load((const " + type + " *) (" + ptr + "))";
+    return "*(const " + type + " *) (" + ptr + ")";
+}
+
+std::string store_stmt(const std::string &type, const std::string &ptr, const std::string &value, bool nt) {
+    if (nt) return "__builtin_nontemporal_store(" + value + ", (" + type + " *) (" + ptr + "));";
+    return "*(" + type + " *) (" + ptr + ") = " + value + ";";
+}
+
 uint32_t ceil_div_u32(size_t a, size_t b) {
     size_t r = (a + b - 1) / b;
     if (r > 0x7fffffffull) fail("kernel grid too large: ", r);
@@ -442,7 +475,9 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
     }
     for (size_t k = 1; k < operands.size(); k++) {
         bool vload = vec > 1 && c.strides[k][rank - 1] == 1;
-        if (vload) ss << "            r" << k << "[u] = *(const V" << k << " *) (p" << k << " + off[u][" << k << "]);\n";
+        if (vload)
+            ss << "            r" << k << "[u] = "
+               << load_expr("V" + std::to_string(k), "p" + std::to_string(k) + " + off[u][" + std::to_string(k) + "]", is_streaming(operands[k])) << ";\n";
         else ss << "            r" << k << "[u] = p" << k << "[off[u][" << k << "]];\n";
     }
     ss << "        }\n    }\n";
@@ -460,7 +495,7 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
             return call + ")";
         }()) << ";\n            }\n";
         int64_t os = c.strides[0][rank - 1];
-        if (os == 1) ss << "            *(V0 *) (p0 + off[u][0]) = out;\n";
+        if (os == 1) ss << "            " << store_stmt("V0", "p0 + off[u][0]", "out", is_streaming(operands[0])) << "\n";
         else {
             // output is not contiguous along the vector axis (never picked by pick_vec, kept for completeness)
             ss << "#pragma unroll\n            for (int j = 0; j < VEC; j++) p0[off[u][0] + (idx_t) j * (idx_t) " << os << "] = out[j];\n";
@@ -579,7 +614,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         ss << "        if (r < (idx_t) " << red_vecs << ") {\n            idx_t o = o_in;\n";
         emit_decompose(ss, "            ", "r", rdims, rstrides, {"o"});
         if (vec > 1) {
-            ss << "            const V v = *(const V *) (in + o);\n#pragma unroll\n";
+            ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
             ss << "            for (int j = 0; j < " << vec << "; j++) acc[(i + j) & 3] = kn_f(acc[(i + j) & 3], " << from_storage(dtype, "v[j]") << ");\n";
         } else {
             ss << "            acc[i & 3] = kn_f(acc[i & 3], " << from_storage(dtype, "in[o]") << ");\n";
@@ -633,7 +668,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         ss << "#pragma unroll 4\n        for (idx_t r = ty; r < (idx_t) " << red_size << "; r += (idx_t) " << TY << ") {\n            idx_t o = o_in;\n";
         emit_decompose(ss, "            ", "r", rc.shape, rc.strides, {"o"});
         if (vec > 1) {
-            ss << "            const V v = *(const V *) (in + o);\n#pragma unroll\n";
+            ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
             ss << "            for (int j = 0; j < " << vec << "; j++) acc[j] = kn_f(acc[j], " << from_storage(dtype, "v[j]") << ");\n";
         } else {
             ss << "            acc[0] = kn_f(acc[0], " << from_storage(dtype, "in[o]") << ");\n";
@@ -687,10 +722,12 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
 
     bool softmax = desc.kind == RowKernelDesc::Softmax;
     KernelSpec spec;
-    spec.name = "kn_row";
+    spec.name = softmax ? "kn_softmax" : "kn_layernorm";
     spec.n_ptrs = ops.size();
     size_t static_size = concrete_size(static_shape);
     if (static_size == 0 || size == 0) return spec;
+    // the normalised value is x * (1 / denom) instead of x / denom: one division per row, at most one ulp apart
+    static const bool use_rcp = !(getenv("KNHIP_ROW_RCP") && !atoi(getenv("KNHIP_ROW_RCP")));
 
     Collapsed sc = collapse_axes(static_shape, static_strides, true);
 
@@ -718,14 +755,18 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     size_t G = 1024;
     for (size_t g : {1, 4, 16, 64, 256, 1024}) {
         size_t per_lane = (nv + g - 1) / g;
-        if (per_lane <= (g >= 256 ? (g == 1024 ? MAX_ITEMS : 8) : (g == 1 ? 2 : 4))) {
+        static const size_t wave_items = getenv("KNHIP_ROW_WAVE_ITEMS") ? (size_t) atoi(getenv("KNHIP_ROW_WAVE_ITEMS")) : 4;
+        static const size_t block_items = getenv("KNHIP_ROW_BLOCK_ITEMS") ? (size_t) atoi(getenv("KNHIP_ROW_BLOCK_ITEMS")) : 8;
+        size_t limit = g == 1024 ? MAX_ITEMS : g == 256 ? block_items : g == 64 ? wave_items : g == 1 ? 2 : 4;
+        if (per_lane <= limit) {
             G = g;
             break;
         }
     }
     size_t items = (nv + G - 1) / G;
     bool cached = items <= MAX_ITEMS;
-    size_t block = std::max<size_t>(G, 256);
+    static const size_t min_block = getenv("KNHIP_ROW_MIN_BLOCK") ? (size_t) atoi(getenv("KNHIP_ROW_MIN_BLOCK")) : 256;
+    size_t block = std::max<size_t>(G, min_block);
     size_t rows_per_block = block / G;
     size_t nw = G / 64;  // waves per row when a row spans several waves
     bool idx64 = !fits_i32(ops, std::max(static_size, size) + 4096);
@@ -768,9 +809,9 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
 
     ss << "#define VEC " << vec << "\n#define ITEMS " << items << "\n#define G " << G << "\n";
     ss << "KN_DEV float kn_max(float a, float b) { return fmaxf(a, b); }\nKN_DEV float kn_add(float a, float b) { return a + b; }\n";
-    ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void kn_row(KnPtrs ptrs) {\n";
+    ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
     for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
-    if (nw > 1) ss << "    __shared__ float lds[" << nw << "];\n";
+    if (nw > 1) ss << "    __shared__ float lds_m[" << nw << "], lds_s[" << nw << "];\n";
     ss << "    const idx_t row = (idx_t) blockIdx.x * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / G);\n";
     ss << "    const idx_t lane = (idx_t) (threadIdx.x % G);\n";
     if (nw <= 1) ss << "    if (row >= (idx_t) " << static_size << ") return;\n";
@@ -783,7 +824,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     // the reduction helper: over G lanes of a wave, or over the waves of the workgroup
     auto reduce = [&](const std::string &var, const char *f) {
         if (G == 1) return;
-        if (nw > 1) ss << "    " << var << " = kn_block_reduce<" << nw << ">(" << var << ", " << f << ", lds);\n";
+        if (nw > 1) ss << "    " << var << " = kn_block_reduce<" << nw << ">(" << var << ", " << f << ", lds_" << var << ");\n";
         else ss << "    " << var << " = kn_group_reduce<G>(" << var << ", " << f << ");\n";
     };
     // load one vector position `i` (in vector units along the axis) and run the prologue on it
@@ -791,7 +832,9 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_pre[k]) continue;
             std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
-            if (vec > 1 && axis_strides[k] == 1) ss << indent << "const V" << k << " a" << k << " = *(const V" << k << " *) (p" << k << " + " << o << ");\n";
+            if (vec > 1 && axis_strides[k] == 1)
+                ss << indent << "const V" << k << " a" << k << " = "
+                   << load_expr("V" + std::to_string(k), "p" + std::to_string(k) + " + " + o, cached && is_streaming(ops[k])) << ";\n";
             else ss << indent << "const S" << k << " a" << k << " = p" << k << "[" << o << "];\n";
         }
         ss << indent << "for (int j = 0; j < VEC; j++) " << dst << "[j] = kn_pre(";
@@ -805,38 +848,56 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         ss << ");\n";
     };
     // run the epilogue on normalised values `src[j]` of vector position `i` and store
-    auto emit_post_store = [&](const std::string &indent, const std::string &i, const std::string &src) {
+    // the epilogue operands of vector position `i`: loaded into `prefix<k>`, either declared on the spot or
+    // assigned to an element of a register array that was declared earlier (`slot`)
+    auto emit_post_loads = [&](const std::string &indent, const std::string &i, const std::string &slot) {
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_post[k]) continue;
             std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
-            if (vec > 1 && axis_strides[k] == 1) ss << indent << "const V" << k << " b" << k << " = *(const V" << k << " *) (p" << k << " + " << o << ");\n";
-            else ss << indent << "const S" << k << " b" << k << " = p" << k << "[" << o << "];\n";
+            bool v = vec > 1 && axis_strides[k] == 1;
+            std::string lhs = slot.empty() ? std::string("const ") + (v ? "V" : "S") + std::to_string(k) + " b" + std::to_string(k)
+                                           : "b" + std::to_string(k) + "[" + slot + "]";
+            if (v) ss << indent << lhs << " = " << load_expr("V" + std::to_string(k), "p" + std::to_string(k) + " + " + o, is_streaming(ops[k])) << ";\n";
+            else ss << indent << lhs << " = p" << k << "[" << o << "];\n";
         }
+    };
+    auto emit_post_store = [&](const std::string &indent, const std::string &i, const std::string &src, const std::string &slot) {
+        if (slot.empty()) emit_post_loads(indent, i, "");
+        const std::string pick = slot.empty() ? std::string() : "[" + slot + "]";
         std::string o0 = "(base[0] + " + i + " * (idx_t) " + i64_str(axis_strides[0] * (int64_t) vec) + ")";
         auto call = [&](const std::string &j) {
             std::string c = "kn_post(" + src + "[" + j + "]";
             for (size_t k = 1; k < ops.size(); k++) {
                 if (!in_post[k]) continue;
-                std::string e = (vec > 1 && axis_strides[k] == 1) ? "b" + std::to_string(k) + "[" + j + "]" : "b" + std::to_string(k);
+                std::string e = "b" + std::to_string(k) + pick + ((vec > 1 && axis_strides[k] == 1) ? "[" + j + "]" : "");
                 c += ", " + from_storage(ops[k].dtype, e);
             }
             return to_storage(ops[0].dtype, c + ")");
         };
         if (vec > 1) {
             ss << indent << "V0 o;\n" << indent << "for (int j = 0; j < VEC; j++) o[j] = " << call("j") << ";\n";
-            ss << indent << "*(V0 *) (p0 + " << o0 << ") = o;\n";
+            ss << indent << store_stmt("V0", "p0 + " + o0, "o", is_streaming(ops[0])) << "\n";
         } else {
             ss << indent << "p0[" << o0 << "] = " << call("0") << ";\n";
         }
     };
 
     const std::string valid = nw > 1 ? std::string("(row < (idx_t) ") + std::to_string(static_size) + ")" : std::string("true");
+    // Epilogue operands (gamma, beta, ...) are requested together with the row itself when they fit in registers,
+    // so that their latency overlaps with the reductions instead of following them.
+    size_t n_post = 0;
+    for (size_t k = 1; k < ops.size(); k++) n_post += in_post[k] ? 1 : 0;
+    bool prefetch_post = cached && n_post > 0 && n_post * items * vec <= 64;
     if (cached) {
+        if (prefetch_post)
+            for (size_t k = 1; k < ops.size(); k++)
+                if (in_post[k]) ss << "    " << ((vec > 1 && axis_strides[k] == 1) ? "V" : "S") << k << " b" << k << "[ITEMS];\n";
         ss << "    float x[ITEMS][VEC];\n";
         ss << "    float m = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
         ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
         ss << "        if (i < (idx_t) " << nv << " && " << valid << ") {\n";
         emit_load_pre("            ", "i", "x[it]");
+        if (prefetch_post) emit_post_loads("            ", "i", "it");
         if (softmax) ss << "            for (int j = 0; j < VEC; j++) m = fmaxf(m, x[it][j]);\n";
         else ss << "            for (int j = 0; j < VEC; j++) m += x[it][j];\n";
         ss << "        } else {\n            for (int j = 0; j < VEC; j++) x[it][j] = " << (softmax ? "-KN_INF" : "0.0f") << ";\n        }\n    }\n";
@@ -855,11 +916,12 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "            x[it][j] = d;\n            s += d * d;\n        }\n    }\n";
             reduce("s", "kn_add");
             ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
-            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / denom;\n    }\n";
+            if (use_rcp) ss << "    const float rdenom = 1.0f / denom;\n#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] * rdenom;\n    }\n";
+            else ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / denom;\n    }\n";
         }
         ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
         ss << "        if (i < (idx_t) " << nv << " && " << valid << ") {\n";
-        emit_post_store("            ", "i", "x[it]");
+        emit_post_store("            ", "i", "x[it]", prefetch_post ? "it" : "");
         ss << "        }\n    }\n}\n";
     } else {
         // rows too long for registers: stream the row three times (the re-reads come from cache)
@@ -884,7 +946,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         emit_load_pre("        ", "i", "t");
         if (softmax) ss << "        for (int j = 0; j < VEC; j++) t[j] = expf(t[j] - m) / s;\n";
         else ss << "        for (int j = 0; j < VEC; j++) t[j] = (t[j] - mean) / denom;\n";
-        emit_post_store("        ", "i", "t");
+        emit_post_store("        ", "i", "t", "");
         ss << "    }\n}\n";
     }
 

@@ -678,8 +678,11 @@ Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &opt
         for (auto &op : planner.steps[si].operands) touch(op.tensor.ptr, si);
     for (auto &t : plan.outputs)
         if (t.ptr.kind == BufferKind::Shared) live[t.ptr.index].second = step_count;
-    for (auto &t : plan.inputs)
-        if (t.ptr.kind == BufferKind::Shared) live[t.ptr.index].first = 0;
+    for (auto &t : plan.inputs) {
+        if (t.ptr.kind != BufferKind::Shared) continue;
+        live[t.ptr.index].first = 0;
+        if (options.preserve_inputs) live[t.ptr.index].second = step_count;
+    }
 
     // ---- arena layout: constants first
     size_t cursor = 0;

@@ -75,6 +75,8 @@ constexpr size_t ARENA_ALIGN = 256;
 struct PlannerOptions {
     bool compile = true;          // compile the generated kernels (can be switched off to inspect the plan only)
     bool fuse_row_epilogue = true;  // fold elementwise consumers of a layernorm / softmax into the row kernel
+    // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
+    bool preserve_inputs = false;
 };
 
 Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &options);

@@ -54,10 +54,11 @@ class Profile:
 class HipExecutor:
     """`HipExecutor(device, graph, batch_size)` / `evaluate(inputs) -> outputs`."""
 
-    def __init__(self, device, graph, batch_size, plan_only=False):
+    def __init__(self, device, graph, batch_size, plan_only=False, preserve_inputs=False):
         index = device.index if isinstance(device, HipDevice) else int(device)
         h = c_void_p()
-        check(lib.knhip_executor_new(index, graph._h, batch_size, int(plan_only), byref(h)))
+        flags = (1 if plan_only else 0) | (2 if preserve_inputs else 0)
+        check(lib.knhip_executor_new(index, graph._h, batch_size, flags, byref(h)))
         self._h = h
         self.device = index
         self.batch_size = batch_size
