@@ -227,6 +227,16 @@ int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, s
 int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed);
 int knhip_executor_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed);
 
+/* Layout algebra hooks for tests (kn-cuda-eval/src/shape.rs:25-285). Strides are in elements.
+ * flags: *simple = row-major contiguous, *dense = covers its span exactly once in some axis order (shape.rs:67-73).
+ * view: *ok = 0 when the view cannot be expressed as a stride edit (shape.rs:135-189).
+ * slice: shape.rs:83-96. Output arrays need `rank` (view: `new_rank`) entries. */
+int knhip_strided_flags(const size_t *shape, const int64_t *strides, size_t rank, int *simple, int *dense);
+int knhip_strided_view(const size_t *shape, const int64_t *strides, size_t rank, const size_t *new_shape,
+                       size_t new_rank, int *ok, int64_t *new_strides);
+int knhip_strided_slice(const size_t *shape, const int64_t *strides, size_t rank, size_t axis, size_t start, size_t end,
+                        size_t step, size_t *out_shape, int64_t *out_strides);
+
 /* kernel compile cache counters (autokernel/common.rs:14-46) */
 int knhip_compile_stats(size_t *compiled, size_t *memory_hits, size_t *disk_hits);
 

@@ -707,6 +707,44 @@ int knhip_executor_str(const knhip_executor *ex, char *buf, size_t cap, size_t *
     });
 }
 
+int knhip_strided_flags(const size_t *shape, const int64_t *strides, size_t rank, int *simple, int *dense) {
+    return guarded([&] {
+        KN_REQUIRE(simple != nullptr && dense != nullptr && (rank == 0 || (shape != nullptr && strides != nullptr)));
+        StridedShape s(std::vector<size_t>(shape, shape + rank), std::vector<int64_t>(strides, strides + rank));
+        *simple = s.has_simple_strides() ? 1 : 0;
+        *dense = s.has_dense_strides() ? 1 : 0;
+        return KNHIP_OK;
+    });
+}
+
+int knhip_strided_view(const size_t *shape, const int64_t *strides, size_t rank, const size_t *new_shape, size_t new_rank,
+                       int *ok, int64_t *new_strides) {
+    return guarded([&] {
+        KN_REQUIRE(ok != nullptr && (rank == 0 || (shape != nullptr && strides != nullptr)));
+        KN_REQUIRE(new_rank == 0 || (new_shape != nullptr && new_strides != nullptr));
+        StridedShape s(std::vector<size_t>(shape, shape + rank), std::vector<int64_t>(strides, strides + rank));
+        auto v = s.view(std::vector<size_t>(new_shape, new_shape + new_rank));
+        *ok = v.has_value() ? 1 : 0;
+        if (v)
+            for (size_t i = 0; i < new_rank; i++) new_strides[i] = v->strides()[i];
+        return KNHIP_OK;
+    });
+}
+
+int knhip_strided_slice(const size_t *shape, const int64_t *strides, size_t rank, size_t axis, size_t start, size_t end,
+                        size_t step, size_t *out_shape, int64_t *out_strides) {
+    return guarded([&] {
+        KN_REQUIRE(shape != nullptr && strides != nullptr && out_shape != nullptr && out_strides != nullptr);
+        StridedShape s(std::vector<size_t>(shape, shape + rank), std::vector<int64_t>(strides, strides + rank));
+        StridedShape r = s.slice(axis, SliceRange::make(start, end, step));
+        for (size_t i = 0; i < rank; i++) {
+            out_shape[i] = r.shape()[i];
+            out_strides[i] = r.strides()[i];
+        }
+        return KNHIP_OK;
+    });
+}
+
 int knhip_compile_stats(size_t *compiled, size_t *memory_hits, size_t *disk_hits) {
     return guarded([&] {
         KN_REQUIRE(compiled != nullptr && memory_hits != nullptr && disk_hits != nullptr);
