@@ -3,9 +3,15 @@
 // One workgroup of 4 waves computes a 128 x 128 tile of D = A * B; every wave owns a 64 x 64 quadrant as 2 x 2
 // MFMA tiles of 32 x 32 (64 accumulator registers per lane). The K dimension is walked in slices of 16 that are
 // staged through LDS as As[k][m] and Bs[k][n]; the next slice is fetched into registers while the current one is
-// multiplied. Operand elements are addressed through small functors, so the same main loop serves strided
-// batched GEMM (any row/column/batch strides) and convolution as an implicit GEMM (the B operand gathers input
-// patches on the fly, with zero padding) with bias + residual + relu applied to the accumulators before the store.
+// multiplied. Operand slices are fetched by small loader objects, so the same main loop serves strided batched
+// GEMM (any row / column / batch strides) and convolution as an implicit GEMM (the B operand gathers input
+// patches on the fly, with zero padding), with bias + residual + relu applied to the accumulators before the store.
+//
+// Loaders come in three flavours, picked on the host per operand:
+//   VecOuter  the non-K axis is contiguous (stride 1) and rows are 16 byte aligned: one 128 bit load moves 4
+//             neighbouring m (or n) of one k, stored to LDS as one 128 bit write
+//   VecK      the K axis is contiguous: one 128 bit load moves 4 neighbouring k of one m (or n)
+//   Scalar    anything else (arbitrary strides), and every tile that sticks out of the matrix
 #include <hip/hip_runtime.h>
 
 #include "../mfma_kernels.h"
@@ -18,66 +24,179 @@ constexpr int BM = 128, BN = 128, BK = 16, THREADS = 256;
 constexpr int LDS_STRIDE = BM + 4;  // keeps rows 16 byte aligned and shifts successive k rows by 4 banks
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// ---- operand accessors for plain strided GEMM
-struct GemmA {
+enum LoadMode { Scalar = 0, VecOuter = 1, VecK = 2 };
+
+// A [outer, K] operand addressed as p[outer * so + k * sk]; `outer` is m for A and n for B.
+struct StridedOperand {
     const float *p;
-    long long sm, sk;
-    int M, K;
-    __device__ __forceinline__ float load(int m, int k) const { return (m < M && k < K) ? p[m * sm + k * sk] : 0.0f; }
-    __device__ __forceinline__ bool lanes_along_k() const { return (sk < 0 ? -sk : sk) < (sm < 0 ? -sm : sm); }
+    long long so, sk;
+    int outer_size, K;
 };
-struct GemmB {
-    const float *p;
-    long long sk, sn;
-    int K, N;
-    __device__ __forceinline__ float load(int k, int n) const { return (k < K && n < N) ? p[k * sk + n * sn] : 0.0f; }
-    __device__ __forceinline__ bool lanes_along_k() const { return (sk < 0 ? -sk : sk) < (sn < 0 ? -sn : sn); }
+
+// Fetches one BK x 128 slice of a strided operand into 8 registers per thread and writes it to LDS as [k][outer].
+template <int MODE>
+struct StridedLoader {
+    StridedOperand op;
+    int o0;        // first outer index of this workgroup's tile
+    bool interior; // the tile lies completely inside the matrix along the outer axis
+    float r[8];
+
+    __device__ __forceinline__ StridedLoader(const StridedOperand &operand, int outer0)
+        : op(operand), o0(outer0), interior(outer0 + 128 <= operand.outer_size) {}
+
+    __device__ __forceinline__ void fetch(int k0) {
+        const int t = threadIdx.x;
+        if (MODE == VecOuter && interior && k0 + BK <= op.K) {
+            // thread -> (k = t / 32 (+8), outer = 4 * (t % 32) ..)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int k = (t >> 5) + 8 * h, o = (t & 31) * 4;
+                const floatx4 v = *(const floatx4 *) (op.p + (long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk);
+#pragma unroll
+                for (int j = 0; j < 4; j++) r[4 * h + j] = v[j];
+            }
+        } else if (MODE == VecK && interior && k0 + BK <= op.K) {
+            // thread -> (outer = t / 4 (+64), k = 4 * (t % 4) ..)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int o = (t >> 2) + 64 * h, k = (t & 3) * 4;
+                const floatx4 v = *(const floatx4 *) (op.p + (long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk);
+#pragma unroll
+                for (int j = 0; j < 4; j++) r[4 * h + j] = v[j];
+            }
+        } else {
+            // lanes run along whichever axis has the smaller stride
+            const bool along_k = (op.sk < 0 ? -op.sk : op.sk) < (op.so < 0 ? -op.so : op.so);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int e = t + THREADS * i;
+                const int o = along_k ? (e >> 4) : (e & 127);
+                const int k = along_k ? (e & 15) : (e >> 7);
+                const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
+                r[i] = ok ? op.p[(long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk] : 0.0f;
+            }
+        }
+    }
+
+    // the layout decision has to match the one `fetch` took for the same slice
+    __device__ __forceinline__ void stage(float (*lds)[LDS_STRIDE], int k0) const {
+        const int t = threadIdx.x;
+        if (MODE == VecOuter && interior && k0 + BK <= op.K) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int k = (t >> 5) + 8 * h, o = (t & 31) * 4;
+                floatx4 v;
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = r[4 * h + j];
+                *(floatx4 *) &lds[k][o] = v;
+            }
+        } else if (MODE == VecK && interior && k0 + BK <= op.K) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int o = (t >> 2) + 64 * h, k = (t & 3) * 4;
+#pragma unroll
+                for (int j = 0; j < 4; j++) lds[k + j][o] = r[4 * h + j];
+            }
+        } else {
+            const bool along_k = (op.sk < 0 ? -op.sk : op.sk) < (op.so < 0 ? -op.so : op.so);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const int e = t + THREADS * i;
+                const int o = along_k ? (e >> 4) : (e & 127);
+                const int k = along_k ? (e & 15) : (e >> 7);
+                lds[k][o] = r[i];
+            }
+        }
+    }
 };
+
+// Input patches of a convolution as the B operand: k = (c, fy, fx), n = (image, oy, ox). Every thread keeps one
+// fixed n for the whole K loop, so the position is decomposed once; KH / KW are compile-time constants (0 = read
+// them from the parameters) so that splitting k costs multiplications instead of divisions.
+template <int KH, int KW>
+struct PatchLoader {
+    const float *base;  // input of this thread's image, or null when n is out of range
+    int K, in_h, in_w, kh, kw, iy0, ix0;
+    float r[8];
+
+    __device__ __forceinline__ PatchLoader(const ConvParams &p, int n0) {
+        kh = KH ? KH : p.kernel_h;
+        kw = KW ? KW : p.kernel_w;
+        K = p.in_c * kh * kw;
+        in_h = p.in_h;
+        in_w = p.in_w;
+        const int n = n0 + (threadIdx.x & 127);
+        const int ohw = p.out_h * p.out_w;
+        const long long total = (long long) p.batch * ohw;
+        if (n < total) {
+            const int img = n / ohw, pos = n - img * ohw;
+            const int oy = pos / p.out_w, ox = pos - oy * p.out_w;
+            iy0 = oy * p.stride_y - p.pad_y;
+            ix0 = ox * p.stride_x - p.pad_x;
+            base = p.input + (long long) img * p.in_c * in_h * in_w;
+        } else {
+            base = nullptr;
+            iy0 = ix0 = 0;
+        }
+    }
+
+    __device__ __forceinline__ void fetch(int k0) {
+        const int khw = kh * kw;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int k = k0 + (threadIdx.x >> 7) + 2 * i;
+            const int c = k / khw, rem = k - c * khw;
+            const int fy = rem / kw, fx = rem - fy * kw;
+            const int iy = iy0 + fy, ix = ix0 + fx;
+            const bool ok = base != nullptr && k < K && iy >= 0 && iy < in_h && ix >= 0 && ix < in_w;
+            r[i] = ok ? base[((long long) c * in_h + iy) * in_w + ix] : 0.0f;
+        }
+    }
+
+    __device__ __forceinline__ void stage(float (*lds)[LDS_STRIDE], int) const {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int k = (threadIdx.x >> 7) + 2 * i;
+            lds[k][threadIdx.x & 127] = r[i];
+        }
+    }
+};
+
 struct GemmStore {
     float *p;
     long long sm, sn;
     int M, N;
-    __device__ __forceinline__ void store(int m, int n, float v) const {
-        if (m < M && n < N) p[m * sm + n * sn] = v;
+    __device__ __forceinline__ void prepare(int, int) {}
+    __device__ __forceinline__ void store(int m, int n, int, float v) const {
+        if (m < M && n < N) p[(long long) m * sm + (long long) n * sn] = v;
     }
 };
 
-// ---- operand accessors for convolution: D[ko][pos] = sum_k filter[ko][k] * patch[k][pos]
-struct ConvA {  // the filter, dense [out_c, in_c * kh * kw]
-    const float *p;
-    int M, K;
-    __device__ __forceinline__ float load(int m, int k) const { return (m < M && k < K) ? p[(long long) m * K + k] : 0.0f; }
-    __device__ __forceinline__ bool lanes_along_k() const { return true; }
-};
-struct ConvB {  // input patches, gathered from the dense NCHW input; n runs over (image, oy, ox)
-    const float *p;
-    int K, N;  // K = in_c * kh * kw, N = batch * out_h * out_w
-    int in_c, in_h, in_w, out_h, out_w, kh, kw, sy, sx, py, px;
-    __device__ __forceinline__ float load(int k, int n) const {
-        if (k >= K || n >= N) return 0.0f;
-        int khw = kh * kw, ohw = out_h * out_w;
-        int c = k / khw, r = k - c * khw;
-        int fy = r / kw, fx = r - fy * kw;
-        int img = n / ohw, pos = n - img * ohw;
-        int oy = pos / out_w, ox = pos - oy * out_w;
-        int iy = oy * sy + fy - py, ix = ox * sx + fx - px;
-        if (iy < 0 || iy >= in_h || ix < 0 || ix >= in_w) return 0.0f;
-        return p[(((long long) img * in_c + c) * in_h + iy) * in_w + ix];
-    }
-    __device__ __forceinline__ bool lanes_along_k() const { return false; }
-};
 struct ConvStore {
     float *p;
     const float *bias;
     const float *res;
     long long bias_stride;
-    int M, N, ohw;  // out_c, batch * out_h * out_w, out_h * out_w
+    int M, ohw;  // out_c, out_h * out_w
+    long long N; // batch * out_h * out_w
     int relu;
-    __device__ __forceinline__ void store(int m, int n, float v) const {
-        if (m < M && n < N) {
-            int img = n / ohw, pos = n - img * ohw;
-            long long o = ((long long) img * M + m) * ohw + pos;
+    long long col_base[2];  // offset of (image, 0, position) for the two columns this lane owns
+    bool col_ok[2];
+
+    __device__ __forceinline__ void prepare(int col0, int col1) {
+        const int cols[2] = {col0, col1};
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            col_ok[j] = cols[j] < N;
+            const int img = cols[j] / ohw, pos = cols[j] - img * ohw;
+            col_base[j] = (long long) img * M * ohw + pos;
+        }
+    }
+    __device__ __forceinline__ void store(int m, int, int j, float v) const {
+        if (m < M && col_ok[j]) {
+            const long long o = col_base[j] + (long long) m * ohw;
             if (res) v += res[o];
             if (bias) v += bias[m * bias_stride];
             if (relu) v = fmaxf(v, 0.0f);
@@ -86,44 +205,13 @@ struct ConvStore {
     }
 };
 
-template <typename A, typename B, typename S>
-__device__ __forceinline__ void mfma_tile_loop(const A &a, const B &b, const S &s, int K) {
-    __shared__ float As[BK][LDS_STRIDE];
-    __shared__ float Bs[BK][LDS_STRIDE];
+template <typename LA, typename LB, typename S>
+__device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int K, int m0, int n0) {
+    __shared__ __attribute__((aligned(16))) float As[BK][LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[BK][LDS_STRIDE];
 
-    const int t = threadIdx.x;
-    const int lane = t & 63, wave = t >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-
-    // each thread moves 8 elements of each operand per slice; lanes run along the axis that is contiguous in memory
-    const bool a_k = a.lanes_along_k(), b_k = b.lanes_along_k();
-    float ra[8], rb[8];
-
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            int e = t + THREADS * i;
-            int am = a_k ? (e >> 4) : (e & (BM - 1));
-            int ak = a_k ? (e & (BK - 1)) : (e >> 7);
-            ra[i] = a.load(m0 + am, k0 + ak);
-            int bn = b_k ? (e >> 4) : (e & (BN - 1));
-            int bk = b_k ? (e & (BK - 1)) : (e >> 7);
-            rb[i] = b.load(k0 + bk, n0 + bn);
-        }
-    };
-    auto stage = [&]() {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            int e = t + THREADS * i;
-            int am = a_k ? (e >> 4) : (e & (BM - 1));
-            int ak = a_k ? (e & (BK - 1)) : (e >> 7);
-            As[ak][am] = ra[i];
-            int bn = b_k ? (e >> 4) : (e & (BN - 1));
-            int bk = b_k ? (e & (BK - 1)) : (e >> 7);
-            Bs[bk][bn] = rb[i];
-        }
-    };
 
     floatx16 acc[2][2];
 #pragma unroll
@@ -133,12 +221,17 @@ __device__ __forceinline__ void mfma_tile_loop(const A &a, const B &b, const S &
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    fetch(0);
+    la.fetch(0);
+    lb.fetch(0);
     for (int k0 = 0; k0 < K; k0 += BK) {
         __syncthreads();  // the previous slice has been consumed
-        stage();
+        la.stage(As, k0);
+        lb.stage(Bs, k0);
         __syncthreads();
-        if (k0 + BK < K) fetch(k0 + BK);
+        if (k0 + BK < K) {
+            la.fetch(k0 + BK);
+            lb.fetch(k0 + BK);
+        }
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
             const int kr = kk + (lane >> 5), c = lane & 31;
@@ -152,33 +245,81 @@ __device__ __forceinline__ void mfma_tile_loop(const A &a, const B &b, const S &
     }
 
     // accumulator layout of the 32x32 tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32
+    const int col0 = n0 + wn * 64 + (lane & 31);
+    s.prepare(col0, col0 + 32);
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                int col = n0 + wn * 64 + j * 32 + (lane & 31);
-                s.store(row, col, acc[i][j][v]);
+                const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                s.store(row, col0 + 32 * j, j, acc[i][j][v]);
             }
 }
 
-__global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
-    const int bz = blockIdx.z;
-    GemmA a{p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k};
-    GemmB b{p.b + bz * p.b_sb, p.b_sk, p.b_sn, p.k, p.n};
-    GemmStore s{p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
-    mfma_tile_loop(a, b, s, p.k);
+// Tiles are numbered so that the workgroups that run at the same time (consecutive ids) share rows of tiles:
+// groups of 8 tile rows are walked column by column.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) {
+    const int id = blockIdx.x;
+    const int group_rows = 8;
+    const int per_group = group_rows * tiles_n;
+    const int g = id / per_group, in_g = id - g * per_group;
+    const int rows_here = min(group_rows, tiles_m - g * group_rows);
+    *tm = g * group_rows + in_g % rows_here;
+    *tn = in_g / rows_here;
 }
 
+template <int A_MODE, int B_MODE>
+__global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
+    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    const int bz = blockIdx.y;
+    const int m0 = tm * BM, n0 = tn * BN;
+    StridedLoader<A_MODE> la(StridedOperand{p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
+    StridedLoader<B_MODE> lb(StridedOperand{p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+    GemmStore s{p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
+    mfma_tile_loop(la, lb, s, p.k, m0, n0);
+}
+
+template <int A_MODE, int KH, int KW>
 __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
-    const int K = p.in_c * p.kernel_h * p.kernel_w, ohw = p.out_h * p.out_w, N = p.batch * ohw;
-    ConvA a{p.filter, p.out_c, K};
-    ConvB b{p.input, K, N, p.in_c, p.in_h, p.in_w, p.out_h, p.out_w,
-            p.kernel_h, p.kernel_w, p.stride_y, p.stride_x, p.pad_y, p.pad_x};
-    ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, N, ohw, p.relu};
-    mfma_tile_loop(a, b, s, K);
+    const int kh = KH ? KH : p.kernel_h, kw = KW ? KW : p.kernel_w;
+    const int K = p.in_c * kh * kw, ohw = p.out_h * p.out_w;
+    const long long N = (long long) p.batch * ohw;
+    const int tiles_m = (p.out_c + BM - 1) / BM, tiles_n = (int) ((N + BN - 1) / BN);
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    StridedLoader<A_MODE> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
+    PatchLoader<KH, KW> lb(p, n0);
+    ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
+    mfma_tile_loop(la, lb, s, K, m0, n0);
+}
+
+// Pick the widest loader an operand allows: `so` / `sk` are the strides of the outer and the K axis.
+int pick_mode(const float *ptr, long long so, long long sk, long long batch_stride, int batch) {
+    const bool aligned = ((uintptr_t) ptr % 16 == 0) && (batch <= 1 || batch_stride % 4 == 0);
+    if (!aligned) return Scalar;
+    if (so == 1 && sk % 4 == 0) return VecOuter;
+    if (sk == 1 && so % 4 == 0) return VecK;
+    return Scalar;
+}
+
+template <int A_MODE>
+void launch_gemm_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+    switch (b_mode) {
+        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK>), grid, dim3(THREADS), 0, stream, p); break;
+        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar>), grid, dim3(THREADS), 0, stream, p); break;
+    }
+}
+
+template <int KH, int KW>
+void launch_conv_k(int a_mode, dim3 grid, hipStream_t stream, const ConvParams &p) {
+    if (a_mode == VecK) hipLaunchKernelGGL((conv_f32_kernel<VecK, KH, KW>), grid, dim3(THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((conv_f32_kernel<Scalar, KH, KW>), grid, dim3(THREADS), 0, stream, p);
 }
 
 }  // namespace
@@ -197,19 +338,30 @@ int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
         q.c_sm = p.c_sn; q.c_sn = p.c_sm;
         p = q;
     }
-    dim3 grid((p.n + BN - 1) / BN, (p.m + BM - 1) / BM, p.batch);
-    if (grid.y > 65535 || grid.z > 65535) return (int) hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(THREADS), 0, stream, p);
+    const long long tiles = (long long) ((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
+    if (tiles > 0x7fffffffll || p.batch > 65535) return (int) hipErrorInvalidConfiguration;
+    dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
+    const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.a_sb, p.batch);
+    const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.b_sb, p.batch);
+    switch (a_mode) {
+        case VecOuter: launch_gemm_b<VecOuter>(b_mode, grid, stream, p); break;
+        case VecK: launch_gemm_b<VecK>(b_mode, grid, stream, p); break;
+        default: launch_gemm_b<Scalar>(b_mode, grid, stream, p); break;
+    }
     return (int) hipGetLastError();
 }
 
 int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
-    long long positions = (long long) p.batch * p.out_h * p.out_w;
+    const long long positions = (long long) p.batch * p.out_h * p.out_w;
     if (positions <= 0 || p.out_c <= 0) return 0;
-    if (positions > 0x7fffffffll) return (int) hipErrorInvalidValue;
-    dim3 grid((unsigned) ((positions + BN - 1) / BN), (p.out_c + BM - 1) / BM, 1);
-    if (grid.y > 65535) return (int) hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL(conv_f32_kernel, grid, dim3(THREADS), 0, stream, p);
+    const long long tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
+    if (positions > 0x7fffffffll || tiles > 0x7fffffffll) return (int) hipErrorInvalidValue;
+    dim3 grid((unsigned) tiles, 1, 1);
+    const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
+    const int a_mode = ((uintptr_t) p.filter % 16 == 0 && K % 4 == 0) ? VecK : Scalar;
+    if (p.kernel_h == 3 && p.kernel_w == 3) launch_conv_k<3, 3>(a_mode, grid, stream, p);
+    else if (p.kernel_h == 1 && p.kernel_w == 1) launch_conv_k<1, 1>(a_mode, grid, stream, p);
+    else launch_conv_k<0, 0>(a_mode, grid, stream, p);
     return (int) hipGetLastError();
 }
 

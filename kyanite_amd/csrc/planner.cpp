@@ -458,10 +458,12 @@ private:
             const Operation &op = graph[curr].operation;
             if (op.kind == OpKind::Binary && op.binary == BinaryOp::Max) {
                 Value l = op.inputs[0], r = op.inputs[1];
-                if (!(can_fuse(l) && can_fuse(r))) return R::done(std::nullopt);
+                // only the activation input has to be exclusive to this relu: the zero it is compared with is a
+                // constant that the builder shares between all relus of the same shape
                 if (graph.is_const_zero(l)) curr = r;
                 else if (graph.is_const_zero(r)) curr = l;
                 else return R::done(std::nullopt);
+                if (!can_fuse(curr)) return R::done(std::nullopt);
                 relu = true;
             }
         }
