@@ -298,6 +298,199 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
     mfma_tile_loop(la, lb, s, K, m0, n0);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// "Plane" convolution: stride 1, same-size output, image width a power of two. Instead of gathering the im2col
+// matrix, every K slice (CB input channels x KH x KW taps) stages the raw input rows that the tile's 128 output
+// positions touch into LDS once, as [channel][group][row][W], and the MFMA B operand is read straight from those
+// planes: position n of the tile sits at a fixed per-lane offset, tap (c, fy, fx) adds a wave-uniform offset, and
+// taps that fall left or right of the image are masked to zero (rows above / below are stored as zero rows).
+// Global -> LDS traffic for B drops by KH * KW and no per-element index arithmetic is left in the K loop.
+// A tile is either R = 128 / W whole output rows of one image (H * W >= 128) or G = 128 / (H * W) whole images.
+constexpr int CB = 8;             // input channels per K slice
+constexpr int PLANE_MAX_VEC = 3;  // 128 bit loads per thread and slice for the B planes
+constexpr int PLANE_SLACK = 4;    // floats in front of / behind the planes that masked taps may touch
+constexpr int PLANE_LDS = PLANE_MAX_VEC * THREADS * 4 + 2 * PLANE_SLACK;
+
+struct PlaneGeom {
+    int rows;            // R: output rows per group
+    int groups;          // G: images per tile (1 when a tile is part of one image)
+    int tiles_per_image; // H * W / 128, or 0 when a tile holds whole images
+    int plane_rows;      // R + KH - 1
+    int w4_shift, g_shift, rw_shift;  // log2 of W / 4, G, R * W
+    int n_vec;           // CB * G * plane_rows * W / 4
+};
+
+template <int KH, int KW>
+__global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, PlaneGeom g) {
+    constexpr int KS = CB * KH * KW;      // K slice
+    constexpr int A_VEC = KS / 4;         // 128 bit loads per filter row and slice
+    constexpr int A_ITERS = BM * A_VEC / THREADS;
+    constexpr int A_STRIDE = BM + 5;      // odd, spreads the transposing stores over the banks
+    static_assert(KS % 4 == 0 && (BM * A_VEC) % THREADS == 0 && KS % 2 == 0, "slice shape");
+    __shared__ float As[KS][A_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[PLANE_LDS];
+
+    const int W = p.in_w, H = p.in_h, C = p.in_c;
+    const int K = C * KH * KW, ohw = H * W;
+    const long long N = (long long) p.batch * ohw;
+    const int tiles_m = (p.out_c + BM - 1) / BM, tiles_n = (int) ((N + BN - 1) / BN);
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    int img0, oy0;
+    if (g.tiles_per_image) {
+        img0 = tn / g.tiles_per_image;
+        oy0 = (tn - img0 * g.tiles_per_image) * g.rows;
+    } else {
+        img0 = tn * g.groups;
+        oy0 = 0;
+    }
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, c32 = lane & 31;
+    const int plane = g.plane_rows * W, gplane = plane << g.g_shift;  // floats per (c, g) and per c
+
+    // ---- B planes: what this thread moves per slice (the same places every slice, only the channel base moves)
+    const float *b_src[PLANE_MAX_VEC];
+    bool b_live[PLANE_MAX_VEC];
+#pragma unroll
+    for (int i = 0; i < PLANE_MAX_VEC; i++) {
+        const int e = t + THREADS * i;
+        const int w4 = e & ((1 << g.w4_shift) - 1), t1 = e >> g.w4_shift;
+        const int t2 = t1 / g.plane_rows, prow = t1 - t2 * g.plane_rows;
+        const int gg = t2 & (g.groups - 1), c = t2 >> g.g_shift;
+        const int iy = oy0 + prow - p.pad_y, img = img0 + gg;
+        const bool ok = e < g.n_vec && iy >= 0 && iy < H && img < p.batch;
+        b_live[i] = e < g.n_vec;
+        b_src[i] = ok ? p.input + (((long long) img * C + c) * H + iy) * W + 4 * w4 : nullptr;
+    }
+    // ---- A (filter) rows: K contiguous
+    const float *a_src[A_ITERS];
+    int a_dst[A_ITERS];
+#pragma unroll
+    for (int i = 0; i < A_ITERS; i++) {
+        const int e = t + THREADS * i, row = e / A_VEC, q = e - row * A_VEC;
+        a_src[i] = (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
+        a_dst[i] = 4 * q * A_STRIDE + row;
+    }
+    // ---- where this lane's two output positions sit inside a plane, and which taps stay inside the image
+    int lane_base[2];
+    bool pair_ok[2][KW];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int n = wn * 64 + 32 * j + c32;
+        const int gl = n >> g.rw_shift, rem = n & ((1 << g.rw_shift) - 1), col = rem & (W - 1);
+        lane_base[j] = PLANE_SLACK + gl * plane + rem - p.pad_x;
+#pragma unroll
+        for (int fx = 0; fx < KW; fx++) {
+            // the upper half of the wave multiplies the next k, whose fx is one further (cyclically)
+            const int f = half ? (fx + 1) % KW : fx;
+            pair_ok[j][fx] = (unsigned) (col + f - p.pad_x) < (unsigned) W;
+        }
+    }
+
+    floatx4 ra[A_ITERS], rb[PLANE_MAX_VEC];
+    auto fetch = [&](int c0) {
+        const long long a_off = (long long) c0 * KH * KW, b_off = (long long) c0 * ohw;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++)
+            ra[i] = a_src[i] ? *(const floatx4 *) (a_src[i] + a_off) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < PLANE_MAX_VEC; i++)
+            rb[i] = b_src[i] ? *(const floatx4 *) (b_src[i] + b_off) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    };
+    auto stage = [&]() {
+        float *a_flat = &As[0][0];
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) a_flat[a_dst[i] + j * A_STRIDE] = ra[i][j];
+#pragma unroll
+        for (int i = 0; i < PLANE_MAX_VEC; i++)
+            if (b_live[i]) *(floatx4 *) &Bs[PLANE_SLACK + 4 * (t + THREADS * i)] = rb[i];
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    if (t < 2 * PLANE_SLACK) Bs[t < PLANE_SLACK ? t : PLANE_LDS - 2 * PLANE_SLACK + t] = 0.0f;
+    fetch(0);
+    for (int c0 = 0; c0 < C; c0 += CB) {
+        __syncthreads();
+        stage();
+        __syncthreads();
+        if (c0 + CB < C) fetch(c0 + CB);
+#pragma unroll
+        for (int kk = 0; kk < KS; kk += 2) {
+            // taps of k = kk (lower half of the wave) and k = kk + 1 (upper half); all compile-time
+            const int ca = kk / (KH * KW), fya = (kk / KW) % KH, fxa = kk % KW;
+            const int cb = (kk + 1) / (KH * KW), fyb = ((kk + 1) / KW) % KH, fxb = (kk + 1) % KW;
+            const int off_a = ca * gplane + fya * W + fxa, off_b = cb * gplane + fyb * W + fxb;
+            const int koff = half ? off_b : off_a;
+            const float a0 = As[kk + half][wm * 64 + c32], a1 = As[kk + half][wm * 64 + 32 + c32];
+            float b0 = Bs[lane_base[0] + koff], b1 = Bs[lane_base[1] + koff];
+            b0 = pair_ok[0][fxa] ? b0 : 0.0f;
+            b1 = pair_ok[1][fxa] ? b1 : 0.0f;
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+    }
+
+    ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
+    const int col0 = n0 + wn * 64 + c32;
+    s.prepare(col0, col0 + 32);
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+                s.store(row, col0 + 32 * j, j, acc[i][j][v]);
+            }
+}
+
+int log2_exact(int x) {
+    int s = 0;
+    while ((1 << s) < x) s++;
+    return (1 << s) == x ? s : -1;
+}
+
+// Fills `g` and returns true when the plane kernel covers this convolution.
+bool plane_geometry(const ConvParams &p, PlaneGeom *g) {
+    if (p.kernel_h != 3 || p.kernel_w != 3 || p.stride_y != 1 || p.stride_x != 1) return false;
+    if (p.pad_y != 1 || p.pad_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
+    if (p.in_c % CB != 0 || (uintptr_t) p.input % 16 != 0 || (uintptr_t) p.filter % 16 != 0) return false;
+    const int W = p.in_w, H = p.in_h;
+    if (W < 4 || W > BN || log2_exact(W) < 0) return false;
+    const long long hw = (long long) H * W;
+    if (hw >= BN) {
+        if (hw % BN != 0) return false;
+        g->rows = BN / W;
+        g->groups = 1;
+        g->tiles_per_image = (int) (hw / BN);
+    } else {
+        if (BN % hw != 0) return false;
+        g->rows = H;
+        g->groups = (int) (BN / hw);
+        g->tiles_per_image = 0;
+    }
+    g->plane_rows = g->rows + p.kernel_h - 1;
+    g->w4_shift = log2_exact(W / 4);
+    g->g_shift = log2_exact(g->groups);
+    g->rw_shift = log2_exact(g->rows * W);
+    g->n_vec = CB * g->groups * g->plane_rows * W / 4;
+    if (g->g_shift < 0 || g->rw_shift < 0 || g->n_vec > PLANE_MAX_VEC * THREADS) return false;
+    return true;
+}
+
 // Pick the widest loader an operand allows: `so` / `sk` are the strides of the outer and the K axis.
 int pick_mode(const float *ptr, long long so, long long sk, long long batch_stride, int batch) {
     const bool aligned = ((uintptr_t) ptr % 16 == 0) && (batch <= 1 || batch_stride % 4 == 0);
@@ -357,6 +550,11 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     const long long tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
     if (positions > 0x7fffffffll || tiles > 0x7fffffffll) return (int) hipErrorInvalidValue;
     dim3 grid((unsigned) tiles, 1, 1);
+    PlaneGeom geom;
+    if (plane_geometry(p, &geom)) {
+        hipLaunchKernelGGL((conv_plane_kernel<3, 3>), grid, dim3(THREADS), 0, stream, p, geom);
+        return (int) hipGetLastError();
+    }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
     const int a_mode = ((uintptr_t) p.filter % 16 == 0 && K % 4 == 0) ? VecK : Scalar;
     if (p.kernel_h == 3 && p.kernel_w == 3) launch_conv_k<3, 3>(a_mode, grid, stream, p);

@@ -828,3 +828,56 @@ def conv_fused_all():
     y = g.relu(g.add(g.add(g.conv(x, w, 1, 1, 1, 1), bias), x))
     g.output(y)
     return g, 5, [rng.standard_normal((5, 130, 5, 8)).astype(np.float32)], None
+
+
+def _plane_conv_case(seed, batch, c_in, c_out, h, w, fused):
+    """3x3 same-size convolutions whose image width is a power of two take the kernel that stages raw input planes"""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    x = g.input([BATCH, c_in, h, w])
+    filt = g.constant([c_out, c_in, 3, 3], (rng.standard_normal((c_out, c_in, 3, 3)) * 0.1).astype(np.float32))
+    y = g.conv(x, filt, 1, 1, 1, 1)
+    if fused:
+        bias = g.constant([1, c_out, 1, 1], rng.standard_normal(c_out).astype(np.float32))
+        y = g.add(y, bias)
+        if c_in == c_out:
+            y = g.add(y, x)
+        y = g.relu(y)
+    g.output(y)
+    return g, batch, [rng.standard_normal((batch, c_in, h, w)).astype(np.float32)], None
+
+
+@case
+def conv_plane_8x8_odd_batch():
+    """two images per tile, the last tile holds one image only"""
+    return _plane_conv_case(20, 5, 16, 16, 8, 8, True)
+
+
+@case
+def conv_plane_4x4():
+    """eight images per tile, partial last tile, partial tile of output channels"""
+    return _plane_conv_case(21, 11, 8, 5, 4, 4, True)
+
+
+@case
+def conv_plane_16x16_wide_out():
+    """one image spans two tiles; 130 output channels span two tiles of channels"""
+    return _plane_conv_case(22, 2, 24, 130, 16, 16, False)
+
+
+@case
+def conv_plane_64x64():
+    """a tile is two rows of the image, halo rows come from the neighbouring tiles' rows"""
+    return _plane_conv_case(23, 1, 8, 8, 64, 64, True)
+
+
+@case
+def conv_plane_2x128():
+    """a tile is one row of the image"""
+    return _plane_conv_case(24, 2, 8, 3, 2, 128, False)
+
+
+@case
+def conv_plane_32x4():
+    """narrow tall image: a tile is 32 rows"""
+    return _plane_conv_case(25, 3, 16, 7, 64, 4, False)
