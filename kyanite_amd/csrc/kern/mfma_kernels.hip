@@ -1,7 +1,8 @@
 // f32 matrix multiply and fused convolution on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32).
 //
 // One workgroup of 4 waves computes a 128 x 128 tile of D = A * B; every wave owns a 64 x 64 quadrant as 2 x 2
-// MFMA tiles of 32 x 32 (64 accumulator registers per lane). The K dimension is walked in slices of 16 that are
+// MFMA tiles of 32 x 32 (64 accumulator registers per lane). Problems with too few such tiles to fill the chip
+// use 64 x 64 tiles instead (one MFMA tile per wave). The K dimension is walked in slices of 16 that are
 // staged through LDS as As[k][m] and Bs[k][n]; the next slice is fetched into registers while the current one is
 // multiplied. Operand slices are fetched by small loader objects, so the same main loop serves strided batched
 // GEMM (any row / column / batch strides) and convolution as an implicit GEMM (the B operand gathers input
@@ -14,14 +15,18 @@
 //   Scalar    anything else (arbitrary strides), and every tile that sticks out of the matrix
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "../mfma_kernels.h"
 
 namespace kn {
 
 namespace {
 
+// BM x BN is the tile of the plane convolution kernel; the generic kernels take their tile (64 or 128 wide per
+// axis) from the loaders. LDS rows are padded by 4 floats: rows stay 16 byte aligned and successive k rows shift
+// by 4 banks.
 constexpr int BM = 128, BN = 128, BK = 16, THREADS = 256;
-constexpr int LDS_STRIDE = BM + 4;  // keeps rows 16 byte aligned and shifts successive k rows by 4 banks
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -35,24 +40,27 @@ struct StridedOperand {
     int outer_size, K;
 };
 
-// Fetches one BK x 128 slice of a strided operand into 8 registers per thread and writes it to LDS as [k][outer].
-template <int MODE>
+// Fetches one BK x WIDTH slice (WIDTH = 64 or 128) of a strided operand into registers and writes it to LDS as
+// [k][outer].
+template <int MODE, int WIDTH>
 struct StridedLoader {
+    static constexpr int EPT = BK * WIDTH / THREADS;  // elements per thread
+    static constexpr int LDS_STRIDE = WIDTH + 4;
     StridedOperand op;
     int o0;        // first outer index of this workgroup's tile
     bool interior; // the tile lies completely inside the matrix along the outer axis
-    float r[8];
+    float r[EPT];
 
     __device__ __forceinline__ StridedLoader(const StridedOperand &operand, int outer0)
-        : op(operand), o0(outer0), interior(outer0 + 128 <= operand.outer_size) {}
+        : op(operand), o0(outer0), interior(outer0 + WIDTH <= operand.outer_size) {}
 
     __device__ __forceinline__ void fetch(int k0) {
         const int t = threadIdx.x;
         if (MODE == VecOuter && interior && k0 + BK <= op.K) {
-            // thread -> (k = t / 32 (+8), outer = 4 * (t % 32) ..)
+            // thread -> (k = t / (WIDTH / 4) (+ ..), outer = 4 * (t % (WIDTH / 4)) ..)
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int k = (t >> 5) + 8 * h, o = (t & 31) * 4;
+            for (int h = 0; h < EPT / 4; h++) {
+                const int k = t / (WIDTH / 4) + (THREADS * 4 / WIDTH) * h, o = (t % (WIDTH / 4)) * 4;
                 const floatx4 v = *(const floatx4 *) (op.p + (long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk);
 #pragma unroll
                 for (int j = 0; j < 4; j++) r[4 * h + j] = v[j];
@@ -60,7 +68,7 @@ struct StridedLoader {
         } else if (MODE == VecK && interior && k0 + BK <= op.K) {
             // thread -> (outer = t / 4 (+64), k = 4 * (t % 4) ..)
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < EPT / 4; h++) {
                 const int o = (t >> 2) + 64 * h, k = (t & 3) * 4;
                 const floatx4 v = *(const floatx4 *) (op.p + (long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk);
 #pragma unroll
@@ -70,10 +78,10 @@ struct StridedLoader {
             // lanes run along whichever axis has the smaller stride
             const bool along_k = (op.sk < 0 ? -op.sk : op.sk) < (op.so < 0 ? -op.so : op.so);
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
+            for (int i = 0; i < EPT; i++) {
                 const int e = t + THREADS * i;
-                const int o = along_k ? (e >> 4) : (e & 127);
-                const int k = along_k ? (e & 15) : (e >> 7);
+                const int o = along_k ? (e >> 4) : (e % WIDTH);
+                const int k = along_k ? (e & 15) : (e / WIDTH);
                 const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
                 r[i] = ok ? op.p[(long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk] : 0.0f;
             }
@@ -85,8 +93,8 @@ struct StridedLoader {
         const int t = threadIdx.x;
         if (MODE == VecOuter && interior && k0 + BK <= op.K) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int k = (t >> 5) + 8 * h, o = (t & 31) * 4;
+            for (int h = 0; h < EPT / 4; h++) {
+                const int k = t / (WIDTH / 4) + (THREADS * 4 / WIDTH) * h, o = (t % (WIDTH / 4)) * 4;
                 floatx4 v;
 #pragma unroll
                 for (int j = 0; j < 4; j++) v[j] = r[4 * h + j];
@@ -94,7 +102,7 @@ struct StridedLoader {
             }
         } else if (MODE == VecK && interior && k0 + BK <= op.K) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
+            for (int h = 0; h < EPT / 4; h++) {
                 const int o = (t >> 2) + 64 * h, k = (t & 3) * 4;
 #pragma unroll
                 for (int j = 0; j < 4; j++) lds[k + j][o] = r[4 * h + j];
@@ -102,10 +110,10 @@ struct StridedLoader {
         } else {
             const bool along_k = (op.sk < 0 ? -op.sk : op.sk) < (op.so < 0 ? -op.so : op.so);
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
+            for (int i = 0; i < EPT; i++) {
                 const int e = t + THREADS * i;
-                const int o = along_k ? (e >> 4) : (e & 127);
-                const int k = along_k ? (e & 15) : (e >> 7);
+                const int o = along_k ? (e >> 4) : (e % WIDTH);
+                const int k = along_k ? (e & 15) : (e / WIDTH);
                 lds[k][o] = r[i];
             }
         }
@@ -115,11 +123,13 @@ struct StridedLoader {
 // Input patches of a convolution as the B operand: k = (c, fy, fx), n = (image, oy, ox). Every thread keeps one
 // fixed n for the whole K loop, so the position is decomposed once; KH / KW are compile-time constants (0 = read
 // them from the parameters) so that splitting k costs multiplications instead of divisions.
-template <int KH, int KW>
+template <int KH, int KW, int WIDTH>
 struct PatchLoader {
+    static constexpr int EPT = BK * WIDTH / THREADS;
+    static constexpr int LDS_STRIDE = WIDTH + 4;
     const float *base;  // input of this thread's image, or null when n is out of range
     int K, in_h, in_w, kh, kw, iy0, ix0;
-    float r[8];
+    float r[EPT];
 
     __device__ __forceinline__ PatchLoader(const ConvParams &p, int n0) {
         kh = KH ? KH : p.kernel_h;
@@ -127,7 +137,7 @@ struct PatchLoader {
         K = p.in_c * kh * kw;
         in_h = p.in_h;
         in_w = p.in_w;
-        const int n = n0 + (threadIdx.x & 127);
+        const int n = n0 + (threadIdx.x % WIDTH);
         const int ohw = p.out_h * p.out_w;
         const long long total = (long long) p.batch * ohw;
         if (n < total) {
@@ -145,8 +155,8 @@ struct PatchLoader {
     __device__ __forceinline__ void fetch(int k0) {
         const int khw = kh * kw;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int k = k0 + (threadIdx.x >> 7) + 2 * i;
+        for (int i = 0; i < EPT; i++) {
+            const int k = k0 + threadIdx.x / WIDTH + (THREADS / WIDTH) * i;
             const int c = k / khw, rem = k - c * khw;
             const int fy = rem / kw, fx = rem - fy * kw;
             const int iy = iy0 + fy, ix = ix0 + fx;
@@ -157,9 +167,9 @@ struct PatchLoader {
 
     __device__ __forceinline__ void stage(float (*lds)[LDS_STRIDE], int) const {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int k = (threadIdx.x >> 7) + 2 * i;
-            lds[k][threadIdx.x & 127] = r[i];
+        for (int i = 0; i < EPT; i++) {
+            const int k = threadIdx.x / WIDTH + (THREADS / WIDTH) * i;
+            lds[k][threadIdx.x % WIDTH] = r[i];
         }
     }
 };
@@ -205,19 +215,20 @@ struct ConvStore {
     }
 };
 
-template <typename LA, typename LB, typename S>
+// MI x NI: MFMA tiles per wave; the workgroup tile is (64 * MI) x (64 * NI) with the 4 waves arranged 2 x 2.
+template <int MI, int NI, typename LA, typename LB, typename S>
 __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int K, int m0, int n0) {
-    __shared__ __attribute__((aligned(16))) float As[BK][LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) float Bs[BK][LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float As[BK][LA::LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Bs[BK][LB::LDS_STRIDE];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    floatx16 acc[2][2];
+    floatx16 acc[MI][NI];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NI; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
@@ -235,25 +246,29 @@ __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int K, int 
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
             const int kr = kk + (lane >> 5), c = lane & 31;
-            const float a0 = As[kr][wm * 64 + c], a1 = As[kr][wm * 64 + 32 + c];
-            const float b0 = Bs[kr][wn * 64 + c], b1 = Bs[kr][wn * 64 + 32 + c];
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            float a[MI], b[NI];
+#pragma unroll
+            for (int i = 0; i < MI; i++) a[i] = As[kr][wm * 32 * MI + 32 * i + c];
+#pragma unroll
+            for (int j = 0; j < NI; j++) b[j] = Bs[kr][wn * 32 * NI + 32 * j + c];
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NI; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
     }
 
     // accumulator layout of the 32x32 tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32
-    const int col0 = n0 + wn * 64 + (lane & 31);
+    const int col0 = n0 + wn * 32 * NI + (lane & 31);
     s.prepare(col0, col0 + 32);
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NI; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int row = m0 + wm * 32 * MI + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 s.store(row, col0 + 32 * j, j, acc[i][j][v]);
             }
 }
@@ -270,32 +285,35 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
     *tn = in_g / rows_here;
 }
 
-template <int A_MODE, int B_MODE>
+// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64)
+template <int A_MODE, int B_MODE, int TI>
 __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
-    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    constexpr int T = 64 * TI;
+    const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
-    const int m0 = tm * BM, n0 = tn * BN;
-    StridedLoader<A_MODE> la(StridedOperand{p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
-    StridedLoader<B_MODE> lb(StridedOperand{p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+    const int m0 = tm * T, n0 = tn * T;
+    StridedLoader<A_MODE, T> la(StridedOperand{p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
+    StridedLoader<B_MODE, T> lb(StridedOperand{p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
     GemmStore s{p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
-    mfma_tile_loop(la, lb, s, p.k, m0, n0);
+    mfma_tile_loop<TI, TI>(la, lb, s, p.k, m0, n0);
 }
 
-template <int A_MODE, int KH, int KW>
+template <int A_MODE, int KH, int KW, int TI>
 __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
+    constexpr int T = 64 * TI;
     const int kh = KH ? KH : p.kernel_h, kw = KW ? KW : p.kernel_w;
     const int K = p.in_c * kh * kw, ohw = p.out_h * p.out_w;
     const long long N = (long long) p.batch * ohw;
-    const int tiles_m = (p.out_c + BM - 1) / BM, tiles_n = (int) ((N + BN - 1) / BN);
+    const int tiles_m = (p.out_c + T - 1) / T, tiles_n = (int) ((N + T - 1) / T);
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
-    const int m0 = tm * BM, n0 = tn * BN;
-    StridedLoader<A_MODE> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
-    PatchLoader<KH, KW> lb(p, n0);
+    const int m0 = tm * T, n0 = tn * T;
+    StridedLoader<A_MODE, T> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
+    PatchLoader<KH, KW, T> lb(p, n0);
     ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
-    mfma_tile_loop(la, lb, s, K, m0, n0);
+    mfma_tile_loop<TI, TI>(la, lb, s, K, m0, n0);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -500,19 +518,44 @@ int pick_mode(const float *ptr, long long so, long long sk, long long batch_stri
     return Scalar;
 }
 
-template <int A_MODE>
+template <int A_MODE, int TI>
 void launch_gemm_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter>), grid, dim3(THREADS), 0, stream, p); break;
-        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK>), grid, dim3(THREADS), 0, stream, p); break;
-        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter, TI>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK, TI>), grid, dim3(THREADS), 0, stream, p); break;
+        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar, TI>), grid, dim3(THREADS), 0, stream, p); break;
     }
 }
 
-template <int KH, int KW>
+template <int TI>
+void launch_gemm_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+    switch (a_mode) {
+        case VecOuter: launch_gemm_b<VecOuter, TI>(b_mode, grid, stream, p); break;
+        case VecK: launch_gemm_b<VecK, TI>(b_mode, grid, stream, p); break;
+        default: launch_gemm_b<Scalar, TI>(b_mode, grid, stream, p); break;
+    }
+}
+
+template <int KH, int KW, int TI>
 void launch_conv_k(int a_mode, dim3 grid, hipStream_t stream, const ConvParams &p) {
-    if (a_mode == VecK) hipLaunchKernelGGL((conv_f32_kernel<VecK, KH, KW>), grid, dim3(THREADS), 0, stream, p);
-    else hipLaunchKernelGGL((conv_f32_kernel<Scalar, KH, KW>), grid, dim3(THREADS), 0, stream, p);
+    if (a_mode == VecK) hipLaunchKernelGGL((conv_f32_kernel<VecK, KH, KW, TI>), grid, dim3(THREADS), 0, stream, p);
+    else hipLaunchKernelGGL((conv_f32_kernel<Scalar, KH, KW, TI>), grid, dim3(THREADS), 0, stream, p);
+}
+
+template <int TI>
+void launch_conv_t(int a_mode, dim3 grid, hipStream_t stream, const ConvParams &p) {
+    if (p.kernel_h == 3 && p.kernel_w == 3) launch_conv_k<3, 3, TI>(a_mode, grid, stream, p);
+    else if (p.kernel_h == 1 && p.kernel_w == 1) launch_conv_k<1, 1, TI>(a_mode, grid, stream, p);
+    else launch_conv_k<0, 0, TI>(a_mode, grid, stream, p);
+}
+
+// 128 x 128 tiles unless there are too few of them to give every compute unit two workgroups.
+int small_tile_threshold() {
+    static const int value = [] {
+        const char *env = getenv("KNHIP_SMALL_TILE_BELOW");
+        return env ? atoi(env) : 512;
+    }();
+    return value;
 }
 
 }  // namespace
@@ -531,35 +574,36 @@ int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
         q.c_sm = p.c_sn; q.c_sn = p.c_sm;
         p = q;
     }
-    const long long tiles = (long long) ((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
+    const long long big_tiles = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128);
+    const bool small = big_tiles * p.batch < small_tile_threshold();
+    const long long tiles = small ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) : big_tiles;
     if (tiles > 0x7fffffffll || p.batch > 65535) return (int) hipErrorInvalidConfiguration;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.a_sb, p.batch);
     const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.b_sb, p.batch);
-    switch (a_mode) {
-        case VecOuter: launch_gemm_b<VecOuter>(b_mode, grid, stream, p); break;
-        case VecK: launch_gemm_b<VecK>(b_mode, grid, stream, p); break;
-        default: launch_gemm_b<Scalar>(b_mode, grid, stream, p); break;
-    }
+    if (small) launch_gemm_a<1>(a_mode, b_mode, grid, stream, p);
+    else launch_gemm_a<2>(a_mode, b_mode, grid, stream, p);
     return (int) hipGetLastError();
 }
 
 int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     const long long positions = (long long) p.batch * p.out_h * p.out_w;
     if (positions <= 0 || p.out_c <= 0) return 0;
-    const long long tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
-    if (positions > 0x7fffffffll || tiles > 0x7fffffffll) return (int) hipErrorInvalidValue;
-    dim3 grid((unsigned) tiles, 1, 1);
+    const long long big_tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
+    if (positions > 0x7fffffffll || big_tiles > 0x7fffffffll / 4) return (int) hipErrorInvalidValue;
     PlaneGeom geom;
     if (plane_geometry(p, &geom)) {
-        hipLaunchKernelGGL((conv_plane_kernel<3, 3>), grid, dim3(THREADS), 0, stream, p, geom);
+        hipLaunchKernelGGL((conv_plane_kernel<3, 3>), dim3((unsigned) big_tiles), dim3(THREADS), 0, stream, p, geom);
         return (int) hipGetLastError();
     }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
     const int a_mode = ((uintptr_t) p.filter % 16 == 0 && K % 4 == 0) ? VecK : Scalar;
-    if (p.kernel_h == 3 && p.kernel_w == 3) launch_conv_k<3, 3>(a_mode, grid, stream, p);
-    else if (p.kernel_h == 1 && p.kernel_w == 1) launch_conv_k<1, 1>(a_mode, grid, stream, p);
-    else launch_conv_k<0, 0>(a_mode, grid, stream, p);
+    if (big_tiles < small_tile_threshold()) {
+        const long long tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64);
+        launch_conv_t<1>(a_mode, dim3((unsigned) tiles), stream, p);
+    } else {
+        launch_conv_t<2>(a_mode, dim3((unsigned) big_tiles), stream, p);
+    }
     return (int) hipGetLastError();
 }
 
