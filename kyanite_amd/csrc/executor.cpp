@@ -75,9 +75,9 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
         Launch &l = launches_[si];
         for (auto &op : step.operands) l.ptrs.push_back(arena_ + plan_.resolve(op.tensor.ptr));
         if (step.kind == StepKind::MatMul) {
-            step.gemm.a = (const float *) l.ptrs[0];
-            step.gemm.b = (const float *) l.ptrs[1];
-            step.gemm.c = (float *) l.ptrs[2];
+            step.gemm.a = l.ptrs[0];
+            step.gemm.b = l.ptrs[1];
+            step.gemm.c = l.ptrs[2];
         } else if (step.kind == StepKind::Conv) {
             size_t k = 0;
             step.conv.input = (const float *) l.ptrs[k++];
@@ -172,7 +172,10 @@ void HipExecutor::launch_step(size_t index, hipEvent_t start, hipEvent_t stop) {
     }
     if (start) hip_check(hipEventRecord(start, stream_), "hipEventRecord");
     switch (step.kind) {
-        case StepKind::MatMul: hip_check((hipError_t) launch_gemm_f32(step.gemm, stream_), "matmul launch"); break;
+        case StepKind::MatMul:
+            hip_check((hipError_t) (step.gemm_f16 ? launch_gemm_f16(step.gemm, stream_) : launch_gemm_f32(step.gemm, stream_)),
+                      "matmul launch");
+            break;
         case StepKind::Conv: hip_check((hipError_t) launch_conv_f32(step.conv, stream_), "conv launch"); break;
         default: {
             void *args[] = {l.ptrs.data()};

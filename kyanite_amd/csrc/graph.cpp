@@ -684,7 +684,7 @@ Value Graph::batched_mat_mul(Value left, Value right) {
 
 Value Graph::softmax(Value input, size_t axis) {
     const ValueInfo &info = (*this)[input];
-    if (info.dtype != DType::F32) fail("Softmax input must be f32");
+    if (info.dtype != DType::F32 && info.dtype != DType::F16) fail("Softmax input must be f32 or f16");
     info.shape.assert_has_axis(axis);
     Operation op;
     op.kind = OpKind::Softmax;
@@ -695,7 +695,7 @@ Value Graph::softmax(Value input, size_t axis) {
 
 Value Graph::layernorm(Value input, size_t axis, float eps) {
     const ValueInfo &info = (*this)[input];
-    if (info.dtype != DType::F32) fail("Layernorm input must be f32");
+    if (info.dtype != DType::F32 && info.dtype != DType::F16) fail("Layernorm input must be f32 or f16");
     info.shape.assert_has_axis(axis);
     Operation op;
     op.kind = OpKind::Layernorm;
@@ -708,7 +708,7 @@ Value Graph::layernorm(Value input, size_t axis, float eps) {
 Value Graph::reduce(Value input, std::vector<size_t> axes, ReduceOp rop) {
     const ValueInfo &info = (*this)[input];
     for (size_t a : axes) info.shape.assert_has_axis(a);
-    if (rop == ReduceOp::Mean && info.dtype != DType::F32) fail("Mean input must be f32");
+    if (rop == ReduceOp::Mean && info.dtype != DType::F32 && info.dtype != DType::F16) fail("Mean input must be f32 or f16");
     if (axes.empty()) return input;
     Shape new_shape = info.shape.replace_all(axes, Shape());
     Operation op;

@@ -1,0 +1,234 @@
+// f16 matrix multiply with f32 accumulation on the CDNA4 matrix cores (v_mfma_f32_32x32x16_f16).
+//
+// Same decomposition as the f32 kernel: a workgroup of 4 waves (2 x 2) owns a T x T tile of D = A * B (T = 128 or
+// 64), every wave (T / 2) x (T / 2) of it as 32 x 32 MFMA tiles. K is walked in slices of 64 that sit in LDS as
+// As[m][k] and Bs[n][k], K contiguous with rows padded by 8 halves: a lane's MFMA operand (8 consecutive k of one
+// row) is one 128 bit LDS read, and operands whose K axis is contiguous in memory (activations, `linear` weights,
+// K^T of attention) move global -> register -> LDS as 128 bit vectors without being transposed. The next slice is
+// fetched into registers while the current one is multiplied; the result is rounded to f16 once, at the store.
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#include "../mfma_kernels.h"
+
+namespace kn {
+
+namespace {
+
+typedef _Float16 half_t;
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 64, THREADS = 256, LDS_K = BK + 8;
+
+enum LoadMode { Scalar = 0, VecOuter = 1, VecK = 2 };
+
+struct Operand {
+    const half_t *p;
+    long long so, sk;  // element strides of the outer (m or n) and the K axis
+    int outer_size, K;
+};
+
+// Fetches a T x BK slice into registers and writes it to LDS as [outer][k]. Vector modes need every vector to lie
+// completely inside or outside the matrix, which the host guarantees (sizes divisible by 8 along the vector axis).
+template <int MODE, int T>
+struct Loader {
+    static constexpr int NVEC = T * BK / 8 / THREADS;  // 128 bit vectors per thread and slice
+    Operand op;
+    int o0;
+    halfx8 r[NVEC];
+
+    __device__ __forceinline__ Loader(const Operand &operand, int outer0) : op(operand), o0(outer0) {}
+
+    __device__ __forceinline__ void fetch(int k0) {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int h = 0; h < NVEC; h++) {
+            if (MODE == VecK) {
+                // 8 vectors cover the 64 k of one row
+                const int o = t / 8 + (THREADS / 8) * h, k = (t % 8) * 8;
+                const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
+                if (ok) r[h] = *(const halfx8 *) (op.p + (long long) (o0 + o) * op.so + (k0 + k));
+                else r[h] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+            } else if (MODE == VecOuter) {
+                // T / 8 vectors cover the T outer indices of one k
+                const int k = t / (T / 8) + (THREADS * 8 / T) * h, o = (t % (T / 8)) * 8;
+                const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
+                if (ok) r[h] = *(const halfx8 *) (op.p + (long long) (k0 + k) * op.sk + (o0 + o));
+                else r[h] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+            } else {
+                // lanes run along k within a row
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int e = (t + THREADS * h) * 8 + j;
+                    const int o = e / BK, k = e % BK;
+                    const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
+                    r[h][j] = ok ? op.p[(long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk] : (half_t) 0;
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void stage(half_t (*lds)[LDS_K]) const {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int h = 0; h < NVEC; h++) {
+            if (MODE == VecK) {
+                const int o = t / 8 + (THREADS / 8) * h, k = (t % 8) * 8;
+                *(halfx8 *) &lds[o][k] = r[h];
+            } else if (MODE == VecOuter) {
+                const int k = t / (T / 8) + (THREADS * 8 / T) * h, o = (t % (T / 8)) * 8;
+#pragma unroll
+                for (int j = 0; j < 8; j++) lds[o + j][k] = r[h][j];
+            } else {
+                const int e = (t + THREADS * h) * 8;
+                *(halfx8 *) &lds[e / BK][e % BK] = r[h];
+            }
+        }
+    }
+};
+
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) {
+    const int id = blockIdx.x;
+    const int group_rows = 8;
+    const int per_group = group_rows * tiles_n;
+    const int g = id / per_group, in_g = id - g * per_group;
+    const int rows_here = min(group_rows, tiles_m - g * group_rows);
+    *tm = g * group_rows + in_g % rows_here;
+    *tn = in_g / rows_here;
+}
+
+// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64)
+template <int A_MODE, int B_MODE, int TI>
+__global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
+    constexpr int T = 64 * TI;
+    __shared__ __attribute__((aligned(16))) half_t As[T][LDS_K];
+    __shared__ __attribute__((aligned(16))) half_t Bs[T][LDS_K];
+
+    const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    const int bz = blockIdx.y;
+    const int m0 = tm * T, n0 = tn * T;
+    Loader<A_MODE, T> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
+    Loader<B_MODE, T> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1, c = lane & 31, half = lane >> 5;
+
+    floatx16 acc[TI][TI];
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TI; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    la.fetch(0);
+    lb.fetch(0);
+    for (int k0 = 0; k0 < p.k; k0 += BK) {
+        __syncthreads();  // the previous slice has been consumed
+        la.stage(As);
+        lb.stage(Bs);
+        __syncthreads();
+        if (k0 + BK < p.k) {
+            la.fetch(k0 + BK);
+            lb.fetch(k0 + BK);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            // lane l supplies 8 consecutive k (starting at 8 * (l / 32)) of row / column l % 32
+            halfx8 a[TI], b[TI];
+#pragma unroll
+            for (int i = 0; i < TI; i++) a[i] = *(const halfx8 *) &As[wm * 32 * TI + 32 * i + c][kk + 8 * half];
+#pragma unroll
+            for (int j = 0; j < TI; j++) b[j] = *(const halfx8 *) &Bs[wn * 32 * TI + 32 * j + c][kk + 8 * half];
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TI; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // accumulator layout of the 32x32 tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32
+    half_t *out = (half_t *) p.c + bz * p.c_sb;
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TI; j++) {
+            const int col = n0 + wn * 32 * TI + 32 * j + c;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wm * 32 * TI + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+                if (row < p.m && col < p.n) out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) acc[i][j][v];
+            }
+        }
+}
+
+// `so` / `sk`: element strides of the outer and the K axis; vectors of 8 halves must be aligned and must not
+// straddle the edge of the matrix.
+int pick_mode(const void *ptr, long long so, long long sk, int outer_size, int k, long long batch_stride, int batch) {
+    const bool aligned = ((uintptr_t) ptr % 16 == 0) && (batch <= 1 || batch_stride % 8 == 0);
+    if (!aligned) return Scalar;
+    if (sk == 1 && so % 8 == 0 && k % 8 == 0) return VecK;
+    if (so == 1 && sk % 8 == 0 && outer_size % 8 == 0) return VecOuter;
+    return Scalar;
+}
+
+template <int A_MODE, int TI>
+void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+    switch (b_mode) {
+        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI>), grid, dim3(THREADS), 0, stream, p); break;
+        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI>), grid, dim3(THREADS), 0, stream, p); break;
+    }
+}
+
+template <int TI>
+void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+    switch (a_mode) {
+        case VecOuter: launch_b<VecOuter, TI>(b_mode, grid, stream, p); break;
+        case VecK: launch_b<VecK, TI>(b_mode, grid, stream, p); break;
+        default: launch_b<Scalar, TI>(b_mode, grid, stream, p); break;
+    }
+}
+
+int small_tile_threshold() {
+    static const int value = [] {
+        const char *env = getenv("KNHIP_SMALL_TILE_BELOW");
+        return env ? atoi(env) : 512;
+    }();
+    return value;
+}
+
+}  // namespace
+
+int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
+    GemmParams p = params;
+    if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
+    // put the axis of C that is contiguous in memory on the MFMA column (lane) axis: D^T = B^T * A^T
+    auto mag = [](long long x) { return x < 0 ? -x : x; };
+    if (mag(p.c_sm) < mag(p.c_sn)) {
+        GemmParams q = p;
+        q.a = p.b; q.b = p.a;
+        q.m = p.n; q.n = p.m;
+        q.a_sb = p.b_sb; q.a_sm = p.b_sn; q.a_sk = p.b_sk;
+        q.b_sb = p.a_sb; q.b_sk = p.a_sk; q.b_sn = p.a_sm;
+        q.c_sm = p.c_sn; q.c_sn = p.c_sm;
+        p = q;
+    }
+    const long long big_tiles = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128);
+    const bool small = big_tiles * p.batch < small_tile_threshold();
+    const long long tiles = small ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) : big_tiles;
+    if (tiles > 0x7fffffffll || p.batch > 65535) return (int) hipErrorInvalidConfiguration;
+    dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
+    const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);
+    const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
+    if (small) launch_a<1>(a_mode, b_mode, grid, stream, p);
+    else launch_a<2>(a_mode, b_mode, grid, stream, p);
+    return (int) hipGetLastError();
+}
+
+}  // namespace kn

@@ -294,9 +294,9 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
     const int m0 = tm * T, n0 = tn * T;
-    StridedLoader<A_MODE, T> la(StridedOperand{p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
-    StridedLoader<B_MODE, T> lb(StridedOperand{p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
-    GemmStore s{p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
+    StridedLoader<A_MODE, T> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
+    StridedLoader<B_MODE, T> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+    GemmStore s{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
     mfma_tile_loop<TI, TI>(la, lb, s, p.k, m0, n0);
 }
 
@@ -510,7 +510,7 @@ bool plane_geometry(const ConvParams &p, PlaneGeom *g) {
 }
 
 // Pick the widest loader an operand allows: `so` / `sk` are the strides of the outer and the K axis.
-int pick_mode(const float *ptr, long long so, long long sk, long long batch_stride, int batch) {
+int pick_mode(const void *ptr, long long so, long long sk, long long batch_stride, int batch) {
     const bool aligned = ((uintptr_t) ptr % 16 == 0) && (batch <= 1 || batch_stride % 4 == 0);
     if (!aligned) return Scalar;
     if (so == 1 && sk % 4 == 0) return VecOuter;

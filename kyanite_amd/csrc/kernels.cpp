@@ -802,9 +802,11 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         });
         ss << "    return " << res << ";\n}\n";
     };
-    KN_ASSERT(desc.pre.nodes.back().dtype == DType::F32);
+    // f16 rows are held, reduced and normalised in f32; the normalised value is rounded to f16 before the epilogue
+    const DType row_dtype = desc.pre.nodes.back().dtype;
+    KN_ASSERT(row_dtype == DType::F32 || row_dtype == DType::F16);
     KN_ASSERT(desc.post.nodes.back().dtype == ops[0].dtype);
-    emit_fn("kn_pre", desc.pre, in_pre, false, DType::F32);
+    emit_fn("kn_pre", desc.pre, in_pre, false, row_dtype);
     emit_fn("kn_post", desc.post, in_post, true, ops[0].dtype);
 
     ss << "#define VEC " << vec << "\n#define ITEMS " << items << "\n#define G " << G << "\n";
@@ -866,7 +868,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         const std::string pick = slot.empty() ? std::string() : "[" + slot + "]";
         std::string o0 = "(base[0] + " + i + " * (idx_t) " + i64_str(axis_strides[0] * (int64_t) vec) + ")";
         auto call = [&](const std::string &j) {
-            std::string c = "kn_post(" + src + "[" + j + "]";
+            std::string c = row_dtype == DType::F16 ? "kn_post(kn_r16(" + src + "[" + j + "])" : "kn_post(" + src + "[" + j + "]";
             for (size_t k = 1; k < ops.size(); k++) {
                 if (!in_post[k]) continue;
                 std::string e = "b" + std::to_string(k) + pick + ((vec > 1 && axis_strides[k] == 1) ? "[" + j + "]" : "");

@@ -10,10 +10,11 @@ struct ihipStream_t;
 namespace kn {
 
 // C[b, i, j] = sum_k A[b, i, k] * B[b, k, j]; element strides are arbitrary (zero batch stride = broadcast operand).
+// The element type (float or _Float16, the same for all three matrices) is fixed by the launch function.
 struct GemmParams {
-    const float *a;
-    const float *b;
-    float *c;
+    const void *a;
+    const void *b;
+    void *c;
     int batch, m, n, k;
     long long a_sb, a_sm, a_sk;
     long long b_sb, b_sk, b_sn;
@@ -38,6 +39,8 @@ struct ConvParams {
 
 // Both return a hipError_t value (0 = success).
 int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
+// f16 operands and result, f32 accumulation, one rounding (to nearest even) at the store
+int launch_gemm_f16(const GemmParams &p, ihipStream_t *stream);
 int launch_conv_f32(const ConvParams &p, ihipStream_t *stream);
 
 }  // namespace kn

@@ -13,7 +13,7 @@ std::string Step::str() const {
     std::ostringstream ss;
     ss << step_kind_name(kind) << " value=" << debug_value;
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
-    if (kind == StepKind::MatMul) ss << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k;
+    if (kind == StepKind::MatMul) ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k;
     else if (kind == StepKind::Conv)
         ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="
            << conv.kernel_h << "x" << conv.kernel_w << (conv_has_bias ? " +bias" : "") << (conv_has_res ? " +res" : "")
@@ -248,14 +248,14 @@ private:
             case OpKind::MatMul: return visit_matmul(value, op.inputs[0], op.inputs[1], true);
             case OpKind::Unary: case OpKind::Binary: return visit_fused_scalar(value);
             case OpKind::Softmax: case OpKind::Layernorm: {
-                KN_ASSERT(result_dtype == DType::F32);
+                KN_ASSERT(result_dtype == DType::F32 || result_dtype == DType::F16);
                 auto row = visit_row_inputs(value);
                 if (!row.ok) return VT::missing(row.need);
                 // no elementwise consumer was fused: the epilogue is the identity
                 ScalarExpr post;
                 ScalarNode n;
                 n.kind = ScalarNode::Load;
-                n.dtype = DType::F32;
+                n.dtype = result_dtype;
                 n.operand = SIZE_MAX;
                 post.nodes.push_back(n);
                 return VT::done(push_row_kernel(value, value, row.value, post, {}));
@@ -263,7 +263,7 @@ private:
             case OpKind::Reduce: {
                 KN_TRY(input, visit(op.inputs[0]));
                 PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
-                if (op.reduce == ReduceOp::Mean) KN_ASSERT(result_dtype == DType::F32);
+                if (op.reduce == ReduceOp::Mean) KN_ASSERT(result_dtype == DType::F32 || result_dtype == DType::F16);
                 Step step;
                 step.kind = StepKind::ReduceOp;
                 step.kernel = make_reduce_kernel(kop(input), kop(output), op.axes, op.reduce);
@@ -327,10 +327,11 @@ private:
         FusedRow row;
         row.axis = op.axis();
         row.eps = op.eps;
+        const DType dt = graph[value].dtype;
         auto load = [&](size_t operand) {
             ScalarNode n;
             n.kind = ScalarNode::Load;
-            n.dtype = DType::F32;
+            n.dtype = dt;
             n.operand = operand;
             row.pre.nodes.push_back(n);
             return row.pre.nodes.size() - 1;
@@ -339,12 +340,12 @@ private:
             if (!alpha) return x;
             ScalarNode c;
             c.kind = ScalarNode::Const;
-            c.dtype = DType::F32;
+            c.dtype = dt;
             c.constant = *alpha;
             row.pre.nodes.push_back(c);
             ScalarNode m;
             m.kind = ScalarNode::Binary;
-            m.dtype = DType::F32;
+            m.dtype = dt;
             m.binary = BinaryOp::Mul;
             m.a = x;
             m.b = row.pre.nodes.size() - 1;
@@ -373,7 +374,7 @@ private:
                 size_t b = scaled(r.value.first, load(2));
                 ScalarNode add;
                 add.kind = ScalarNode::Binary;
-                add.dtype = DType::F32;
+                add.dtype = dt;
                 add.binary = BinaryOp::Add;
                 add.a = a;
                 add.b = b;
@@ -426,17 +427,19 @@ private:
 
     // planner.rs:606-648
     VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first) {
-        if (graph[value].dtype != DType::F32) fail("GPU matmul only supports f32, got ", dtype_name(graph[value].dtype));
+        const DType dt = graph[value].dtype;
+        if (dt != DType::F32 && dt != DType::F16) fail("GPU matmul only supports f32 and f16, got ", dtype_name(dt));
         KN_TRY(left, visit(left_v));
         KN_TRY(right, visit(right_v));
         KN_ASSERT(left.shape.rank() == 3 && right.shape.rank() == 3);
         size_t b = left.shape.shape()[0], m = left.shape.shape()[1], k = left.shape.shape()[2], n = right.shape.shape()[2];
-        PlanTensor result = batch_first ? alloc_tensor_shared({b, m, n}, DType::F32)
-                                        : alloc_tensor_shared({m, b, n}, DType::F32).permute({1, 0, 2});
+        PlanTensor result = batch_first ? alloc_tensor_shared({b, m, n}, dt)
+                                        : alloc_tensor_shared({m, b, n}, dt).permute({1, 0, 2});
         if (b * m * n != 0) {
             KN_ASSERT(b <= INT32_MAX && m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX);
             Step step;
             step.kind = StepKind::MatMul;
+            step.gemm_f16 = dt == DType::F16;
             GemmParams &g = step.gemm;
             g.batch = (int) b; g.m = (int) m; g.n = (int) n; g.k = (int) k;
             g.a_sb = left.shape.strides()[0]; g.a_sm = left.shape.strides()[1]; g.a_sk = left.shape.strides()[2];

@@ -35,6 +35,7 @@ struct Step {
     std::shared_ptr<const CodeObject> code;
     // matrix-core kernels; the pointers are filled in when the plan is realised
     GemmParams gemm{};
+    bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
     ConvParams conv{};
     bool conv_has_bias = false, conv_has_res = false;
 

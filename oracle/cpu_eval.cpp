@@ -16,7 +16,8 @@
 // element sequentially in f32, which is tolerance-equal, not bit-equal, to the reference's CPU path.
 //
 // Deviation: binary operations, matmul and conv on f64 operands are evaluated (the reference panics for f64
-// pairs, dtype.rs:460-483); F16 (absent from the reference) computes in f32 and rounds every result to f16.
+// pairs, dtype.rs:460-483); F16 (absent from the reference) loads f16, computes and accumulates in f32 and rounds the
+// result of every operation of the graph to f16 once (reduce, mean, softmax, layernorm and matmul included).
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -604,9 +605,25 @@ void split_axis(const std::vector<size_t> &shape, size_t axis, size_t *outer, si
 
 float rust_max(float a, float b) { return std::isnan(a) ? b : (std::isnan(b) ? a : (a > b ? a : b)); }
 
+// F16 tensors (absent from the reference) as f32 and back: row operations load f16, compute in f32 and round once.
+Tensor widen_f16(const Tensor &x) {
+    Tensor out = Tensor::make(F32, x.shape);
+    size_t n = out.len();
+    for (size_t i = 0; i < n; i++) out.ptr<float>()[i] = h2f(x.ptr<uint16_t>()[i]);
+    return out;
+}
+
+Tensor narrow_f16(const Tensor &x) {
+    Tensor out = Tensor::make(F16, x.shape);
+    size_t n = x.len();
+    for (size_t i = 0; i < n; i++) out.ptr<uint16_t>()[i] = f2h(x.ptr<float>()[i]);
+    return out;
+}
+
 Tensor eval_softmax(const Tensor &x, size_t axis) {
     // cpu.rs:443-458
-    if (x.dtype != F32) die("oracle: softmax input must be f32");
+    if (x.dtype == F16) return narrow_f16(eval_softmax(widen_f16(x), axis));
+    if (x.dtype != F32) die("oracle: softmax input must be f32 or f16");
     Tensor out = Tensor::make(F32, x.shape);
     size_t outer, len, inner;
     split_axis(x.shape, axis, &outer, &len, &inner);
@@ -631,7 +648,8 @@ Tensor eval_softmax(const Tensor &x, size_t axis) {
 
 Tensor eval_layernorm(const Tensor &x, size_t axis, float eps) {
     // cpu.rs:461-479: biased variance, eps inside the square root
-    if (x.dtype != F32) die("oracle: layernorm input must be f32");
+    if (x.dtype == F16) return narrow_f16(eval_layernorm(widen_f16(x), axis, eps));
+    if (x.dtype != F32) die("oracle: layernorm input must be f32 or f16");
     Tensor out = Tensor::make(F32, x.shape);
     size_t outer, len, inner;
     split_axis(x.shape, axis, &outer, &len, &inner);
@@ -681,13 +699,14 @@ Tensor eval_reduce(const Node &nd, const Tensor &x, const std::vector<size_t> &o
         if (curr.dtype == F16) {
             const uint16_t *s = curr.ptr<uint16_t>();
             uint16_t *d = next.ptr<uint16_t>();
-            // every partial result is an f16 value
+            // f32 accumulation over the lane, one rounding at the end
             float ident = nd.sub == Prod ? 1.0f : nd.sub == RMin ? INFINITY : nd.sub == RMax ? -INFINITY : 0.0f;
             uint8_t bop = nd.sub == Prod ? Mul : nd.sub == RMin ? Min : nd.sub == RMax ? Max : Add;
             for (size_t o = 0; o < outer; o++)
                 for (size_t i = 0; i < inner; i++) {
                     float acc = ident;
-                    for (size_t j = 0; j < len; j++) acc = h2f(f2h(binary_scalar<float>(bop, acc, h2f(s[o * len * inner + j * inner + i]))));
+                    for (size_t j = 0; j < len; j++) acc = binary_scalar<float>(bop, acc, h2f(s[o * len * inner + j * inner + i]));
+                    if (nd.sub == Mean) acc = acc / (float) len;
                     d[o * inner + i] = f2h(acc);
                 }
         } else {

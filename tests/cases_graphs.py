@@ -881,3 +881,90 @@ def conv_plane_2x128():
 def conv_plane_32x4():
     """narrow tall image: a tile is 32 rows"""
     return _plane_conv_case(25, 3, 16, 7, 64, 4, False)
+
+
+# ---- f16 storage with f32 arithmetic (an extension over the reference IR, which has no f16)
+
+def _f16(rng, *shape, scale=1.0):
+    return (rng.standard_normal(shape) * scale).astype(np.float16)
+
+
+@case
+def f16_elementwise_chain():
+    g = Graph()
+    rng = np.random.default_rng(30)
+    x = g.input([BATCH, 40], DType.F16)
+    w = g.constant([1, 40], _f16(rng, 1, 40))
+    y = g.mul(g.add(x, w), g.scalar(0.5, DType.F16))
+    y = g.unary(UnaryOp.EXP, y)
+    g.output_all([y, g.value_cast(y, DType.F32), g.value_cast(g.value_cast(y, DType.F32), DType.F16)])
+    return g, 3, [_f16(rng, 3, 40)], None
+
+
+@case
+def f16_matmul_layouts():
+    """K-contiguous (linear), N-contiguous and transposed-result operands, sizes that are multiples of 8"""
+    g = Graph()
+    rng = np.random.default_rng(31)
+    a = g.input([72, 136], DType.F16)
+    w = g.constant([200, 136], _f16(rng, 200, 136, scale=0.1))
+    b = g.constant([136, 64], _f16(rng, 136, 64, scale=0.1))
+    lin = g.linear(a, w)
+    nn = g.mat_mul(a, b)
+    g.output_all([lin, nn, g.permute(lin, [1, 0])])
+    return g, 0, [_f16(rng, 72, 136)], None
+
+
+@case
+def f16_matmul_odd_sizes():
+    """nothing is a multiple of 8: every operand goes through the element-wise loader"""
+    g = Graph()
+    rng = np.random.default_rng(32)
+    a = g.input([3, 37, 45], DType.F16)
+    b = g.input([3, 45, 51], DType.F16)
+    g.output(g.batched_mat_mul(a, b))
+    return g, 0, [_f16(rng, 3, 37, 45), _f16(rng, 3, 45, 51)], None
+
+
+@case
+def f16_matmul_big_tiles():
+    """enough tiles for the 128 x 128 kernel, with partial tiles on both axes and a K tail"""
+    g = Graph()
+    rng = np.random.default_rng(33)
+    a = g.input([16, 264, 200], DType.F16)
+    b = g.input([16, 328, 200], DType.F16)
+    g.output(g.batched_mat_mul(a, g.permute(b, [0, 2, 1])))
+    return g, 0, [_f16(rng, 16, 264, 200, scale=0.2), _f16(rng, 16, 328, 200, scale=0.2)], None
+
+
+@case
+def f16_attention():
+    """softmax(q k^T / sqrt(d) + causal mask) v, all in f16"""
+    g = Graph()
+    rng = np.random.default_rng(34)
+    heads, seq, d = 4, 48, 32
+    q = g.input([heads, seq, d], DType.F16)
+    k = g.input([heads, seq, d], DType.F16)
+    v = g.input([heads, seq, d], DType.F16)
+    mask = np.where(np.tril(np.ones((seq, seq), bool)), 0.0, -np.inf).astype(np.float16)
+    scores = g.batched_mat_mul(q, g.permute(k, [0, 2, 1]))
+    scores = g.add(g.mul(scores, g.scalar(1.0 / np.sqrt(d), DType.F16)), g.constant([1, seq, seq], mask))
+    out = g.batched_mat_mul(g.softmax(scores, 2), v)
+    g.output(out)
+    return g, 0, [_f16(rng, heads, seq, d), _f16(rng, heads, seq, d), _f16(rng, heads, seq, d)], None
+
+
+@case
+def f16_norms():
+    """layernorm with gamma / beta, RMSNorm from primitives, mean / sum / max reductions"""
+    g = Graph()
+    rng = np.random.default_rng(35)
+    x = g.input([BATCH, 6, 256], DType.F16)
+    gamma = g.constant([1, 1, 256], (1.0 + 0.1 * rng.standard_normal(256)).astype(np.float16))
+    beta = g.constant([1, 1, 256], _f16(rng, 256, scale=0.1))
+    ln = g.add(g.mul(g.layernorm(x, 2, 1e-5), gamma), beta)
+    ms = g.reduce(g.mul(x, x), [2], ReduceOp.MEAN)
+    rms = g.unary(UnaryOp.SQRT, g.add(g.view(ms, [BATCH, 6, 1]), g.scalar(1e-5, DType.F16)))
+    rn = g.mul(g.binary(BinaryOp.DIV, x, rms), gamma)
+    g.output_all([ln, rn, g.reduce(x, [2], ReduceOp.SUM), g.reduce(x, [1], ReduceOp.MAX), g.softmax(x, 1)])
+    return g, 5, [_f16(rng, 5, 6, 256)], None
