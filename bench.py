@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
-"""Benchmark of the HIP executor on the bandwidth-bound operator graphs (BASELINE.json configs[1]).
+"""Benchmark of the HIP executor. One JSON line per run.
 
-One step = one `run_async` (device only, inputs resident in HBM) of ONE executor whose graph holds the four
-operator graphs side by side, so the four kernels run back to back on one stream:
+Default workload `bandwidth` (BASELINE.json configs[1], the configuration the metric is quoted on): one step =
+one `run_async` (device only, inputs resident in HBM) of ONE executor whose graph holds the four operator graphs
+side by side, so the four kernels run back to back on one stream:
   (a) y = tanh-GELU(x * a + b) + r on [64, 1024, 1024] with a, b broadcast from [1024]
   (b) softmax over the last axis of [32, 16, 512, 512]
   (c) layernorm over the last axis of [8192, 4096] with gamma / beta, eps 1e-5
@@ -11,11 +12,22 @@ The metric is graph evaluations per second (four per step). The JSON line also c
 achieved HBM bandwidth (algorithmic bytes / launch duration measured with HIP events on the executor's stream)
 against the 8 TB/s peak, and the oracle (`cpu_eval_graph` restatement) timed on one host core.
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
+The other workloads run one of the remaining configurations the same way (one step = one evaluation of the graph):
+  --workload mlp     configs[0]  tiny MLP, batch 8 (launch latency)
+  --workload resnet  configs[2]  AlphaZero style ResNet tower, f32, batch 1024
+  --workload llama   configs[3]  2 layer LLaMA style decoder, f16, sequence 512
+  --workload unet    configs[4]  Stable-Diffusion style UNet block, f32, batch 2
+For these the roofline entry is the kernel family with the largest share of the step (identical launches are
+averaged), against the MFMA peak when it is a matmul / conv and against the HBM peak otherwise; the parity check
+and the CPU baseline use a bounded sample of the same workload that the oracle finishes in seconds (stated in
+`cpu_baseline.sample`), chosen so that the GPU result at full size must reproduce it.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -23,6 +35,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0}
 
 # HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` (KiB per dispatch),
 # each scaled by what the same counter reads for a kernel of known traffic (y = 2 * x on [64,1024,1024]:
@@ -35,31 +48,56 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def main():
-    parser = argparse.ArgumentParser()
-    parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=50)
-    parser.add_argument("--warmup", type=int, default=5)
-    parser.add_argument("--no-cpu-baseline", action="store_true", help="skip the timed CPU oracle leg and parity check")
-    parser.add_argument("--copy-probe", action="store_true",
-                        help="also launch y = 2 * x on [64,1024,1024] once (a kernel of known traffic, 536,870,912 B, "
-                             "to calibrate hardware counters against)")
-    parser.add_argument("--order", default="abcd", help="order of the four graphs inside one step (letters a-d)")
-    parser.add_argument("--kernel-iters", type=int, default=20, help="profiled runs for the per-kernel timing")
-    args = parser.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this build runs on exactly one GPU (one executor, one arena, no collectives); "
-              f"--gpus {args.gpus} is not supported", file=sys.stderr)
-        sys.exit(2)
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
+
+def rel_error(expected, actual):
+    """max |a - e| / max(|e|, 0.5 * rms(e)) over the finite entries; non-finite entries must agree exactly."""
+    import numpy as np
+    e64, a64 = np.asarray(expected, np.float64), np.asarray(actual, np.float64)
+    special = ~np.isfinite(e64)
+    if special.any() and not np.array_equal(e64[special], a64[special], equal_nan=True):
+        return float("inf")
+    e64, a64 = e64[~special], a64[~special]
+    if e64.size == 0:
+        return 0.0
+    floor = max(0.5 * np.sqrt(np.mean(e64 * e64)), 1e-30)
+    return float(np.max(np.abs(a64 - e64) / np.maximum(np.abs(e64), floor)))
+
+
+def timed_steps(ex, steps, warmup):
+    for _ in range(warmup):
+        ex.run_async()
+    ex.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ex.run_async()
+    ex.synchronize()
+    return time.perf_counter() - t0
+
+
+def per_step_seconds(ex, iters):
+    """Average launch duration of every step: HIP events around each launch, on the stream the kernels run on."""
+    import numpy as np
+    ex.set_profile(True)
+    per_step = np.zeros(ex.step_count())
+    for _ in range(iters):
+        ex.run_async()
+        per_step += np.asarray(ex.last_profile().step_seconds)
+    ex.set_profile(False)
+    return per_step / iters
+
+
+# ------------------------------------------------------------------------------------------------ bandwidth graphs
+
+def run_bandwidth(args, device):
     import numpy as np
 
-    from kyanite_amd import Graph, HipDevice, HipExecutor
+    from kyanite_amd import Graph, HipExecutor
     from kyanite_amd.configs import BANDWIDTH_CONFIGS
 
-    device = HipDevice(0)
     t_setup = time.time()
-
     # one graph that holds the four operator graphs side by side
     combined = Graph()
     parts = []  # (name, sub graph, first input index, input count, algorithmic bytes, input factory)
@@ -84,9 +122,8 @@ def main():
             ex.upload_input(first + k, x)
         host_inputs[name] = inputs
     for i in range(ex.step_count()):
-        print(f"[bench] step {i}: {ex.step_str(i)}", file=sys.stderr, flush=True)
-    print(f"[bench] setup took {time.time() - t_setup:.1f} s, arena {ex.mem_usage['arena_bytes'] / 2**20:.0f} MiB",
-          file=sys.stderr, flush=True)
+        log(f"step {i}: {ex.step_str(i)}")
+    log(f"setup took {time.time() - t_setup:.1f} s, arena {ex.mem_usage['arena_bytes'] / 2**20:.0f} MiB")
 
     if args.copy_probe:
         pg = Graph()
@@ -96,29 +133,15 @@ def main():
         probe.upload_input(0, np.ones((64, 1024, 1024), np.float32))
         probe.run_async()
         probe.synchronize()
-        print(f"[bench] copy probe launched: {probe.step_str(0)}", file=sys.stderr, flush=True)
+        log(f"copy probe launched: {probe.step_str(0)}")
         del probe
 
-    # ---- the timed region: K steps between two synchronisations
-    for _ in range(args.warmup):
-        ex.run_async()
-    ex.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        ex.run_async()
-    ex.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    evals_per_s = len(parts) * args.steps / elapsed
+    steps = args.steps if args.steps is not None else 50
+    elapsed = timed_steps(ex, steps, args.warmup)
+    ms_per_step = elapsed / steps * 1e3
+    evals_per_s = len(parts) * steps / elapsed
 
-    # ---- per-kernel launch durations: HIP events around every step, on the stream the kernels run on
-    ex.set_profile(True)
-    per_step = np.zeros(ex.step_count())
-    for _ in range(args.kernel_iters):
-        ex.run_async()
-        per_step += np.asarray(ex.last_profile().step_seconds)
-    ex.set_profile(False)
-    per_step /= args.kernel_iters
+    per_step = per_step_seconds(ex, args.kernel_iters)
     kernels = {}
     for i, (name, _, _, _, algo_bytes, _) in enumerate(parts):
         ms = per_step[i] * 1e3
@@ -140,25 +163,22 @@ def main():
             dt = time.perf_counter() - t
             cpu_seconds += dt
             sample_desc.append(f"{name} {dt:.2f} s")
-            actual = ex.download_output(i)
-            e64, a64 = expected[0].astype(np.float64), actual.astype(np.float64)
-            floor = 0.1 * np.sqrt(np.mean(e64 * e64))
-            err = float(np.max(np.abs(a64 - e64) / np.maximum(np.abs(e64), floor)))
+            err = rel_error(expected[0], ex.download_output(i))
             kernels[name]["max_rel_err_vs_oracle"] = float(f"{err:.3e}")
             if not err <= 1e-4:
-                print(f"[bench] PARITY FAILURE on {name}: max relative error {err:.3e}", file=sys.stderr)
+                log(f"PARITY FAILURE on {name}: max relative error {err:.3e}")
                 sys.exit(1)
         cpu_baseline = {"value": round(len(parts) / cpu_seconds, 4), "unit": "graph evals/s", "cores": 1, "kind": "port",
                         "sample": "oracle (C++ restatement of cpu_eval_graph, single thread) on the whole workload, one "
                                   "evaluation of each graph at full shape: " + ", ".join(sample_desc)}
 
     dom = kernels[dominant]
-    result = {
+    return {
         "metric": "graph evals/sec at 1 GPU (bandwidth-bound op graphs 2a-2d, device only)",
         "value": round(evals_per_s, 2),
         "unit": "graph evals/s",
         "n_gpus": 1,
-        "steps": args.steps,
+        "steps": steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
@@ -176,6 +196,229 @@ def main():
         "cpu_baseline": cpu_baseline,
         "device": device.name(),
     }
+
+
+# ------------------------------------------------------------------------------------------------ whole-model graphs
+
+def kernel_table(ex, per_step):
+    """Identical launches (same step description apart from the value id) grouped into one entry."""
+    groups = {}
+    for i in range(ex.step_count()):
+        sig = re.sub(r" value=\d+", "", ex.step_str(i))
+        sig = re.sub(r' id="[^"]*"', "", sig)
+        flops, nbytes = ex.step_work(i)
+        grp = groups.setdefault(sig, {"launches": 0, "total_s": 0.0, "flops": flops, "bytes": nbytes})
+        grp["launches"] += 1
+        grp["total_s"] += float(per_step[i])
+    table = []
+    for sig, grp in groups.items():
+        avg = grp["total_s"] / grp["launches"]
+        f16 = " f16 " in sig or sig.endswith(" f16")
+        entry = {"kernel": sig, "launches": grp["launches"], "avg_ms": round(avg * 1e3, 5),
+                 "share": 0.0, "total_ms": round(grp["total_s"] * 1e3, 5)}
+        if grp["flops"] > 0:
+            tf = grp["flops"] / avg / 1e12
+            peak = MFMA_PEAK_TFLOPS["f16" if f16 else "f32"]
+            entry.update({"flops": grp["flops"], "achieved_tflops": round(tf, 2), "mfma_frac": round(tf / peak, 4),
+                          "mfma_peak_tflops": peak})
+        gbs = grp["bytes"] / avg / 1e9
+        entry.update({"algorithmic_bytes": grp["bytes"], "achieved_gbs": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)})
+        table.append(entry)
+    total = sum(e["total_ms"] for e in table) or 1.0
+    for e in table:
+        e["share"] = round(e["total_ms"] / total, 4)
+    table.sort(key=lambda e: -e["total_ms"])
+    return table
+
+
+def roofline_of(entry):
+    # a matmul / conv is priced against the matrix cores unless its arithmetic intensity puts it under the HBM roof
+    if "achieved_tflops" in entry and entry["mfma_frac"] >= entry["hbm_frac"]:
+        return {"bound": "mfma", "kernel": entry["kernel"], "achieved": entry["achieved_tflops"],
+                "peak": entry["mfma_peak_tflops"], "unit": "TFLOP/s", "frac": entry["mfma_frac"], "traffic": None}
+    return {"bound": "hbm", "kernel": entry["kernel"], "achieved": entry["achieved_gbs"], "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": entry["hbm_frac"], "traffic": None}
+
+
+def run_model(args, device, workload):
+    import numpy as np
+
+    from kyanite_amd import HipExecutor
+    from kyanite_amd import configs
+
+    t_setup = time.time()
+    dtype, tol = "f32", 1e-4
+    if workload == "mlp":
+        batch = 8
+        graph, inputs = configs.build_tiny_mlp(seed=0, batch=batch)
+        flops = 2 * batch * (16 * 32 + 32 * 10)
+        desc = "BASELINE configs[0]: tiny MLP 16->32->10 with softmax, f32, batch 8"
+        default_steps = 5000
+    elif workload == "resnet":
+        batch = 1024
+        graph, make_inputs, flop_per_pos = configs.build_resnet_tower(seed=0)
+        inputs = make_inputs(batch)
+        flops = flop_per_pos * batch
+        desc = "BASELINE configs[2]: AlphaZero style ResNet tower (10 blocks x 128 channels on 8x8, policy + value heads), f32, batch 1024"
+        default_steps = 20
+    elif workload == "llama":
+        batch = 0
+        graph, make_inputs, flops = configs.build_llama(seed=0)
+        inputs = make_inputs()
+        dtype, tol = "f16", 2e-2
+        desc = ("BASELINE configs[3]: 2 layer LLaMA style decoder, d_model 4096, 32 heads, FFN 11008, f16 weights and "
+                "activations with f32 accumulation, batch 1, prefill of 512 tokens")
+        default_steps = 20
+    elif workload == "unet":
+        batch = 0
+        graph, make_inputs, flops = configs.build_unet_block(seed=0)
+        inputs = make_inputs()
+        desc = ("BASELINE configs[4]: Stable-Diffusion style UNet block (ResBlock 320 channels at 64x64 + spatial "
+                "transformer with self / cross attention and GEGLU), f32, batch 2")
+        default_steps = 10
+    else:
+        raise SystemExit(f"unknown workload {workload}")
+    log(f"graph built in {time.time() - t_setup:.1f} s")
+
+    ex = HipExecutor(device, graph, batch, preserve_inputs=True)
+    for k, x in enumerate(inputs):
+        ex.upload_input(k, x)
+    log(f"setup took {time.time() - t_setup:.1f} s, {ex.step_count()} steps, arena {ex.mem_usage['arena_bytes'] / 2**20:.0f} MiB")
+
+    steps = args.steps if args.steps is not None else default_steps
+    elapsed = timed_steps(ex, steps, args.warmup)
+    ms_per_step = elapsed / steps * 1e3
+    evals_per_s = steps / elapsed
+
+    per_step = per_step_seconds(ex, min(args.kernel_iters, 5))
+    table = kernel_table(ex, per_step)
+    for e in table[:12]:
+        log(f"{e['share'] * 100:5.1f}%  {e['launches']:3d} x {e['avg_ms']:9.4f} ms  "
+            f"{e.get('achieved_tflops', 0):8.2f} TFLOP/s  {e['achieved_gbs']:8.1f} GB/s  {e['kernel'][:110]}")
+    extra = {}
+
+    # ---- parity on a bounded sample the full-size run must reproduce, and the same sample as CPU baseline
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_eval_graph
+        gpu_outputs = [ex.download_output(i) for i in range(len(ex.output_info))]
+        if workload == "mlp":
+            n = 1000
+            t = time.perf_counter()
+            for _ in range(n):
+                expected = cpu_eval_graph(graph, batch, inputs)
+            cpu_seconds = (time.perf_counter() - t) / n
+            compare = list(zip(expected, gpu_outputs))
+            cpu_evals = 1.0 / cpu_seconds
+            sample = f"{n} evaluations of the whole graph at batch 8 ({cpu_seconds * 1e6:.1f} us each)"
+        elif workload == "resnet":
+            rows = 16  # positions are independent of each other: the first rows of the batch must match
+            t = time.perf_counter()
+            expected = cpu_eval_graph(graph, rows, [x[:rows] for x in inputs])
+            cpu_seconds = time.perf_counter() - t
+            compare = [(e, g[:rows]) for e, g in zip(expected, gpu_outputs)]
+            cpu_evals = rows / cpu_seconds / batch
+            sample = (f"the first {rows} of the 1024 positions ({cpu_seconds:.2f} s), scaled to evaluations of 1024 "
+                      f"positions; the GPU's first {rows} rows at batch 1024 are checked against them")
+        elif workload == "llama":
+            rows = 16  # causal attention: the first tokens do not depend on the later ones
+            small, _, _ = configs.build_llama(seed=0, seq=rows)
+            t = time.perf_counter()
+            expected = cpu_eval_graph(small, 0, [inputs[0][:, :rows]])
+            cpu_seconds = time.perf_counter() - t
+            compare = [(expected[0], gpu_outputs[0][:, :rows])]
+            cpu_evals = rows / cpu_seconds / 512
+            sample = (f"the same decoder on the first {rows} of the 512 tokens ({cpu_seconds:.2f} s), scaled to "
+                      f"evaluations of 512 tokens; by causality the GPU's first {rows} output rows at sequence 512 are "
+                      "checked against them")
+        else:
+            # samples of the batch are independent: the first one at full resolution
+            one, _, _ = configs.build_unet_block(seed=0, batch=1)
+            t = time.perf_counter()
+            expected = cpu_eval_graph(one, 0, [x[:1] for x in inputs])
+            cpu_seconds = time.perf_counter() - t
+            compare = [(expected[0], gpu_outputs[0][:1])]
+            cpu_evals = 1.0 / cpu_seconds / 2
+            sample = (f"the first of the 2 samples at full resolution ({cpu_seconds:.2f} s), scaled to evaluations of "
+                      "batch 2; the GPU's first sample at batch 2 is checked against it")
+        worst = 0.0
+        for e, a in compare:
+            assert e.shape == a.shape and e.dtype == a.dtype, (e.shape, a.shape, e.dtype, a.dtype)
+            worst = max(worst, rel_error(e, a))
+        extra["max_rel_err_vs_oracle"] = float(f"{worst:.3e}")
+        if not worst <= tol:
+            log(f"PARITY FAILURE on {workload}: max relative error {worst:.3e} exceeds {tol:.0e}")
+            sys.exit(1)
+        cpu_baseline = {"value": float(f"{cpu_evals:.4g}"), "unit": "graph evals/s", "cores": 1, "kind": "port",
+                        "sample": "oracle (C++ restatement of cpu_eval_graph, single thread) on " + sample}
+
+    if workload == "mlp":
+        # the reference's executor contract includes the copies: time `evaluate` (H2D, launches, D2H) as well
+        n = 2000
+        for _ in range(20):
+            ex.evaluate(inputs)
+        t = time.perf_counter()
+        for _ in range(n):
+            ex.evaluate(inputs)
+        dt = (time.perf_counter() - t) / n
+        extra["evaluate_with_copies_us"] = round(dt * 1e6, 2)
+        extra["evaluate_with_copies_evals_per_s"] = round(1.0 / dt, 1)
+
+    mfma_s = sum(float(per_step[i]) for i in range(ex.step_count()) if ex.step_work(i)[0] > 0)
+    mfma_flops = sum(ex.step_work(i)[0] for i in range(ex.step_count()))
+    if mfma_s > 0:
+        peak = MFMA_PEAK_TFLOPS[dtype]
+        extra["matmul_conv_total"] = {"ms": round(mfma_s * 1e3, 4), "tflops": round(mfma_flops / mfma_s / 1e12, 2),
+                                      "mfma_frac": round(mfma_flops / mfma_s / 1e12 / peak, 4)}
+    result = {
+        "metric": f"graph evals/sec at 1 GPU ({workload}, device only)",
+        "value": round(evals_per_s, 3),
+        "unit": "graph evals/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {"workload": desc, "inputs_resident_in_hbm": True, "flop_per_eval": flops,
+                   "whole_graph_tflops": round(flops * evals_per_s / 1e12, 2)},
+        "roofline": roofline_of(table[0]),
+        "kernels": table[:16],
+        "cpu_baseline": cpu_baseline,
+        "device": device.name(),
+    }
+    result.update(extra)
+    return result
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=None, help="timed steps (default: 50 for the bandwidth graphs)")
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--workload", default="bandwidth", choices=["bandwidth", "mlp", "resnet", "llama", "unet"])
+    parser.add_argument("--no-cpu-baseline", action="store_true", help="skip the timed CPU oracle leg and parity check")
+    parser.add_argument("--copy-probe", action="store_true",
+                        help="also launch y = 2 * x on [64,1024,1024] once (a kernel of known traffic, 536,870,912 B, "
+                             "to calibrate hardware counters against)")
+    parser.add_argument("--order", default="abcd", help="order of the four graphs inside one step (letters a-d)")
+    parser.add_argument("--kernel-iters", type=int, default=20, help="profiled runs for the per-kernel timing")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on exactly one GPU (one executor, one arena, no collectives); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    from kyanite_amd import HipDevice
+
+    device = HipDevice(0)
+    if args.workload == "bandwidth":
+        result = run_bandwidth(args, device)
+    else:
+        result = run_model(args, device, args.workload)
     print(json.dumps(result))
 
 

@@ -224,6 +224,10 @@ int knhip_executor_step_count(const knhip_executor *ex, size_t *count);
 /* kind: 0 conv, 1 mat_mul, 2 scalar_op, 3 reduce_op, 4 softmax_op, 5 layernorm_op, 6 gather_op */
 int knhip_executor_step_kind(const knhip_executor *ex, size_t index, int *kind);
 int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed);
+/* algorithmic work of one launch of the step, for roofline reports next to the per-step times of the profile
+ * (the role of the per-kernel lines of kn-cuda-eval/src/executor.rs:269-289 and profile_net.rs:147-171):
+ * flops = 2 * multiply-adds of a conv / mat_mul step (0 for the others), bytes = every distinct operand element once */
+int knhip_executor_step_work(const knhip_executor *ex, size_t index, double *flops, double *bytes);
 int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed);
 int knhip_executor_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed);
 

@@ -4,7 +4,7 @@ There is no fallback: if the library is missing (run `python kyanite_amd/build.p
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int64, c_size_t, c_uint8, c_uint32, c_uint64, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_uint8, c_uint32, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libknhip.so")
@@ -124,6 +124,7 @@ SIGNATURES = {
     "knhip_executor_step_count": [E, PZ],
     "knhip_executor_step_kind": [E, c_size_t, POINTER(c_int)],
     "knhip_executor_step_str": [E, c_size_t, c_char_p, c_size_t, PZ],
+    "knhip_executor_step_work": [E, c_size_t, POINTER(c_double), POINTER(c_double)],
     "knhip_executor_step_source": [E, c_size_t, c_char_p, c_size_t, PZ],
     "knhip_executor_str": [E, c_char_p, c_size_t, PZ],
     "knhip_strided_flags": [PZ, POINTER(c_int64), c_size_t, POINTER(c_int), POINTER(c_int)],

@@ -55,6 +55,17 @@ def normal(seed, stream, shape, mean=0.0, std=1.0):
     return out.reshape(shape)
 
 
+_LARGE_CACHE = {}
+
+
+def cached_normal(seed, stream, shape, std, np_dtype):
+    """`normal` for large weight tensors that several graphs of one process share (full size and sample builds)."""
+    key = (seed, stream, tuple(shape), float(std), np.dtype(np_dtype).str)
+    if key not in _LARGE_CACHE:
+        _LARGE_CACHE[key] = normal(seed, stream, shape, std=std).astype(np_dtype)
+    return _LARGE_CACHE[key]
+
+
 def bernoulli(seed, stream, shape, p):
     return (uniform(seed, stream, shape) < p).astype(np.float32)
 
@@ -187,3 +198,172 @@ def build_resnet_tower(seed=0, channels=128, blocks=10, board=8, in_planes=21, p
     macs = (in_planes * 9 * channels * hw + blocks * 2 * channels * 9 * channels * hw + channels * policy_channels * hw +
             policy_channels * hw * policy_size + channels * value_channels * hw + value_channels * hw * value_hidden + value_hidden)
     return g, inputs, 2 * macs  # flop per position
+
+
+# ---------------------------------------------------------------------------------------------- config 4
+
+def build_llama(seed=0, layers=2, seq=512, d_model=4096, heads=32, ffn=11008, eps=1e-6, rope_base=10000.0,
+                dtype=DType.F16):
+    """LLaMA style decoder on one sequence: RMSNorm, rotary embedding on Q / K, causal softmax attention, SwiGLU
+    feed-forward, residual adds; f16 weights / activations (f32 accumulation inside every operation).
+    Everything is spelled with primitive operations: RMSNorm = x / sqrt(mean(x * x) + eps) * g, rotary = slices +
+    mul + sub / add + concat, the causal mask = an added constant holding -inf, SiLU = x * sigmoid(x).
+    Weights N(0, 0.02), norm gains 1, input embeddings N(0, 1) of shape [1, seq, d_model].
+    Returns (graph, make_inputs, flop per evaluation). Because of the causal mask, the first t rows of the output
+    depend only on the first t rows of the input."""
+    np_dt = DType(dtype).numpy
+    d_head = d_model // heads
+    assert d_head * heads == d_model and d_head % 2 == 0
+    g = Graph()
+    stream = [400]
+
+    def weight(co, ci):
+        stream[0] += 1
+        return g.constant([co, ci], cached_normal(seed, stream[0], (co, ci), 0.02, np_dt))
+
+    def const(shape, array):
+        return g.constant(list(shape), np.ascontiguousarray(array).astype(np_dt))
+
+    def rmsnorm(x):
+        ms = g.view(g.reduce(g.mul(x, x), [1], ReduceOp.MEAN), [seq, 1])
+        rms = g.unary(UnaryOp.SQRT, g.add(ms, g.scalar(eps, dtype)))
+        gain = const((1, d_model), np.ones((1, d_model)))
+        return g.mul(g.binary(BinaryOp.DIV, x, rms), gain)
+
+    # rotary tables, HF layout: the two halves of a head rotate against each other
+    half = d_head // 2
+    inv_freq = rope_base ** (-np.arange(half, dtype=np.float64) * 2.0 / d_head)
+    angles = np.arange(seq, dtype=np.float64)[:, None] * inv_freq[None, :]
+    cos_t = const((1, seq, half), np.cos(angles)[None])
+    sin_t = const((1, seq, half), np.sin(angles)[None])
+
+    def rotary(t):  # [heads, seq, d_head]
+        a = g.slice(t, 2, 0, half)
+        b = g.slice(t, 2, half, d_head)
+        ra = g.sub(g.mul(a, cos_t), g.mul(b, sin_t))
+        rb = g.add(g.mul(b, cos_t), g.mul(a, sin_t))
+        return g.concat([ra, rb], 2)
+
+    def split_heads(t):  # [seq, d_model] -> [heads, seq, d_head]
+        return g.permute(g.view(t, [seq, heads, d_head]), [1, 0, 2])
+
+    mask = const((1, seq, seq), np.where(np.tril(np.ones((seq, seq), bool)), 0.0, -np.inf))
+    scale = g.scalar(1.0 / math.sqrt(d_head), dtype)
+
+    x_in = g.input([1, seq, d_model], dtype)
+    x = g.view(x_in, [seq, d_model])
+    for _ in range(layers):
+        h = rmsnorm(x)
+        q = rotary(split_heads(g.linear(h, weight(d_model, d_model))))
+        k = rotary(split_heads(g.linear(h, weight(d_model, d_model))))
+        v = split_heads(g.linear(h, weight(d_model, d_model)))
+        scores = g.batched_mat_mul(q, g.permute(k, [0, 2, 1]))
+        probs = g.softmax(g.add(g.mul(scores, scale), mask), 2)
+        ctx = g.permute(g.batched_mat_mul(probs, v), [1, 0, 2])
+        x = g.add(x, g.linear(g.view(ctx, [seq, d_model]), weight(d_model, d_model)))
+        h = rmsnorm(x)
+        gate = g.linear(h, weight(ffn, d_model))
+        up = g.linear(h, weight(ffn, d_model))
+        act = g.mul(g.mul(gate, g.sigmoid(gate)), up)
+        x = g.add(x, g.linear(act, weight(d_model, ffn)))
+    g.output(g.view(x, [1, seq, d_model]))
+
+    def inputs(rows=seq):
+        return [normal(seed, 399, (1, seq, d_model))[:, :rows].astype(np_dt)]
+
+    macs = layers * (4 * seq * d_model * d_model + 2 * heads * seq * seq * d_head + 3 * seq * d_model * ffn)
+    return g, inputs, 2 * macs
+
+
+# ---------------------------------------------------------------------------------------------- config 5
+
+def build_unet_block(seed=0, batch=2, channels=320, size=64, groups=32, heads=8, time_dim=1280, ctx_len=77,
+                     ctx_dim=768, ffn_mult=4):
+    """Stable-Diffusion style UNet block, f32: ResBlock (GroupNorm + SiLU + 3x3 conv, twice, with the projected
+    timestep embedding added in between and the residual at the end) followed by a spatial transformer over the
+    size * size tokens (layernorm + self-attention, layernorm + cross-attention to the context, layernorm + GEGLU
+    feed-forward; linear projections in and out, residual around the whole transformer).
+    GroupNorm is lowered as the reference's ONNX loader does it (kn-graph/src/onnx/load.rs:513-568): view as
+    [N, groups, rest], layernorm over the last axis, view back, then scale and shift per channel.
+    Inputs: latent [N, C, size, size], timestep embedding [N, time_dim], context [N, ctx_len, ctx_dim], all N(0, 1);
+    weights N(0, 0.02), norm scales 1 + N(0, 0.02). Returns (graph, make_inputs, flop per evaluation)."""
+    g = Graph()
+    stream = [500]
+    C, hw, d_head = channels, size * size, channels // heads
+    assert d_head * heads == C and C % groups == 0
+
+    def rnd(shape, std=0.02, mean=0.0):
+        stream[0] += 1
+        return g.constant(list(shape), normal(seed, stream[0], tuple(shape), mean=mean, std=std))
+
+    def linear(x, co, ci, bias=True):
+        y = g.linear(x, rnd((co, ci)))
+        return g.add(y, rnd((1, co))) if bias else y
+
+    def silu(x):
+        return g.mul(x, g.sigmoid(x))
+
+    def group_norm(x, eps):
+        y = g.layernorm(g.view(x, [batch, groups, (C // groups) * hw]), 2, eps)
+        y = g.view(y, [batch, C, size, size])
+        return g.add(g.mul(y, rnd((1, C, 1, 1), mean=1.0)), rnd((1, C, 1, 1)))
+
+    def layer_norm(x):  # [batch * hw, C]
+        return g.add(g.mul(g.layernorm(x, 1, 1e-5), rnd((1, C), mean=1.0)), rnd((1, C)))
+
+    def conv3(x):
+        return g.add(g.conv(x, rnd((C, C, 3, 3)), 1, 1, 1, 1), rnd((1, C, 1, 1)))
+
+    def attention(x, ctx, ctx_tokens, ctx_width):
+        # x [batch * hw, C]; ctx [batch * ctx_tokens, ctx_width]
+        def heads_of(t, tokens):  # [batch * tokens, C] -> [batch * heads, tokens, d_head]
+            t = g.permute(g.view(t, [batch, tokens, heads, d_head]), [0, 2, 1, 3])
+            return g.view(t, [batch * heads, tokens, d_head])
+
+        q = heads_of(linear(x, C, C, bias=False), hw)
+        k = heads_of(linear(ctx, C, ctx_width, bias=False), ctx_tokens)
+        v = heads_of(linear(ctx, C, ctx_width, bias=False), ctx_tokens)
+        scores = g.mul(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), g.scalar(1.0 / math.sqrt(d_head)))
+        out = g.batched_mat_mul(g.softmax(scores, 2), v)  # [batch * heads, hw, d_head]
+        out = g.permute(g.view(out, [batch, heads, hw, d_head]), [0, 2, 1, 3])
+        return linear(g.view(out, [batch * hw, C]), C, C)
+
+    latent = g.input([batch, C, size, size])
+    t_emb = g.input([batch, time_dim])
+    context = g.input([batch, ctx_len, ctx_dim])
+
+    # ---- ResBlock
+    h = conv3(silu(group_norm(latent, 1e-5)))
+    h = g.add(h, g.view(linear(silu(t_emb), C, time_dim), [batch, C, 1, 1]))
+    h = conv3(silu(group_norm(h, 1e-5)))
+    res = g.add(latent, h)
+
+    # ---- spatial transformer
+    t = group_norm(res, 1e-6)
+    t = g.view(g.permute(g.view(t, [batch, C, hw]), [0, 2, 1]), [batch * hw, C])  # tokens
+    t = linear(t, C, C)
+    n = layer_norm(t)
+    t = g.add(t, attention(n, n, hw, C))
+    ctx2 = g.view(context, [batch * ctx_len, ctx_dim])
+    t = g.add(t, attention(layer_norm(t), ctx2, ctx_len, ctx_dim))
+    inner = C * ffn_mult
+    n = layer_norm(t)
+    proj = linear(n, 2 * inner, C)
+    value, gate = g.slice(proj, 1, 0, inner), g.slice(proj, 1, inner, 2 * inner)
+    gelu = g.mul(g.mul(gate, g.scalar(0.5)),
+                 g.add(g.unary(UnaryOp.ERF, g.mul(gate, g.scalar(1.0 / math.sqrt(2.0)))), g.scalar(1.0)))
+    t = g.add(t, linear(g.mul(value, gelu), C, inner))
+    t = linear(t, C, C)
+    t = g.view(g.permute(g.view(t, [batch, hw, C]), [0, 2, 1]), [batch, C, size, size])
+    g.output(g.add(res, t))
+
+    def inputs():
+        return [normal(seed, 497, (batch, C, size, size)), normal(seed, 498, (batch, time_dim)),
+                normal(seed, 499, (batch, ctx_len, ctx_dim))]
+
+    tok = batch * hw
+    macs = (2 * tok * C * C * 9 + batch * time_dim * C + 2 * tok * C * C  # convs, time projection, proj in / out
+            + 4 * tok * C * C + 2 * batch * heads * hw * hw * d_head  # self-attention
+            + 2 * tok * C * C + 2 * batch * ctx_len * ctx_dim * C + 2 * batch * heads * hw * ctx_len * d_head  # cross
+            + tok * C * 2 * inner + tok * inner * C)  # GEGLU feed-forward
+    return g, inputs, 2 * macs

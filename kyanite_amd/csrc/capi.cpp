@@ -693,6 +693,16 @@ int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, s
     });
 }
 
+int knhip_executor_step_work(const knhip_executor *ex, size_t index, double *flops, double *bytes) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr && flops != nullptr && bytes != nullptr);
+        const kn::Step &step = ex->ex.plan().steps.at(index);
+        *flops = step.flops();
+        *bytes = step.bytes();
+        return KNHIP_OK;
+    });
+}
+
 int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed) {
     return guarded([&] {
         KN_REQUIRE(ex != nullptr);

@@ -24,6 +24,26 @@ std::string Step::str() const {
     return ss.str();
 }
 
+double Step::flops() const {
+    if (kind == StepKind::MatMul) return 2.0 * gemm.batch * gemm.m * gemm.n * gemm.k;
+    if (kind == StepKind::Conv)
+        return 2.0 * conv.batch * conv.out_c * conv.out_h * conv.out_w * conv.in_c * conv.kernel_h * conv.kernel_w;
+    return 0.0;
+}
+
+double Step::bytes() const {
+    double total = 0.0;
+    for (auto &op : operands) {
+        double elements = 1.0;
+        const auto &shape = op.tensor.shape.shape();
+        const auto &strides = op.tensor.shape.strides();
+        for (size_t a = 0; a < shape.size(); a++)
+            if (strides[a] != 0) elements *= (double) shape[a];
+        total += elements * (double) dtype_bytes(op.tensor.dtype);
+    }
+    return total;
+}
+
 size_t Plan::resolve(const PlanPtr &ptr) const {
     size_t base;
     switch (ptr.kind) {

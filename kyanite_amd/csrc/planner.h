@@ -40,6 +40,10 @@ struct Step {
     bool conv_has_bias = false, conv_has_res = false;
 
     std::string str() const;
+    // Algorithmic work of one launch: multiply-add flops of a MatMul / Conv step (0 otherwise) and the bytes of
+    // every distinct operand element (a broadcast axis counts once), which is what a perfect kernel would move.
+    double flops() const;
+    double bytes() const;
 };
 
 struct MemoryUsage {  // planner.rs:67-81

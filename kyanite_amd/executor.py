@@ -1,7 +1,7 @@
 """HipExecutor and the runtime device selector, mirroring kn-cuda-eval's CudaExecutor
 (executor.rs:60-266) and kn-runtime's Device / PreparedGraph (kn-runtime/src/lib.rs:68-126)."""
 import ctypes
-from ctypes import byref, c_float, c_int, c_size_t, c_void_p
+from ctypes import byref, c_double, c_float, c_int, c_size_t, c_void_p
 
 import numpy as np
 
@@ -180,6 +180,12 @@ class HipExecutor:
             check(lib.knhip_executor_step_kind(self._h, i, byref(k)))
             kinds.append(STEP_KINDS[k.value])
         return kinds
+
+    def step_work(self, i):
+        """(flops, bytes) of one launch of step `i`: multiply-add flops for conv / mat_mul, algorithmic bytes for all."""
+        flops, nbytes = c_double(), c_double()
+        check(lib.knhip_executor_step_work(self._h, i, byref(flops), byref(nbytes)))
+        return flops.value, nbytes.value
 
     def step_str(self, i):
         return get_string(lib.knhip_executor_step_str, self._h, i)

@@ -968,3 +968,28 @@ def f16_norms():
     rn = g.mul(g.binary(BinaryOp.DIV, x, rms), gamma)
     g.output_all([ln, rn, g.reduce(x, [2], ReduceOp.SUM), g.reduce(x, [1], ReduceOp.MAX), g.softmax(x, 1)])
     return g, 5, [_f16(rng, 5, 6, 256)], None
+
+
+# ---- miniature versions of the benchmark configurations (same builders, small sizes)
+
+@case
+def config_llama_small():
+    from kyanite_amd.configs import build_llama
+    g, make_inputs, _ = build_llama(seed=1, layers=2, seq=24, d_model=64, heads=4, ffn=176)
+    return g, 0, make_inputs(), None
+
+
+@case
+def config_llama_f32_small():
+    """the same decoder in f32: the tight f32 bar applies to every kernel of the graph"""
+    from kyanite_amd.configs import build_llama
+    g, make_inputs, _ = build_llama(seed=2, layers=1, seq=40, d_model=96, heads=3, ffn=200, dtype=DType.F32)
+    return g, 0, make_inputs(), None
+
+
+@case
+def config_unet_block_small():
+    from kyanite_amd.configs import build_unet_block
+    g, make_inputs, _ = build_unet_block(seed=2, batch=2, channels=32, size=8, groups=4, heads=2, time_dim=48, ctx_len=5,
+                                         ctx_dim=24)
+    return g, 0, make_inputs(), None

@@ -15,11 +15,15 @@ TOLERANCE_REL_DIFF = 0.001
 
 # The tighter bar this project states for its own GPU path against the oracle:
 #   max over elements of |actual - expected| / max(|expected|, FLOOR_FRACTION * rms(expected)) <= F32_MAX_REL.
-# The floor is needed because sums that cancel to (almost) zero carry the rounding of their large terms: an f32
-# contraction over K terms is only reproducible to about eps * sqrt(K) of the tensor's scale under reordering,
-# i.e. ~6e-6 * rms for K = 11008, so the floor sits at a tenth of the tensor's rms.
+# The floor is needed because sums that cancel to (almost) zero carry the rounding of their large terms. Two f32
+# evaluations of one K-term contraction that differ only in summation order differ by about
+# sqrt(2) * (eps / 2) * sqrt(K) * rms per element (one sigma), and the largest of millions of elements sits near
+# five sigma: 7e-6 * rms for K = 1152 and 1.1e-5 * rms for K = 2880 (both measured on the ResNet and UNet
+# configurations at full size, where they match this estimate), 2.2e-5 * rms for K = 11008. A floor of half the
+# tensor's rms keeps that noise a factor of two under the 1e-4 bar for the longest contraction of any configuration;
+# a real defect (wrong index, dropped term) shows up as an error of the order of the rms itself.
 F32_MAX_REL = 1e-4
-FLOOR_FRACTION = 0.1
+FLOOR_FRACTION = 0.5
 # f16 tensors (f16 storage, f32 arithmetic, one rounding per operation; not part of the reference IR): 2e-2
 F16_MAX_REL = 2e-2
 

@@ -209,3 +209,40 @@ def test_float_min_max_ignore_nan():
     g.output_all([g.binary(BinaryOp.MIN, a, b), g.binary(BinaryOp.MAX, a, b)])
     lo, hi = cpu_eval_graph(g, 0, [np.array([np.nan, 1.0, np.nan], np.float32), np.array([2.0, np.nan, np.nan], np.float32)])
     assert lo[0] == 2.0 and lo[1] == 1.0 and np.isnan(lo[2]) and hi[0] == 2.0 and hi[1] == 1.0 and np.isnan(hi[2])
+
+
+def test_f16_operations_round_once_from_f64_results():
+    """f16 (not in the reference IR): every operation is the f64 library result rounded to f16, up to the last
+    f16 bit (f32 arithmetic before the rounding can move a value that sits next to a rounding boundary)."""
+    rng = np.random.default_rng(40)
+
+    def ulps(a, b):
+        a, b = np.asarray(a, np.float16), np.asarray(b, np.float16)
+        assert a.shape == b.shape and a.dtype == np.float16
+        ia, ib = a.view(np.int16).astype(np.int32), b.view(np.int16).astype(np.int32)
+        ia, ib = np.where(ia < 0, -(ia & 0x7FFF), ia), np.where(ib < 0, -(ib & 0x7FFF), ib)
+        return int(np.max(np.abs(ia - ib)))
+
+    x = rng.standard_normal((6, 40)).astype(np.float16)
+    w = (rng.standard_normal((40, 9)) * 0.3).astype(np.float16)
+    x64, w64 = x.astype(np.float64), w.astype(np.float64)
+    g = Graph()
+    xi = g.input([6, 40], DType.F16)
+    mm = g.mat_mul(xi, g.constant([40, 9], w))
+    g.output_all([mm, g.softmax(xi, 1), g.layernorm(xi, 1, 1e-3), g.reduce(xi, [1], ReduceOp.SUM),
+                  g.reduce(xi, [0], ReduceOp.MEAN), g.mul(xi, xi), g.unary(UnaryOp.EXP, xi)])
+    got = cpu_eval_graph(g, 0, [x])
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    mean = x64.mean(axis=1, keepdims=True)
+    var = ((x64 - mean) ** 2).mean(axis=1, keepdims=True)
+    want = [x64 @ w64, e / e.sum(axis=1, keepdims=True), (x64 - mean) / np.sqrt(var + 1e-3), x64.sum(axis=1),
+            x64.mean(axis=0), x64 * x64, np.exp(x64)]
+    for y, t in zip(got, want):
+        assert y.dtype == np.float16
+        assert ulps(y, t.astype(np.float16)) <= 1
+    # a long sum accumulates in f32, not f16: an f16 accumulator would get stuck at 2048 (2048 + 1 rounds to 2048)
+    long = np.concatenate([np.ones(4096), np.full(4096, 2.0 ** -10)]).astype(np.float16)
+    g = Graph()
+    g.output(g.reduce(g.input([8192], DType.F16), [0], ReduceOp.SUM))
+    (s,) = cpu_eval_graph(g, 0, [long])
+    assert s.dtype == np.float16 and float(s) == 4100.0
