@@ -149,6 +149,10 @@ int knhip_graph_value_axes(const knhip_graph *g, knhip_value value, size_t *buf,
 int knhip_graph_value_constant(const knhip_graph *g, knhip_value value, const void **data, size_t *bytes);
 /* graph.rs:490-527: 1 in *is_single and the element in `element` (8 bytes of room) when every element is equal */
 int knhip_graph_as_single_const(const knhip_graph *g, knhip_value value, int *is_single, void *element);
+/* Graph::as_const (graph.rs:435-474): the value computed on the host when it only depends on constants through
+ * layout operations, unary / binary operations, reduce, gather and concat. *needed = byte size of the dense
+ * row-major result (its shape and dtype are those of the value); the bytes are copied when cap >= *needed. */
+int knhip_graph_as_const(const knhip_graph *g, knhip_value value, int *is_const, void *data, size_t cap, size_t *needed);
 
 /* kn-graph/src/shape.rs:353-365. `actual` holds the concatenated dims of all inputs. *status: 0 ok, 1 different
  * length, 2 constant mismatch, 3 batch conflict, 4 impossible batch value; *has_batch 0 when any batch size fits */

@@ -102,6 +102,7 @@ SIGNATURES = {
     "knhip_graph_value_axes": [G, V, PZ, c_size_t],
     "knhip_graph_value_constant": [G, V, POINTER(c_void_p), PZ],
     "knhip_graph_as_single_const": [G, V, POINTER(c_int), c_void_p],
+    "knhip_graph_as_const": [G, V, POINTER(c_int), c_void_p, c_size_t, PZ],
     "knhip_graph_infer_batch_size": [G, PZ, PZ, c_size_t, POINTER(c_int), POINTER(c_int), POINTER(c_uint64)],
     "knhip_optimizer_settings_default": [POINTER(OptimizerSettingsT)],
     "knhip_graph_optimize": [G, POINTER(OptimizerSettingsT), POINTER(G)],

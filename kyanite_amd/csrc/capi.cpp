@@ -442,6 +442,17 @@ int knhip_graph_as_single_const(const knhip_graph *g, knhip_value value, int *is
     });
 }
 
+int knhip_graph_as_const(const knhip_graph *g, knhip_value value, int *is_const, void *data, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(g != nullptr && is_const != nullptr && needed != nullptr);
+        auto c = g->graph.as_const(value);
+        *is_const = c.has_value() ? 1 : 0;
+        *needed = c ? c->nbytes() : 0;
+        if (c && data != nullptr && cap >= c->nbytes() && c->nbytes() > 0) std::memcpy(data, c->bytes(), c->nbytes());
+        return KNHIP_OK;
+    });
+}
+
 int knhip_graph_infer_batch_size(const knhip_graph *g, const size_t *actual, const size_t *ranks, size_t input_count,
                                  int *status, int *has_batch, uint64_t *batch) {
     return guarded([&] {

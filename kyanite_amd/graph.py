@@ -309,6 +309,18 @@ class Graph:
         dt = self[value].dtype.numpy
         return np.frombuffer(bytes(buf)[: dt.itemsize], dtype=dt)[0]
 
+    def as_const(self, value):
+        """Graph::as_const (graph.rs:435-474): the value as a numpy array when it is computable from constants alone."""
+        info = self[value]
+        flag, needed = c_int(), c_size_t()
+        check(lib.knhip_graph_as_const(self._h, value, byref(flag), None, 0, byref(needed)))
+        if not flag.value:
+            return None
+        dims = [d.fixed_factor for d in info.shape]
+        buf = (c_uint8 * max(needed.value, 1))()
+        check(lib.knhip_graph_as_const(self._h, value, byref(flag), buf, needed.value, byref(needed)))
+        return np.frombuffer(bytes(buf)[: needed.value], dtype=info.dtype.numpy).reshape(dims).copy()
+
     def infer_batch_size(self, actual_shapes):
         """Returns (status, batch) with status 0 on success; batch is None when any batch size fits."""
         flat = [d for s in actual_shapes for d in s]
