@@ -194,6 +194,10 @@ int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const
                             void *const *outputs, const size_t *output_bytes, size_t output_count);
 /* run_async (executor.rs:199-258): launch all steps on the executor's stream, no synchronisation */
 int knhip_executor_run_async(knhip_executor *ex);
+/* No counterpart in the reference (its executor launches step by step, executor.rs:199-206): when enabled, run_async
+ * and evaluate replay the launch list as one HIP graph, captured on the first run. For graphs of many small kernels,
+ * where the launches dominate (tiny MLP at batch 8). Profiled runs still launch step by step. */
+int knhip_executor_set_graph_mode(knhip_executor *ex, int enabled);
 int knhip_executor_synchronize(knhip_executor *ex);
 /* The timing loop of the reference's profile_net (kn-cuda-eval/src/bin/profile_net.rs:146-180, `--skip-io`):
  * `iterations` back-to-back run_async calls bracketed by two HIP events recorded on the executor's stream;

@@ -704,6 +704,14 @@ int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, s
     });
 }
 
+int knhip_executor_set_graph_mode(knhip_executor *ex, int enabled) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        ex->ex.set_graph_mode(enabled != 0);
+        return KNHIP_OK;
+    });
+}
+
 int knhip_executor_step_work(const knhip_executor *ex, size_t index, double *flops, double *bytes) {
     return guarded([&] {
         KN_REQUIRE(ex != nullptr && flops != nullptr && bytes != nullptr);

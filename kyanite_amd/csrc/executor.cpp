@@ -116,6 +116,7 @@ HipExecutor::~HipExecutor() {
     // failures while tearing down are ignored on purpose (the reference does the same in its drop handlers)
     (void) hipSetDevice(device_);
     if (stream_) (void) hipStreamSynchronize(stream_);
+    if (graph_exec_) (void) hipGraphExecDestroy(graph_exec_);
     for (void *p : pinned_inputs_) (void) hipHostFree(p);
     for (void *p : pinned_outputs_) (void) hipHostFree(p);
     for (hipModule_t m : modules_) (void) hipModuleUnload(m);
@@ -194,8 +195,28 @@ void HipExecutor::run_async() {
     if (current != device_) hip_check(hipSetDevice(device_), "hipSetDevice");
 
     if (!profile_) {
-        for (size_t si = 0; si < plan_.steps.size(); si++) launch_step(si);
         last_profile_ = std::nullopt;
+        if (graph_mode_ && !plan_.steps.empty()) {
+            if (!graph_exec_) {
+                // the launch list is fixed for the lifetime of the executor (same kernels, same arena addresses)
+                hipGraph_t graph = nullptr;
+                hip_check(hipStreamBeginCapture(stream_, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+                try {
+                    for (size_t si = 0; si < plan_.steps.size(); si++) launch_step(si);
+                } catch (...) {
+                    (void) hipStreamEndCapture(stream_, &graph);
+                    if (graph) (void) hipGraphDestroy(graph);
+                    throw;
+                }
+                hip_check(hipStreamEndCapture(stream_, &graph), "hipStreamEndCapture");
+                hipError_t e = hipGraphInstantiate(&graph_exec_, graph, nullptr, nullptr, 0);
+                (void) hipGraphDestroy(graph);
+                hip_check(e, "hipGraphInstantiate");
+            }
+            hip_check(hipGraphLaunch(graph_exec_, stream_), "hipGraphLaunch");
+            return;
+        }
+        for (size_t si = 0; si < plan_.steps.size(); si++) launch_step(si);
         return;
     }
 

@@ -42,6 +42,12 @@ public:
     // `iterations` back-to-back runs timed with events on the executor's stream; elapsed milliseconds in total
     float time_runs(size_t iterations);
 
+    // Replay the launch list as one HIP graph (captured from the executor's stream on the first run after switching
+    // it on) instead of launching every step: one submission per evaluation, for graphs of small kernels where the
+    // launches dominate. Profiled runs always launch step by step.
+    void set_graph_mode(bool on) { graph_mode_ = on; }
+    bool graph_mode() const { return graph_mode_; }
+
     void set_profile(bool on) { profile_ = on; }
     const std::optional<Profile> &last_profile() const { return last_profile_; }
 
@@ -73,6 +79,8 @@ private:
     std::vector<HostTensor> tensor_outputs_;
     bool profile_ = false;
     std::optional<Profile> last_profile_;
+    bool graph_mode_ = false;
+    hipGraphExec_t graph_exec_ = nullptr;
 };
 
 void hip_check(hipError_t e, const char *what);

@@ -149,6 +149,10 @@ class HipExecutor:
         check(lib.knhip_executor_stream(self._h, byref(p)))
         return p.value or 0
 
+    def set_graph_mode(self, enabled):
+        """Replay the launch list as one HIP graph (captured on the first run) instead of launching every step."""
+        check(lib.knhip_executor_set_graph_mode(self._h, int(enabled)))
+
     def set_profile(self, enabled):
         check(lib.knhip_executor_set_profile(self._h, int(enabled)))
 
