@@ -809,19 +809,55 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     emit_fn("kn_pre", desc.pre, in_pre, false, row_dtype);
     emit_fn("kn_post", desc.post, in_post, true, ops[0].dtype);
 
+    // Epilogue operands (gamma, beta, ...) are requested together with the row itself when they fit in registers,
+    // so that their latency overlaps with the reductions instead of following them.
+    size_t n_post = 0;
+    bool post_row_invariant = true;  // the epilogue operands only vary along the normalised axis
+    for (size_t k = 1; k < ops.size(); k++) {
+        if (!in_post[k]) continue;
+        n_post++;
+        for (size_t a = 0; a < sc.rank(); a++) post_row_invariant &= sc.strides[k][a] == 0;
+    }
+    bool prefetch_post = cached && n_post > 0 && n_post * items * vec <= 64;
+    // When they are the same for every row, a group of lanes walks over `seq` rows one after another and loads
+    // them once, as long as enough workgroups remain to fill the chip.
+    size_t seq = 1;
+    if (prefetch_post && post_row_invariant) {
+        // measured on [8192, 4096] with gamma / beta: 2 or 4 rows per group are no faster than 1 (49.5 us against
+        // 54.6 / 55.9 us), so this stays off unless asked for
+        static const size_t max_seq = getenv("KNHIP_ROW_SEQ") ? (size_t) atoi(getenv("KNHIP_ROW_SEQ")) : 1;
+        for (size_t c = max_seq; c > 1; c /= 2)
+            if (static_size / (rows_per_block * c) >= 2048) {
+                seq = c;
+                break;
+            }
+    }
+    // Rows and vector positions past the end are clamped for addressing and masked afterwards, so that the loads of
+    // a row are straight-line code that the compiler can issue back to back (a branch per load would make every
+    // load wait for the one before it).
+    const bool check_row = static_size % (rows_per_block * seq) != 0;
+    const bool check_i = cached && items * G != nv;
+
     ss << "#define VEC " << vec << "\n#define ITEMS " << items << "\n#define G " << G << "\n";
     ss << "KN_DEV float kn_max(float a, float b) { return fmaxf(a, b); }\nKN_DEV float kn_add(float a, float b) { return a + b; }\n";
-    ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
+    // Holding the epilogue operands across rows costs a few registers more than the 64 per lane that full
+    // occupancy allows; the compiler is told to stay within them (it has the slack: at most one spill was seen).
+    ss << "extern \"C\" __global__ " << (seq > 1 ? "__attribute__((amdgpu_waves_per_eu(8, 8))) " : "") << "__launch_bounds__("
+       << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
     for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
     if (nw > 1) ss << "    __shared__ float lds_m[" << nw << "], lds_s[" << nw << "];\n";
-    ss << "    const idx_t row = (idx_t) blockIdx.x * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / G);\n";
     ss << "    const idx_t lane = (idx_t) (threadIdx.x % G);\n";
-    if (nw <= 1) ss << "    if (row >= (idx_t) " << static_size << ") return;\n";
     ss << "    idx_t base[" << ops.size() << "];\n    for (int k = 0; k < " << ops.size() << "; k++) base[k] = 0;\n";
-    {
+    const std::string row0 = "((idx_t) blockIdx.x * (idx_t) " + std::to_string(rows_per_block) + " + (idx_t) (threadIdx.x / G))";
+    auto emit_row_setup = [&]() {
         std::vector<std::string> offs;
         for (size_t k = 0; k < ops.size(); k++) offs.push_back("base[" + std::to_string(k) + "]");
-        emit_decompose(ss, "    ", "row", sc.shape, sc.strides, offs);
+        if (check_row) ss << "    const idx_t rowc = row < (idx_t) " << static_size << " ? row : (idx_t) " << (static_size - 1) << ";\n";
+        emit_decompose(ss, "    ", check_row ? "rowc" : "row", sc.shape, sc.strides, offs);
+    };
+    if (seq == 1) {
+        ss << "    const idx_t row = " << row0 << ";\n";
+        emit_row_setup();
     }
     // the reduction helper: over G lanes of a wave, or over the waves of the workgroup
     auto reduce = [&](const std::string &var, const char *f) {
@@ -829,25 +865,36 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         if (nw > 1) ss << "    " << var << " = kn_block_reduce<" << nw << ">(" << var << ", " << f << ", lds_" << var << ");\n";
         else ss << "    " << var << " = kn_group_reduce<G>(" << var << ", " << f << ");\n";
     };
-    // load one vector position `i` (in vector units along the axis) and run the prologue on it
-    auto emit_load_pre = [&](const std::string &indent, const std::string &i, const std::string &dst) {
+    // the prologue operands of vector position `i` (in vector units along the axis): loaded into `a<k>`, either
+    // declared on the spot or assigned to an element of a register array that was declared earlier (`slot`)
+    auto emit_pre_loads = [&](const std::string &indent, const std::string &i, const std::string &slot) {
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_pre[k]) continue;
             std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
-            if (vec > 1 && axis_strides[k] == 1)
-                ss << indent << "const V" << k << " a" << k << " = "
-                   << load_expr("V" + std::to_string(k), "p" + std::to_string(k) + " + " + o, cached && is_streaming(ops[k])) << ";\n";
-            else ss << indent << "const S" << k << " a" << k << " = p" << k << "[" << o << "];\n";
+            bool v = vec > 1 && axis_strides[k] == 1;
+            std::string lhs = slot.empty() ? std::string("const ") + (v ? "V" : "S") + std::to_string(k) + " a" + std::to_string(k)
+                                           : "a" + std::to_string(k) + "[" + slot + "]";
+            if (v) ss << indent << lhs << " = "
+                      << load_expr("V" + std::to_string(k), "p" + std::to_string(k) + " + " + o, cached && is_streaming(ops[k])) << ";\n";
+            else ss << indent << lhs << " = p" << k << "[" << o << "];\n";
         }
+    };
+    // run the prologue on the loaded operands
+    auto emit_pre_apply = [&](const std::string &indent, const std::string &dst, const std::string &slot) {
+        const std::string pick = slot.empty() ? std::string() : "[" + slot + "]";
         ss << indent << "for (int j = 0; j < VEC; j++) " << dst << "[j] = kn_pre(";
         bool first = true;
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_pre[k]) continue;
-            std::string e = (vec > 1 && axis_strides[k] == 1) ? "a" + std::to_string(k) + "[j]" : "a" + std::to_string(k);
+            std::string e = "a" + std::to_string(k) + pick + ((vec > 1 && axis_strides[k] == 1) ? "[j]" : "");
             ss << (first ? "" : ", ") << from_storage(ops[k].dtype, e);
             first = false;
         }
         ss << ");\n";
+    };
+    auto emit_load_pre = [&](const std::string &indent, const std::string &i, const std::string &dst) {
+        emit_pre_loads(indent, i, "");
+        emit_pre_apply(indent, dst, "");
     };
     // run the epilogue on normalised values `src[j]` of vector position `i` and store
     // the epilogue operands of vector position `i`: loaded into `prefix<k>`, either declared on the spot or
@@ -884,25 +931,40 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         }
     };
 
-    const std::string valid = nw > 1 ? std::string("(row < (idx_t) ") + std::to_string(static_size) + ")" : std::string("true");
-    // Epilogue operands (gamma, beta, ...) are requested together with the row itself when they fit in registers,
-    // so that their latency overlaps with the reductions instead of following them.
-    size_t n_post = 0;
-    for (size_t k = 1; k < ops.size(); k++) n_post += in_post[k] ? 1 : 0;
-    bool prefetch_post = cached && n_post > 0 && n_post * items * vec <= 64;
+    const std::string valid = check_row ? std::string("(row < (idx_t) ") + std::to_string(static_size) + ")" : std::string("true");
     if (cached) {
-        if (prefetch_post)
-            for (size_t k = 1; k < ops.size(); k++)
-                if (in_post[k]) ss << "    " << ((vec > 1 && axis_strides[k] == 1) ? "V" : "S") << k << " b" << k << "[ITEMS];\n";
+        const std::string item_index = std::string("        const idx_t i = lane + (idx_t) it * (idx_t) G;\n") +
+            (check_i ? "        const idx_t ic = i < (idx_t) " + std::to_string(nv) + " ? i : (idx_t) " + std::to_string(nv - 1) + ";\n"
+                     : std::string("        const idx_t ic = i;\n"));
+        for (size_t k = 1; k < ops.size(); k++) {
+            const char *t = (vec > 1 && axis_strides[k] == 1) ? "V" : "S";
+            if (in_pre[k]) ss << "    " << t << k << " a" << k << "[ITEMS];\n";
+            if (in_post[k] && prefetch_post) ss << "    " << t << k << " b" << k << "[ITEMS];\n";
+        }
+        if (seq > 1) {
+            // the epilogue operands once, then the rows of this group one after another
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n" << item_index;
+            emit_post_loads("        ", "ic", "it");
+            ss << "    }\n";
+            ss << "    for (int rs = 0; rs < " << seq << "; rs++) {\n";
+            ss << "    const idx_t row = " << row0 << " * (idx_t) " << seq << " + (idx_t) rs;\n";
+            ss << "    for (int k = 0; k < " << ops.size() << "; k++) base[k] = 0;\n";
+            emit_row_setup();
+        }
+        // every load of the row first, then the arithmetic
+        ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n" << item_index;
+        emit_pre_loads("        ", "ic", "it");
+        if (prefetch_post && seq == 1) emit_post_loads("        ", "ic", "it");
+        ss << "    }\n";
         ss << "    float x[ITEMS][VEC];\n";
         ss << "    float m = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
         ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
-        ss << "        if (i < (idx_t) " << nv << " && " << valid << ") {\n";
-        emit_load_pre("            ", "i", "x[it]");
-        if (prefetch_post) emit_post_loads("            ", "i", "it");
-        if (softmax) ss << "            for (int j = 0; j < VEC; j++) m = fmaxf(m, x[it][j]);\n";
-        else ss << "            for (int j = 0; j < VEC; j++) m += x[it][j];\n";
-        ss << "        } else {\n            for (int j = 0; j < VEC; j++) x[it][j] = " << (softmax ? "-KN_INF" : "0.0f") << ";\n        }\n    }\n";
+        emit_pre_apply("        ", "x[it]", "it");
+        if (check_i)
+            ss << "        if (!(i < (idx_t) " << nv << ")) for (int j = 0; j < VEC; j++) x[it][j] = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
+        if (softmax) ss << "        for (int j = 0; j < VEC; j++) m = fmaxf(m, x[it][j]);\n";
+        else ss << "        for (int j = 0; j < VEC; j++) m += x[it][j];\n";
+        ss << "    }\n";
         reduce("m", softmax ? "kn_max" : "kn_add");
         ss << "    float s = 0.0f;\n";
         if (softmax) {
@@ -922,9 +984,12 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             else ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / denom;\n    }\n";
         }
         ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
-        ss << "        if (i < (idx_t) " << nv << " && " << valid << ") {\n";
+        std::string guard;
+        if (check_i) guard = "i < (idx_t) " + std::to_string(nv);
+        if (check_row) guard += (guard.empty() ? "" : " && ") + valid;
+        ss << "        " << (guard.empty() ? std::string() : "if (" + guard + ") ") << "{\n";
         emit_post_store("            ", "i", "x[it]", prefetch_post ? "it" : "");
-        ss << "        }\n    }\n}\n";
+        ss << "        }\n    }\n" << (seq > 1 ? "    }\n" : "") << "}\n";
     } else {
         // rows too long for registers: stream the row three times (the re-reads come from cache)
         ss << "    float t[VEC];\n";
@@ -954,9 +1019,10 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
 
     spec.source = ss.str();
     spec.block = (uint32_t) block;
-    spec.grid = ceil_div_u32(static_size, rows_per_block);
+    spec.grid = ceil_div_u32(static_size, rows_per_block * seq);
     std::ostringstream note;
     note << (softmax ? "softmax" : "layernorm") << " G=" << G << " vec=" << vec << " items=" << items << (cached ? " cached" : " streamed");
+    if (seq > 1) note << " rows=" << seq;
     spec.strategy = note.str();
     return spec;
 }

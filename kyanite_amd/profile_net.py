@@ -76,8 +76,8 @@ def profile_sweep(device, graph):
 
 
 def profile_cpu(graph, batch, n):
-    raise SystemExit("--cpu: the CPU evaluator of this repository is test infrastructure (oracle/) and is not shipped "
-                     "with the executor; `python bench.py` times it on the benchmark graphs and reports it as cpu_baseline")
+    raise SystemExit("--cpu: this package ships no CPU evaluator (the one in this repository is test infrastructure); "
+                     "`python bench.py` times it on the benchmark graphs and reports it as cpu_baseline")
 
 
 def main(argv=None):

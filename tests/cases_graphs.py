@@ -993,3 +993,16 @@ def config_unet_block_small():
     g, make_inputs, _ = build_unet_block(seed=2, batch=2, channels=32, size=8, groups=4, heads=2, time_dim=48, ctx_len=5,
                                          ctx_dim=24)
     return g, 0, make_inputs(), None
+
+
+@case
+def layernorm_affine_many_rows():
+    """enough rows that a workgroup walks over several of them with gamma / beta held in registers; the last
+    workgroup runs out of rows part way"""
+    g = Graph()
+    rng = np.random.default_rng(50)
+    x = g.input([4099, 2048])
+    gamma = g.constant([1, 2048], (1.0 + 0.1 * rng.standard_normal((1, 2048))).astype(np.float32))
+    beta = g.constant([1, 2048], (0.1 * rng.standard_normal((1, 2048))).astype(np.float32))
+    g.output(g.add(g.mul(g.layernorm(x, 1, 1e-5), gamma), beta))
+    return g, 0, [rng.standard_normal((4099, 2048)).astype(np.float32) * 3.0 + 0.5], None
