@@ -26,7 +26,7 @@ namespace {
 // BM x BN is the tile of the plane convolution kernel; the generic kernels take their tile (64 or 128 wide per
 // axis) from the loaders. LDS rows are padded by 4 floats: rows stay 16 byte aligned and successive k rows shift
 // by 4 banks.
-constexpr int BM = 128, BN = 128, BK = 16, THREADS = 256;
+constexpr int BM = 128, BN = 128, THREADS = 256;
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -41,11 +41,17 @@ struct StridedOperand {
 };
 
 // Fetches one BK x WIDTH slice (WIDTH = 64 or 128) of a strided operand into registers and writes it to LDS as
-// [k][outer].
-template <int MODE, int WIDTH>
+// [k][outer]. BK is 16, or 64 for the 64 wide tiles of problems with a long K axis: those are chosen when there is
+// little work per compute unit, and deeper slices keep more bytes in flight per round trip to memory (measured:
+// 8 x 4096 x 4096 171 -> 148 us, 512 x 4096 x 4096 224 -> 212 us; with K of a few hundred the shallow slices win).
+template <int MODE, int WIDTH, int BK_>
 struct StridedLoader {
+    static constexpr int BK = BK_;
     static constexpr int EPT = BK * WIDTH / THREADS;  // elements per thread
-    static constexpr int LDS_STRIDE = WIDTH + 4;
+    // Rows padded by 4 keep the 128 bit stores of the VecOuter mode aligned. The transposing stores of the VecK mode
+    // write 4 * (BK / 4) different k rows per wave: with 64 deep slices an odd stride spreads them over all banks
+    // (two lanes per bank, the minimum), a multiple of 4 would pile them onto two groups of four banks.
+    static constexpr int LDS_STRIDE = (MODE == VecK && BK > 16) ? WIDTH + 1 : WIDTH + 4;
     StridedOperand op;
     int o0;        // first outer index of this workgroup's tile
     bool interior; // the tile lies completely inside the matrix along the outer axis
@@ -69,7 +75,7 @@ struct StridedLoader {
             // thread -> (outer = t / 4 (+64), k = 4 * (t % 4) ..)
 #pragma unroll
             for (int h = 0; h < EPT / 4; h++) {
-                const int o = (t >> 2) + 64 * h, k = (t & 3) * 4;
+                const int o = t / (BK / 4) + (THREADS * 4 / BK) * h, k = (t % (BK / 4)) * 4;
                 const floatx4 v = *(const floatx4 *) (op.p + (long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk);
 #pragma unroll
                 for (int j = 0; j < 4; j++) r[4 * h + j] = v[j];
@@ -80,8 +86,8 @@ struct StridedLoader {
 #pragma unroll
             for (int i = 0; i < EPT; i++) {
                 const int e = t + THREADS * i;
-                const int o = along_k ? (e >> 4) : (e % WIDTH);
-                const int k = along_k ? (e & 15) : (e / WIDTH);
+                const int o = along_k ? (e / BK) : (e % WIDTH);
+                const int k = along_k ? (e % BK) : (e / WIDTH);
                 const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
                 r[i] = ok ? op.p[(long long) (o0 + o) * op.so + (long long) (k0 + k) * op.sk] : 0.0f;
             }
@@ -103,7 +109,7 @@ struct StridedLoader {
         } else if (MODE == VecK && interior && k0 + BK <= op.K) {
 #pragma unroll
             for (int h = 0; h < EPT / 4; h++) {
-                const int o = (t >> 2) + 64 * h, k = (t & 3) * 4;
+                const int o = t / (BK / 4) + (THREADS * 4 / BK) * h, k = (t % (BK / 4)) * 4;
 #pragma unroll
                 for (int j = 0; j < 4; j++) lds[k + j][o] = r[4 * h + j];
             }
@@ -112,8 +118,8 @@ struct StridedLoader {
 #pragma unroll
             for (int i = 0; i < EPT; i++) {
                 const int e = t + THREADS * i;
-                const int o = along_k ? (e >> 4) : (e % WIDTH);
-                const int k = along_k ? (e & 15) : (e / WIDTH);
+                const int o = along_k ? (e / BK) : (e % WIDTH);
+                const int k = along_k ? (e % BK) : (e / WIDTH);
                 lds[k][o] = r[i];
             }
         }
@@ -123,8 +129,9 @@ struct StridedLoader {
 // Input patches of a convolution as the B operand: k = (c, fy, fx), n = (image, oy, ox). Every thread keeps one
 // fixed n for the whole K loop, so the position is decomposed once; KH / KW are compile-time constants (0 = read
 // them from the parameters) so that splitting k costs multiplications instead of divisions.
-template <int KH, int KW, int WIDTH>
+template <int KH, int KW, int WIDTH, int BK_>
 struct PatchLoader {
+    static constexpr int BK = BK_;
     static constexpr int EPT = BK * WIDTH / THREADS;
     static constexpr int LDS_STRIDE = WIDTH + 4;
     const float *base;  // input of this thread's image, or null when n is out of range
@@ -218,6 +225,8 @@ struct ConvStore {
 // MI x NI: MFMA tiles per wave; the workgroup tile is (64 * MI) x (64 * NI) with the 4 waves arranged 2 x 2.
 template <int MI, int NI, typename LA, typename LB, typename S>
 __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int K, int m0, int n0) {
+    constexpr int BK = LA::BK;
+    static_assert(LA::BK == LB::BK, "both operands advance by the same slice");
     __shared__ __attribute__((aligned(16))) float As[BK][LA::LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) float Bs[BK][LB::LDS_STRIDE];
 
@@ -285,8 +294,8 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
     *tn = in_g / rows_here;
 }
 
-// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64)
-template <int A_MODE, int B_MODE, int TI>
+// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64); BK: depth of a K slice
+template <int A_MODE, int B_MODE, int TI, int BK>
 __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
     constexpr int T = 64 * TI;
     const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
@@ -294,15 +303,15 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
     const int m0 = tm * T, n0 = tn * T;
-    StridedLoader<A_MODE, T> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
-    StridedLoader<B_MODE, T> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+    StridedLoader<A_MODE, T, BK> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
+    StridedLoader<B_MODE, T, BK> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
     GemmStore s{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
     mfma_tile_loop<TI, TI>(la, lb, s, p.k, m0, n0);
 }
 
 template <int A_MODE, int KH, int KW, int TI>
 __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
-    constexpr int T = 64 * TI;
+    constexpr int T = 64 * TI, BK = 16;
     const int kh = KH ? KH : p.kernel_h, kw = KW ? KW : p.kernel_w;
     const int K = p.in_c * kh * kw, ohw = p.out_h * p.out_w;
     const long long N = (long long) p.batch * ohw;
@@ -310,8 +319,8 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * T, n0 = tn * T;
-    StridedLoader<A_MODE, T> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
-    PatchLoader<KH, KW, T> lb(p, n0);
+    StridedLoader<A_MODE, T, BK> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
+    PatchLoader<KH, KW, T, BK> lb(p, n0);
     ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
     mfma_tile_loop<TI, TI>(la, lb, s, K, m0, n0);
 }
@@ -518,21 +527,21 @@ int pick_mode(const void *ptr, long long so, long long sk, long long batch_strid
     return Scalar;
 }
 
-template <int A_MODE, int TI>
+template <int A_MODE, int TI, int BK>
 void launch_gemm_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter, TI>), grid, dim3(THREADS), 0, stream, p); break;
-        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK, TI>), grid, dim3(THREADS), 0, stream, p); break;
-        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar, TI>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter, TI, BK>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK, TI, BK>), grid, dim3(THREADS), 0, stream, p); break;
+        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar, TI, BK>), grid, dim3(THREADS), 0, stream, p); break;
     }
 }
 
-template <int TI>
+template <int TI, int BK>
 void launch_gemm_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
     switch (a_mode) {
-        case VecOuter: launch_gemm_b<VecOuter, TI>(b_mode, grid, stream, p); break;
-        case VecK: launch_gemm_b<VecK, TI>(b_mode, grid, stream, p); break;
-        default: launch_gemm_b<Scalar, TI>(b_mode, grid, stream, p); break;
+        case VecOuter: launch_gemm_b<VecOuter, TI, BK>(b_mode, grid, stream, p); break;
+        case VecK: launch_gemm_b<VecK, TI, BK>(b_mode, grid, stream, p); break;
+        default: launch_gemm_b<Scalar, TI, BK>(b_mode, grid, stream, p); break;
     }
 }
 
@@ -581,8 +590,9 @@ int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
     dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.a_sb, p.batch);
     const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.b_sb, p.batch);
-    if (small) launch_gemm_a<1>(a_mode, b_mode, grid, stream, p);
-    else launch_gemm_a<2>(a_mode, b_mode, grid, stream, p);
+    if (small && p.k >= 2048) launch_gemm_a<1, 64>(a_mode, b_mode, grid, stream, p);
+    else if (small) launch_gemm_a<1, 16>(a_mode, b_mode, grid, stream, p);
+    else launch_gemm_a<2, 16>(a_mode, b_mode, grid, stream, p);
     return (int) hipGetLastError();
 }
 
