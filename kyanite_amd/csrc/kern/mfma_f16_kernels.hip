@@ -1,11 +1,12 @@
 // f16 matrix multiply with f32 accumulation on the CDNA4 matrix cores (v_mfma_f32_32x32x16_f16).
 //
 // Same decomposition as the f32 kernel: a workgroup of 4 waves (2 x 2) owns a T x T tile of D = A * B (T = 128 or
-// 64), every wave (T / 2) x (T / 2) of it as 32 x 32 MFMA tiles. K is walked in slices of 64 that sit in LDS as
+// 64), every wave (T / 2) x (T / 2) of it as 32 x 32 MFMA tiles. K is walked in slices of BK that sit in LDS as
 // As[m][k] and Bs[n][k], K contiguous with rows padded by 8 halves: a lane's MFMA operand (8 consecutive k of one
 // row) is one 128 bit LDS read, and operands whose K axis is contiguous in memory (activations, `linear` weights,
-// K^T of attention) move global -> register -> LDS as 128 bit vectors without being transposed. The next slice is
-// fetched into registers while the current one is multiplied; the result is rounded to f16 once, at the store.
+// K^T of attention) move global -> register -> LDS as 128 bit vectors without being transposed.
+// The slices are double buffered in LDS: while slice s is multiplied, slice s + 1 waits in registers and slice
+// s + 2 is in flight from memory; one barrier per slice. The result is rounded to f16 once, at the store.
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
@@ -20,7 +21,7 @@ typedef _Float16 half_t;
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BK = 64, THREADS = 256, LDS_K = BK + 8;
+constexpr int THREADS = 256;
 
 enum LoadMode { Scalar = 0, VecOuter = 1, VecK = 2 };
 
@@ -32,9 +33,11 @@ struct Operand {
 
 // Fetches a T x BK slice into registers and writes it to LDS as [outer][k]. Vector modes need every vector to lie
 // completely inside or outside the matrix, which the host guarantees (sizes divisible by 8 along the vector axis).
-template <int MODE, int T>
+template <int MODE, int T, int BK>
 struct Loader {
     static constexpr int NVEC = T * BK / 8 / THREADS;  // 128 bit vectors per thread and slice
+    static constexpr int LDS_K = BK + 8;
+    static_assert(NVEC >= 1, "slice too small for the workgroup");
     Operand op;
     int o0;
     halfx8 r[NVEC];
@@ -46,8 +49,8 @@ struct Loader {
 #pragma unroll
         for (int h = 0; h < NVEC; h++) {
             if (MODE == VecK) {
-                // 8 vectors cover the 64 k of one row
-                const int o = t / 8 + (THREADS / 8) * h, k = (t % 8) * 8;
+                // BK / 8 vectors cover the k of one row
+                const int o = t / (BK / 8) + (THREADS * 8 / BK) * h, k = (t % (BK / 8)) * 8;
                 const bool ok = (o0 + o) < op.outer_size && (k0 + k) < op.K;
                 if (ok) r[h] = *(const halfx8 *) (op.p + (long long) (o0 + o) * op.so + (k0 + k));
                 else r[h] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -75,7 +78,7 @@ struct Loader {
 #pragma unroll
         for (int h = 0; h < NVEC; h++) {
             if (MODE == VecK) {
-                const int o = t / 8 + (THREADS / 8) * h, k = (t % 8) * 8;
+                const int o = t / (BK / 8) + (THREADS * 8 / BK) * h, k = (t % (BK / 8)) * 8;
                 *(halfx8 *) &lds[o][k] = r[h];
             } else if (MODE == VecOuter) {
                 const int k = t / (T / 8) + (THREADS * 8 / T) * h, o = (t % (T / 8)) * 8;
@@ -99,20 +102,21 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
     *tn = in_g / rows_here;
 }
 
-// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64)
-template <int A_MODE, int B_MODE, int TI>
+// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64); BK: depth of a K slice;
+// NBUF: LDS buffers per operand (2 = double buffered, one barrier per slice; 1 = two barriers per slice)
+template <int A_MODE, int B_MODE, int TI, int BK, int NBUF>
 __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
-    constexpr int T = 64 * TI;
-    __shared__ __attribute__((aligned(16))) half_t As[T][LDS_K];
-    __shared__ __attribute__((aligned(16))) half_t Bs[T][LDS_K];
+    constexpr int T = 64 * TI, LDS_K = BK + 8;
+    __shared__ __attribute__((aligned(16))) half_t As[NBUF][T][LDS_K];
+    __shared__ __attribute__((aligned(16))) half_t Bs[NBUF][T][LDS_K];
 
     const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
     const int m0 = tm * T, n0 = tn * T;
-    Loader<A_MODE, T> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
-    Loader<B_MODE, T> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+    Loader<A_MODE, T, BK> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
+    Loader<B_MODE, T, BK> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1, c = lane & 31, half = lane >> 5;
@@ -125,30 +129,43 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+    const int slices = (p.k + BK - 1) / BK;
     la.fetch(0);
     lb.fetch(0);
-    for (int k0 = 0; k0 < p.k; k0 += BK) {
-        __syncthreads();  // the previous slice has been consumed
-        la.stage(As);
-        lb.stage(Bs);
-        __syncthreads();
-        if (k0 + BK < p.k) {
-            la.fetch(k0 + BK);
-            lb.fetch(k0 + BK);
-        }
+    la.stage(As[0]);
+    lb.stage(Bs[0]);
+    __syncthreads();
+    if (slices > 1) {
+        la.fetch(BK);
+        lb.fetch(BK);
+    }
+    for (int s = 0; s < slices; s++) {
+        const int cur = NBUF == 2 ? (s & 1) : 0;
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 16) {
             // lane l supplies 8 consecutive k (starting at 8 * (l / 32)) of row / column l % 32
             halfx8 a[TI], b[TI];
 #pragma unroll
-            for (int i = 0; i < TI; i++) a[i] = *(const halfx8 *) &As[wm * 32 * TI + 32 * i + c][kk + 8 * half];
+            for (int i = 0; i < TI; i++) a[i] = *(const halfx8 *) &As[cur][wm * 32 * TI + 32 * i + c][kk + 8 * half];
 #pragma unroll
-            for (int j = 0; j < TI; j++) b[j] = *(const halfx8 *) &Bs[wn * 32 * TI + 32 * j + c][kk + 8 * half];
+            for (int j = 0; j < TI; j++) b[j] = *(const halfx8 *) &Bs[cur][wn * 32 * TI + 32 * j + c][kk + 8 * half];
 #pragma unroll
             for (int i = 0; i < TI; i++)
 #pragma unroll
                 for (int j = 0; j < TI; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (NBUF == 1) __syncthreads();  // the slice has been consumed by every wave
+        if (s + 1 < slices) {
+            // double buffered: the other buffer was last read in iteration s - 1, which every wave has left through
+            // the barrier below
+            la.stage(As[NBUF == 2 ? cur ^ 1 : 0]);
+            lb.stage(Bs[NBUF == 2 ? cur ^ 1 : 0]);
+        }
+        __syncthreads();
+        if (s + 2 < slices) {
+            la.fetch((s + 2) * BK);
+            lb.fetch((s + 2) * BK);
         }
     }
 
@@ -177,28 +194,30 @@ int pick_mode(const void *ptr, long long so, long long sk, int outer_size, int k
     return Scalar;
 }
 
-template <int A_MODE, int TI>
+template <int A_MODE, int TI, int BK, int NBUF>
 void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI>), grid, dim3(THREADS), 0, stream, p); break;
-        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI>), grid, dim3(THREADS), 0, stream, p); break;
-        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p); break;
+        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p); break;
     }
 }
 
-template <int TI>
+template <int TI, int BK, int NBUF>
 void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
     switch (a_mode) {
-        case VecOuter: launch_b<VecOuter, TI>(b_mode, grid, stream, p); break;
-        case VecK: launch_b<VecK, TI>(b_mode, grid, stream, p); break;
-        default: launch_b<Scalar, TI>(b_mode, grid, stream, p); break;
+        case VecOuter: launch_b<VecOuter, TI, BK, NBUF>(b_mode, grid, stream, p); break;
+        case VecK: launch_b<VecK, TI, BK, NBUF>(b_mode, grid, stream, p); break;
+        default: launch_b<Scalar, TI, BK, NBUF>(b_mode, grid, stream, p); break;
     }
 }
 
+// 128 x 128 tiles unless there are fewer of them than compute units (measured: 344 tiles 85 us against 112 us with
+// 64 x 64 tiles, 128 tiles 56 us against 47 us).
 int small_tile_threshold() {
     static const int value = [] {
         const char *env = getenv("KNHIP_SMALL_TILE_BELOW");
-        return env ? atoi(env) : 512;
+        return env ? atoi(env) : 256;
     }();
     return value;
 }
@@ -226,8 +245,11 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);
     const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
-    if (small) launch_a<1>(a_mode, b_mode, grid, stream, p);
-    else launch_a<2>(a_mode, b_mode, grid, stream, p);
+    // Measured on 128 x 128 tiles (TFLOP/s at 4096^3 / 8192^3): BK 64 single buffered 594 / 757, BK 64 double
+    // buffered 643 / 718, BK 128 single buffered 672 / 744. All of them sit at the rate at which the L2 can feed
+    // the compute units at this tile size (64 flop per byte fetched from L2, about 12 TB/s -> 770 TFLOP/s).
+    if (small) launch_a<1, 64, 2>(a_mode, b_mode, grid, stream, p);
+    else launch_a<2, 128, 1>(a_mode, b_mode, grid, stream, p);
     return (int) hipGetLastError();
 }
 
