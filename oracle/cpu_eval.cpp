@@ -10,7 +10,9 @@
 //
 // What pins it (see tests/test_oracle_*.py): the expected vectors the reference's own tests hold (elementwise
 // sweep values, softplus, casts, flip, repeat, gather, linear, affine / batch-norm folding, clamp, broadcast add,
-// chained scalar ops, complex multiply) and closed forms / numpy brute force for what those leave open.
+// chained scalar ops, complex multiply), the four ONNX + check-data fixtures of the reference's tests
+// (kn-cuda-eval/tests/data, whole-graph outputs reproduced to 2e-7 ... 2e-6 relative) and closed forms / numpy
+// brute force for what those leave open.
 // Parity unpinned at the bit level: the accumulation order inside ndarray's `sum_axis` / `mean_axis` / `dot`
 // (third party, not in the reference tree) - softmax, layernorm, conv and matmul here accumulate each output
 // element sequentially in f32, which is tolerance-equal, not bit-equal, to the reference's CPU path.
