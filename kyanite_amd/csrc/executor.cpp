@@ -78,6 +78,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             step.gemm.a = l.ptrs[0];
             step.gemm.b = l.ptrs[1];
             step.gemm.c = l.ptrs[2];
+            step.gemm.workspace = l.ptrs.size() > 3 ? l.ptrs[3] : nullptr;
         } else if (step.kind == StepKind::Conv) {
             size_t k = 0;
             step.conv.input = (const float *) l.ptrs[k++];

@@ -1,0 +1,73 @@
+// Launch decisions for the MFMA matrix multiply kernels: operand orientation, tile size, slice depth and the split
+// of the K axis. Kept apart from the kernels so that the planner can reserve the split-K workspace in the arena.
+#include <cstdlib>
+
+#include "mfma_kernels.h"
+
+namespace kn {
+
+namespace {
+
+int env_int(const char *name, int fallback) {
+    const char *env = getenv(name);
+    return env && *env ? atoi(env) : fallback;
+}
+
+}  // namespace
+
+GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
+    GemmLaunchPlan lp{};
+    GemmParams p = params;
+    // put the axis of C that is contiguous in memory on the MFMA column (lane) axis: D^T = B^T * A^T
+    auto mag = [](long long x) { return x < 0 ? -x : x; };
+    if (mag(p.c_sm) < mag(p.c_sn)) {
+        GemmParams q = p;
+        q.a = p.b; q.b = p.a;
+        q.m = p.n; q.n = p.m;
+        q.a_sb = p.b_sb; q.a_sm = p.b_sn; q.a_sk = p.b_sk;
+        q.b_sb = p.a_sb; q.b_sk = p.a_sk; q.b_sn = p.a_sm;
+        q.c_sm = p.c_sn; q.c_sn = p.c_sm;
+        p = q;
+    }
+    lp.p = p;
+    lp.split_k = 1;
+    lp.k_chunk = p.k;
+    if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return lp;
+
+    // 128 x 128 tiles unless there are too few of them to fill the chip. Measured thresholds: f32 344 tiles run
+    // 534 us on 64 x 64 tiles against 597 us, 512 tiles 734 us against 662 us; f16 344 tiles 112 us against 85 us,
+    // 128 tiles 47 us against 56 us. An output no wider than 64 would leave most of a 128 wide tile unused
+    // (16 x [4096 x 4096] x [4096 x 40] in f32: 450 us on 64 x 64 tiles against 682 us).
+    static const int threshold_env = env_int("KNHIP_SMALL_TILE_BELOW", -1);
+    const long long threshold = threshold_env >= 0 ? threshold_env : (f16 ? 256 : 512);
+    static const int split_enabled = env_int("KNHIP_SPLIT_K", 1);
+    const long long big_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch;
+    const bool narrow = p.m <= 64 || p.n <= 64;
+    // With a long K axis and too few tiles, 128 x 128 tiles split along K keep the higher arithmetic intensity
+    // per byte fetched from L2 and still fill the chip.
+    const bool can_split = split_enabled && p.k >= 1024;
+    lp.small_tile = narrow || (big_blocks < threshold && !(can_split && big_blocks < 256));
+    const long long blocks = lp.small_tile ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch : big_blocks;
+    if (f16) lp.bk = lp.small_tile ? 64 : 128;
+    else lp.bk = lp.small_tile && p.k >= 2048 ? 64 : 16;
+
+    if (can_split && blocks < 256) {
+        const int min_chunk = f16 ? 512 : 256;  // K elements a split should at least cover
+        long long s = (512 + blocks - 1) / blocks;
+        if (s > p.k / min_chunk) s = p.k / min_chunk;
+        if (s > 1) {
+            long long chunk = (p.k + s - 1) / s;
+            chunk = (chunk + lp.bk - 1) / lp.bk * lp.bk;
+            s = (p.k + chunk - 1) / chunk;
+            const unsigned long long bytes = (unsigned long long) s * p.batch * p.m * p.n * 4ull;
+            if (s > 1 && bytes <= (256ull << 20)) {
+                lp.split_k = (int) s;
+                lp.k_chunk = (int) chunk;
+                lp.workspace_bytes = (size_t) bytes;
+            }
+        }
+    }
+    return lp;
+}
+
+}  // namespace kn

@@ -105,7 +105,7 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
 // TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64); BK: depth of a K slice;
 // NBUF: LDS buffers per operand (2 = double buffered, one barrier per slice; 1 = two barriers per slice)
 template <int A_MODE, int B_MODE, int TI, int BK, int NBUF>
-__global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
+__global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p, int k_chunk) {
     constexpr int T = 64 * TI, LDS_K = BK + 8;
     __shared__ __attribute__((aligned(16))) half_t As[NBUF][T][LDS_K];
     __shared__ __attribute__((aligned(16))) half_t Bs[NBUF][T][LDS_K];
@@ -115,8 +115,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
     const int m0 = tm * T, n0 = tn * T;
-    Loader<A_MODE, T, BK> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
-    Loader<B_MODE, T, BK> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
+    // split K: workgroup z of gridDim.z multiplies its own range of k and stores an f32 partial product
+    const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
+    Loader<A_MODE, T, BK> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
+    Loader<B_MODE, T, BK> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1, c = lane & 31, half = lane >> 5;
@@ -129,15 +131,15 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    const int slices = (p.k + BK - 1) / BK;
-    la.fetch(0);
-    lb.fetch(0);
+    const int slices = (k_end - k_begin + BK - 1) / BK;
+    la.fetch(k_begin);
+    lb.fetch(k_begin);
     la.stage(As[0]);
     lb.stage(Bs[0]);
     __syncthreads();
     if (slices > 1) {
-        la.fetch(BK);
-        lb.fetch(BK);
+        la.fetch(k_begin + BK);
+        lb.fetch(k_begin + BK);
     }
     for (int s = 0; s < slices; s++) {
         const int cur = NBUF == 2 ? (s & 1) : 0;
@@ -164,13 +166,15 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
         }
         __syncthreads();
         if (s + 2 < slices) {
-            la.fetch((s + 2) * BK);
-            lb.fetch((s + 2) * BK);
+            la.fetch(k_begin + (s + 2) * BK);
+            lb.fetch(k_begin + (s + 2) * BK);
         }
     }
 
     // accumulator layout of the 32x32 tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32
     half_t *out = (half_t *) p.c + bz * p.c_sb;
+    float *partial = (float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n;
+    const bool split = gridDim.z > 1;
 #pragma unroll
     for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -179,7 +183,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p) {
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 32 * TI + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
-                if (row < p.m && col < p.n) out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) acc[i][j][v];
+                if (row < p.m && col < p.n) {
+                    if (split) partial[(long long) row * p.n + col] = acc[i][j][v];
+                    else out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) acc[i][j][v];
+                }
             }
         }
 }
@@ -195,64 +202,44 @@ int pick_mode(const void *ptr, long long so, long long sk, int outer_size, int k
 }
 
 template <int A_MODE, int TI, int BK, int NBUF>
-void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p); break;
-        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p); break;
-        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p, kc); break;
+        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p, kc); break;
+        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p, kc); break;
     }
 }
 
 template <int TI, int BK, int NBUF>
-void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
     switch (a_mode) {
-        case VecOuter: launch_b<VecOuter, TI, BK, NBUF>(b_mode, grid, stream, p); break;
-        case VecK: launch_b<VecK, TI, BK, NBUF>(b_mode, grid, stream, p); break;
-        default: launch_b<Scalar, TI, BK, NBUF>(b_mode, grid, stream, p); break;
+        case VecOuter: launch_b<VecOuter, TI, BK, NBUF>(b_mode, grid, stream, p, kc); break;
+        case VecK: launch_b<VecK, TI, BK, NBUF>(b_mode, grid, stream, p, kc); break;
+        default: launch_b<Scalar, TI, BK, NBUF>(b_mode, grid, stream, p, kc); break;
     }
-}
-
-// 128 x 128 tiles unless there are fewer of them than compute units (measured: 344 tiles 85 us against 112 us with
-// 64 x 64 tiles, 128 tiles 56 us against 47 us).
-int small_tile_threshold() {
-    static const int value = [] {
-        const char *env = getenv("KNHIP_SMALL_TILE_BELOW");
-        return env ? atoi(env) : 256;
-    }();
-    return value;
 }
 
 }  // namespace
 
 int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
-    GemmParams p = params;
-    if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
-    // put the axis of C that is contiguous in memory on the MFMA column (lane) axis: D^T = B^T * A^T
-    auto mag = [](long long x) { return x < 0 ? -x : x; };
-    if (mag(p.c_sm) < mag(p.c_sn)) {
-        GemmParams q = p;
-        q.a = p.b; q.b = p.a;
-        q.m = p.n; q.n = p.m;
-        q.a_sb = p.b_sb; q.a_sm = p.b_sn; q.a_sk = p.b_sk;
-        q.b_sb = p.a_sb; q.b_sk = p.a_sk; q.b_sn = p.a_sm;
-        q.c_sm = p.c_sn; q.c_sn = p.c_sm;
-        p = q;
-    }
-    const long long big_tiles = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128);
-    // an output no wider than 64 would leave most of a 128 wide tile unused (measured on 16 x [4096 x 4096] x
-    // [4096 x 40] in f32: 682 us with 128 x 128 tiles, 450 us with 64 x 64)
-    const bool small = big_tiles * p.batch < small_tile_threshold() || p.m <= 64 || p.n <= 64;
-    const long long tiles = small ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) : big_tiles;
-    if (tiles > 0x7fffffffll || p.batch > 65535) return (int) hipErrorInvalidConfiguration;
-    dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
+    if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
+    const GemmLaunchPlan lp = plan_gemm_launch(params, true);
+    const GemmParams &p = lp.p;
+    const int t = lp.small_tile ? 64 : 128;
+    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t);
+    if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
+    if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
+    dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);
     const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
     // Measured on 128 x 128 tiles (TFLOP/s at 4096^3 / 8192^3): BK 64 single buffered 594 / 757, BK 64 double
     // buffered 643 / 718, BK 128 single buffered 672 / 744. All of them sit at the rate at which the L2 can feed
     // the compute units at this tile size (64 flop per byte fetched from L2, about 12 TB/s -> 770 TFLOP/s).
-    if (small) launch_a<1, 64, 2>(a_mode, b_mode, grid, stream, p);
-    else launch_a<2, 128, 1>(a_mode, b_mode, grid, stream, p);
-    return (int) hipGetLastError();
+    if (lp.small_tile) launch_a<1, 64, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    else launch_a<2, 128, 1>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    int e = (int) hipGetLastError();
+    if (e == 0 && lp.split_k > 1) e = launch_gemm_reduce_partials(p, lp.split_k, true, stream);
+    return e;
 }
 
 }  // namespace kn

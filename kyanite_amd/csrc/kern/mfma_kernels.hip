@@ -224,7 +224,7 @@ struct ConvStore {
 
 // MI x NI: MFMA tiles per wave; the workgroup tile is (64 * MI) x (64 * NI) with the 4 waves arranged 2 x 2.
 template <int MI, int NI, typename LA, typename LB, typename S>
-__device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int K, int m0, int n0) {
+__device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int k_begin, int K, int m0, int n0) {
     constexpr int BK = LA::BK;
     static_assert(LA::BK == LB::BK, "both operands advance by the same slice");
     __shared__ __attribute__((aligned(16))) float As[BK][LA::LDS_STRIDE];
@@ -241,9 +241,9 @@ __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int K, int 
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    la.fetch(0);
-    lb.fetch(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
+    la.fetch(k_begin);
+    lb.fetch(k_begin);
+    for (int k0 = k_begin; k0 < K; k0 += BK) {
         __syncthreads();  // the previous slice has been consumed
         la.stage(As, k0);
         lb.stage(Bs, k0);
@@ -296,17 +296,21 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
 
 // TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64); BK: depth of a K slice
 template <int A_MODE, int B_MODE, int TI, int BK>
-__global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p) {
+__global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p, int k_chunk) {
     constexpr int T = 64 * TI;
     const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
     const int m0 = tm * T, n0 = tn * T;
-    StridedLoader<A_MODE, T, BK> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, p.k}, m0);
-    StridedLoader<B_MODE, T, BK> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, p.k}, n0);
-    GemmStore s{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
-    mfma_tile_loop<TI, TI>(la, lb, s, p.k, m0, n0);
+    // split K: workgroup z of gridDim.z multiplies its own range of k and stores an f32 partial product
+    const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
+    StridedLoader<A_MODE, T, BK> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
+    StridedLoader<B_MODE, T, BK> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
+    GemmStore s = gridDim.z > 1
+        ? GemmStore{(float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n, p.n, 1, p.m, p.n}
+        : GemmStore{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
+    mfma_tile_loop<TI, TI>(la, lb, s, k_begin, k_end, m0, n0);
 }
 
 template <int A_MODE, int KH, int KW, int TI>
@@ -322,7 +326,7 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
     StridedLoader<A_MODE, T, BK> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
     PatchLoader<KH, KW, T, BK> lb(p, n0);
     ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
-    mfma_tile_loop<TI, TI>(la, lb, s, K, m0, n0);
+    mfma_tile_loop<TI, TI>(la, lb, s, 0, K, m0, n0);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -528,21 +532,35 @@ int pick_mode(const void *ptr, long long so, long long sk, long long batch_strid
 }
 
 template <int A_MODE, int TI, int BK>
-void launch_gemm_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+void launch_gemm_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter, TI, BK>), grid, dim3(THREADS), 0, stream, p); break;
-        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK, TI, BK>), grid, dim3(THREADS), 0, stream, p); break;
-        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar, TI, BK>), grid, dim3(THREADS), 0, stream, p); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecOuter, TI, BK>), grid, dim3(THREADS), 0, stream, p, kc); break;
+        case VecK: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, VecK, TI, BK>), grid, dim3(THREADS), 0, stream, p, kc); break;
+        default: hipLaunchKernelGGL((gemm_f32_kernel<A_MODE, Scalar, TI, BK>), grid, dim3(THREADS), 0, stream, p, kc); break;
     }
 }
 
 template <int TI, int BK>
-void launch_gemm_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p) {
+void launch_gemm_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
     switch (a_mode) {
-        case VecOuter: launch_gemm_b<VecOuter, TI, BK>(b_mode, grid, stream, p); break;
-        case VecK: launch_gemm_b<VecK, TI, BK>(b_mode, grid, stream, p); break;
-        default: launch_gemm_b<Scalar, TI, BK>(b_mode, grid, stream, p); break;
+        case VecOuter: launch_gemm_b<VecOuter, TI, BK>(b_mode, grid, stream, p, kc); break;
+        case VecK: launch_gemm_b<VecK, TI, BK>(b_mode, grid, stream, p, kc); break;
+        default: launch_gemm_b<Scalar, TI, BK>(b_mode, grid, stream, p, kc); break;
     }
+}
+
+// Sums the split-K partial products [batch][split][m][n] (f32, dense) into C.
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p, int split) {
+    const long long mn = (long long) p.m * p.n;
+    const long long e = (long long) blockIdx.x * 256 + threadIdx.x;
+    if (e >= mn) return;
+    const int bz = blockIdx.y;
+    const float *part = (const float *) p.workspace + (long long) bz * split * mn + e;
+    float total = 0.0f;
+    for (int s = 0; s < split; s++) total += part[s * mn];
+    const long long row = e / p.n, col = e - row * p.n;
+    ((OutT *) p.c)[bz * p.c_sb + row * p.c_sm + col * p.c_sn] = (OutT) total;
 }
 
 template <int KH, int KW, int TI>
@@ -558,7 +576,7 @@ void launch_conv_t(int a_mode, dim3 grid, hipStream_t stream, const ConvParams &
     else launch_conv_k<0, 0, TI>(a_mode, grid, stream, p);
 }
 
-// 128 x 128 tiles unless there are too few of them to give every compute unit two workgroups.
+// convolutions: 128 x 128 tiles unless there are too few of them to give every compute unit two workgroups
 int small_tile_threshold() {
     static const int value = [] {
         const char *env = getenv("KNHIP_SMALL_TILE_BELOW");
@@ -569,33 +587,31 @@ int small_tile_threshold() {
 
 }  // namespace
 
+int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipStream_t *stream) {
+    const long long mn = (long long) p.m * p.n;
+    dim3 grid((unsigned) ((mn + 255) / 256), (unsigned) p.batch, 1);
+    if (f16) hipLaunchKernelGGL((gemm_reduce_partials_kernel<_Float16>), grid, dim3(256), 0, stream, p, split);
+    else hipLaunchKernelGGL((gemm_reduce_partials_kernel<float>), grid, dim3(256), 0, stream, p, split);
+    return (int) hipGetLastError();
+}
+
 int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
-    GemmParams p = params;
-    if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
-    // put the axis of C that is contiguous in memory on the MFMA column (lane) axis: D^T = B^T * A^T
-    auto mag = [](long long x) { return x < 0 ? -x : x; };
-    if (mag(p.c_sm) < mag(p.c_sn)) {
-        GemmParams q = p;
-        q.a = p.b; q.b = p.a;
-        q.m = p.n; q.n = p.m;
-        q.a_sb = p.b_sb; q.a_sm = p.b_sn; q.a_sk = p.b_sk;
-        q.b_sb = p.a_sb; q.b_sk = p.a_sk; q.b_sn = p.a_sm;
-        q.c_sm = p.c_sn; q.c_sn = p.c_sm;
-        p = q;
-    }
-    const long long big_tiles = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128);
-    // an output no wider than 64 would leave most of a 128 wide tile unused (measured on 16 x [4096 x 4096] x
-    // [4096 x 40] in f32: 682 us with 128 x 128 tiles, 450 us with 64 x 64)
-    const bool small = big_tiles * p.batch < small_tile_threshold() || p.m <= 64 || p.n <= 64;
-    const long long tiles = small ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) : big_tiles;
-    if (tiles > 0x7fffffffll || p.batch > 65535) return (int) hipErrorInvalidConfiguration;
-    dim3 grid((unsigned) tiles, (unsigned) p.batch, 1);
+    if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
+    const GemmLaunchPlan lp = plan_gemm_launch(params, false);
+    const GemmParams &p = lp.p;
+    const int t = lp.small_tile ? 64 : 128;
+    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t);
+    if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
+    if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
+    dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.a_sb, p.batch);
     const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.b_sb, p.batch);
-    if (small && p.k >= 2048) launch_gemm_a<1, 64>(a_mode, b_mode, grid, stream, p);
-    else if (small) launch_gemm_a<1, 16>(a_mode, b_mode, grid, stream, p);
-    else launch_gemm_a<2, 16>(a_mode, b_mode, grid, stream, p);
-    return (int) hipGetLastError();
+    if (lp.small_tile && lp.bk == 64) launch_gemm_a<1, 64>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    else if (lp.small_tile) launch_gemm_a<1, 16>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    else launch_gemm_a<2, 16>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    int e = (int) hipGetLastError();
+    if (e == 0 && lp.split_k > 1) e = launch_gemm_reduce_partials(p, lp.split_k, false, stream);
+    return e;
 }
 
 int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {

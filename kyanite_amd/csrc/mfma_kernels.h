@@ -19,7 +19,23 @@ struct GemmParams {
     long long a_sb, a_sm, a_sk;
     long long b_sb, b_sk, b_sn;
     long long c_sb, c_sm, c_sn;
+    // f32 scratch for partial products when the launch splits the K axis (`GemmLaunchPlan::workspace_bytes`
+    // bytes, 256 byte aligned); may be null otherwise
+    void *workspace = nullptr;
 };
+
+// How a matrix multiply is launched; a pure function of the shapes, strides and alignments, so the planner can ask
+// for it ahead of time (to reserve the workspace) and the launch reproduces it.
+struct GemmLaunchPlan {
+    GemmParams p;            // operands swapped where needed so that the contiguous axis of C is the column axis
+    bool small_tile;         // 64 x 64 workgroup tiles instead of 128 x 128
+    int bk;                  // depth of a K slice
+    int split_k;             // workgroups along K per output tile (1 = no split)
+    int k_chunk;             // K elements per split, a multiple of bk
+    size_t workspace_bytes;  // split_k * batch * m * n * 4 when split_k > 1, else 0
+};
+GemmLaunchPlan plan_gemm_launch(const GemmParams &p, bool f16);
+
 
 // out[n, ko, oy, ox] = act(sum_{c, fy, fx} in[n, c, oy*sy + fy - py, ox*sx + fx - px] * filter[ko, c, fy, fx]
 //                          + bias[ko] + res[n, ko, oy, ox])
@@ -41,6 +57,8 @@ struct ConvParams {
 int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
 // f16 operands and result, f32 accumulation, one rounding (to nearest even) at the store
 int launch_gemm_f16(const GemmParams &p, ihipStream_t *stream);
+// second pass of a split-K launch: C = sum of the f32 partial products in the workspace (`p` already oriented)
+int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipStream_t *stream);
 int launch_conv_f32(const ConvParams &p, ihipStream_t *stream);
 
 }  // namespace kn

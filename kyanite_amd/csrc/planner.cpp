@@ -33,7 +33,9 @@ double Step::flops() const {
 
 double Step::bytes() const {
     double total = 0.0;
-    for (auto &op : operands) {
+    for (size_t i = 0; i < operands.size(); i++) {
+        if (kind == StepKind::MatMul && i >= 3) break;  // split-K scratch is not algorithmic traffic
+        auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
         const auto &strides = op.tensor.shape.strides();
@@ -466,6 +468,11 @@ private:
             g.b_sb = right.shape.strides()[0]; g.b_sk = right.shape.strides()[1]; g.b_sn = right.shape.strides()[2];
             g.c_sb = result.shape.strides()[0]; g.c_sm = result.shape.strides()[1]; g.c_sn = result.shape.strides()[2];
             step.operands = {{left, OperandKind::In}, {right, OperandKind::In}, {result, OperandKind::Out}};
+            // a launch that splits the K axis needs scratch for its f32 partial products: a shared buffer that is
+            // live for this step only
+            const GemmLaunchPlan lp = plan_gemm_launch(g, step.gemm_f16);
+            if (lp.workspace_bytes > 0)
+                step.operands.push_back({alloc_tensor_shared({lp.workspace_bytes / 4}, DType::F32), OperandKind::Out});
             push(std::move(step), value);
         }
         return VT::done(result);

@@ -1006,3 +1006,41 @@ def layernorm_affine_many_rows():
     beta = g.constant([1, 2048], (0.1 * rng.standard_normal((1, 2048))).astype(np.float32))
     g.output(g.add(g.mul(g.layernorm(x, 1, 1e-5), gamma), beta))
     return g, 0, [rng.standard_normal((4099, 2048)).astype(np.float32) * 3.0 + 0.5], None
+
+
+# ---- long contractions with few output tiles: the launch splits the K axis and sums f32 partial products
+
+@case
+def matmul_split_k_skinny_f32():
+    """8 rows (64 x 64 tiles), K = 4100 with a ragged last slice, N = 200 with a partial tile"""
+    g = Graph()
+    rng = np.random.default_rng(60)
+    a = g.input([BATCH, 4100])
+    w = g.constant([200, 4100], (rng.standard_normal((200, 4100)) * 0.05).astype(np.float32))
+    g.output(g.linear(a, w))
+    return g, 8, [rng.standard_normal((8, 4100)).astype(np.float32)], None
+
+
+@case
+def matmul_split_k_big_tiles_f32():
+    """2 batches of 200 x 2304 x 330: 128 x 128 tiles with partial tiles on both axes, K split"""
+    g = Graph()
+    rng = np.random.default_rng(61)
+    a = g.input([2, 200, 2304])
+    b = g.input([2, 2304, 330])
+    y = g.batched_mat_mul(a, b)
+    g.output_all([y, g.permute(y, [0, 2, 1])])
+    return g, 0, [rng.standard_normal((2, 200, 2304)).astype(np.float32) * 0.1,
+                  rng.standard_normal((2, 2304, 330)).astype(np.float32)], None
+
+
+@case
+def matmul_split_k_f16():
+    """f16 operands, f32 partial products, one rounding after the sum: big tiles (136 x 264) and skinny (16 rows)"""
+    g = Graph()
+    rng = np.random.default_rng(62)
+    a = g.input([136, 4352], DType.F16)
+    w = g.constant([264, 4352], _f16(rng, 264, 4352, scale=0.05))
+    s = g.input([16, 4352], DType.F16)
+    g.output_all([g.linear(a, w), g.linear(s, w)])
+    return g, 0, [_f16(rng, 136, 4352), _f16(rng, 16, 4352)], None
