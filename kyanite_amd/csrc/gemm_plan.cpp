@@ -46,7 +46,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // With a long K axis and too few tiles, 128 x 128 tiles split along K keep the higher arithmetic intensity
     // per byte fetched from L2 and still fill the chip.
     const bool can_split = split_enabled && p.k >= 1024;
-    lp.small_tile = narrow || (big_blocks < threshold && !(can_split && big_blocks < 256));
+    lp.small_tile = narrow || (big_blocks < threshold && !(can_split && p.k >= 2048 && big_blocks < 256));
     const long long blocks = lp.small_tile ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch : big_blocks;
     if (f16) lp.bk = lp.small_tile ? 64 : 128;
     else lp.bk = lp.small_tile && p.k >= 2048 ? 64 : 16;

@@ -102,6 +102,51 @@ template<int NW, typename T, typename F> KN_DEV T kn_block_reduce(T v, F f, T *l
     }
     return v;
 }
+
+// Mean and centred sum of squares of a row out of per-lane statistics over `cnt` elements each, combined pairwise
+// (Chan, Golub, LeVeque: M2 = M2a + M2b + (mean_b - mean_a)^2 * n / 2 for equal counts; no cancellation), in ONE
+// pass over the G lanes of a group. Both partners of an exchange compute bit-identical results.
+template<int G> KN_DEV void kn_group_stats(float &mean, float &m2, float cnt) {
+#pragma unroll
+    for (int m = 1; m < G; m <<= 1) {
+        const float om = kn_shfl_xor(mean, m), o2 = kn_shfl_xor(m2, m);
+        const float d = om - mean;
+        m2 = (m2 + o2) + d * d * (cnt * 0.5f);
+        mean = (mean + om) * 0.5f;
+        cnt *= 2.0f;
+    }
+}
+
+// the same over a workgroup of NW waves (a power of two), with one barrier; `lds` holds 2 * NW floats
+template<int NW> KN_DEV void kn_block_stats(float &mean, float &m2, float cnt, float *lds) {
+    kn_group_stats<64>(mean, m2, cnt);
+    if constexpr (NW > 1) {
+        cnt *= 64.0f;
+        if ((threadIdx.x & 63) == 0) {
+            lds[2 * (threadIdx.x >> 6)] = mean;
+            lds[2 * (threadIdx.x >> 6) + 1] = m2;
+        }
+        __syncthreads();
+        float ms[NW], qs[NW];
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            ms[w] = lds[2 * w];
+            qs[w] = lds[2 * w + 1];
+        }
+#pragma unroll
+        for (int n = NW; n > 1; n >>= 1) {
+#pragma unroll
+            for (int i = 0; i < n / 2; i++) {
+                const float d = ms[2 * i + 1] - ms[2 * i];
+                qs[i] = (qs[2 * i] + qs[2 * i + 1]) + d * d * (cnt * 0.5f);
+                ms[i] = (ms[2 * i] + ms[2 * i + 1]) * 0.5f;
+            }
+            cnt *= 2.0f;
+        }
+        mean = ms[0];
+        m2 = qs[0];
+    }
+}
 )KN";
 }
 
@@ -845,7 +890,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     ss << "extern \"C\" __global__ " << (seq > 1 ? "__attribute__((amdgpu_waves_per_eu(8, 8))) " : "") << "__launch_bounds__("
        << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
     for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
-    if (nw > 1) ss << "    __shared__ float lds_m[" << nw << "], lds_s[" << nw << "];\n";
+    if (nw > 1) ss << "    __shared__ float lds_m[" << nw << "], lds_s[" << nw << "], lds_st[" << 2 * nw << "];\n";
     ss << "    const idx_t lane = (idx_t) (threadIdx.x % G);\n";
     ss << "    idx_t base[" << ops.size() << "];\n    for (int k = 0; k < " << ops.size() << "; k++) base[k] = 0;\n";
     const std::string row0 = "((idx_t) blockIdx.x * (idx_t) " + std::to_string(rows_per_block) + " + (idx_t) (threadIdx.x / G))";
@@ -965,7 +1010,12 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         if (softmax) ss << "        for (int j = 0; j < VEC; j++) m = fmaxf(m, x[it][j]);\n";
         else ss << "        for (int j = 0; j < VEC; j++) m += x[it][j];\n";
         ss << "    }\n";
-        reduce("m", softmax ? "kn_max" : "kn_add");
+        // layernorm with the same number of elements in every lane: per-lane mean and centred sum of squares,
+        // combined pairwise in a single pass over the lanes instead of one pass for the mean and one for the
+        // variance (one barrier instead of two when a row spans several waves)
+        static const bool one_pass_env = !(getenv("KNHIP_ROW_ONE_PASS") && !atoi(getenv("KNHIP_ROW_ONE_PASS")));
+        const bool one_pass = !softmax && !check_i && G > 1 && one_pass_env;
+        if (!one_pass) reduce("m", softmax ? "kn_max" : "kn_add");
         ss << "    float s = 0.0f;\n";
         if (softmax) {
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
@@ -973,12 +1023,22 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "            x[it][j] = e;\n            s += e;\n        }\n    }\n";
             reduce("s", "kn_add");
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / s;\n    }\n";
+        } else if (one_pass) {
+            const size_t cnt = items * vec;
+            ss << "    float mean = m / (float) " << cnt << ".0f;\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n";
+            ss << "        for (int j = 0; j < VEC; j++) {\n            const float d = x[it][j] - mean;\n            s += d * d;\n        }\n    }\n";
+            if (nw > 1) ss << "    kn_block_stats<" << nw << ">(mean, s, (float) " << cnt << ".0f, lds_st);\n";
+            else ss << "    kn_group_stats<G>(mean, s, (float) " << cnt << ".0f);\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] - mean;\n    }\n";
         } else {
             ss << "    const float mean = m / (float) " << size << ".0f;\n";
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
             ss << "        for (int j = 0; j < VEC; j++) {\n            const float d = (i < (idx_t) " << nv << ") ? (x[it][j] - mean) : 0.0f;\n";
             ss << "            x[it][j] = d;\n            s += d * d;\n        }\n    }\n";
             reduce("s", "kn_add");
+        }
+        if (!softmax) {
             ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
             if (use_rcp) ss << "    const float rdenom = 1.0f / denom;\n#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] * rdenom;\n    }\n";
             else ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / denom;\n    }\n";
