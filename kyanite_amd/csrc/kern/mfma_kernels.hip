@@ -331,12 +331,12 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
 
 // ---------------------------------------------------------------------------------------------------------------
 // "Plane" convolution: stride 1, same-size output, image width a power of two. Instead of gathering the im2col
-// matrix, every K slice (CB input channels x KH x KW taps) stages the raw input rows that the tile's 128 output
-// positions touch into LDS once, as [channel][group][row][W], and the MFMA B operand is read straight from those
+// matrix, every K slice (CB input channels x KH x KW taps) stages the raw input rows that the tile's TN = 128 or
+// 64 output positions touch into LDS once, as [channel][group][row][W], and the MFMA B operand is read straight from those
 // planes: position n of the tile sits at a fixed per-lane offset, tap (c, fy, fx) adds a wave-uniform offset, and
 // taps that fall left or right of the image are masked to zero (rows above / below are stored as zero rows).
 // Global -> LDS traffic for B drops by KH * KW and no per-element index arithmetic is left in the K loop.
-// A tile is either R = 128 / W whole output rows of one image (H * W >= 128) or G = 128 / (H * W) whole images.
+// A tile is either R = TN / W whole output rows of one image (H * W >= TN) or G = TN / (H * W) whole images.
 constexpr int CB = 8;             // input channels per K slice
 constexpr int PLANE_MAX_VEC = 3;  // 128 bit loads per thread and slice for the B planes
 constexpr int PLANE_SLACK = 4;    // floats in front of / behind the planes that masked taps may touch
@@ -351,8 +351,10 @@ struct PlaneGeom {
     int n_vec;           // CB * G * plane_rows * W / 4
 };
 
-template <int KH, int KW>
+// NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64)
+template <int KH, int KW, int NJ>
 __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, PlaneGeom g) {
+    constexpr int TN = 64 * NJ;  // positions per tile
     constexpr int KS = CB * KH * KW;      // K slice
     constexpr int A_VEC = KS / 4;         // 128 bit loads per filter row and slice
     constexpr int A_ITERS = BM * A_VEC / THREADS;
@@ -364,10 +366,10 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     const int W = p.in_w, H = p.in_h, C = p.in_c;
     const int K = C * KH * KW, ohw = H * W;
     const long long N = (long long) p.batch * ohw;
-    const int tiles_m = (p.out_c + BM - 1) / BM, tiles_n = (int) ((N + BN - 1) / BN);
+    const int tiles_m = (p.out_c + BM - 1) / BM, tiles_n = (int) ((N + TN - 1) / TN);
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
-    const int m0 = tm * BM, n0 = tn * BN;
+    const int m0 = tm * BM, n0 = tn * TN;
     int img0, oy0;
     if (g.tiles_per_image) {
         img0 = tn / g.tiles_per_image;
@@ -404,12 +406,12 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         a_src[i] = (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
         a_dst[i] = 4 * q * A_STRIDE + row;
     }
-    // ---- where this lane's two output positions sit inside a plane, and which taps stay inside the image
-    int lane_base[2];
-    bool pair_ok[2][KW];
+    // ---- where this lane's output positions sit inside a plane, and which taps stay inside the image
+    int lane_base[NJ];
+    bool pair_ok[NJ][KW];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int n = wn * 64 + 32 * j + c32;
+    for (int j = 0; j < NJ; j++) {
+        const int n = wn * 32 * NJ + 32 * j + c32;
         const int gl = n >> g.rw_shift, rem = n & ((1 << g.rw_shift) - 1), col = rem & (W - 1);
         lane_base[j] = PLANE_SLACK + gl * plane + rem - p.pad_x;
 #pragma unroll
@@ -441,11 +443,11 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             if (b_live[i]) *(floatx4 *) &Bs[PLANE_SLACK + 4 * (t + THREADS * i)] = rb[i];
     };
 
-    floatx16 acc[2][2];
+    floatx16 acc[2][NJ];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
@@ -464,23 +466,26 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             const int off_a = ca * gplane + fya * W + fxa, off_b = cb * gplane + fyb * W + fxb;
             const int koff = half ? off_b : off_a;
             const float a0 = As[kk + half][wm * 64 + c32], a1 = As[kk + half][wm * 64 + 32 + c32];
-            float b0 = Bs[lane_base[0] + koff], b1 = Bs[lane_base[1] + koff];
-            b0 = pair_ok[0][fxa] ? b0 : 0.0f;
-            b1 = pair_ok[1][fxa] ? b1 : 0.0f;
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            float b[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                b[j] = Bs[lane_base[j] + koff];
+                b[j] = pair_ok[j][fxa] ? b[j] : 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; j++) acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b[j], acc[0][j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < NJ; j++) acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b[j], acc[1][j], 0, 0, 0);
         }
     }
 
     ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
-    const int col0 = n0 + wn * 64 + c32;
+    const int col0 = n0 + wn * 32 * NJ + c32;
     s.prepare(col0, col0 + 32);
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
@@ -495,22 +500,22 @@ int log2_exact(int x) {
 }
 
 // Fills `g` and returns true when the plane kernel covers this convolution.
-bool plane_geometry(const ConvParams &p, PlaneGeom *g) {
+bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     if (p.kernel_h != 3 || p.kernel_w != 3 || p.stride_y != 1 || p.stride_x != 1) return false;
     if (p.pad_y != 1 || p.pad_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
     if (p.in_c % CB != 0 || (uintptr_t) p.input % 16 != 0 || (uintptr_t) p.filter % 16 != 0) return false;
     const int W = p.in_w, H = p.in_h;
-    if (W < 4 || W > BN || log2_exact(W) < 0) return false;
+    if (W < 4 || W > tn || log2_exact(W) < 0) return false;
     const long long hw = (long long) H * W;
-    if (hw >= BN) {
-        if (hw % BN != 0) return false;
-        g->rows = BN / W;
+    if (hw >= tn) {
+        if (hw % tn != 0) return false;
+        g->rows = tn / W;
         g->groups = 1;
-        g->tiles_per_image = (int) (hw / BN);
+        g->tiles_per_image = (int) (hw / tn);
     } else {
-        if (BN % hw != 0) return false;
+        if (tn % hw != 0) return false;
         g->rows = H;
-        g->groups = (int) (BN / hw);
+        g->groups = (int) (tn / hw);
         g->tiles_per_image = 0;
     }
     g->plane_rows = g->rows + p.kernel_h - 1;
@@ -620,8 +625,15 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     const long long big_tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
     if (positions > 0x7fffffffll || big_tiles > 0x7fffffffll / 4) return (int) hipErrorInvalidValue;
     PlaneGeom geom;
-    if (plane_geometry(p, &geom)) {
-        hipLaunchKernelGGL((conv_plane_kernel<3, 3>), dim3((unsigned) big_tiles), dim3(THREADS), 0, stream, p, geom);
+    static const int plane_wide_from = getenv("KNHIP_CONV_PLANE_WIDE_FROM") ? atoi(getenv("KNHIP_CONV_PLANE_WIDE_FROM")) : 512;
+    // 128 x 64 tiles until there are two 128 x 128 ones per compute unit. Measured on 128 -> 128 channels, 8 x 8
+    // images (us, narrow / wide): batch 64 55 / 89, 256 62 / 95, 512 105 / 103, 1024 208 / 187.
+    int tn = big_tiles >= plane_wide_from ? 128 : 64;
+    if (tn == 64 && !plane_geometry(p, tn, &geom)) tn = 128;  // images wider than 64 only fit the wide tile
+    if (plane_geometry(p, tn, &geom)) {
+        const long long tiles = ((positions + tn - 1) / tn) * ((p.out_c + BM - 1) / BM);
+        if (tn == 128) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2>), dim3((unsigned) tiles), dim3(THREADS), 0, stream, p, geom);
+        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1>), dim3((unsigned) tiles), dim3(THREADS), 0, stream, p, geom);
         return (int) hipGetLastError();
     }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
