@@ -252,19 +252,32 @@ __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int k_begin
             la.fetch(k0 + BK);
             lb.fetch(k0 + BK);
         }
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
+        // the operands of step kk + 2 are read from LDS before the MFMAs of step kk are issued
+        auto read_step = [&](int kk, float (&a)[MI], float (&b)[NI]) {
             const int kr = kk + (lane >> 5), c = lane & 31;
-            float a[MI], b[NI];
 #pragma unroll
             for (int i = 0; i < MI; i++) a[i] = As[kr][wm * 32 * MI + 32 * i + c];
 #pragma unroll
             for (int j = 0; j < NI; j++) b[j] = Bs[kr][wn * 32 * NI + 32 * j + c];
+        };
+        float a[MI], b[NI];
+        read_step(0, a, b);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float na[MI], nb[NI];
+            if (kk + 2 < BK) read_step(kk + 2, na, nb);
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads in front of the MFMAs
 #pragma unroll
             for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < NI; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            if (kk + 2 < BK) {
+#pragma unroll
+                for (int i = 0; i < MI; i++) a[i] = na[i];
+#pragma unroll
+                for (int j = 0; j < NI; j++) b[j] = nb[j];
+            }
         }
     }
 
@@ -458,24 +471,45 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         stage();
         __syncthreads();
         if (c0 + CB < C) fetch(c0 + CB);
-#pragma unroll
-        for (int kk = 0; kk < KS; kk += 2) {
-            // taps of k = kk (lower half of the wave) and k = kk + 1 (upper half); all compile-time
+        // The operands of step kk + 2 are read from LDS before the MFMAs of step kk are issued, so that the LDS
+        // latency runs under the matrix instructions instead of in front of them.
+        auto read_step = [&](int kk, float &a0, float &a1, float (&b)[NJ]) {
+            // taps of k = kk (lower half of the wave) and k = kk + 1 (upper half); all compile-time after unrolling
             const int ca = kk / (KH * KW), fya = (kk / KW) % KH, fxa = kk % KW;
             const int cb = (kk + 1) / (KH * KW), fyb = ((kk + 1) / KW) % KH, fxb = (kk + 1) % KW;
             const int off_a = ca * gplane + fya * W + fxa, off_b = cb * gplane + fyb * W + fxb;
             const int koff = half ? off_b : off_a;
-            const float a0 = As[kk + half][wm * 64 + c32], a1 = As[kk + half][wm * 64 + 32 + c32];
-            float b[NJ];
+            a0 = As[kk + half][wm * 64 + c32];
+            a1 = As[kk + half][wm * 64 + 32 + c32];
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                b[j] = Bs[lane_base[j] + koff];
-                b[j] = pair_ok[j][fxa] ? b[j] : 0.0f;
-            }
+            for (int j = 0; j < NJ; j++) b[j] = Bs[lane_base[j] + koff];
+        };
+        // taps outside the image are masked when the value is consumed, not when it is read, so that nothing
+        // waits for the LDS in front of the MFMAs
+        auto mask_step = [&](int kk, float (&b)[NJ]) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) b[j] = pair_ok[j][kk % KW] ? b[j] : 0.0f;
+        };
+        float a0, a1, b[NJ];
+        read_step(0, a0, a1, b);
+        mask_step(0, b);
+#pragma unroll
+        for (int kk = 0; kk < KS; kk += 2) {
+            float na0 = 0.0f, na1 = 0.0f, nb[NJ];
+            if (kk + 2 < KS) read_step(kk + 2, na0, na1, nb);
+            __builtin_amdgcn_sched_barrier(0);  // keep the reads in front of the MFMAs
 #pragma unroll
             for (int j = 0; j < NJ; j++) acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b[j], acc[0][j], 0, 0, 0);
 #pragma unroll
             for (int j = 0; j < NJ; j++) acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b[j], acc[1][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kk + 2 < KS) {
+                a0 = na0;
+                a1 = na1;
+#pragma unroll
+                for (int j = 0; j < NJ; j++) b[j] = nb[j];
+                mask_step(kk + 2, b);
+            }
         }
     }
 
