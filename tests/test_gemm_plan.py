@@ -1,0 +1,59 @@
+"""Launch decisions of the matrix multiply (no device needed): which shapes reserve a split-K workspace in the
+arena, and that the workspace is the size the launch will use (split * batch * m * n f32 values)."""
+import re
+
+import numpy as np
+
+from kyanite_amd import DType, Graph, HipExecutor
+
+
+def plan(m, n, k, batch=1, dtype=DType.F32):
+    g = Graph()
+    a = g.input([batch, m, k], dtype)
+    b = g.input([batch, k, n], dtype)
+    g.output(g.batched_mat_mul(a, b))
+    ex = HipExecutor(0, g, 0, plan_only=True)
+    assert ex.step_count() == 1
+    text = ex.step_str(0)
+    shapes = re.findall(r"f(?:16|32)\[([0-9, ]*)\]", text.split("operands:")[1])
+    workspace = int(shapes[3]) if len(shapes) > 3 else 0
+    return workspace, ex
+
+
+def test_no_split_when_the_tiles_fill_the_chip():
+    for m, n, k in ((4096, 4096, 4096), (1024, 4672, 2048), (512, 11008, 4096)):
+        assert plan(m, n, k)[0] == 0
+    assert plan(512, 11008, 4096, dtype=DType.F16)[0] == 0
+    # short contractions never split, however few tiles there are
+    assert plan(8, 32, 16)[0] == 0 and plan(64, 64, 512)[0] == 0
+
+
+def test_split_for_long_contractions_with_few_tiles():
+    # 512 x 4096 x 4096: 128 tiles of 128 x 128 on 256 compute units -> 4 splits of 1024
+    ws, _ = plan(512, 4096, 4096, dtype=DType.F16)
+    assert ws == 4 * 512 * 4096
+    ws, _ = plan(512, 4096, 4096)
+    assert ws == 4 * 512 * 4096
+    # skinny: 8 rows, 64 tiles of 64 x 64 -> 8 splits of 512
+    ws, _ = plan(8, 4096, 4096)
+    assert ws == 8 * 8 * 4096
+    # the workspace counts every batch
+    ws, _ = plan(200, 330, 2304, batch=2)
+    assert ws % (2 * 200 * 330) == 0 and ws // (2 * 200 * 330) >= 2
+
+
+def test_workspace_is_scratch_for_its_step_only():
+    # two split matmuls in a row share the same arena bytes for their workspaces
+    g = Graph()
+    x = g.input([8, 4096])
+    w1 = g.constant([4096, 4096], np.zeros((4096, 4096), np.float32))
+    w2 = g.constant([4096, 4096], np.ones((4096, 4096), np.float32))
+    g.output(g.linear(g.linear(x, w1), w2))
+    ex = HipExecutor(0, g, 0, plan_only=True)
+    assert ex.step_kinds() == ["mat_mul", "mat_mul"]
+    usage = ex.mem_usage
+    one_workspace = 8 * 8 * 4096 * 4
+    assert usage["shared_bytes"] < 2 * one_workspace + 3 * 8 * 4096 * 4 + 4096
+    # algorithmic bytes of the step do not include the workspace
+    flops, nbytes = ex.step_work(0)
+    assert flops == 2 * 8 * 4096 * 4096 and nbytes == 4 * (8 * 4096 + 4096 * 4096 + 8 * 4096)
