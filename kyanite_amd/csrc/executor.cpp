@@ -78,7 +78,9 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             step.gemm.a = l.ptrs[0];
             step.gemm.b = l.ptrs[1];
             step.gemm.c = l.ptrs[2];
-            step.gemm.workspace = l.ptrs.size() > 3 ? l.ptrs[3] : nullptr;
+            size_t next = 3;
+            step.gemm.addend = step.gemm_has_addend ? l.ptrs[next++] : nullptr;
+            step.gemm.workspace = l.ptrs.size() > next ? l.ptrs[next] : nullptr;
         } else if (step.kind == StepKind::Conv) {
             size_t k = 0;
             step.conv.input = (const float *) l.ptrs[k++];

@@ -27,6 +27,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         q.a_sb = p.b_sb; q.a_sm = p.b_sn; q.a_sk = p.b_sk;
         q.b_sb = p.a_sb; q.b_sk = p.a_sk; q.b_sn = p.a_sm;
         q.c_sm = p.c_sn; q.c_sn = p.c_sm;
+        q.d_sm = p.d_sn; q.d_sn = p.d_sm;
         p = q;
     }
     lp.p = p;

@@ -175,6 +175,8 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p, int k_c
     half_t *out = (half_t *) p.c + bz * p.c_sb;
     float *partial = (float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n;
     const bool split = gridDim.z > 1;
+    // the epilogue of a split launch is applied by the pass that sums the partial products
+    const half_t *addend = p.addend ? (const half_t *) p.addend + bz * p.d_sb : nullptr;
 #pragma unroll
     for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -184,8 +186,14 @@ __global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p, int k_c
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 32 * TI + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
                 if (row < p.m && col < p.n) {
-                    if (split) partial[(long long) row * p.n + col] = acc[i][j][v];
-                    else out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) acc[i][j][v];
+                    if (split) {
+                        partial[(long long) row * p.n + col] = acc[i][j][v];
+                    } else {
+                        half_t r = (half_t) acc[i][j][v];
+                        if (addend) r = (half_t) ((float) r + (float) addend[(long long) row * p.d_sm + (long long) col * p.d_sn]);
+                        if (p.relu) r = r > (half_t) 0 ? r : (half_t) 0;
+                        out[(long long) row * p.c_sm + (long long) col * p.c_sn] = r;
+                    }
                 }
             }
         }

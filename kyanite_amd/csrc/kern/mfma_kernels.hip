@@ -185,9 +185,16 @@ struct GemmStore {
     float *p;
     long long sm, sn;
     int M, N;
+    const float *addend;  // optional epilogue operand (null = none), with its own strides
+    long long dm, dn;
+    int relu;
     __device__ __forceinline__ void prepare(int, int) {}
     __device__ __forceinline__ void store(int m, int n, int, float v) const {
-        if (m < M && n < N) p[(long long) m * sm + (long long) n * sn] = v;
+        if (m < M && n < N) {
+            if (addend) v += addend[(long long) m * dm + (long long) n * dn];
+            if (relu) v = fmaxf(v, 0.0f);
+            p[(long long) m * sm + (long long) n * sn] = v;
+        }
     }
 };
 
@@ -320,9 +327,12 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p, int k_c
     const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
     StridedLoader<A_MODE, T, BK> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
     StridedLoader<B_MODE, T, BK> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
+    // the epilogue of a split launch is applied by the pass that sums the partial products
     GemmStore s = gridDim.z > 1
-        ? GemmStore{(float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n, p.n, 1, p.m, p.n}
-        : GemmStore{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n};
+        ? GemmStore{(float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n, p.n, 1, p.m, p.n,
+                    nullptr, 0, 0, 0}
+        : GemmStore{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n,
+                    p.addend ? (const float *) p.addend + bz * p.d_sb : nullptr, p.d_sm, p.d_sn, p.relu};
     mfma_tile_loop<TI, TI>(la, lb, s, k_begin, k_end, m0, n0);
 }
 
@@ -599,6 +609,10 @@ __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p,
     float total = 0.0f;
     for (int s = 0; s < split; s++) total += part[s * mn];
     const long long row = e / p.n, col = e - row * p.n;
+    // rounding to the output type after the product and after the sum, like separate operations would
+    total = (float) (OutT) total;
+    if (p.addend) total = (float) (OutT) (total + (float) ((const OutT *) p.addend)[bz * p.d_sb + row * p.d_sm + col * p.d_sn]);
+    if (p.relu) total = fmaxf(total, 0.0f);
     ((OutT *) p.c)[bz * p.c_sb + row * p.c_sm + col * p.c_sn] = (OutT) total;
 }
 

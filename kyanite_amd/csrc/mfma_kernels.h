@@ -19,6 +19,12 @@ struct GemmParams {
     long long a_sb, a_sm, a_sk;
     long long b_sb, b_sk, b_sn;
     long long c_sb, c_sm, c_sn;
+    // optional epilogue: C = act(A * B + D) with D addressed by element strides like C (zero = broadcast) and
+    // act = max(., 0) when `relu` is set; for f16 the product and the sum are each rounded to f16, like separate
+    // operations would
+    const void *addend = nullptr;
+    long long d_sb = 0, d_sm = 0, d_sn = 0;
+    int relu = 0;
     // f32 scratch for partial products when the launch splits the K axis (`GemmLaunchPlan::workspace_bytes`
     // bytes, 256 byte aligned); may be null otherwise
     void *workspace = nullptr;

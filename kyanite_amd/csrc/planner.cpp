@@ -13,7 +13,9 @@ std::string Step::str() const {
     std::ostringstream ss;
     ss << step_kind_name(kind) << " value=" << debug_value;
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
-    if (kind == StepKind::MatMul) ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k;
+    if (kind == StepKind::MatMul)
+        ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
+           << (gemm_has_addend ? " +add" : "") << (gemm.relu ? " relu" : "");
     else if (kind == StepKind::Conv)
         ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="
            << conv.kernel_h << "x" << conv.kernel_w << (conv_has_bias ? " +bias" : "") << (conv_has_res ? " +res" : "")
@@ -34,7 +36,7 @@ double Step::flops() const {
 double Step::bytes() const {
     double total = 0.0;
     for (size_t i = 0; i < operands.size(); i++) {
-        if (kind == StepKind::MatMul && i >= 3) break;  // split-K scratch is not algorithmic traffic
+        if (kind == StepKind::MatMul && i >= (gemm_has_addend ? 4u : 3u)) break;  // split-K scratch is not algorithmic traffic
         auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
@@ -199,6 +201,11 @@ private:
     VT visit_single_new(Value value) {
         {
             auto fused = try_visit_fused_conv(value);
+            if (!fused.ok) return VT::missing(fused.need);
+            if (fused.value) return VT::done(*fused.value);
+        }
+        if (options.fuse_matmul_epilogue) {
+            auto fused = try_visit_fused_matmul(value);
             if (!fused.ok) return VT::missing(fused.need);
             if (fused.value) return VT::done(*fused.value);
         }
@@ -448,7 +455,77 @@ private:
     }
 
     // planner.rs:606-648
-    VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first) {
+    // Not in the reference (its matmuls are plain library calls): an elementwise tail of a matmul of the form
+    //   max(., 0)?  <-  (. + d)?  <-  view*  <-  MatMul
+    // whose intermediate values are hidden and used once is folded into the matmul's store, d being any tensor of
+    // the result's shape (a broadcast bias, a residual). Returns nullopt when `value` is not such a tail.
+    Visit<std::optional<PlanTensor>> try_visit_fused_matmul(Value value) {
+        using R = Visit<std::optional<PlanTensor>>;
+        const DType dt = graph[value].dtype;
+        if (dt != DType::F32 && dt != DType::F16) return R::done(std::nullopt);
+        Value curr = value;
+        bool relu = false;
+        {
+            const Operation &op = graph[curr].operation;
+            if (op.kind == OpKind::Binary && op.binary == BinaryOp::Max) {
+                Value l = op.inputs[0], r = op.inputs[1];
+                if (graph.is_const_zero(l)) curr = r;
+                else if (graph.is_const_zero(r)) curr = l;
+                else return R::done(std::nullopt);
+                if (!can_fuse(curr)) return R::done(std::nullopt);
+                relu = true;
+            }
+        }
+        // through views down to the matmul, as long as every link is hidden and used once (`from` itself is the
+        // operand of the operation above and has been checked by the caller)
+        auto matmul_under = [&](Value from) -> std::optional<Value> {
+            Value v = from;
+            while (graph[v].operation.kind == OpKind::View) {
+                Value inner = graph[v].operation.inputs[0];
+                if (!can_fuse(inner)) return std::nullopt;
+                v = inner;
+            }
+            if (graph[v].operation.kind != OpKind::MatMul) return std::nullopt;
+            return v;
+        };
+        std::optional<Value> addend;
+        std::optional<Value> mm;
+        {
+            const Operation &op = graph[curr].operation;
+            if (op.kind == OpKind::Binary && op.binary == BinaryOp::Add) {
+                Value l = op.inputs[0], r = op.inputs[1];
+                if (can_fuse(l)) mm = matmul_under(l);
+                if (mm) addend = r;
+                else if (can_fuse(r) && (mm = matmul_under(r))) addend = l;
+            } else if (relu) {
+                mm = matmul_under(curr);
+            }
+        }
+        if (!mm || (!relu && !addend)) return R::done(std::nullopt);
+        if (map.count(*mm)) return R::done(std::nullopt);
+
+        const ConcreteShape final_shape = graph[value].shape.eval(batch_size);
+        const ConcreteShape mm_shape = graph[*mm].shape.eval(batch_size);
+        std::optional<PlanTensor> addend_t;
+        if (addend) {
+            auto at = visit(*addend);
+            if (!at.ok) return R::missing(at.need);
+            // the operand in the matmul's own [b, m, n] shape; an operand whose layout cannot follow the views
+            // between the matmul and the sum is not fused
+            KN_ASSERT(at.value.shape.shape() == final_shape);
+            addend_t = at.value.view(mm_shape);
+            if (!addend_t) return R::done(std::nullopt);
+        }
+        const Operation &mop = graph[*mm].operation;
+        auto result = visit_matmul(value, mop.inputs[0], mop.inputs[1], true, addend_t, relu);
+        if (!result.ok) return R::missing(result.need);
+        auto viewed = result.value.view(final_shape);
+        KN_ASSERT(viewed.has_value(), "a dense matmul result can always be viewed");
+        return R::done(*viewed);
+    }
+
+    VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first,
+                    const std::optional<PlanTensor> &addend = std::nullopt, bool relu = false) {
         const DType dt = graph[value].dtype;
         if (dt != DType::F32 && dt != DType::F16) fail("GPU matmul only supports f32 and f16, got ", dtype_name(dt));
         KN_TRY(left, visit(left_v));
@@ -468,6 +545,13 @@ private:
             g.b_sb = right.shape.strides()[0]; g.b_sk = right.shape.strides()[1]; g.b_sn = right.shape.strides()[2];
             g.c_sb = result.shape.strides()[0]; g.c_sm = result.shape.strides()[1]; g.c_sn = result.shape.strides()[2];
             step.operands = {{left, OperandKind::In}, {right, OperandKind::In}, {result, OperandKind::Out}};
+            if (addend) {
+                KN_ASSERT(addend->dtype == dt && addend->shape.shape() == ConcreteShape({b, m, n}));
+                g.d_sb = addend->shape.strides()[0]; g.d_sm = addend->shape.strides()[1]; g.d_sn = addend->shape.strides()[2];
+                step.gemm_has_addend = true;
+                step.operands.push_back({*addend, OperandKind::In});
+            }
+            g.relu = relu ? 1 : 0;
             // a launch that splits the K axis needs scratch for its f32 partial products: a shared buffer that is
             // live for this step only
             const GemmLaunchPlan lp = plan_gemm_launch(g, step.gemm_f16);

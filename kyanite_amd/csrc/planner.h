@@ -36,6 +36,7 @@ struct Step {
     // matrix-core kernels; the pointers are filled in when the plan is realised
     GemmParams gemm{};
     bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
+    bool gemm_has_addend = false;  // operand 3 is the tensor added in the epilogue
     ConvParams conv{};
     bool conv_has_bias = false, conv_has_res = false;
 
@@ -80,6 +81,7 @@ constexpr size_t ARENA_ALIGN = 256;
 struct PlannerOptions {
     bool compile = true;          // compile the generated kernels (can be switched off to inspect the plan only)
     bool fuse_row_epilogue = true;  // fold elementwise consumers of a layernorm / softmax into the row kernel
+    bool fuse_matmul_epilogue = true;  // fold `+ d` and `max(., 0)` after a matmul into the matmul's store
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
 };

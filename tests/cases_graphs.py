@@ -1044,3 +1044,53 @@ def matmul_split_k_f16():
     s = g.input([16, 4352], DType.F16)
     g.output_all([g.linear(a, w), g.linear(s, w)])
     return g, 0, [_f16(rng, 136, 4352), _f16(rng, 16, 4352)], None
+
+
+# ---- elementwise tails folded into the matmul's store
+
+@case
+def matmul_bias_relu_fused():
+    """relu(x W^T + b), x W^T + b, relu(x W^T) and a residual sum, with partial tiles; one launch each"""
+    g = Graph()
+    rng = np.random.default_rng(70)
+    x = g.input([BATCH, 70])
+    w = g.constant([130, 70], (rng.standard_normal((130, 70)) * 0.2).astype(np.float32))
+    b = g.constant([1, 130], rng.standard_normal((1, 130)).astype(np.float32))
+    w2 = g.constant([70, 130], (rng.standard_normal((70, 130)) * 0.2).astype(np.float32))
+    h = g.relu(g.add(g.linear(x, w), b))
+    y = g.add(x, g.linear(h, w2))  # residual: the addend is a full tensor
+    g.output_all([y, g.add(g.linear(y, w), b), g.relu(g.linear(y, w))])
+    return g, 9, [rng.standard_normal((9, 70)).astype(np.float32)], None
+
+
+@case
+def matmul_epilogue_layouts():
+    """batched product with a bias per row (the addend is broadcast along the contiguous axis) and a transposed
+    result, so the launch swaps its operands"""
+    g = Graph()
+    rng = np.random.default_rng(71)
+    a = g.input([3, 40, 24])
+    b = g.input([3, 24, 56])
+    row_bias = g.constant([1, 40, 1], rng.standard_normal((1, 40, 1)).astype(np.float32))
+    col_bias = g.constant([3, 1, 56], rng.standard_normal((3, 1, 56)).astype(np.float32))
+    a2 = g.input([3, 40, 24])
+    y = g.relu(g.add(g.batched_mat_mul(a, b), row_bias))
+    z = g.add(g.batched_mat_mul(a2, b), col_bias)
+    g.output_all([y, g.permute(z, [0, 2, 1])])
+    return g, 0, [rng.standard_normal((3, 40, 24)).astype(np.float32), rng.standard_normal((3, 24, 56)).astype(np.float32),
+                  rng.standard_normal((3, 40, 24)).astype(np.float32)], None
+
+
+@case
+def matmul_epilogue_split_k_f16():
+    """f16: product, sum and relu each round to f16; the long contraction is split, so the tail runs in the pass
+    that sums the partial products"""
+    g = Graph()
+    rng = np.random.default_rng(72)
+    x = g.input([24, 4352], DType.F16)
+    w = g.constant([136, 4352], _f16(rng, 136, 4352, scale=0.05))
+    b = g.constant([1, 136], _f16(rng, 1, 136))
+    small = g.constant([136, 136], _f16(rng, 136, 136, scale=0.1))
+    h = g.relu(g.add(g.linear(x, w), b))
+    g.output_all([h, g.add(h, g.linear(h, small))])
+    return g, 0, [_f16(rng, 24, 4352)], None
