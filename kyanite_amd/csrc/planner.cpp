@@ -259,16 +259,44 @@ private:
                 return VT::done(output);
             }
             case OpKind::Concat: {
-                std::vector<PlanTensor> ins;
+                // planner.rs:394-412 copies every input into its slice of the result. An input that is an
+                // elementwise chain nobody else uses is computed straight into its slice instead (one kernel
+                // less per input and no intermediate buffer).
+                struct Piece {
+                    std::optional<PlanTensor> tensor;  // a materialised input, copied
+                    std::optional<ScalarBlock> block;  // or a chain evaluated in place
+                    Value value;
+                };
+                std::vector<Piece> pieces;
                 for (Value x : op.inputs) {
-                    KN_TRY(t, visit(x));
-                    ins.push_back(t);
+                    Piece piece;
+                    piece.value = x;
+                    const OpKind kind = graph[x].operation.kind;
+                    if (!map.count(x) && can_fuse(x) && (kind == OpKind::Unary || kind == OpKind::Binary)) {
+                        ScalarBlock block;
+                        block.operands.push_back(PlanTensor());  // placeholder for the result
+                        block.loaded.push_back(std::nullopt);
+                        auto root = visit_fused_scalar_recurse(x, block, true);
+                        if (!root.ok) return VT::missing(root.need);
+                        if (!block.row_value) piece.block = std::move(block);
+                    }
+                    if (!piece.block) {
+                        KN_TRY(t, visit(x));
+                        piece.tensor = t;
+                    }
+                    pieces.push_back(std::move(piece));
                 }
                 PlanTensor result = alloc_tensor_shared(result_shape, result_dtype);
                 size_t axis = op.axis(), start = 0;
-                for (auto &in : ins) {
-                    size_t len = in.shape.shape()[axis];
-                    plan_copy_tensor(in, result.slice(axis, SliceRange{start, start + len, 1}), value);
+                for (auto &piece : pieces) {
+                    size_t len = graph[piece.value].shape.eval(batch_size)[axis];
+                    PlanTensor target = result.slice(axis, SliceRange{start, start + len, 1});
+                    if (piece.block) {
+                        piece.block->operands[0] = target;
+                        plan_scalar_op(piece.block->expr, piece.block->operands, piece.value);
+                    } else {
+                        plan_copy_tensor(*piece.tensor, target, value);
+                    }
                     start += len;
                 }
                 return VT::done(result);
