@@ -598,22 +598,38 @@ void launch_gemm_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const 
     }
 }
 
-// Sums the split-K partial products [batch][split][m][n] (f32, dense) into C.
-template <typename OutT>
+// Sums the split-K partial products [batch][split][m][n] (f32, dense) into C and applies the epilogue. VEC = 4:
+// every thread owns four neighbouring columns (n a multiple of 4, C and the addend contiguous or broadcast along n).
+template <typename OutT, int VEC>
 __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p, int split) {
     const long long mn = (long long) p.m * p.n;
-    const long long e = (long long) blockIdx.x * 256 + threadIdx.x;
+    const long long e = ((long long) blockIdx.x * 256 + threadIdx.x) * VEC;
     if (e >= mn) return;
     const int bz = blockIdx.y;
     const float *part = (const float *) p.workspace + (long long) bz * split * mn + e;
-    float total = 0.0f;
-    for (int s = 0; s < split; s++) total += part[s * mn];
+    float total[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) total[j] = 0.0f;
+    for (int s = 0; s < split; s++) {
+        if (VEC == 4) {
+            const floatx4 v = *(const floatx4 *) (part + s * mn);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) total[j] += v[j];
+        } else {
+            total[0] += part[s * mn];
+        }
+    }
     const long long row = e / p.n, col = e - row * p.n;
-    // rounding to the output type after the product and after the sum, like separate operations would
-    total = (float) (OutT) total;
-    if (p.addend) total = (float) (OutT) (total + (float) ((const OutT *) p.addend)[bz * p.d_sb + row * p.d_sm + col * p.d_sn]);
-    if (p.relu) total = fmaxf(total, 0.0f);
-    ((OutT *) p.c)[bz * p.c_sb + row * p.c_sm + col * p.c_sn] = (OutT) total;
+    OutT *out = (OutT *) p.c + bz * p.c_sb + row * p.c_sm + col * p.c_sn;
+    const OutT *addend = p.addend ? (const OutT *) p.addend + bz * p.d_sb + row * p.d_sm + col * p.d_sn : nullptr;
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        // rounding to the output type after the product and after the sum, like separate operations would
+        float v = (float) (OutT) total[j];
+        if (addend) v = (float) (OutT) (v + (float) addend[j * p.d_sn]);
+        if (p.relu) v = fmaxf(v, 0.0f);
+        out[j * p.c_sn] = (OutT) v;
+    }
 }
 
 template <int KH, int KW, int TI>
@@ -642,9 +658,13 @@ int small_tile_threshold() {
 
 int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipStream_t *stream) {
     const long long mn = (long long) p.m * p.n;
-    dim3 grid((unsigned) ((mn + 255) / 256), (unsigned) p.batch, 1);
-    if (f16) hipLaunchKernelGGL((gemm_reduce_partials_kernel<_Float16>), grid, dim3(256), 0, stream, p, split);
-    else hipLaunchKernelGGL((gemm_reduce_partials_kernel<float>), grid, dim3(256), 0, stream, p, split);
+    const bool vec = p.n % 4 == 0 && p.c_sn == 1 && (uintptr_t) p.workspace % 16 == 0;
+    const long long threads = vec ? mn / 4 : mn;
+    dim3 grid((unsigned) ((threads + 255) / 256), (unsigned) p.batch, 1);
+    if (f16 && vec) hipLaunchKernelGGL((gemm_reduce_partials_kernel<_Float16, 4>), grid, dim3(256), 0, stream, p, split);
+    else if (f16) hipLaunchKernelGGL((gemm_reduce_partials_kernel<_Float16, 1>), grid, dim3(256), 0, stream, p, split);
+    else if (vec) hipLaunchKernelGGL((gemm_reduce_partials_kernel<float, 4>), grid, dim3(256), 0, stream, p, split);
+    else hipLaunchKernelGGL((gemm_reduce_partials_kernel<float, 1>), grid, dim3(256), 0, stream, p, split);
     return (int) hipGetLastError();
 }
 
