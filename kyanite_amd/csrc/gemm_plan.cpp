@@ -48,13 +48,23 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // per byte fetched from L2 and still fill the chip.
     const bool can_split = split_enabled && p.k >= 1024;
     lp.small_tile = narrow || (big_blocks < threshold && !(can_split && p.k >= 2048 && big_blocks < 256));
-    const long long blocks = lp.small_tile ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch : big_blocks;
-    if (f16) lp.bk = lp.small_tile ? 64 : 128;
+    // f16 with so few tiles that the K axis gets split anyway: 256 x 128 tiles (8 waves), which fetch a quarter
+    // fewer bytes from L2 per flop and halve the partial products per split. Measured (us, 128 x 128 against
+    // 256 x 128): 512 x 4096 x 4096 43 / 38, 512 x 4096 x 11008 89 / 75; without a split they do not pay:
+    // 512 x 11008 x 4096 82 / 87, 8192^3 1454 / 1439.
+    static const int tall_below = env_int("KNHIP_F16_TALL_BELOW", 128);
+    const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch;
+    lp.tall_tile = f16 && !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8 && can_split &&
+                   p.k >= 2048 && tall_blocks < tall_below;
+    long long blocks = lp.small_tile ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch : big_blocks;
+    if (lp.tall_tile) blocks = tall_blocks;
+    if (f16) lp.bk = lp.small_tile || lp.tall_tile ? 64 : 128;
     else lp.bk = lp.small_tile && p.k >= 2048 ? 64 : 16;
 
-    if (can_split && blocks < 256) {
+    const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
+    if (can_split && blocks < split_below) {
         const int min_chunk = f16 ? 512 : 256;  // K elements a split should at least cover
-        long long s = (512 + blocks - 1) / blocks;
+        long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;
         if (s > 1) {
             long long chunk = (p.k + s - 1) / s;

@@ -21,7 +21,6 @@ typedef _Float16 half_t;
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int THREADS = 256;
 
 enum LoadMode { Scalar = 0, VecOuter = 1, VecK = 2 };
 
@@ -33,7 +32,8 @@ struct Operand {
 
 // Fetches a T x BK slice into registers and writes it to LDS as [outer][k]. Vector modes need every vector to lie
 // completely inside or outside the matrix, which the host guarantees (sizes divisible by 8 along the vector axis).
-template <int MODE, int T, int BK>
+// THREADS: size of the workgroup that shares the slice.
+template <int MODE, int T, int BK, int THREADS>
 struct Loader {
     static constexpr int NVEC = T * BK / 8 / THREADS;  // 128 bit vectors per thread and slice
     static constexpr int LDS_K = BK + 8;
@@ -102,23 +102,25 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
     *tn = in_g / rows_here;
 }
 
-// TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64); BK: depth of a K slice;
-// NBUF: LDS buffers per operand (2 = double buffered, one barrier per slice; 1 = two barriers per slice)
-template <int A_MODE, int B_MODE, int TI, int BK, int NBUF>
-__global__ __launch_bounds__(THREADS) void gemm_f16_kernel(GemmParams p, int k_chunk) {
-    constexpr int T = 64 * TI, LDS_K = BK + 8;
-    __shared__ __attribute__((aligned(16))) half_t As[NBUF][T][LDS_K];
-    __shared__ __attribute__((aligned(16))) half_t Bs[NBUF][T][LDS_K];
+// TI: MFMA tiles per wave and axis; WM: waves along M (2 along N), so the workgroup tile is (32 TI WM) x (64 TI):
+// 128 x 128 (TI 2, WM 2), 64 x 64 (TI 1, WM 2) or 256 x 128 with 8 waves (TI 2, WM 4), which fetches a quarter less
+// from L2 per flop. BK: depth of a K slice; NBUF: LDS buffers per operand (2 = double buffered, one barrier per
+// slice; 1 = two barriers per slice)
+template <int A_MODE, int B_MODE, int TI, int BK, int NBUF, int WM>
+__global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_chunk) {
+    constexpr int TM = 32 * TI * WM, TN = 64 * TI, LDS_K = BK + 8, THREADS = 128 * WM;
+    __shared__ __attribute__((aligned(16))) half_t As[NBUF][TM][LDS_K];
+    __shared__ __attribute__((aligned(16))) half_t Bs[NBUF][TN][LDS_K];
 
-    const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
+    const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int bz = blockIdx.y;
-    const int m0 = tm * T, n0 = tn * T;
+    const int m0 = tm * TM, n0 = tn * TN;
     // split K: workgroup z of gridDim.z multiplies its own range of k and stores an f32 partial product
     const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
-    Loader<A_MODE, T, BK> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
-    Loader<B_MODE, T, BK> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
+    Loader<A_MODE, TM, BK, THREADS> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
+    Loader<B_MODE, TN, BK, THREADS> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1, c = lane & 31, half = lane >> 5;
@@ -209,21 +211,22 @@ int pick_mode(const void *ptr, long long so, long long sk, int outer_size, int k
     return Scalar;
 }
 
-template <int A_MODE, int TI, int BK, int NBUF>
+template <int A_MODE, int TI, int BK, int NBUF, int WM>
 void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
+    const dim3 block(128 * WM);
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p, kc); break;
-        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p, kc); break;
-        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF>), grid, dim3(THREADS), 0, stream, p, kc); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc); break;
+        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc); break;
+        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc); break;
     }
 }
 
-template <int TI, int BK, int NBUF>
+template <int TI, int BK, int NBUF, int WM>
 void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
     switch (a_mode) {
-        case VecOuter: launch_b<VecOuter, TI, BK, NBUF>(b_mode, grid, stream, p, kc); break;
-        case VecK: launch_b<VecK, TI, BK, NBUF>(b_mode, grid, stream, p, kc); break;
-        default: launch_b<Scalar, TI, BK, NBUF>(b_mode, grid, stream, p, kc); break;
+        case VecOuter: launch_b<VecOuter, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc); break;
+        case VecK: launch_b<VecK, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc); break;
+        default: launch_b<Scalar, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc); break;
     }
 }
 
@@ -233,8 +236,8 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
     const GemmLaunchPlan lp = plan_gemm_launch(params, true);
     const GemmParams &p = lp.p;
-    const int t = lp.small_tile ? 64 : 128;
-    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t);
+    const int t = lp.small_tile ? 64 : 128, t_m = lp.tall_tile ? 256 : t;
+    const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t - 1) / t);
     if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
@@ -243,8 +246,9 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     // Measured on 128 x 128 tiles (TFLOP/s at 4096^3 / 8192^3): BK 64 single buffered 594 / 757, BK 64 double
     // buffered 643 / 718, BK 128 single buffered 672 / 744. All of them sit at the rate at which the L2 can feed
     // the compute units at this tile size (64 flop per byte fetched from L2, about 12 TB/s -> 770 TFLOP/s).
-    if (lp.small_tile) launch_a<1, 64, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
-    else launch_a<2, 128, 1>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    if (lp.small_tile) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    else if (lp.tall_tile) launch_a<2, 64, 1, 4>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    else launch_a<2, 128, 1, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
     int e = (int) hipGetLastError();
     if (e == 0 && lp.split_k > 1) e = launch_gemm_reduce_partials(p, lp.split_k, true, stream);
     return e;

@@ -35,6 +35,7 @@ struct GemmParams {
 struct GemmLaunchPlan {
     GemmParams p;            // operands swapped where needed so that the contiguous axis of C is the column axis
     bool small_tile;         // 64 x 64 workgroup tiles instead of 128 x 128
+    bool tall_tile;          // f16 only: 256 x 128 workgroup tiles (8 waves)
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)
     int k_chunk;             // K elements per split, a multiple of bk

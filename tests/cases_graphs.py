@@ -1094,3 +1094,30 @@ def matmul_epilogue_split_k_f16():
     h = g.relu(g.add(g.linear(x, w), b))
     g.output_all([h, g.add(h, g.linear(h, small))])
     return g, 0, [_f16(rng, 24, 4352)], None
+
+
+@case
+def f16_matmul_tall_tiles():
+    """256 x 128 workgroup tiles (8 waves, K split): 500 rows (12 rows of the second tile missing), 200 and 264
+    columns (partial tiles), K = 2088 with a ragged last slice; N-contiguous and K-contiguous right operands"""
+    g = Graph()
+    rng = np.random.default_rng(80)
+    a = g.input([2, 500, 2088], DType.F16)
+    b = g.input([2, 2088, 200], DType.F16)
+    w = g.constant([264, 2088], _f16(rng, 264, 2088, scale=0.05))
+    bias = g.constant([1, 264], _f16(rng, 1, 264))
+    y = g.batched_mat_mul(a, b)
+    z = g.relu(g.add(g.linear(g.view(a, [1000, 2088]), w), bias))
+    g.output_all([y, z])
+    return g, 0, [_f16(rng, 2, 500, 2088, scale=0.2), _f16(rng, 2, 2088, 200, scale=0.1)], None
+
+
+@case
+def f16_matmul_tall_tiles_split_k():
+    """256 x 128 tiles with the K axis split: 512 x 384 x 4104"""
+    g = Graph()
+    rng = np.random.default_rng(81)
+    a = g.input([512, 4104], DType.F16)
+    w = g.constant([384, 4104], _f16(rng, 384, 4104, scale=0.05))
+    g.output(g.linear(a, w))
+    return g, 0, [_f16(rng, 512, 4104)], None
