@@ -1121,3 +1121,19 @@ def f16_matmul_tall_tiles_split_k():
     w = g.constant([384, 4104], _f16(rng, 384, 4104, scale=0.05))
     g.output(g.linear(a, w))
     return g, 0, [_f16(rng, 512, 4104)], None
+
+
+@case
+def matmul_narrow_output_f32():
+    """outputs at most 64 wide with many rows (64 x 64 tiles whatever the tile count): short K (slices of 16) and
+    long K (slices of 64), ragged rows, columns and K"""
+    g = Graph()
+    rng = np.random.default_rng(90)
+    a = g.input([32, 1100, 50])
+    b = g.input([32, 50, 40])
+    c = g.input([16, 2100, 2060])
+    d = g.input([16, 2060, 24])
+    g.output_all([g.batched_mat_mul(a, b), g.batched_mat_mul(c, d)])
+    return g, 0, [rng.standard_normal((32, 1100, 50)).astype(np.float32), rng.standard_normal((32, 50, 40)).astype(np.float32),
+                  (rng.standard_normal((16, 2100, 2060)) * 0.05).astype(np.float32),
+                  rng.standard_normal((16, 2060, 24)).astype(np.float32)], None
