@@ -188,10 +188,23 @@ struct GemmStore {
     const float *addend;  // optional epilogue operand (null = none), with its own strides
     long long dm, dn;
     int relu;
-    __device__ __forceinline__ void prepare(int, int) {}
-    __device__ __forceinline__ void store(int m, int n, int, float v) const {
+    // what `prepare` derives for the two columns this lane owns
+    const float *d_col[2];  // addend at (row 0, column), or null
+    float d_bias[2];        // its value when the addend does not depend on the row (a bias): loaded once
+    bool row_invariant;
+
+    __device__ __forceinline__ void prepare(int col0, int col1) {
+        const int cols[2] = {col0, col1};
+        row_invariant = addend != nullptr && dm == 0;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            d_col[j] = addend != nullptr && cols[j] < N ? addend + (long long) cols[j] * dn : nullptr;
+            d_bias[j] = row_invariant && d_col[j] ? *d_col[j] : 0.0f;
+        }
+    }
+    __device__ __forceinline__ void store(int m, int n, int j, float v) const {
         if (m < M && n < N) {
-            if (addend) v += addend[(long long) m * dm + (long long) n * dn];
+            if (addend) v += row_invariant ? d_bias[j] : d_col[j][(long long) m * dm];
             if (relu) v = fmaxf(v, 0.0f);
             p[(long long) m * sm + (long long) n * sn] = v;
         }
@@ -259,32 +272,19 @@ __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int k_begin
             la.fetch(k0 + BK);
             lb.fetch(k0 + BK);
         }
-        // the operands of step kk + 2 are read from LDS before the MFMAs of step kk are issued
-        auto read_step = [&](int kk, float (&a)[MI], float (&b)[NI]) {
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
             const int kr = kk + (lane >> 5), c = lane & 31;
+            float a[MI], b[NI];
 #pragma unroll
             for (int i = 0; i < MI; i++) a[i] = As[kr][wm * 32 * MI + 32 * i + c];
 #pragma unroll
             for (int j = 0; j < NI; j++) b[j] = Bs[kr][wn * 32 * NI + 32 * j + c];
-        };
-        float a[MI], b[NI];
-        read_step(0, a, b);
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            float na[MI], nb[NI];
-            if (kk + 2 < BK) read_step(kk + 2, na, nb);
-            __builtin_amdgcn_sched_barrier(0);  // keep the reads in front of the MFMAs
 #pragma unroll
             for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < NI; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
-            if (kk + 2 < BK) {
-#pragma unroll
-                for (int i = 0; i < MI; i++) a[i] = na[i];
-#pragma unroll
-                for (int j = 0; j < NI; j++) b[j] = nb[j];
-            }
         }
     }
 
@@ -330,9 +330,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p, int k_c
     // the epilogue of a split launch is applied by the pass that sums the partial products
     GemmStore s = gridDim.z > 1
         ? GemmStore{(float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n, p.n, 1, p.m, p.n,
-                    nullptr, 0, 0, 0}
+                    nullptr, 0, 0, 0, {nullptr, nullptr}, {0.0f, 0.0f}, false}
         : GemmStore{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n,
-                    p.addend ? (const float *) p.addend + bz * p.d_sb : nullptr, p.d_sm, p.d_sn, p.relu};
+                    p.addend ? (const float *) p.addend + bz * p.d_sb : nullptr, p.d_sm, p.d_sn, p.relu,
+                    {nullptr, nullptr}, {0.0f, 0.0f}, false};
     mfma_tile_loop<TI, TI>(la, lb, s, k_begin, k_end, m0, n0);
 }
 
@@ -481,45 +482,24 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         stage();
         __syncthreads();
         if (c0 + CB < C) fetch(c0 + CB);
-        // The operands of step kk + 2 are read from LDS before the MFMAs of step kk are issued, so that the LDS
-        // latency runs under the matrix instructions instead of in front of them.
-        auto read_step = [&](int kk, float &a0, float &a1, float (&b)[NJ]) {
-            // taps of k = kk (lower half of the wave) and k = kk + 1 (upper half); all compile-time after unrolling
+#pragma unroll
+        for (int kk = 0; kk < KS; kk += 2) {
+            // taps of k = kk (lower half of the wave) and k = kk + 1 (upper half); all compile-time
             const int ca = kk / (KH * KW), fya = (kk / KW) % KH, fxa = kk % KW;
             const int cb = (kk + 1) / (KH * KW), fyb = ((kk + 1) / KW) % KH, fxb = (kk + 1) % KW;
             const int off_a = ca * gplane + fya * W + fxa, off_b = cb * gplane + fyb * W + fxb;
             const int koff = half ? off_b : off_a;
-            a0 = As[kk + half][wm * 64 + c32];
-            a1 = As[kk + half][wm * 64 + 32 + c32];
+            const float a0 = As[kk + half][wm * 64 + c32], a1 = As[kk + half][wm * 64 + 32 + c32];
+            float b[NJ];
 #pragma unroll
-            for (int j = 0; j < NJ; j++) b[j] = Bs[lane_base[j] + koff];
-        };
-        // taps outside the image are masked when the value is consumed, not when it is read, so that nothing
-        // waits for the LDS in front of the MFMAs
-        auto mask_step = [&](int kk, float (&b)[NJ]) {
-#pragma unroll
-            for (int j = 0; j < NJ; j++) b[j] = pair_ok[j][kk % KW] ? b[j] : 0.0f;
-        };
-        float a0, a1, b[NJ];
-        read_step(0, a0, a1, b);
-        mask_step(0, b);
-#pragma unroll
-        for (int kk = 0; kk < KS; kk += 2) {
-            float na0 = 0.0f, na1 = 0.0f, nb[NJ];
-            if (kk + 2 < KS) read_step(kk + 2, na0, na1, nb);
-            __builtin_amdgcn_sched_barrier(0);  // keep the reads in front of the MFMAs
+            for (int j = 0; j < NJ; j++) {
+                b[j] = Bs[lane_base[j] + koff];
+                b[j] = pair_ok[j][fxa] ? b[j] : 0.0f;
+            }
 #pragma unroll
             for (int j = 0; j < NJ; j++) acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b[j], acc[0][j], 0, 0, 0);
 #pragma unroll
             for (int j = 0; j < NJ; j++) acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b[j], acc[1][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (kk + 2 < KS) {
-                a0 = na0;
-                a1 = na1;
-#pragma unroll
-                for (int j = 0; j < NJ; j++) b[j] = nb[j];
-                mask_step(kk + 2, b);
-            }
         }
     }
 
