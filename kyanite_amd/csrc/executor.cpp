@@ -50,6 +50,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     if (!plan_only) HipDevice::check(device);
     PlannerOptions options;
     options.preserve_inputs = preserve_inputs;
+    if (const char *e = getenv("KNHIP_FUSE_ATTENTION")) options.fuse_attention = atoi(e) != 0;
     plan_ = plan_graph(graph, batch_size, options);
     for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
     if (plan_only) return;
@@ -74,7 +75,12 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
         Step &step = plan_.steps[si];
         Launch &l = launches_[si];
         for (auto &op : step.operands) l.ptrs.push_back(arena_ + plan_.resolve(op.tensor.ptr));
-        if (step.kind == StepKind::MatMul) {
+        if (step.kind == StepKind::MatMul && step.attention) {
+            step.attn.q = (const float *) l.ptrs[0];
+            step.attn.k = (const float *) l.ptrs[1];
+            step.attn.v = (const float *) l.ptrs[2];
+            step.attn.o = (float *) l.ptrs[3];
+        } else if (step.kind == StepKind::MatMul) {
             step.gemm.a = l.ptrs[0];
             step.gemm.b = l.ptrs[1];
             step.gemm.c = l.ptrs[2];
@@ -177,6 +183,10 @@ void HipExecutor::launch_step(size_t index, hipEvent_t start, hipEvent_t stop) {
     if (start) hip_check(hipEventRecord(start, stream_), "hipEventRecord");
     switch (step.kind) {
         case StepKind::MatMul:
+            if (step.attention) {
+                hip_check((hipError_t) launch_attention_f32(step.attn, stream_), "attention launch");
+                break;
+            }
             hip_check((hipError_t) (step.gemm_f16 ? launch_gemm_f16(step.gemm, stream_) : launch_gemm_f32(step.gemm, stream_)),
                       "matmul launch");
             break;

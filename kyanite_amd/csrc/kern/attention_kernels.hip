@@ -1,0 +1,196 @@
+// Fused attention in f32 on the CDNA4 matrix cores: O = softmax(scale * Q K^T) V without the score matrix ever
+// leaving the compute unit. It replaces the three launches that the reference plans for this chain (batched matmul,
+// softmax, batched matmul: kn-cuda-eval/src/planner.rs:606-648 and :418-476), which move the [Lq, Lk] scores through
+// memory four times.
+//
+// A workgroup of 4 waves owns 128 queries of one batch entry, a wave 32 of them, and walks the keys in blocks of 64
+// that sit in LDS (K as [key][k], V as [key][dim], zero padded). Everything is computed transposed, keys (then dims)
+// along the rows and queries along the columns of the 32 x 32 MFMA tiles:
+//   S^T = K Q^T      A operand: a row of K from LDS, B operand: Q, held in registers for the whole kernel
+//   O^T += V^T P^T   A operand: a column of V from LDS, B operand: P^T
+// In this orientation a lane owns one query (column l % 32), so the softmax statistics of a row of the scores are
+// per-lane values (plus one exchange between the two halves of the wave), and the accumulator registers of S^T are,
+// as they are, B operands of the second product: register v of half h holds key 8 (v / 4) + 4 h + v % 4 of the
+// tile, and the sum over keys may run in any order, so step v of the second product simply takes that key from V.
+// The softmax is the usual running one: a maximum and a sum per query, the output rescaled when the maximum moves.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "../mfma_kernels.h"
+
+namespace kn {
+
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int THREADS = 256;  // 4 waves
+constexpr int BQ = 128;       // queries per workgroup
+constexpr int BKEYS = 64;     // keys per block
+
+// DK: width of Q and K (a multiple of 8); DVT: 32-wide tiles that cover the width of V
+template <int DK, int DVT>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) void attention_f32_kernel(AttentionParams p) {
+    constexpr int DV = 32 * DVT, KS = DK + 4, VS = DV + 4, HALF = DK / 2;  // row strides that spread the LDS banks
+    static_assert(DK % 8 == 0 && BKEYS * 4 == THREADS, "unsupported shape");
+    __shared__ __attribute__((aligned(16))) float Ks[BKEYS][KS];
+    __shared__ __attribute__((aligned(16))) float Vs[BKEYS][VS];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 31, h = lane >> 5;
+    const int bz = blockIdx.y;
+    const int query = blockIdx.x * BQ + wave * 32 + c;
+    const float *kp = p.k + bz * p.k_sb, *vp = p.v + bz * p.v_sb;
+
+    // Q^T operand: lane (query c, half h) holds k = h * HALF + t for step t, pre-multiplied by scale * log2(e) so
+    // that the exponentials are plain exp2
+    float qf[HALF];
+    {
+        const float factor = p.scale * 1.44269504088896340736f;
+        const float *qp = p.q + bz * p.q_sb + (long long) query * p.q_sm;
+#pragma unroll
+        for (int t = 0; t < HALF; t++) qf[t] = query < p.lq ? qp[(long long) (h * HALF + t) * p.q_sk] * factor : 0.0f;
+    }
+
+    // Global -> register -> LDS: thread t moves elements t % 4, t % 4 + 4, ... of key t / 4 of the block, so that
+    // one 32 bit offset per thread (and a wave-uniform base per step) addresses all of them. Strides are not
+    // negative (the host checks).
+    constexpr int K_PER_THREAD = DK / 4, V_PER_THREAD = DV / 4;
+    const int my_key = threadIdx.x >> 2, sub = threadIdx.x & 3;
+    const unsigned koff = (unsigned) (my_key * p.k_sn + sub * p.k_sk), voff = (unsigned) (my_key * p.v_sk + sub * p.v_sn);
+    float kreg[K_PER_THREAD], vreg[V_PER_THREAD];
+    auto fetch = [&](int key0) {
+        const float *kb = kp + (long long) key0 * p.k_sn, *vb = vp + (long long) key0 * p.v_sk;
+        const bool valid = key0 + my_key < p.lk;
+#pragma unroll
+        for (int i = 0; i < K_PER_THREAD; i++) kreg[i] = valid ? (kb + (long long) 4 * i * p.k_sk)[koff] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < V_PER_THREAD; i++)
+            vreg[i] = valid && 4 * i + sub < p.dv ? (vb + (long long) 4 * i * p.v_sn)[voff] : 0.0f;
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < K_PER_THREAD; i++) Ks[my_key][4 * i + sub] = kreg[i];
+#pragma unroll
+        for (int i = 0; i < V_PER_THREAD; i++) Vs[my_key][4 * i + sub] = vreg[i];
+    };
+
+    floatx16 oacc[DVT];
+#pragma unroll
+    for (int t = 0; t < DVT; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) oacc[t][v] = 0.0f;
+    float row_max = -INFINITY, row_sum = 0.0f;  // row_sum: this half's share of the keys only
+
+    fetch(0);
+    for (int key0 = 0; key0 < p.lk; key0 += BKEYS) {
+        stage();
+        __syncthreads();
+        if (key0 + BKEYS < p.lk) fetch(key0 + BKEYS);
+
+        // scores of 2 x 32 keys against the wave's 32 queries
+        floatx16 st[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) st[j][v] = 0.0f;
+#pragma unroll
+        for (int t4 = 0; t4 < HALF / 4; t4++) {
+            floatx4 a[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) a[j] = *(const floatx4 *) &Ks[32 * j + c][h * HALF + 4 * t4];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    st[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][u], qf[4 * t4 + u], st[j], 0, 0, 0);
+        }
+        if (key0 + BKEYS > p.lk) {
+            // keys past the end take no part
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    if (key0 + 32 * j + 8 * (v >> 2) + 4 * h + (v & 3) >= p.lk) st[j][v] = -INFINITY;
+        }
+
+        float block_max = st[0][0];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) block_max = fmaxf(block_max, st[j][v]);
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
+        const float new_max = fmaxf(row_max, block_max);
+        const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);  // 0 for the first block
+        row_max = new_max;
+        float block_sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                st[j][v] = __builtin_amdgcn_exp2f(st[j][v] - new_max);
+                block_sum += st[j][v];
+            }
+        row_sum = row_sum * alpha + block_sum;
+#pragma unroll
+        for (int t = 0; t < DVT; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) oacc[t][v] *= alpha;
+
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int s = 0; s < 16; s++) {
+                const int key = 32 * j + 8 * (s >> 2) + 4 * h + (s & 3);
+#pragma unroll
+                for (int t = 0; t < DVT; t++)
+                    oacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[key][32 * t + c], st[j][s], oacc[t], 0, 0, 0);
+            }
+        __syncthreads();  // the block has been consumed by every wave
+    }
+
+    row_sum += __shfl_xor(row_sum, 32);
+    if (query < p.lq) {
+        const float inv = 1.0f / row_sum;
+        float *op = p.o + bz * p.o_sb + (long long) query * p.o_sm;
+#pragma unroll
+        for (int t = 0; t < DVT; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int d = 32 * t + 8 * (v >> 2) + 4 * h + (v & 3);
+                if (d < p.dv) op[(long long) d * p.o_sn] = oacc[t][v] * inv;
+            }
+    }
+}
+
+}  // namespace
+
+bool attention_supported(int dk, int dv) {
+    return (dk == 32 || dk == 40 || dk == 64) && dv >= 1 && dv <= 64;
+}
+
+int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream) {
+    if (p.batch <= 0 || p.lq <= 0 || p.dv <= 0) return 0;
+    if (!attention_supported(p.dk, p.dv) || p.lk <= 0 || p.batch > 65535) return (int) hipErrorInvalidValue;
+    const dim3 grid((unsigned) ((p.lq + BQ - 1) / BQ), (unsigned) p.batch), block(THREADS);
+    const bool wide = p.dv > 32;
+    switch (p.dk) {
+        case 32:
+            if (wide) hipLaunchKernelGGL((attention_f32_kernel<32, 2>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((attention_f32_kernel<32, 1>), grid, block, 0, stream, p);
+            break;
+        case 40:
+            if (wide) hipLaunchKernelGGL((attention_f32_kernel<40, 2>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((attention_f32_kernel<40, 1>), grid, block, 0, stream, p);
+            break;
+        default:
+            if (wide) hipLaunchKernelGGL((attention_f32_kernel<64, 2>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((attention_f32_kernel<64, 1>), grid, block, 0, stream, p);
+            break;
+    }
+    return (int) hipGetLastError();
+}
+
+}  // namespace kn

@@ -92,8 +92,20 @@ struct Loader {
     }
 };
 
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) {
-    const int id = blockIdx.x;
+// Tiles are numbered in bands of 8 tile rows, column by column within a band, so 8 k consecutive numbers are a patch
+// of 8 x k tiles. Workgroups are handed to the 8 XCDs (each with its own L2) in turn, workgroup i to XCD i % 8;
+// the renumbering below gives every XCD runs of `xcd_chunk` consecutive tile numbers (as many as it runs at a time),
+// so that the workgroups sharing an L2 cover one compact patch and find each other's operand tiles there.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_chunk, int *tm, int *tn) {
+    int id = blockIdx.x;
+    if (xcd_chunk > 0) {
+        const int per_round = 8 * xcd_chunk;
+        const int full = (int) (gridDim.x / per_round) * per_round;  // the tail keeps its numbers
+        if (id < full) {
+            const int xcd = id & 7, local = id >> 3;
+            id = ((local / xcd_chunk) * 8 + xcd) * xcd_chunk + local % xcd_chunk;
+        }
+    }
     const int group_rows = 8;
     const int per_group = group_rows * tiles_n;
     const int g = id / per_group, in_g = id - g * per_group;
@@ -107,14 +119,14 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
 // from L2 per flop. BK: depth of a K slice; NBUF: LDS buffers per operand (2 = double buffered, one barrier per
 // slice; 1 = two barriers per slice)
 template <int A_MODE, int B_MODE, int TI, int BK, int NBUF, int WM>
-__global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_chunk) {
+__global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_chunk, int xcd_chunk) {
     constexpr int TM = 32 * TI * WM, TN = 64 * TI, LDS_K = BK + 8, THREADS = 128 * WM;
     __shared__ __attribute__((aligned(16))) half_t As[NBUF][TM][LDS_K];
     __shared__ __attribute__((aligned(16))) half_t Bs[NBUF][TN][LDS_K];
 
     const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    tile_of_block(tiles_m, tiles_n, xcd_chunk, &tm, &tn);
     const int bz = blockIdx.y;
     const int m0 = tm * TM, n0 = tn * TN;
     // split K: workgroup z of gridDim.z multiplies its own range of k and stores an f32 partial product
@@ -212,21 +224,21 @@ int pick_mode(const void *ptr, long long so, long long sk, int outer_size, int k
 }
 
 template <int A_MODE, int TI, int BK, int NBUF, int WM>
-void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
+void launch_b(int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc, int xc) {
     const dim3 block(128 * WM);
     switch (b_mode) {
-        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc); break;
-        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc); break;
-        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc); break;
+        case VecOuter: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecOuter, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc, xc); break;
+        case VecK: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, VecK, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc, xc); break;
+        default: hipLaunchKernelGGL((gemm_f16_kernel<A_MODE, Scalar, TI, BK, NBUF, WM>), grid, block, 0, stream, p, kc, xc); break;
     }
 }
 
 template <int TI, int BK, int NBUF, int WM>
-void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc) {
+void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmParams &p, int kc, int xc) {
     switch (a_mode) {
-        case VecOuter: launch_b<VecOuter, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc); break;
-        case VecK: launch_b<VecK, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc); break;
-        default: launch_b<Scalar, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc); break;
+        case VecOuter: launch_b<VecOuter, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc, xc); break;
+        case VecK: launch_b<VecK, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc, xc); break;
+        default: launch_b<Scalar, TI, BK, NBUF, WM>(b_mode, grid, stream, p, kc, xc); break;
     }
 }
 
@@ -246,9 +258,12 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     // Measured on 128 x 128 tiles (TFLOP/s at 4096^3 / 8192^3): BK 64 single buffered 594 / 757, BK 64 double
     // buffered 643 / 718, BK 128 single buffered 672 / 744. All of them sit at the rate at which the L2 can feed
     // the compute units at this tile size (64 flop per byte fetched from L2, about 12 TB/s -> 770 TFLOP/s).
-    if (lp.small_tile) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
-    else if (lp.tall_tile) launch_a<2, 64, 1, 4>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
-    else launch_a<2, 128, 1, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    // workgroups an XCD (32 compute units) runs at a time: 1 per compute unit for the tall tiles, else 2
+    static const int xc_env = getenv("KNHIP_XCD_CHUNK") ? atoi(getenv("KNHIP_XCD_CHUNK")) : -1;
+    const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile ? 32 : 64);
+    if (lp.small_tile) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
+    else if (lp.tall_tile) launch_a<2, 64, 1, 4>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
+    else launch_a<2, 128, 1, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     int e = (int) hipGetLastError();
     if (e == 0 && lp.split_k > 1) e = launch_gemm_reduce_partials(p, lp.split_k, true, stream);
     return e;

@@ -60,7 +60,26 @@ struct ConvParams {
     int relu;
 };
 
-// Both return a hipError_t value (0 = success).
+// O[b] = softmax(scale * Q[b] K[b]^T) V[b] with the softmax along the keys; Q is [batch, lq, dk], K [batch, lk, dk],
+// V [batch, lk, dv], O [batch, lq, dv], all f32 with arbitrary element strides (batch, row, column in that order;
+// zero batch stride = broadcast operand).
+struct AttentionParams {
+    const float *q;
+    const float *k;
+    const float *v;
+    float *o;
+    int batch, lq, lk, dk, dv;
+    long long q_sb, q_sm, q_sk;
+    long long k_sb, k_sn, k_sk;  // k_sn: between keys, k_sk: along dk
+    long long v_sb, v_sk, v_sn;  // v_sk: between keys, v_sn: along dv
+    long long o_sb, o_sm, o_sn;
+    float scale;
+};
+// widths the fused kernel is built for; other chains run as matmul, softmax, matmul
+bool attention_supported(int dk, int dv);
+
+// All return a hipError_t value (0 = success).
+int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream);
 int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
 // f16 operands and result, f32 accumulation, one rounding (to nearest even) at the store
 int launch_gemm_f16(const GemmParams &p, ihipStream_t *stream);

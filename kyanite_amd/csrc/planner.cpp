@@ -1,5 +1,6 @@
 #include "planner.h"
 
+#include <cmath>
 #include <map>
 
 namespace kn {
@@ -13,7 +14,9 @@ std::string Step::str() const {
     std::ostringstream ss;
     ss << step_kind_name(kind) << " value=" << debug_value;
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
-    if (kind == StepKind::MatMul)
+    if (kind == StepKind::MatMul && attention)
+        ss << " attention f32 b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
+    else if (kind == StepKind::MatMul)
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm.relu ? " relu" : "");
     else if (kind == StepKind::Conv)
@@ -27,6 +30,7 @@ std::string Step::str() const {
 }
 
 double Step::flops() const {
+    if (kind == StepKind::MatMul && attention) return 2.0 * attn.batch * attn.lq * attn.lk * (attn.dk + attn.dv);
     if (kind == StepKind::MatMul) return 2.0 * gemm.batch * gemm.m * gemm.n * gemm.k;
     if (kind == StepKind::Conv)
         return 2.0 * conv.batch * conv.out_c * conv.out_h * conv.out_w * conv.in_c * conv.kernel_h * conv.kernel_w;
@@ -36,7 +40,7 @@ double Step::flops() const {
 double Step::bytes() const {
     double total = 0.0;
     for (size_t i = 0; i < operands.size(); i++) {
-        if (kind == StepKind::MatMul && i >= (gemm_has_addend ? 4u : 3u)) break;  // split-K scratch is not algorithmic traffic
+        if (kind == StepKind::MatMul && !attention && i >= (gemm_has_addend ? 4u : 3u)) break;  // split-K scratch is not algorithmic traffic
         auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
@@ -204,6 +208,11 @@ private:
             if (!fused.ok) return VT::missing(fused.need);
             if (fused.value) return VT::done(*fused.value);
         }
+        if (options.fuse_attention) {
+            auto fused = try_visit_fused_attention(value);
+            if (!fused.ok) return VT::missing(fused.need);
+            if (fused.value) return VT::done(*fused.value);
+        }
         if (options.fuse_matmul_epilogue) {
             auto fused = try_visit_fused_matmul(value);
             if (!fused.ok) return VT::missing(fused.need);
@@ -337,6 +346,14 @@ private:
         if (can_fuse(input) && permutation == std::vector<size_t>{1, 0, 2} && !map.count(input)) {
             const Operation &iop = graph[input].operation;
             if (iop.kind == OpKind::MatMul) {
+                if (options.fuse_attention) {
+                    auto fused = try_visit_fused_attention(input, false);
+                    if (!fused.ok) return VT::missing(fused.need);
+                    if (fused.value) {
+                        insert_mapping(input, *fused.value);
+                        return VT::done(fused.value->permute(permutation));
+                    }
+                }
                 // avoid a non-dense result for the typical attention matmul: write directly in [m, b, n] order
                 KN_TRY(mm, visit_matmul(input, iop.inputs[0], iop.inputs[1], false));
                 insert_mapping(input, mm);
@@ -550,6 +567,81 @@ private:
         auto viewed = result.value.view(final_shape);
         KN_ASSERT(viewed.has_value(), "a dense matmul result can always be viewed");
         return R::done(*viewed);
+    }
+
+    // matmul(softmax(matmul(q, kt) [* or / constant], last axis), v) in f32, every intermediate value hidden and used
+    // once: the scores stay on the compute unit instead of passing through memory between three launches
+    // (planner.rs:606-648, :418-476 plan them separately).
+    Visit<std::optional<PlanTensor>> try_visit_fused_attention(Value value, bool batch_first = true) {
+        using R = Visit<std::optional<PlanTensor>>;
+        const ValueInfo &info = graph[value];
+        if (info.operation.kind != OpKind::MatMul || info.dtype != DType::F32) return R::done(std::nullopt);
+        const Value probs = info.operation.inputs[0], v_v = info.operation.inputs[1];
+        const Operation &sop = graph[probs].operation;
+        if (sop.kind != OpKind::Softmax || sop.axis() != 2 || !can_fuse(probs) || map.count(probs)) return R::done(std::nullopt);
+        Value scores = sop.inputs[0];
+        if (!can_fuse(scores) || map.count(scores)) return R::done(std::nullopt);
+        float scale = 1.0f;
+        {
+            const Operation &op = graph[scores].operation;
+            if (op.kind == OpKind::Binary && (op.binary == BinaryOp::Mul || op.binary == BinaryOp::Div)) {
+                Value l = op.inputs[0], r = op.inputs[1];
+                auto rc = graph.as_single_const(r);
+                auto lc = op.binary == BinaryOp::Mul ? graph.as_single_const(l) : std::nullopt;
+                Value inner;
+                std::optional<DScalar> factor;
+                if (rc) { inner = l; factor = rc; }
+                else if (lc) { inner = r; factor = lc; }
+                else return R::done(std::nullopt);
+                if (factor->dtype != DType::F32 || !can_fuse(inner) || map.count(inner)) return R::done(std::nullopt);
+                scale = op.binary == BinaryOp::Mul ? (float) factor->f : 1.0f / (float) factor->f;
+                if (!(scale > 0.0f) || !std::isfinite(scale)) return R::done(std::nullopt);
+                scores = inner;
+            }
+        }
+        const Operation &mop = graph[scores].operation;
+        if (mop.kind != OpKind::MatMul || graph[scores].dtype != DType::F32) return R::done(std::nullopt);
+        const Value q_v = mop.inputs[0], kt_v = mop.inputs[1];
+        const ConcreteShape q_shape = graph[q_v].shape.eval(batch_size), kt_shape = graph[kt_v].shape.eval(batch_size);
+        const ConcreteShape v_shape = graph[v_v].shape.eval(batch_size);
+        const size_t b = q_shape[0], lq = q_shape[1], dk = q_shape[2], lk = kt_shape[2], dv = v_shape[2];
+        if (b == 0 || lq == 0 || lk == 0 || b > 65535 || lq > INT32_MAX || lk > INT32_MAX) return R::done(std::nullopt);
+        if (dk > 1024 || dv > 1024 || !attention_supported((int) dk, (int) dv)) return R::done(std::nullopt);
+
+        auto q = visit(q_v);
+        if (!q.ok) return R::missing(q.need);
+        auto kt = visit(kt_v);
+        if (!kt.ok) return R::missing(kt.need);
+        auto v = visit(v_v);
+        if (!v.ok) return R::missing(v.need);
+        // the kernel addresses a block of 64 keys with 32 bit offsets from the block's base
+        auto fits = [](const PlanTensor &t) {
+            for (size_t a = 1; a < 3; a++) {
+                const long long s = t.shape.strides()[a];
+                if (s < 0 || s > (1ll << 20)) return false;
+            }
+            return true;
+        };
+        if (!fits(kt.value) || !fits(v.value)) return R::done(std::nullopt);
+
+        PlanTensor result = batch_first ? alloc_tensor_shared({b, lq, dv}, DType::F32)
+                                        : alloc_tensor_shared({lq, b, dv}, DType::F32).permute({1, 0, 2});
+        Step step;
+        step.kind = StepKind::MatMul;
+        step.attention = true;
+        AttentionParams &a = step.attn;
+        a.batch = (int) b; a.lq = (int) lq; a.lk = (int) lk; a.dk = (int) dk; a.dv = (int) dv;
+        a.scale = scale;
+        const auto &qs = q.value.shape.strides(), &ks = kt.value.shape.strides(), &vs = v.value.shape.strides();
+        const auto &os = result.shape.strides();
+        a.q_sb = qs[0]; a.q_sm = qs[1]; a.q_sk = qs[2];
+        a.k_sb = ks[0]; a.k_sk = ks[1]; a.k_sn = ks[2];  // the operand is K^T: [b, dk, lk]
+        a.v_sb = vs[0]; a.v_sk = vs[1]; a.v_sn = vs[2];
+        a.o_sb = os[0]; a.o_sm = os[1]; a.o_sn = os[2];
+        step.operands = {{q.value, OperandKind::In}, {kt.value, OperandKind::In}, {v.value, OperandKind::In},
+                         {result, OperandKind::Out}};
+        push(std::move(step), value);
+        return R::done(result);
     }
 
     VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first,

@@ -37,6 +37,9 @@ struct Step {
     GemmParams gemm{};
     bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
     bool gemm_has_addend = false;  // operand 3 is the tensor added in the epilogue
+    // a MatMul step that is a whole softmax(scale * Q K^T) V chain in one launch; operands Q, K, V, O
+    bool attention = false;
+    AttentionParams attn{};
     ConvParams conv{};
     bool conv_has_bias = false, conv_has_res = false;
 
@@ -82,6 +85,7 @@ struct PlannerOptions {
     bool compile = true;          // compile the generated kernels (can be switched off to inspect the plan only)
     bool fuse_row_epilogue = true;  // fold elementwise consumers of a layernorm / softmax into the row kernel
     bool fuse_matmul_epilogue = true;  // fold `+ d` and `max(., 0)` after a matmul into the matmul's store
+    bool fuse_attention = true;  // matmul, softmax, matmul chains in f32 run as one launch
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
 };

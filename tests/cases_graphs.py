@@ -990,7 +990,7 @@ def config_llama_f32_small():
 @case
 def config_unet_block_small():
     from kyanite_amd.configs import build_unet_block
-    g, make_inputs, _ = build_unet_block(seed=2, batch=2, channels=32, size=8, groups=4, heads=2, time_dim=48, ctx_len=5,
+    g, make_inputs, _ = build_unet_block(seed=2, batch=2, channels=64, size=8, groups=4, heads=2, time_dim=48, ctx_len=5,
                                          ctx_dim=24)
     return g, 0, make_inputs(), None
 
@@ -1137,3 +1137,74 @@ def matmul_narrow_output_f32():
     return g, 0, [rng.standard_normal((32, 1100, 50)).astype(np.float32), rng.standard_normal((32, 50, 40)).astype(np.float32),
                   (rng.standard_normal((16, 2100, 2060)) * 0.05).astype(np.float32),
                   rng.standard_normal((16, 2060, 24)).astype(np.float32)], None
+
+
+def _attention_case(seed, b, lq, lk, dk, dv, scale_op, layout):
+    """softmax(scale * Q K^T) V; `layout` picks how the operands reach the products: 'dense' [b, rows, width]
+    inputs with K permuted, 'heads' [rows, b, width] inputs permuted like an attention layer does (strided
+    operands, result permuted back), 'v_transposed' V stored [b, dv, lk]"""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    if layout == "heads":
+        q_in, k_in, v_in = g.input([lq, b, dk]), g.input([lk, b, dk]), g.input([lk, b, dv])
+        q, kt, v = g.permute(q_in, [1, 0, 2]), g.permute(k_in, [1, 2, 0]), g.permute(v_in, [1, 0, 2])
+        shapes = [(lq, b, dk), (lk, b, dk), (lk, b, dv)]
+    else:
+        q, k_in = g.input([b, lq, dk]), g.input([b, lk, dk])
+        kt = g.permute(k_in, [0, 2, 1])
+        if layout == "v_transposed":
+            v = g.permute(g.input([b, dv, lk]), [0, 2, 1])
+            shapes = [(b, lq, dk), (b, lk, dk), (b, dv, lk)]
+        else:
+            v = g.input([b, lk, dv])
+            shapes = [(b, lq, dk), (b, lk, dk), (b, lk, dv)]
+    scores = g.batched_mat_mul(q, kt)
+    if scale_op == "mul":
+        scores = g.mul(scores, g.scalar(1.0 / np.sqrt(dk)))
+    elif scale_op == "mul_left":
+        scores = g.mul(g.scalar(1.0 / np.sqrt(dk)), scores)
+    elif scale_op == "div":
+        scores = g.binary(BinaryOp.DIV, scores, g.scalar(float(np.sqrt(dk))))
+    out = g.batched_mat_mul(g.softmax(scores, 2), v)
+    if layout == "heads":
+        out = g.view(g.permute(out, [1, 0, 2]), [lq, b * dv])
+    g.output(out)
+    return g, 0, [rng.standard_normal(shape).astype(np.float32) for shape in shapes], None
+
+
+@case
+def attention_fused_ragged():
+    """one launch for the whole chain; 200 queries and 77 keys (partial blocks of both), width 40"""
+    return _attention_case(100, 3, 200, 77, 40, 40, "mul", "dense")
+
+
+@case
+def attention_fused_heads_layout():
+    """operands that are permuted views (row strides b * width), result written in [lq, b, dv] order; width 64"""
+    return _attention_case(101, 4, 128, 256, 64, 64, "div", "heads")
+
+
+@case
+def attention_fused_narrow_v():
+    """width 32, V narrower than one tile and stored transposed, no scale, the scale on the left"""
+    a = _attention_case(102, 2, 70, 130, 32, 24, "none", "v_transposed")
+    return a
+
+
+@case
+def attention_fused_many_blocks():
+    """enough keys that the running maximum and sum are rescaled many times; large score range"""
+    g, b, inputs, _ = _attention_case(103, 2, 256, 1000, 40, 40, "mul_left", "dense")
+    inputs[0] *= 4.0
+    return g, b, inputs, None
+
+
+@case
+def attention_chain_not_fused():
+    """the scores are an output as well, so the chain has to stay three launches"""
+    g = Graph()
+    rng = np.random.default_rng(104)
+    q, k, v = g.input([2, 50, 40]), g.input([2, 60, 40]), g.input([2, 60, 40])
+    probs = g.softmax(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), 2)
+    g.output_all([g.batched_mat_mul(probs, v), probs])
+    return g, 0, [rng.standard_normal(s).astype(np.float32) for s in [(2, 50, 40), (2, 60, 40), (2, 60, 40)]], None

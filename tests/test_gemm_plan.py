@@ -57,3 +57,35 @@ def test_workspace_is_scratch_for_its_step_only():
     # algorithmic bytes of the step do not include the workspace
     flops, nbytes = ex.step_work(0)
     assert flops == 2 * 8 * 4096 * 4096 and nbytes == 4 * (8 * 4096 + 4096 * 4096 + 8 * 4096)
+
+
+def _attention_graph(dk, dv, dtype=DType.F32, extra_output=False, axis=2):
+    g = Graph()
+    q, k, v = g.input([2, 50, dk], dtype), g.input([2, 60, dk], dtype), g.input([2, 60, dv], dtype)
+    scores = g.mul(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), g.scalar(0.25, dtype))
+    probs = g.softmax(scores, axis)
+    g.output(g.batched_mat_mul(probs, v))
+    if extra_output:
+        g.output(probs)
+    return g
+
+
+def test_attention_chain_is_one_launch():
+    # matmul -> * constant -> softmax over the keys -> matmul in f32 at a supported width: one step, whose work is
+    # both products and whose bytes are Q, K, V and O only
+    ex = HipExecutor(0, _attention_graph(40, 40), 0, plan_only=True)
+    assert ex.step_kinds() == ["mat_mul"]
+    assert "attention" in ex.step_str(0) and "lq=50 lk=60 dk=40 dv=40" in ex.step_str(0)
+    flops, nbytes = ex.step_work(0)
+    assert flops == 2 * 2 * 50 * 60 * (40 + 40)
+    assert nbytes == 4 * 2 * (50 * 40 + 60 * 40 + 60 * 40 + 50 * 40)
+
+
+def test_attention_chain_stays_apart_when_it_must():
+    three = ["mat_mul", "softmax_op", "mat_mul"]
+    # the probabilities are needed elsewhere
+    assert HipExecutor(0, _attention_graph(40, 40, extra_output=True), 0, plan_only=True).step_kinds() == three
+    # a width the fused kernel is not built for, f16, a softmax over the queries
+    assert HipExecutor(0, _attention_graph(24, 40), 0, plan_only=True).step_kinds() == three
+    assert HipExecutor(0, _attention_graph(40, 40, DType.F16), 0, plan_only=True).step_kinds() == three
+    assert HipExecutor(0, _attention_graph(40, 40, axis=1), 0, plan_only=True).step_kinds() == three
