@@ -46,7 +46,11 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     const bool narrow = p.m <= 64 || p.n <= 64;
     // With a long K axis and too few tiles, 128 x 128 tiles split along K keep the higher arithmetic intensity
     // per byte fetched from L2 and still fill the chip.
-    const bool can_split = split_enabled && p.k >= 1024;
+    // A handful of tiles leaves the chip idle while every workgroup walks all of K at one slice per memory round
+    // trip, so there K is split from 256 on (154 x 320 x 768 in f32: 41 us unsplit).
+    const long long small_blocks = (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch;
+    const bool few_tiles = small_blocks < 64;
+    const bool can_split = split_enabled && (p.k >= 1024 || (few_tiles && p.k >= 256));
     lp.small_tile = narrow || (big_blocks < threshold && !(can_split && p.k >= 2048 && big_blocks < 256));
     // f16 with so few tiles that the K axis gets split anyway: 256 x 128 tiles (8 waves), which fetch a quarter
     // fewer bytes from L2 per flop and halve the partial products per split. Measured (us, 128 x 128 against
@@ -56,14 +60,14 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch;
     lp.tall_tile = f16 && !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8 && can_split &&
                    p.k >= 2048 && tall_blocks < tall_below;
-    long long blocks = lp.small_tile ? (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch : big_blocks;
+    long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile ? 64 : 128;
-    else lp.bk = lp.small_tile && p.k >= 2048 ? 64 : 16;
+    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < 512)) ? 64 : 16;
 
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
     if (can_split && blocks < split_below) {
-        const int min_chunk = f16 ? 512 : 256;  // K elements a split should at least cover
+        const int min_chunk = few_tiles ? 128 : (f16 ? 512 : 256);  // K elements a split should at least cover
         long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;
         if (s > 1) {

@@ -24,8 +24,9 @@ def test_no_split_when_the_tiles_fill_the_chip():
     for m, n, k in ((4096, 4096, 4096), (1024, 4672, 2048), (512, 11008, 4096)):
         assert plan(m, n, k)[0] == 0
     assert plan(512, 11008, 4096, dtype=DType.F16)[0] == 0
-    # short contractions never split, however few tiles there are
-    assert plan(8, 32, 16)[0] == 0 and plan(64, 64, 512)[0] == 0
+    # short contractions never split, however few tiles there are; from 256 on a handful of tiles does
+    assert plan(8, 32, 16)[0] == 0 and plan(64, 64, 200)[0] == 0
+    assert plan(64, 64, 512)[0] == 4 * 64 * 64 and plan(1024, 256, 512)[0] == 0
 
 
 def test_split_for_long_contractions_with_few_tiles():
