@@ -23,8 +23,8 @@ namespace kn {
 
 namespace {
 
-// BM x BN is the tile of the plane convolution kernel; the generic kernels take their tile (64 or 128 wide per
-// axis) from the loaders. LDS rows are padded by 4 floats: rows stay 16 byte aligned and successive k rows shift
+// BM x BN is the large tile of the convolution kernels; the generic kernels take their tile (64 or 128 wide per
+// axis) from the loaders, the plane kernel from its template arguments. LDS rows are padded by 4 floats: rows stay 16 byte aligned and successive k rows shift
 // by 4 banks.
 constexpr int BM = 128, BN = 128, THREADS = 256;
 
@@ -375,15 +375,17 @@ struct PlaneGeom {
     int n_vec;           // CB * G * plane_rows * W / 4
 };
 
-// NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64)
-template <int KH, int KW, int NJ>
+// NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64); MI: the same along
+// the output channels (2 -> 128 channels per tile, 1 -> 64)
+template <int KH, int KW, int NJ, int MI>
 __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, PlaneGeom g) {
     constexpr int TN = 64 * NJ;  // positions per tile
+    constexpr int BM = 64 * MI;  // output channels per tile
     constexpr int KS = CB * KH * KW;      // K slice
     constexpr int A_VEC = KS / 4;         // 128 bit loads per filter row and slice
-    constexpr int A_ITERS = BM * A_VEC / THREADS;
+    constexpr int A_ITERS = (BM * A_VEC + THREADS - 1) / THREADS;
     constexpr int A_STRIDE = BM + 5;      // odd, spreads the transposing stores over the banks
-    static_assert(KS % 4 == 0 && (BM * A_VEC) % THREADS == 0 && KS % 2 == 0, "slice shape");
+    static_assert(KS % 4 == 0 && KS % 2 == 0, "slice shape");
     __shared__ float As[KS][A_STRIDE];
     __shared__ __attribute__((aligned(16))) float Bs[PLANE_LDS];
 
@@ -427,8 +429,8 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 #pragma unroll
     for (int i = 0; i < A_ITERS; i++) {
         const int e = t + THREADS * i, row = e / A_VEC, q = e - row * A_VEC;
-        a_src[i] = (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
-        a_dst[i] = 4 * q * A_STRIDE + row;
+        a_src[i] = row < BM && (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
+        a_dst[i] = row < BM ? 4 * q * A_STRIDE + row : -1;
     }
     // ---- where this lane's output positions sit inside a plane, and which taps stay inside the image
     int lane_base[NJ];
@@ -460,16 +462,18 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         float *a_flat = &As[0][0];
 #pragma unroll
         for (int i = 0; i < A_ITERS; i++)
+            if ((BM * A_VEC) % THREADS == 0 || a_dst[i] >= 0) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) a_flat[a_dst[i] + j * A_STRIDE] = ra[i][j];
+                for (int j = 0; j < 4; j++) a_flat[a_dst[i] + j * A_STRIDE] = ra[i][j];
+            }
 #pragma unroll
         for (int i = 0; i < PLANE_MAX_VEC; i++)
             if (b_live[i]) *(floatx4 *) &Bs[PLANE_SLACK + 4 * (t + THREADS * i)] = rb[i];
     };
 
-    floatx16 acc[2][NJ];
+    floatx16 acc[MI][NJ];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < NJ; j++)
 #pragma unroll
@@ -489,17 +493,18 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             const int cb = (kk + 1) / (KH * KW), fyb = ((kk + 1) / KW) % KH, fxb = (kk + 1) % KW;
             const int off_a = ca * gplane + fya * W + fxa, off_b = cb * gplane + fyb * W + fxb;
             const int koff = half ? off_b : off_a;
-            const float a0 = As[kk + half][wm * 64 + c32], a1 = As[kk + half][wm * 64 + 32 + c32];
-            float b[NJ];
+            float a[MI], b[NJ];
+#pragma unroll
+            for (int i = 0; i < MI; i++) a[i] = As[kk + half][wm * 32 * MI + 32 * i + c32];
 #pragma unroll
             for (int j = 0; j < NJ; j++) {
                 b[j] = Bs[lane_base[j] + koff];
                 b[j] = pair_ok[j][fxa] ? b[j] : 0.0f;
             }
 #pragma unroll
-            for (int j = 0; j < NJ; j++) acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b[j], acc[0][j], 0, 0, 0);
+            for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int j = 0; j < NJ; j++) acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b[j], acc[1][j], 0, 0, 0);
+                for (int j = 0; j < NJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
     }
 
@@ -507,12 +512,12 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     const int col0 = n0 + wn * 32 * NJ + c32;
     s.prepare(col0, col0 + 32);
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+                const int row = m0 + wm * 32 * MI + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
                 s.store(row, col0 + 32 * j, j, acc[i][j][v]);
             }
 }
@@ -672,16 +677,32 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     if (positions <= 0 || p.out_c <= 0) return 0;
     const long long big_tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
     if (positions > 0x7fffffffll || big_tiles > 0x7fffffffll / 4) return (int) hipErrorInvalidValue;
+    // Plane kernel tiles (output channels x positions): 128 x 128 or 64 x 64, each wave owning 4 or 1 MFMA tiles of
+    // the result. The waves of all workgroups spread over 1024 SIMDs and the launch takes about as long as the
+    // busiest SIMD: rounds of waves x MFMA tiles per wave. The small tile costs a tenth more per MFMA tile (more LDS
+    // reads and staged planes per flop) but rounds the work off better; the smaller estimate wins. Measured (us,
+    // 128 x 128 / 64 x 64): 128 -> 128 channels on 8 x 8 images, batch 64 89 / 34, 256 94 / 55, 384 98 / 78,
+    // 512 102 / 108, 768 176 / 156, 1024 189 / 206; 320 -> 320 on 2 x 64 x 64 228 / 183; 1280 -> 1280 on
+    // 2 x 16 x 16 818 / 291. (128 x 64 tiles never won against both.)
     PlaneGeom geom;
-    static const int plane_wide_from = getenv("KNHIP_CONV_PLANE_WIDE_FROM") ? atoi(getenv("KNHIP_CONV_PLANE_WIDE_FROM")) : 512;
-    // 128 x 64 tiles until there are two 128 x 128 ones per compute unit. Measured on 128 -> 128 channels, 8 x 8
-    // images (us, narrow / wide): batch 64 55 / 89, 256 62 / 95, 512 105 / 103, 1024 208 / 187.
-    int tn = big_tiles >= plane_wide_from ? 128 : 64;
-    if (tn == 64 && !plane_geometry(p, tn, &geom)) tn = 128;  // images wider than 64 only fit the wide tile
-    if (plane_geometry(p, tn, &geom)) {
-        const long long tiles = ((positions + tn - 1) / tn) * ((p.out_c + BM - 1) / BM);
-        if (tn == 128) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2>), dim3((unsigned) tiles), dim3(THREADS), 0, stream, p, geom);
-        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1>), dim3((unsigned) tiles), dim3(THREADS), 0, stream, p, geom);
+    static const int variant_env = getenv("KNHIP_CONV_PLANE_VARIANT") ? atoi(getenv("KNHIP_CONV_PLANE_VARIANT")) : 0;
+    struct Variant { int bm, tn, id; double unit_cost; };
+    static const Variant variants[2] = {{128, 128, 22, 4 * 1.00}, {64, 64, 11, 1 * 1.10}};
+    const Variant *best = nullptr;
+    double best_cost = 0.0;
+    for (const Variant &v : variants) {
+        if (variant_env && variant_env != v.id) continue;
+        if (!plane_geometry(p, v.tn, &geom)) continue;
+        const long long tiles = ((positions + v.tn - 1) / v.tn) * ((p.out_c + v.bm - 1) / v.bm);
+        const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost;
+        if (!best || cost < best_cost) { best = &v; best_cost = cost; }
+    }
+    if (best) {
+        plane_geometry(p, best->tn, &geom);
+        const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
+        const dim3 grid((unsigned) tiles), block(THREADS);
+        if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2>), grid, block, 0, stream, p, geom);
+        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1>), grid, block, 0, stream, p, geom);
         return (int) hipGetLastError();
     }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
