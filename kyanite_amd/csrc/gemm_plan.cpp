@@ -63,7 +63,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile ? 64 : 128;
-    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < 512)) ? 64 : 16;
+    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
 
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
     if (can_split && blocks < split_below) {
