@@ -51,6 +51,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     PlannerOptions options;
     options.preserve_inputs = preserve_inputs;
     if (const char *e = getenv("KNHIP_FUSE_ATTENTION")) options.fuse_attention = atoi(e) != 0;
+    if (const char *e = getenv("KNHIP_GROUP_MATMULS")) options.group_matmuls = atoi(e) != 0;
     plan_ = plan_graph(graph, batch_size, options);
     for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
     if (plan_only) return;
@@ -80,6 +81,16 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             step.attn.k = (const float *) l.ptrs[1];
             step.attn.v = (const float *) l.ptrs[2];
             step.attn.o = (float *) l.ptrs[3];
+        } else if (step.kind == StepKind::MatMul && step.gemm.groups > 1) {
+            const size_t groups = (size_t) step.gemm.groups;
+            KN_ASSERT(l.ptrs.size() == 1 + 2 * groups);
+            step.gemm.a = l.ptrs[0];
+            for (size_t g = 0; g < groups; g++) {
+                step.gemm.b_group[g] = l.ptrs[1 + g];
+                step.gemm.c_group[g] = l.ptrs[1 + groups + g];
+            }
+            step.gemm.b = step.gemm.b_group[0];
+            step.gemm.c = step.gemm.c_group[0];
         } else if (step.kind == StepKind::MatMul) {
             step.gemm.a = l.ptrs[0];
             step.gemm.b = l.ptrs[1];

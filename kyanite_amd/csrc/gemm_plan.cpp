@@ -42,13 +42,14 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     static const int threshold_env = env_int("KNHIP_SMALL_TILE_BELOW", -1);
     const long long threshold = threshold_env >= 0 ? threshold_env : (f16 ? 256 : 512);
     static const int split_enabled = env_int("KNHIP_SPLIT_K", 1);
-    const long long big_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch;
+    const int groups = p.groups > 1 ? p.groups : 1;
+    const long long big_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch * groups;
     const bool narrow = p.m <= 64 || p.n <= 64;
     // With a long K axis and too few tiles, 128 x 128 tiles split along K keep the higher arithmetic intensity
     // per byte fetched from L2 and still fill the chip.
     // A handful of tiles leaves the chip idle while every workgroup walks all of K at one slice per memory round
     // trip, so there K is split from 256 on (154 x 320 x 768 in f32: 41 us unsplit).
-    const long long small_blocks = (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch;
+    const long long small_blocks = (long long) ((p.m + 63) / 64) * ((p.n + 63) / 64) * p.batch * groups;
     const bool few_tiles = small_blocks < 64;
     const bool can_split = split_enabled && (p.k >= 1024 || (few_tiles && p.k >= 256));
     lp.small_tile = narrow || (big_blocks < threshold && !(can_split && p.k >= 2048 && big_blocks < 256));
@@ -57,8 +58,8 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // 256 x 128): 512 x 4096 x 4096 43 / 38, 512 x 4096 x 11008 89 / 75; without a split they do not pay:
     // 512 x 11008 x 4096 82 / 87, 8192^3 1454 / 1439.
     static const int tall_below = env_int("KNHIP_F16_TALL_BELOW", 128);
-    const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch;
-    lp.tall_tile = f16 && !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8 && can_split &&
+    const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch * groups;
+    lp.tall_tile = f16 && groups == 1 && !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8 && can_split &&
                    p.k >= 2048 && tall_blocks < tall_below;
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
@@ -66,7 +67,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
 
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
-    if (can_split && blocks < split_below) {
+    if (can_split && blocks < split_below && groups == 1) {
         const int min_chunk = few_tiles ? 128 : (f16 ? 512 : 256);  // K elements a split should at least cover
         long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;
@@ -83,6 +84,18 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         }
     }
     return lp;
+}
+
+bool gemm_group_ok(const GemmParams &p, bool f16) {
+    if (p.groups < 2 || p.groups > GEMM_MAX_GROUPS || p.addend != nullptr || p.relu) return false;
+    auto mag = [](long long x) { return x < 0 ? -x : x; };
+    if (mag(p.c_sm) < mag(p.c_sn)) return false;  // the launch would swap the operands
+    // A grouped launch never splits K. Where even all products together leave the chip short of tiles, separate
+    // launches that split K are faster.
+    GemmParams wide = p;
+    wide.groups = 1;
+    wide.n = p.n * p.groups;
+    return plan_gemm_launch(wide, f16).split_k == 1;
 }
 
 }  // namespace kn

@@ -124,15 +124,20 @@ __global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_
     __shared__ __attribute__((aligned(16))) half_t As[NBUF][TM][LDS_K];
     __shared__ __attribute__((aligned(16))) half_t Bs[NBUF][TN][LDS_K];
 
+    // a grouped launch lines the tiles of its products up along n
     const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n, xcd_chunk, &tm, &tn);
+    tile_of_block(tiles_m, tiles_n * p.groups, xcd_chunk, &tm, &tn);
+    const int group = tn / tiles_n;
+    tn -= group * tiles_n;
+    const void *b_base = p.groups > 1 ? p.b_group[group] : p.b;
+    void *c_base = p.groups > 1 ? p.c_group[group] : p.c;
     const int bz = blockIdx.y;
     const int m0 = tm * TM, n0 = tn * TN;
     // split K: workgroup z of gridDim.z multiplies its own range of k and stores an f32 partial product
     const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
     Loader<A_MODE, TM, BK, THREADS> la(Operand{(const half_t *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
-    Loader<B_MODE, TN, BK, THREADS> lb(Operand{(const half_t *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
+    Loader<B_MODE, TN, BK, THREADS> lb(Operand{(const half_t *) b_base + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave >> 1, wn = wave & 1, c = lane & 31, half = lane >> 5;
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_
     }
 
     // accumulator layout of the 32x32 tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32
-    half_t *out = (half_t *) p.c + bz * p.c_sb;
+    half_t *out = (half_t *) c_base + bz * p.c_sb;
     float *partial = (float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n;
     const bool split = gridDim.z > 1;
     // the epilogue of a split launch is applied by the pass that sums the partial products
@@ -249,12 +254,18 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     const GemmLaunchPlan lp = plan_gemm_launch(params, true);
     const GemmParams &p = lp.p;
     const int t = lp.small_tile ? 64 : 128, t_m = lp.tall_tile ? 256 : t;
-    const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t - 1) / t);
+    const int groups = p.groups > 1 ? p.groups : 1;
+    if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
+    const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t - 1) / t) * groups;
     if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);
-    const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
+    int b_mode = pick_mode(groups > 1 ? p.b_group[0] : p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
+    for (int g = 1; g < groups; g++) {  // the loader that every operand of the group allows
+        const int mode = pick_mode(p.b_group[g], p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
+        if (mode != b_mode) b_mode = Scalar;
+    }
     // Measured on 128 x 128 tiles (TFLOP/s at 4096^3 / 8192^3): BK 64 single buffered 594 / 757, BK 64 double
     // buffered 643 / 718, BK 128 single buffered 672 / 744. All of them sit at the rate at which the L2 can feed
     // the compute units at this tile size (64 flop per byte fetched from L2, about 12 TB/s -> 770 TFLOP/s).

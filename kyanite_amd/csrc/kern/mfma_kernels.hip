@@ -318,20 +318,25 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
 template <int A_MODE, int B_MODE, int TI, int BK>
 __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p, int k_chunk) {
     constexpr int T = 64 * TI;
+    // a grouped launch lines the tiles of its products up along n
     const int tiles_m = (p.m + T - 1) / T, tiles_n = (p.n + T - 1) / T;
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    tile_of_block(tiles_m, tiles_n * p.groups, &tm, &tn);
+    const int group = tn / tiles_n;
+    tn -= group * tiles_n;
+    const void *b_base = p.groups > 1 ? p.b_group[group] : p.b;
+    void *c_base = p.groups > 1 ? p.c_group[group] : p.c;
     const int bz = blockIdx.y;
     const int m0 = tm * T, n0 = tn * T;
     // split K: workgroup z of gridDim.z multiplies its own range of k and stores an f32 partial product
     const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
     StridedLoader<A_MODE, T, BK> la(StridedOperand{(const float *) p.a + bz * p.a_sb, p.a_sm, p.a_sk, p.m, k_end}, m0);
-    StridedLoader<B_MODE, T, BK> lb(StridedOperand{(const float *) p.b + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
+    StridedLoader<B_MODE, T, BK> lb(StridedOperand{(const float *) b_base + bz * p.b_sb, p.b_sn, p.b_sk, p.n, k_end}, n0);
     // the epilogue of a split launch is applied by the pass that sums the partial products
     GemmStore s = gridDim.z > 1
         ? GemmStore{(float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n, p.n, 1, p.m, p.n,
                     nullptr, 0, 0, 0, {nullptr, nullptr}, {0.0f, 0.0f}, false}
-        : GemmStore{(float *) p.c + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n,
+        : GemmStore{(float *) c_base + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n,
                     p.addend ? (const float *) p.addend + bz * p.d_sb : nullptr, p.d_sm, p.d_sn, p.relu,
                     {nullptr, nullptr}, {0.0f, 0.0f}, false};
     mfma_tile_loop<TI, TI>(la, lb, s, k_begin, k_end, m0, n0);
@@ -658,12 +663,18 @@ int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
     const GemmLaunchPlan lp = plan_gemm_launch(params, false);
     const GemmParams &p = lp.p;
     const int t = lp.small_tile ? 64 : 128;
-    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t);
+    const int groups = p.groups > 1 ? p.groups : 1;
+    if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
+    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * groups;
     if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.a_sb, p.batch);
-    const int b_mode = pick_mode(p.b, p.b_sn, p.b_sk, p.b_sb, p.batch);
+    int b_mode = pick_mode(groups > 1 ? p.b_group[0] : p.b, p.b_sn, p.b_sk, p.b_sb, p.batch);
+    for (int g = 1; g < groups; g++) {  // the loader that every operand of the group allows
+        const int mode = pick_mode(p.b_group[g], p.b_sn, p.b_sk, p.b_sb, p.batch);
+        if (mode != b_mode) b_mode = Scalar;
+    }
     if (lp.small_tile && lp.bk == 64) launch_gemm_a<1, 64>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
     else if (lp.small_tile) launch_gemm_a<1, 16>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
     else launch_gemm_a<2, 16>(a_mode, b_mode, grid, stream, p, lp.k_chunk);

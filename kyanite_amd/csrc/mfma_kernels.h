@@ -11,6 +11,8 @@ namespace kn {
 
 // C[b, i, j] = sum_k A[b, i, k] * B[b, k, j]; element strides are arbitrary (zero batch stride = broadcast operand).
 // The element type (float or _Float16, the same for all three matrices) is fixed by the launch function.
+constexpr int GEMM_MAX_GROUPS = 4;
+
 struct GemmParams {
     const void *a;
     const void *b;
@@ -25,6 +27,12 @@ struct GemmParams {
     const void *addend = nullptr;
     long long d_sb = 0, d_sm = 0, d_sn = 0;
     int relu = 0;
+    // Grouped launch: `groups` (up to GEMM_MAX_GROUPS) products A * B_g = C_g that share A, all shapes and all
+    // strides, in one launch; b / c are then ignored in favour of b_group / c_group. Not combined with an addend
+    // or a split of the K axis.
+    int groups = 1;
+    const void *b_group[4] = {nullptr, nullptr, nullptr, nullptr};
+    void *c_group[4] = {nullptr, nullptr, nullptr, nullptr};
     // f32 scratch for partial products when the launch splits the K axis (`GemmLaunchPlan::workspace_bytes`
     // bytes, 256 byte aligned); may be null otherwise
     void *workspace = nullptr;
@@ -42,6 +50,8 @@ struct GemmLaunchPlan {
     size_t workspace_bytes;  // split_k * batch * m * n * 4 when split_k > 1, else 0
 };
 GemmLaunchPlan plan_gemm_launch(const GemmParams &p, bool f16);
+// whether `p.groups` products may share one launch: no operand swap, no K split, no epilogue
+bool gemm_group_ok(const GemmParams &p, bool f16);
 
 
 // out[n, ko, oy, ox] = act(sum_{c, fy, fx} in[n, c, oy*sy + fy - py, ox*sx + fx - px] * filter[ko, c, fy, fx]

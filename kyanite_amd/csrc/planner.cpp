@@ -1,5 +1,6 @@
 #include "planner.h"
 
+#include <algorithm>
 #include <cmath>
 #include <map>
 
@@ -16,9 +17,11 @@ std::string Step::str() const {
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
     if (kind == StepKind::MatMul && attention)
         ss << " attention f32 b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
-    else if (kind == StepKind::MatMul)
+    else if (kind == StepKind::MatMul) {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm.relu ? " relu" : "");
+        if (gemm.groups > 1) ss << " x" << gemm.groups << " grouped";
+    }
     else if (kind == StepKind::Conv)
         ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="
            << conv.kernel_h << "x" << conv.kernel_w << (conv_has_bias ? " +bias" : "") << (conv_has_res ? " +res" : "")
@@ -31,7 +34,7 @@ std::string Step::str() const {
 
 double Step::flops() const {
     if (kind == StepKind::MatMul && attention) return 2.0 * attn.batch * attn.lq * attn.lk * (attn.dk + attn.dv);
-    if (kind == StepKind::MatMul) return 2.0 * gemm.batch * gemm.m * gemm.n * gemm.k;
+    if (kind == StepKind::MatMul) return 2.0 * gemm.batch * gemm.m * gemm.n * gemm.k * (gemm.groups > 1 ? gemm.groups : 1);
     if (kind == StepKind::Conv)
         return 2.0 * conv.batch * conv.out_c * conv.out_h * conv.out_w * conv.in_c * conv.kernel_h * conv.kernel_w;
     return 0.0;
@@ -40,7 +43,7 @@ double Step::flops() const {
 double Step::bytes() const {
     double total = 0.0;
     for (size_t i = 0; i < operands.size(); i++) {
-        if (kind == StepKind::MatMul && !attention && i >= (gemm_has_addend ? 4u : 3u)) break;  // split-K scratch is not algorithmic traffic
+        if (kind == StepKind::MatMul && !attention && gemm.groups <= 1 && i >= (gemm_has_addend ? 4u : 3u)) break;  // split-K scratch is not algorithmic traffic
         auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
@@ -311,7 +314,14 @@ private:
                 return VT::done(result);
             }
             case OpKind::Conv: fail("Conv should have been handled by the conv fuser (only rank-4 f32 convolutions are supported)");
-            case OpKind::MatMul: return visit_matmul(value, op.inputs[0], op.inputs[1], true);
+            case OpKind::MatMul: {
+                if (options.group_matmuls) {
+                    auto grouped = try_visit_matmul_group(value);
+                    if (!grouped.ok) return VT::missing(grouped.need);
+                    if (grouped.value) return VT::done(*grouped.value);
+                }
+                return visit_matmul(value, op.inputs[0], op.inputs[1], true);
+            }
             case OpKind::Unary: case OpKind::Binary: return visit_fused_scalar(value);
             case OpKind::Softmax: case OpKind::Layernorm: {
                 KN_ASSERT(result_dtype == DType::F32 || result_dtype == DType::F16);
@@ -642,6 +652,121 @@ private:
                          {result, OperandKind::Out}};
         push(std::move(step), value);
         return R::done(result);
+    }
+
+    // Matmuls of the same left operand with constant right operands of one shape and layout (the q / k / v or gate /
+    // up projections of a transformer layer) run as ONE grouped launch: more tiles to fill the chip with, the left
+    // operand fetched once per tile row, and launches saved. The reference launches them one by one
+    // (planner.rs:606-648).
+    std::unordered_map<Value, std::vector<Value>> matmuls_by_left;
+    std::vector<Value> some_user;  // one of the values that use a value (the only one for values used once)
+    bool matmuls_by_left_built = false;
+
+    // whether the matmul is likely to be folded into the `+ tensor` / relu that consumes it (try_visit_fused_matmul):
+    // such a matmul stays out of groups
+    bool feeds_fused_epilogue(Value mm) const {
+        Value v = mm;
+        while (can_fuse(v)) {
+            const Value user = some_user[v];
+            const Operation &op = graph[user].operation;
+            if (op.kind == OpKind::View) { v = user; continue; }
+            if (op.kind != OpKind::Binary) return false;
+            if (op.binary == BinaryOp::Add) return true;
+            return op.binary == BinaryOp::Max && (graph.is_const_zero(op.inputs[0]) || graph.is_const_zero(op.inputs[1]));
+        }
+        return false;
+    }
+
+    const std::vector<Value> &matmul_siblings(Value left) {
+        if (!matmuls_by_left_built) {
+            matmuls_by_left_built = true;
+            // only values that some output depends on
+            std::vector<char> seen(graph.len(), 0);
+            some_user.assign(graph.len(), 0);
+            std::vector<Value> stack(graph.outputs.begin(), graph.outputs.end());
+            while (!stack.empty()) {
+                Value v = stack.back();
+                stack.pop_back();
+                if (seen[v]) continue;
+                seen[v] = 1;
+                for (Value in : graph[v].operation.inputs) {
+                    some_user[in] = v;
+                    stack.push_back(in);
+                }
+            }
+            for (Value v = 0; v < graph.len(); v++) {
+                const Operation &op = graph[v].operation;
+                if (seen[v] && op.kind == OpKind::MatMul && graph.is_const(op.inputs[1]) && !graph.is_const(op.inputs[0]) &&
+                    !feeds_fused_epilogue(v))
+                    matmuls_by_left[op.inputs[0]].push_back(v);
+            }
+        }
+        static const std::vector<Value> none;
+        auto it = matmuls_by_left.find(left);
+        return it == matmuls_by_left.end() ? none : it->second;
+    }
+
+    Visit<std::optional<PlanTensor>> try_visit_matmul_group(Value value) {
+        using R = Visit<std::optional<PlanTensor>>;
+        const ValueInfo &info = graph[value];
+        const DType dt = info.dtype;
+        if (dt != DType::F32 && dt != DType::F16) return R::done(std::nullopt);
+        const Value left_v = info.operation.inputs[0];
+        std::vector<Value> members{value};
+        for (Value other : matmul_siblings(left_v)) {
+            if (other == value || map.count(other) || members.size() >= (size_t) GEMM_MAX_GROUPS) continue;
+            if (graph[other].dtype != dt || graph[other].shape != info.shape) continue;
+            if (graph[graph[other].operation.inputs[1]].shape != graph[info.operation.inputs[1]].shape) continue;
+            members.push_back(other);
+        }
+        // `value` itself has to be one of the candidates (constant right operand, reachable)
+        {
+            const auto &sib = matmul_siblings(left_v);
+            if (members.size() < 2 || std::find(sib.begin(), sib.end(), value) == sib.end()) return R::done(std::nullopt);
+        }
+        auto left = visit(left_v);
+        if (!left.ok) return R::missing(left.need);
+        std::vector<PlanTensor> rights;
+        for (Value m : members) {
+            auto r = visit(graph[m].operation.inputs[1]);
+            if (!r.ok) return R::missing(r.need);
+            rights.push_back(r.value);
+        }
+        // keep the members whose right operand is laid out like the first one's
+        std::vector<Value> kept{members[0]};
+        std::vector<PlanTensor> kept_rights{rights[0]};
+        for (size_t i = 1; i < members.size(); i++)
+            if (rights[i].shape.strides() == rights[0].shape.strides()) {
+                kept.push_back(members[i]);
+                kept_rights.push_back(rights[i]);
+            }
+        if (kept.size() < 2) return R::done(std::nullopt);
+
+        const PlanTensor &l = left.value, &r0 = kept_rights[0];
+        KN_ASSERT(l.shape.rank() == 3 && r0.shape.rank() == 3);
+        const size_t b = l.shape.shape()[0], m = l.shape.shape()[1], k = l.shape.shape()[2], n = r0.shape.shape()[2];
+        if (b * m * n == 0 || b > INT32_MAX || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return R::done(std::nullopt);
+        Step step;
+        step.kind = StepKind::MatMul;
+        step.gemm_f16 = dt == DType::F16;
+        GemmParams &g = step.gemm;
+        g.batch = (int) b; g.m = (int) m; g.n = (int) n; g.k = (int) k;
+        g.a_sb = l.shape.strides()[0]; g.a_sm = l.shape.strides()[1]; g.a_sk = l.shape.strides()[2];
+        g.b_sb = r0.shape.strides()[0]; g.b_sk = r0.shape.strides()[1]; g.b_sn = r0.shape.strides()[2];
+        g.c_sb = (long long) (m * n); g.c_sm = (long long) n; g.c_sn = 1;
+        g.groups = (int) kept.size();
+        if (!gemm_group_ok(g, step.gemm_f16)) return R::done(std::nullopt);
+
+        step.operands.push_back({l, OperandKind::In});
+        for (auto &r : kept_rights) step.operands.push_back({r, OperandKind::In});
+        std::vector<PlanTensor> results;
+        for (size_t i = 0; i < kept.size(); i++) {
+            results.push_back(alloc_tensor_shared({b, m, n}, dt));
+            step.operands.push_back({results.back(), OperandKind::Out});
+        }
+        push(std::move(step), value);
+        for (size_t i = 1; i < kept.size(); i++) insert_mapping(kept[i], results[i]);
+        return R::done(results[0]);
     }
 
     VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first,

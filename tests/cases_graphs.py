@@ -1208,3 +1208,52 @@ def attention_chain_not_fused():
     probs = g.softmax(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), 2)
     g.output_all([g.batched_mat_mul(probs, v), probs])
     return g, 0, [rng.standard_normal(s).astype(np.float32) for s in [(2, 50, 40), (2, 60, 40), (2, 60, 40)]], None
+
+
+def _shared_left_linears(seed, dtype, m, k, n, count, bias_on=(), relu_on=()):
+    """`count` linear layers of one input; some of them with a bias and / or a relu behind them"""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    np_dtype = np.float16 if dtype == DType.F16 else np.float32
+    x = g.input([m, k], dtype)
+    outs = []
+    for i in range(count):
+        w = g.constant([n, k], (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np_dtype), dtype)
+        y = g.linear(x, w)
+        if i in bias_on:
+            y = g.add(y, g.view(g.constant([n], rng.standard_normal(n).astype(np_dtype), dtype), [1, n]))
+        if i in relu_on:
+            y = g.relu(y)
+        outs.append(y)
+    g.output_all(outs)
+    return g, 0, [rng.standard_normal((m, k)).astype(np_dtype)], None
+
+
+@case
+def matmul_group_qkv_f32():
+    """three projections of one input share a launch; ragged rows and columns"""
+    return _shared_left_linears(110, DType.F32, 600, 320, 328, 3)
+
+
+@case
+def matmul_group_f16():
+    """the same in f16 (128 x 128 tiles, slices of 128)"""
+    return _shared_left_linears(111, DType.F16, 520, 256, 384, 3)
+
+
+@case
+def matmul_group_more_than_one_launch_holds():
+    """six siblings: a group of four and a group of two"""
+    return _shared_left_linears(112, DType.F32, 200, 64, 96, 6)
+
+
+@case
+def matmul_group_with_epilogues():
+    """siblings with a bias or relu behind them keep their fused epilogue, the plain ones still share a launch"""
+    return _shared_left_linears(113, DType.F32, 300, 128, 192, 4, bias_on=(0, 2), relu_on=(2,))
+
+
+@case
+def matmul_group_declined_when_k_would_be_split():
+    """skinny products with a long K run apart, each split along K"""
+    return _shared_left_linears(114, DType.F32, 8, 4096, 256, 2)
