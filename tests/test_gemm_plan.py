@@ -90,3 +90,33 @@ def test_attention_chain_stays_apart_when_it_must():
     assert HipExecutor(0, _attention_graph(24, 40), 0, plan_only=True).step_kinds() == three
     assert HipExecutor(0, _attention_graph(40, 40, DType.F16), 0, plan_only=True).step_kinds() == three
     assert HipExecutor(0, _attention_graph(40, 40, axis=1), 0, plan_only=True).step_kinds() == three
+
+
+def _projections(count, m, k, n, dtype=DType.F32, bias_on=()):
+    g = Graph()
+    x = g.input([m, k], dtype)
+    np_dtype = np.float16 if dtype == DType.F16 else np.float32
+    for i in range(count):
+        y = g.linear(x, g.constant([n, k], np.full((n, k), i + 1, np_dtype), dtype))
+        if i in bias_on:
+            y = g.add(y, g.view(g.constant([n], np.ones(n, np_dtype), dtype), [1, n]))
+        g.output(y)
+    return g
+
+
+def test_projections_of_one_input_share_a_launch():
+    ex = HipExecutor(0, _projections(3, 512, 4096, 4096, DType.F16), 0, plan_only=True)
+    assert ex.step_kinds() == ["mat_mul"] and "x3 grouped" in ex.step_str(0)
+    flops, nbytes = ex.step_work(0)
+    assert flops == 3 * 2 * 512 * 4096 * 4096
+    assert nbytes == 2 * (512 * 4096 + 3 * 4096 * 4096 + 3 * 512 * 4096)
+    # at most four products per launch
+    ex = HipExecutor(0, _projections(6, 256, 64, 128), 0, plan_only=True)
+    assert [("x4" in ex.step_str(i), "x2" in ex.step_str(i)) for i in range(ex.step_count())] == [(True, False), (False, True)]
+    # a product whose bias is folded into its store keeps its own launch
+    ex = HipExecutor(0, _projections(3, 256, 64, 128, bias_on=(1,)), 0, plan_only=True)
+    texts = sorted(ex.step_str(i).split(" operands")[0].split("k=64")[1].strip() for i in range(ex.step_count()))
+    assert texts == ["+add", "x2 grouped"]
+    # where even the group leaves the chip short of tiles, the products run apart and split K
+    ex = HipExecutor(0, _projections(2, 8, 4096, 256), 0, plan_only=True)
+    assert ex.step_count() == 2 and all("grouped" not in ex.step_str(i) for i in range(2))
