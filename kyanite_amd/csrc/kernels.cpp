@@ -565,10 +565,11 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
 // ------------------------------------------------------------------------------------------------ reduce kernel
 
 KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
-                              ReduceOp rop) {
+                              ReduceOp rop, const ScalarExpr *pre) {
     const auto &ishape = input.shape.shape();
-    DType dtype = input.dtype;
-    KN_ASSERT(output.dtype == dtype);
+    // the folded values have the type of the output; with a prologue the loaded operand may be of another type
+    const DType dtype = output.dtype, in_dtype = input.dtype;
+    KN_ASSERT(pre ? pre->nodes.back().dtype == dtype : in_dtype == dtype);
 
     // split axes into kept and reduced
     std::vector<size_t> kept_shape, red_shape;
@@ -606,7 +607,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
 
     std::vector<KernelOperand> both{input, output};
     bool idx64 = !fits_i32(both, std::max(kept_size, red_size) + 4096);
-    size_t es = dtype_bytes(dtype);
+    size_t es = dtype_bytes(in_dtype);
 
     const char *T = compute_type(dtype);
     DScalar identity = reduce_identity(rop, dtype);
@@ -615,7 +616,18 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
 
     std::ostringstream ss;
     emit_header(ss, idx64, 2);
-    ss << "typedef " << storage_type(dtype) << " S;\ntypedef " << T << " T;\n";
+    ss << "typedef " << storage_type(dtype) << " S;\ntypedef " << storage_type(in_dtype) << " SI;\ntypedef " << T << " T;\n";
+    // the value that is folded: the loaded element, or an elementwise expression of it
+    ss << "KN_DEV T kn_pre(" << compute_type(in_dtype) << " x1) {\n";
+    if (pre) {
+        std::string res = emit_expr(ss, *pre, "y", [&](size_t operand) {
+            KN_ASSERT(operand == 1);
+            return std::string("x1");
+        });
+        ss << "    return " << res << ";\n}\n";
+    } else {
+        ss << "    return x1;\n}\n";
+    }
     ss << "KN_DEV T kn_f(T a, T b) { return " << binary_expr(bop, dtype, "a", "b") << "; }\n";
     ss << "KN_DEV T kn_identity() { return " << identity.to_c_str() << "; }\n";
     ss << "KN_DEV T kn_post(T v) { return "
@@ -643,9 +655,9 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
             rdims.back() /= vec;
             rstrides[0].back() *= (int64_t) vec;
         }
-        if (vec > 1) ss << vec_type_decl("V", dtype, vec);
+        if (vec > 1) ss << vec_type_decl("V", in_dtype, vec);
         ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_reduce(KnPtrs ptrs) {\n";
-        ss << "    const S *in = (const S *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
+        ss << "    const SI *in = (const SI *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
         if (G == 256) ss << "    __shared__ T lds[4];\n";
         ss << "    const idx_t row = (idx_t) blockIdx.x * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / " << G << ");\n";
         ss << "    const idx_t lane = (idx_t) (threadIdx.x % " << G << ");\n";
@@ -660,9 +672,9 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         emit_decompose(ss, "            ", "r", rdims, rstrides, {"o"});
         if (vec > 1) {
             ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
-            ss << "            for (int j = 0; j < " << vec << "; j++) acc[(i + j) & 3] = kn_f(acc[(i + j) & 3], " << from_storage(dtype, "v[j]") << ");\n";
+            ss << "            for (int j = 0; j < " << vec << "; j++) acc[(i + j) & 3] = kn_f(acc[(i + j) & 3], " << "kn_pre(" + from_storage(in_dtype, "v[j]") + ")" << ");\n";
         } else {
-            ss << "            acc[i & 3] = kn_f(acc[i & 3], " << from_storage(dtype, "in[o]") << ");\n";
+            ss << "            acc[i & 3] = kn_f(acc[i & 3], " << "kn_pre(" + from_storage(in_dtype, "in[o]") + ")" << ");\n";
         }
         ss << "        }\n    }\n";
         ss << "    T total = kn_f(kn_f(acc[0], acc[1]), kn_f(acc[2], acc[3]));\n";
@@ -679,7 +691,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         if (kc.strides[1].back() == 1 && kc.strides[0].back() == 1) {
             for (vec = 16 / es; vec > 1; vec /= 2) {
                 bool ok = kc.shape.back() % vec == 0 && input.offset_bytes % (int64_t) (vec * es) == 0 &&
-                          output.offset_bytes % (int64_t) (vec * es) == 0;
+                          output.offset_bytes % (int64_t) (vec * dtype_bytes(dtype)) == 0;
                 for (size_t a = 0; a + 1 < kc.rank(); a++)
                     ok &= kc.strides[0][a] % (int64_t) vec == 0 && kc.strides[1][a] % (int64_t) vec == 0;
                 for (size_t a = 0; a < rc.rank(); a++) ok &= rc.strides[0][a] % (int64_t) vec == 0;
@@ -699,9 +711,9 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         kdims.back() /= vec;
         kstrides[0].back() *= (int64_t) vec;
         kstrides[1].back() *= (int64_t) vec;
-        if (vec > 1) ss << vec_type_decl("V", dtype, vec);
+        if (vec > 1) ss << vec_type_decl("V", in_dtype, vec) << vec_type_decl("VO", dtype, vec);
         ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void kn_reduce(KnPtrs ptrs) {\n";
-        ss << "    const S *in = (const S *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
+        ss << "    const SI *in = (const SI *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
         if (TY > 1) ss << "    __shared__ T lds[" << TY << "][" << vec << "][" << TX << "];\n";
         ss << "    const idx_t tx = (idx_t) (threadIdx.x % " << TX << "), ty = (idx_t) (threadIdx.x / " << TX << ");\n";
         ss << "    const idx_t kv = (idx_t) blockIdx.x * (idx_t) " << TX << " + tx;\n";
@@ -714,9 +726,9 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         emit_decompose(ss, "            ", "r", rc.shape, rc.strides, {"o"});
         if (vec > 1) {
             ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
-            ss << "            for (int j = 0; j < " << vec << "; j++) acc[j] = kn_f(acc[j], " << from_storage(dtype, "v[j]") << ");\n";
+            ss << "            for (int j = 0; j < " << vec << "; j++) acc[j] = kn_f(acc[j], " << "kn_pre(" + from_storage(in_dtype, "v[j]") + ")" << ");\n";
         } else {
-            ss << "            acc[0] = kn_f(acc[0], " << from_storage(dtype, "in[o]") << ");\n";
+            ss << "            acc[0] = kn_f(acc[0], " << "kn_pre(" + from_storage(in_dtype, "in[o]") + ")" << ");\n";
         }
         ss << "        }\n    }\n";
         if (TY > 1) {
@@ -727,8 +739,8 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
             ss << "    if (valid) {\n";
         }
         if (vec > 1) {
-            ss << "        V o;\n        for (int j = 0; j < " << vec << "; j++) o[j] = " << to_storage(dtype, "kn_post(acc[j])") << ";\n";
-            ss << "        *(V *) (out + o_out) = o;\n";
+            ss << "        VO o;\n        for (int j = 0; j < " << vec << "; j++) o[j] = " << to_storage(dtype, "kn_post(acc[j])") << ";\n";
+            ss << "        *(VO *) (out + o_out) = o;\n";
         } else {
             ss << "        out[o_out] = " << to_storage(dtype, "kn_post(acc[0])") << ";\n";
         }

@@ -48,9 +48,10 @@ struct KernelOperand {
 // out = expr(loads...). operands[0] is the output; the rest are the loaded operands, all of the same shape.
 KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const ScalarExpr &expr);
 
-// output[kept] = post(fold(op, input[kept, reduced...])) (reduce.rs:35-153)
+// output[kept] = post(fold(op, pre(input[kept, reduced...]))) (reduce.rs:35-153). `pre`: an optional elementwise
+// expression of the loaded element (its only operand is number 1), e.g. the square in a mean of squares.
 KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
-                              ReduceOp op);
+                              ReduceOp op, const ScalarExpr *pre = nullptr);
 
 // Row kernels. The value that gets normalised is `pre(load operands...)`, the value stored is
 // `post(normalised, load operands...)`: this is how a preceding scale / residual add and a following affine

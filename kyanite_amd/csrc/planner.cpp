@@ -337,9 +337,30 @@ private:
                 return VT::done(push_row_kernel(value, value, row.value, post, {}));
             }
             case OpKind::Reduce: {
-                KN_TRY(input, visit(op.inputs[0]));
-                PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
                 if (op.reduce == ReduceOp::Mean) KN_ASSERT(result_dtype == DType::F32 || result_dtype == DType::F16);
+                // An elementwise chain of ONE tensor that only this reduction uses (the square in a mean of
+                // squares) is evaluated on the loaded elements instead of being written out and read back.
+                const Value in_v = op.inputs[0];
+                const OpKind in_kind = graph[in_v].operation.kind;
+                if (!map.count(in_v) && can_fuse(in_v) && (in_kind == OpKind::Unary || in_kind == OpKind::Binary)) {
+                    ScalarBlock block;
+                    block.operands.push_back(PlanTensor());  // placeholder for a result
+                    block.loaded.push_back(std::nullopt);
+                    auto root = visit_fused_scalar_recurse(in_v, block, true);
+                    if (!root.ok) return VT::missing(root.need);
+                    if (!block.row_value && block.operands.size() == 2) {
+                        const PlanTensor &input = block.operands[1];
+                        PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
+                        Step step;
+                        step.kind = StepKind::ReduceOp;
+                        step.kernel = make_reduce_kernel(kop(input), kop(output), op.axes, op.reduce, &block.expr);
+                        step.operands = {{input, OperandKind::In}, {output, OperandKind::Out}};
+                        push(std::move(step), value);
+                        return VT::done(output);
+                    }
+                }
+                KN_TRY(input, visit(in_v));
+                PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
                 Step step;
                 step.kind = StepKind::ReduceOp;
                 step.kernel = make_reduce_kernel(kop(input), kop(output), op.axes, op.reduce);
@@ -437,22 +458,16 @@ private:
             return row.pre.nodes.size() - 1;
         };
         Value input = op.inputs[0];
-        if (op.kind == OpKind::Softmax) {
-            row.kind = RowKernelDesc::Softmax;
-            auto sv = visit_scalable_value(input);
-            if (!sv.ok) return R::missing(sv.need);
-            row.inputs = {sv.value.second};
-            scaled(sv.value.first, load(1));
-            return R::done(row);
-        }
-        row.kind = RowKernelDesc::Layernorm;
+        row.kind = op.kind == OpKind::Softmax ? RowKernelDesc::Softmax : RowKernelDesc::Layernorm;
+        // `a0 * x0 + a1 * x1` in front of the row operation (planner.rs:522-604 for layernorm; here for softmax as
+        // well, which covers `scale * scores + mask`); the operands may be laid out differently (a broadcast mask)
         const Operation &iop = graph[input].operation;
         if (iop.kind == OpKind::Binary && iop.binary == BinaryOp::Add && !map.count(input)) {
             auto l = visit_scalable_value(iop.inputs[0]);
             if (!l.ok) return R::missing(l.need);
             auto r = visit_scalable_value(iop.inputs[1]);
             if (!r.ok) return R::missing(r.need);
-            if (l.value.second.shape == r.value.second.shape) {
+            if (l.value.second.shape.shape() == r.value.second.shape.shape()) {
                 row.inputs = {l.value.second, r.value.second};
                 size_t a = scaled(l.value.first, load(1));
                 size_t b = scaled(r.value.first, load(2));
@@ -465,7 +480,6 @@ private:
                 row.pre.nodes.push_back(add);
                 return R::done(row);
             }
-            // differently laid out operands: fall back to materialising the sum
             auto total = visit(input);
             if (!total.ok) return R::missing(total.need);
             row.inputs = {total.value};
@@ -972,6 +986,13 @@ private:
                         block.row_value = value;
                         n.kind = ScalarNode::Load;
                         n.operand = SIZE_MAX;
+                    } else if (op.kind == OpKind::Broadcast && is_small_elementwise(op.inputs[0])) {
+                        // A broadcast elementwise chain that nobody else uses (`rsqrt(mean + eps)` of a norm) is
+                        // evaluated per element here instead of in a launch of its own.
+                        auto inner = inline_under_broadcast(op.inputs[0], info.shape.eval(batch_size), block);
+                        if (!inner.ok) return inner;
+                        block.value_nodes[value] = inner.value;
+                        return R::done(inner.value);
                     } else {
                         auto t = visit(value);
                         if (!t.ok) return R::missing(t.need);
@@ -986,6 +1007,50 @@ private:
         }
         block.value_nodes[value] = node;
         return R::done(node);
+    }
+
+    bool is_small_elementwise(Value v) const {
+        const OpKind kind = graph[v].operation.kind;
+        return (kind == OpKind::Unary || kind == OpKind::Binary) && can_fuse(v) && !map.count(v);
+    }
+
+    // The nodes of the elementwise chain under a Broadcast, with its leaf tensors broadcast to `target`.
+    Visit<size_t> inline_under_broadcast(Value value, const ConcreteShape &target, ScalarBlock &block) {
+        using R = Visit<size_t>;
+        auto known = block.value_nodes.find(value);
+        if (known != block.value_nodes.end()) return R::done(known->second);
+        const ValueInfo &info = graph[value];
+        const Operation &op = info.operation;
+        ScalarNode n;
+        n.dtype = info.dtype;
+        if (is_small_elementwise(value)) {
+            auto a = inline_under_broadcast(op.inputs[0], target, block);
+            if (!a.ok) return a;
+            n.a = a.value;
+            if (op.kind == OpKind::Unary) {
+                n.kind = ScalarNode::Unary;
+                n.unary = op.unary;
+                n.cast_to = op.cast_to;
+            } else {
+                auto b = inline_under_broadcast(op.inputs[1], target, block);
+                if (!b.ok) return b;
+                n.kind = ScalarNode::Binary;
+                n.binary = op.binary;
+                n.b = b.value;
+            }
+        } else if (auto c = graph.as_single_const(value)) {
+            n.kind = ScalarNode::Const;
+            n.constant = *c;
+        } else {
+            auto t = visit(value);
+            if (!t.ok) return R::missing(t.need);
+            const size_t node = block.load_operand(t.value.broadcast(target));
+            block.value_nodes[value] = node;
+            return R::done(node);
+        }
+        block.expr.nodes.push_back(n);
+        block.value_nodes[value] = block.expr.nodes.size() - 1;
+        return R::done(block.expr.nodes.size() - 1);
     }
 
     // planner.rs:926-931

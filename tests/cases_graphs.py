@@ -1257,3 +1257,55 @@ def matmul_group_with_epilogues():
 def matmul_group_declined_when_k_would_be_split():
     """skinny products with a long K run apart, each split along K"""
     return _shared_left_linears(114, DType.F32, 8, 4096, 256, 2)
+
+
+@case
+def reduce_with_elementwise_prologue():
+    """an elementwise chain of one tensor that only the reduction uses is evaluated inside the reduce kernel:
+    sum of squares along rows (lanes share a row) and along columns (threads own columns), max |x|, and a mean of
+    squares whose input is f16 and whose reduction runs in f32 (the cast is part of the chain)"""
+    g = Graph()
+    rng = np.random.default_rng(120)
+    x = g.input([37, 200])
+    h = g.input([24, 512], DType.F16)
+    y = g.input([300, 64])
+    g.output(g.reduce(g.mul(x, x), [1], ReduceOp.SUM))
+    g.output(g.reduce(g.mul(g.unary(UnaryOp.ABS, x), g.scalar(2.0)), [0], ReduceOp.SUM))
+    g.output(g.reduce(g.unary(UnaryOp.ABS, g.add(y, g.scalar(0.5))), [0, 1], ReduceOp.MAX))
+    hf = g.value_cast(h, DType.F32)
+    g.output(g.reduce(g.mul(hf, hf), [1], ReduceOp.MEAN))
+    g.output(g.reduce(g.mul(h, h), [1], ReduceOp.MEAN))
+    return g, 0, [rng.standard_normal((37, 200)).astype(np.float32), rng.standard_normal((24, 512)).astype(np.float16),
+                  rng.standard_normal((300, 64)).astype(np.float32)], None
+
+
+@case
+def rms_norm_two_launches():
+    """x * rsqrt(mean(x^2) + eps) * w: the square folds into the reduction, the rsqrt of the broadcast mean into the
+    scaling kernel; f32 and f16"""
+    g = Graph()
+    rng = np.random.default_rng(121)
+    outs = []
+    for dtype, np_dtype in ((DType.F32, np.float32), (DType.F16, np.float16)):
+        x = g.input([50, 96], dtype)
+        w = g.constant([1, 96], (1.0 + 0.1 * rng.standard_normal((1, 96))).astype(np_dtype), dtype)
+        ms = g.view(g.reduce(g.mul(x, x), [1], ReduceOp.MEAN), [50, 1])
+        r = g.binary(BinaryOp.DIV, g.scalar(1.0, dtype), g.unary(UnaryOp.SQRT, g.add(ms, g.scalar(1e-5, dtype))))
+        outs.append(g.mul(g.mul(x, g.broadcast(r, [50, 96])), g.broadcast(w, [50, 96])))
+    g.output_all(outs)
+    return g, 0, [rng.standard_normal((50, 96)).astype(np.float32), rng.standard_normal((50, 96)).astype(np.float16)], None
+
+
+@case
+def softmax_scale_and_mask_prologue():
+    """softmax(scale * scores + mask) with a mask that is broadcast over the heads: one kernel; f32 and f16"""
+    g = Graph()
+    rng = np.random.default_rng(122)
+    mask = np.where(np.tril(np.ones((40, 40))) > 0, 0.0, -1e4)
+    outs = []
+    for dtype, np_dtype in ((DType.F32, np.float32), (DType.F16, np.float16)):
+        s = g.input([6, 40, 40], dtype)
+        m = g.broadcast(g.constant([1, 40, 40], mask.astype(np_dtype)[None], dtype), [6, 40, 40])
+        outs.append(g.softmax(g.add(g.mul(s, g.scalar(0.125, dtype)), m), 2))
+    g.output_all(outs)
+    return g, 0, [rng.standard_normal((6, 40, 40)).astype(np.float32) * 4, (rng.standard_normal((6, 40, 40)) * 4).astype(np.float16)], None
