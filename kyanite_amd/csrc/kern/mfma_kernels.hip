@@ -362,14 +362,16 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
 // "Plane" convolution: stride 1, same-size output, image width a power of two. Instead of gathering the im2col
 // matrix, every K slice (CB input channels x KH x KW taps) stages the raw input rows that the tile's TN = 128 or
 // 64 output positions touch into LDS once, as [channel][group][row][W], and the MFMA B operand is read straight from those
-// planes: position n of the tile sits at a fixed per-lane offset, tap (c, fy, fx) adds a wave-uniform offset, and
-// taps that fall left or right of the image are masked to zero (rows above / below are stored as zero rows).
+// planes: position n of the tile sits at a fixed per-lane offset, tap (c, fy, fx) adds a wave-uniform offset. Every
+// plane row has PLANE_PAD zero floats in front of it, so a tap left of the image reads the row's own padding and a
+// tap right of it the next row's (rows above / below the image are stored as zero rows): no masking in the K loop.
 // Global -> LDS traffic for B drops by KH * KW and no per-element index arithmetic is left in the K loop.
 // A tile is either R = TN / W whole output rows of one image (H * W >= TN) or G = TN / (H * W) whole images.
 constexpr int CB = 8;             // input channels per K slice
 constexpr int PLANE_MAX_VEC = 3;  // 128 bit loads per thread and slice for the B planes
-constexpr int PLANE_SLACK = 4;    // floats in front of / behind the planes that masked taps may touch
-constexpr int PLANE_LDS = PLANE_MAX_VEC * THREADS * 4 + 2 * PLANE_SLACK;
+constexpr int PLANE_PAD = 4;      // zero floats in front of every plane row: what a tap left or right of the image reads
+constexpr int PLANE_SLACK = 4;    // zero floats in front of / behind all planes
+constexpr int PLANE_LDS = 2 * PLANE_MAX_VEC * THREADS * 4 + 2 * PLANE_SLACK;  // rows of 4 pixels double with the padding
 
 struct PlaneGeom {
     int rows;            // R: output rows per group
@@ -378,6 +380,7 @@ struct PlaneGeom {
     int plane_rows;      // R + KH - 1
     int w4_shift, g_shift, rw_shift;  // log2 of W / 4, G, R * W
     int n_vec;           // CB * G * plane_rows * W / 4
+    int row_stride;      // W + PLANE_PAD
 };
 
 // NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64); MI: the same along
@@ -412,11 +415,12 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, c32 = lane & 31;
-    const int plane = g.plane_rows * W, gplane = plane << g.g_shift;  // floats per (c, g) and per c
+    const int RS = g.row_stride;
+    const int plane = g.plane_rows * RS, gplane = plane << g.g_shift;  // LDS floats per (c, g) and per c
 
     // ---- B planes: what this thread moves per slice (the same places every slice, only the channel base moves)
     const float *b_src[PLANE_MAX_VEC];
-    bool b_live[PLANE_MAX_VEC];
+    int b_dst[PLANE_MAX_VEC];  // -1: nothing to move
 #pragma unroll
     for (int i = 0; i < PLANE_MAX_VEC; i++) {
         const int e = t + THREADS * i;
@@ -425,7 +429,7 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         const int gg = t2 & (g.groups - 1), c = t2 >> g.g_shift;
         const int iy = oy0 + prow - p.pad_y, img = img0 + gg;
         const bool ok = e < g.n_vec && iy >= 0 && iy < H && img < p.batch;
-        b_live[i] = e < g.n_vec;
+        b_dst[i] = e < g.n_vec ? PLANE_SLACK + t1 * RS + PLANE_PAD + 4 * w4 : -1;
         b_src[i] = ok ? p.input + (((long long) img * C + c) * H + iy) * W + 4 * w4 : nullptr;
     }
     // ---- A (filter) rows: K contiguous
@@ -439,18 +443,11 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     }
     // ---- where this lane's output positions sit inside a plane, and which taps stay inside the image
     int lane_base[NJ];
-    bool pair_ok[NJ][KW];
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
         const int n = wn * 32 * NJ + 32 * j + c32;
-        const int gl = n >> g.rw_shift, rem = n & ((1 << g.rw_shift) - 1), col = rem & (W - 1);
-        lane_base[j] = PLANE_SLACK + gl * plane + rem - p.pad_x;
-#pragma unroll
-        for (int fx = 0; fx < KW; fx++) {
-            // the upper half of the wave multiplies the next k, whose fx is one further (cyclically)
-            const int f = half ? (fx + 1) % KW : fx;
-            pair_ok[j][fx] = (unsigned) (col + f - p.pad_x) < (unsigned) W;
-        }
+        const int gl = n >> g.rw_shift, rem = n & ((1 << g.rw_shift) - 1), col = rem & (W - 1), r = rem >> (g.w4_shift + 2);
+        lane_base[j] = PLANE_SLACK + gl * plane + r * RS + PLANE_PAD + col - p.pad_x;
     }
 
     floatx4 ra[A_ITERS], rb[PLANE_MAX_VEC];
@@ -473,7 +470,7 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             }
 #pragma unroll
         for (int i = 0; i < PLANE_MAX_VEC; i++)
-            if (b_live[i]) *(floatx4 *) &Bs[PLANE_SLACK + 4 * (t + THREADS * i)] = rb[i];
+            if (b_dst[i] >= 0) *(floatx4 *) &Bs[b_dst[i]] = rb[i];
     };
 
     floatx16 acc[MI][NJ];
@@ -484,47 +481,85 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    if (t < 2 * PLANE_SLACK) Bs[t < PLANE_SLACK ? t : PLANE_LDS - 2 * PLANE_SLACK + t] = 0.0f;
+    // the padding is never written again
+    for (int i = t; i < PLANE_LDS; i += THREADS) Bs[i] = 0.0f;
     fetch(0);
     for (int c0 = 0; c0 < C; c0 += CB) {
         __syncthreads();
         stage();
         __syncthreads();
         if (c0 + CB < C) fetch(c0 + CB);
-#pragma unroll
-        for (int kk = 0; kk < KS; kk += 2) {
+        // The operands of step kk + 2 are requested from LDS before the MFMAs of step kk are issued, and the wave
+        // raises its priority while it issues MFMAs. Measured on this loop alone (no global loads, two waves per
+        // SIMD): operands read right before their MFMAs and masked with selects 126 TFLOP/s, without the selects 140,
+        // read one step ahead and with the priority 147, the bare MFMAs 155.
+        float a_next[MI], b_next[NJ];
+        auto read_operands = [&](int kk) {
             // taps of k = kk (lower half of the wave) and k = kk + 1 (upper half); all compile-time
             const int ca = kk / (KH * KW), fya = (kk / KW) % KH, fxa = kk % KW;
             const int cb = (kk + 1) / (KH * KW), fyb = ((kk + 1) / KW) % KH, fxb = (kk + 1) % KW;
-            const int off_a = ca * gplane + fya * W + fxa, off_b = cb * gplane + fyb * W + fxb;
+            const int off_a = ca * gplane + fya * RS + fxa, off_b = cb * gplane + fyb * RS + fxb;
             const int koff = half ? off_b : off_a;
+#pragma unroll
+            for (int i = 0; i < MI; i++) a_next[i] = As[kk + half][wm * 32 * MI + 32 * i + c32];
+#pragma unroll
+            for (int j = 0; j < NJ; j++) b_next[j] = Bs[lane_base[j] + koff];
+        };
+        read_operands(0);
+#pragma unroll
+        for (int kk = 0; kk < KS; kk += 2) {
             float a[MI], b[NJ];
 #pragma unroll
-            for (int i = 0; i < MI; i++) a[i] = As[kk + half][wm * 32 * MI + 32 * i + c32];
+            for (int i = 0; i < MI; i++) a[i] = a_next[i];
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                b[j] = Bs[lane_base[j] + koff];
-                b[j] = pair_ok[j][fxa] ? b[j] : 0.0f;
-            }
+            for (int j = 0; j < NJ; j++) b[j] = b_next[j];
+            if (kk + 2 < KS) read_operands(kk + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < NJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
+    // Epilogue. Bias and residual are requested for a whole MFMA tile row at once (addresses clamped into the tensor
+    // instead of branches around the loads), so their latencies overlap; only the stores are predicated.
     ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
     const int col0 = n0 + wn * 32 * NJ + c32;
     s.prepare(col0, col0 + 32);
 #pragma unroll
-    for (int i = 0; i < MI; i++)
+    for (int i = 0; i < MI; i++) {
+        int row_off[16];  // inside one image: below 2^31 (checked on the host)
+        float bias_v[16];
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
+        for (int v = 0; v < 16; v++) {
+            const int row = m0 + wm * 32 * MI + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+            const int row_c = min(row, p.out_c - 1);
+            row_off[v] = row_c * ohw;
+            bias_v[v] = s.bias ? s.bias[row_c * s.bias_stride] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const long long base = s.col_ok[j] ? s.col_base[j] : 0ll;
+            float res_v[16];
+            if (s.res) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) res_v[v] = s.res[base + row_off[v]];
+            }
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 32 * MI + i * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-                s.store(row, col0 + 32 * j, j, acc[i][j][v]);
+                float x = acc[i][j][v];
+                if (s.res) x += res_v[v];
+                x += bias_v[v];
+                if (s.relu) x = fmaxf(x, 0.0f);
+                if (row < p.out_c && s.col_ok[j]) s.p[base + row_off[v]] = x;
             }
+        }
+    }
 }
 
 int log2_exact(int x) {
@@ -557,7 +592,9 @@ bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     g->g_shift = log2_exact(g->groups);
     g->rw_shift = log2_exact(g->rows * W);
     g->n_vec = CB * g->groups * g->plane_rows * W / 4;
+    g->row_stride = W + PLANE_PAD;
     if (g->g_shift < 0 || g->rw_shift < 0 || g->n_vec > PLANE_MAX_VEC * THREADS) return false;
+    if (CB * g->groups * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
     return true;
 }
 
@@ -688,6 +725,7 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     if (positions <= 0 || p.out_c <= 0) return 0;
     const long long big_tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
     if (positions > 0x7fffffffll || big_tiles > 0x7fffffffll / 4) return (int) hipErrorInvalidValue;
+    if ((long long) p.out_c * p.out_h * p.out_w > 0x7fffffffll) return (int) hipErrorInvalidValue;
     // Plane kernel tiles (output channels x positions): 128 x 128 or 64 x 64, each wave owning 4 or 1 MFMA tiles of
     // the result. The waves of all workgroups spread over 1024 SIMDs and the launch takes about as long as the
     // busiest SIMD: rounds of waves x MFMA tiles per wave. The small tile costs a tenth more per MFMA tile (more LDS
