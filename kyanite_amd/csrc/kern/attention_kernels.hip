@@ -96,16 +96,31 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) st[j][v] = 0.0f;
+        // (LDS operands are requested one step before the MFMAs that use them, and the wave raises its priority
+        // while it issues MFMAs; the scheduling barriers keep that order)
+        {
+            floatx4 a_next[2];
 #pragma unroll
-        for (int t4 = 0; t4 < HALF / 4; t4++) {
-            floatx4 a[2];
+            for (int j = 0; j < 2; j++) a_next[j] = *(const floatx4 *) &Ks[32 * j + c][h * HALF];
 #pragma unroll
-            for (int j = 0; j < 2; j++) a[j] = *(const floatx4 *) &Ks[32 * j + c][h * HALF + 4 * t4];
+            for (int t4 = 0; t4 < HALF / 4; t4++) {
+                floatx4 a[2];
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+                for (int j = 0; j < 2; j++) a[j] = a_next[j];
+                if (t4 + 1 < HALF / 4) {
 #pragma unroll
-                for (int j = 0; j < 2; j++)
-                    st[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][u], qf[4 * t4 + u], st[j], 0, 0, 0);
+                    for (int j = 0; j < 2; j++) a_next[j] = *(const floatx4 *) &Ks[32 * j + c][h * HALF + 4 * (t4 + 1)];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        st[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j][u], qf[4 * t4 + u], st[j], 0, 0, 0);
+                __builtin_amdgcn_s_setprio(0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (key0 + BKEYS > p.lk) {
             // keys past the end take no part
@@ -139,15 +154,36 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
             for (int v = 0; v < 16; v++) oacc[t][v] *= alpha;
 
+        {
+            // steps of the second product in groups of 4 keys (one per accumulator register v % 4)
+            auto key_of = [&](int step) { return 32 * (step >> 4) + 8 * ((step & 15) >> 2) + 4 * h + (step & 3); };
+            float v_next[4][DVT];
+            auto read_v = [&](int step0) {
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+                for (int u = 0; u < 4; u++)
 #pragma unroll
-            for (int s = 0; s < 16; s++) {
-                const int key = 32 * j + 8 * (s >> 2) + 4 * h + (s & 3);
+                    for (int t = 0; t < DVT; t++) v_next[u][t] = Vs[key_of(step0 + u)][32 * t + c];
+            };
+            read_v(0);
 #pragma unroll
-                for (int t = 0; t < DVT; t++)
-                    oacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(Vs[key][32 * t + c], st[j][s], oacc[t], 0, 0, 0);
+            for (int step0 = 0; step0 < 32; step0 += 4) {
+                float vv[4][DVT];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int t = 0; t < DVT; t++) vv[u][t] = v_next[u][t];
+                if (step0 + 4 < 32) read_v(step0 + 4);
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int t = 0; t < DVT; t++)
+                        oacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[u][t], st[(step0 + u) >> 4][(step0 + u) & 15], oacc[t], 0, 0, 0);
+                __builtin_amdgcn_s_setprio(0);
+                __builtin_amdgcn_sched_barrier(0);
             }
+        }
         __syncthreads();  // the block has been consumed by every wave
     }
 
