@@ -77,10 +77,11 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
         Launch &l = launches_[si];
         for (auto &op : step.operands) l.ptrs.push_back(arena_ + plan_.resolve(op.tensor.ptr));
         if (step.kind == StepKind::MatMul && step.attention) {
-            step.attn.q = (const float *) l.ptrs[0];
-            step.attn.k = (const float *) l.ptrs[1];
-            step.attn.v = (const float *) l.ptrs[2];
-            step.attn.o = (float *) l.ptrs[3];
+            step.attn.q = l.ptrs[0];
+            step.attn.k = l.ptrs[1];
+            step.attn.v = l.ptrs[2];
+            step.attn.mask = step.attention_has_mask ? l.ptrs[3] : nullptr;
+            step.attn.o = l.ptrs.back();
         } else if (step.kind == StepKind::MatMul && step.gemm.groups > 1) {
             const size_t groups = (size_t) step.gemm.groups;
             KN_ASSERT(l.ptrs.size() == 1 + 2 * groups);
@@ -195,7 +196,8 @@ void HipExecutor::launch_step(size_t index, hipEvent_t start, hipEvent_t stop) {
     switch (step.kind) {
         case StepKind::MatMul:
             if (step.attention) {
-                hip_check((hipError_t) launch_attention_f32(step.attn, stream_), "attention launch");
+                hip_check((hipError_t) (step.gemm_f16 ? launch_attention_f16(step.attn, stream_) : launch_attention_f32(step.attn, stream_)),
+                          "attention launch");
                 break;
             }
             hip_check((hipError_t) (step.gemm_f16 ? launch_gemm_f16(step.gemm, stream_) : launch_gemm_f32(step.gemm, stream_)),

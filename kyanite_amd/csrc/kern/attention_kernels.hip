@@ -42,14 +42,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int c = lane & 31, h = lane >> 5;
     const int bz = blockIdx.y;
     const int query = blockIdx.x * BQ + wave * 32 + c;
-    const float *kp = p.k + bz * p.k_sb, *vp = p.v + bz * p.v_sb;
+    const float *kp = (const float *) p.k + bz * p.k_sb, *vp = (const float *) p.v + bz * p.v_sb;
 
     // Q^T operand: lane (query c, half h) holds k = h * HALF + t for step t, pre-multiplied by scale * log2(e) so
     // that the exponentials are plain exp2
     float qf[HALF];
     {
         const float factor = p.scale * 1.44269504088896340736f;
-        const float *qp = p.q + bz * p.q_sb + (long long) query * p.q_sm;
+        const float *qp = (const float *) p.q + bz * p.q_sb + (long long) query * p.q_sm;
 #pragma unroll
         for (int t = 0; t < HALF; t++) qf[t] = query < p.lq ? qp[(long long) (h * HALF + t) * p.q_sk] * factor : 0.0f;
     }
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
     row_sum += __shfl_xor(row_sum, 32);
     if (query < p.lq) {
         const float inv = 1.0f / row_sum;
-        float *op = p.o + bz * p.o_sb + (long long) query * p.o_sm;
+        float *op = (float *) p.o + bz * p.o_sb + (long long) query * p.o_sm;
 #pragma unroll
         for (int t = 0; t < DVT; t++)
 #pragma unroll

@@ -70,26 +70,33 @@ struct ConvParams {
     int relu;
 };
 
-// O[b] = softmax(scale * Q[b] K[b]^T) V[b] with the softmax along the keys; Q is [batch, lq, dk], K [batch, lk, dk],
-// V [batch, lk, dv], O [batch, lq, dv], all f32 with arbitrary element strides (batch, row, column in that order;
-// zero batch stride = broadcast operand).
+// O[b] = softmax(scale * Q[b] K[b]^T + mask[b]) V[b] with the softmax along the keys; Q is [batch, lq, dk],
+// K [batch, lk, dk], V [batch, lk, dv], O [batch, lq, dv], mask [batch, lq, lk], with arbitrary element strides (batch,
+// row, column in that order; zero stride = broadcast). The element type (float or _Float16) is fixed by the launch
+// function; the f32 kernel takes no mask, the f16 kernel needs contiguous, 16 byte aligned rows of Q, K and V.
 struct AttentionParams {
-    const float *q;
-    const float *k;
-    const float *v;
-    float *o;
+    const void *q;
+    const void *k;
+    const void *v;
+    void *o;
     int batch, lq, lk, dk, dv;
     long long q_sb, q_sm, q_sk;
     long long k_sb, k_sn, k_sk;  // k_sn: between keys, k_sk: along dk
     long long v_sb, v_sk, v_sn;  // v_sk: between keys, v_sn: along dv
     long long o_sb, o_sm, o_sn;
     float scale;
+    int has_scale = 1;  // f16: whether the scores are multiplied (and rounded) at all
+    const void *mask = nullptr;
+    long long m_sb = 0, m_sq = 0, m_sk = 0;
+    int mask_vec = 0;  // rows of the mask are contiguous and 8 byte aligned
 };
 // widths the fused kernel is built for; other chains run as matmul, softmax, matmul
 bool attention_supported(int dk, int dv);
+bool attention_f16_supported(int dk, int dv);
 
 // All return a hipError_t value (0 = success).
 int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream);
+int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream);
 int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
 // f16 operands and result, f32 accumulation, one rounding (to nearest even) at the store
 int launch_gemm_f16(const GemmParams &p, ihipStream_t *stream);

@@ -16,7 +16,7 @@ std::string Step::str() const {
     ss << step_kind_name(kind) << " value=" << debug_value;
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
     if (kind == StepKind::MatMul && attention)
-        ss << " attention f32 b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
+        ss << " attention " << (gemm_f16 ? "f16" : "f32") << (attention_has_mask ? " +mask" : "") << " b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
     else if (kind == StepKind::MatMul) {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm.relu ? " relu" : "");
@@ -593,22 +593,40 @@ private:
         return R::done(*viewed);
     }
 
-    // matmul(softmax(matmul(q, kt) [* or / constant], last axis), v) in f32, every intermediate value hidden and used
-    // once: the scores stay on the compute unit instead of passing through memory between three launches
-    // (planner.rs:606-648, :418-476 plan them separately).
+    // matmul(softmax(matmul(q, kt) [* or / constant] [+ mask], last axis), v) in f32 (no mask) or f16, every
+    // intermediate value hidden and used once: the scores stay on the compute unit instead of passing through memory
+    // between three or more launches (planner.rs:606-648, :418-476 plan them separately).
     Visit<std::optional<PlanTensor>> try_visit_fused_attention(Value value, bool batch_first = true) {
         using R = Visit<std::optional<PlanTensor>>;
         const ValueInfo &info = graph[value];
-        if (info.operation.kind != OpKind::MatMul || info.dtype != DType::F32) return R::done(std::nullopt);
+        const DType dt = info.dtype;
+        if (info.operation.kind != OpKind::MatMul || (dt != DType::F32 && dt != DType::F16)) return R::done(std::nullopt);
+        const bool f16 = dt == DType::F16;
         const Value probs = info.operation.inputs[0], v_v = info.operation.inputs[1];
         const Operation &sop = graph[probs].operation;
         if (sop.kind != OpKind::Softmax || sop.axis() != 2 || !can_fuse(probs) || map.count(probs)) return R::done(std::nullopt);
         Value scores = sop.inputs[0];
         if (!can_fuse(scores) || map.count(scores)) return R::done(std::nullopt);
+        // f16 only: `... + mask`, either way round; the mask is any tensor of the scores' shape (usually a broadcast)
+        std::optional<Value> mask_v;
+        if (f16 && graph[scores].operation.kind == OpKind::Binary && graph[scores].operation.binary == BinaryOp::Add) {
+            const Value l = graph[scores].operation.inputs[0], r = graph[scores].operation.inputs[1];
+            auto leads_to_matmul = [&](Value v) {
+                if (!can_fuse(v) || map.count(v)) return false;
+                const Operation &op = graph[v].operation;
+                if (op.kind == OpKind::MatMul) return true;
+                return op.kind == OpKind::Binary && op.binary == BinaryOp::Mul;
+            };
+            if (leads_to_matmul(l)) { scores = l; mask_v = r; }
+            else if (leads_to_matmul(r)) { scores = r; mask_v = l; }
+            else return R::done(std::nullopt);
+        }
         float scale = 1.0f;
+        bool has_scale = false;
         {
             const Operation &op = graph[scores].operation;
-            if (op.kind == OpKind::Binary && (op.binary == BinaryOp::Mul || op.binary == BinaryOp::Div)) {
+            // f16 rounds the scaled scores, so a division is not the same as a multiplication there
+            if (op.kind == OpKind::Binary && (op.binary == BinaryOp::Mul || (op.binary == BinaryOp::Div && !f16))) {
                 Value l = op.inputs[0], r = op.inputs[1];
                 auto rc = graph.as_single_const(r);
                 auto lc = op.binary == BinaryOp::Mul ? graph.as_single_const(l) : std::nullopt;
@@ -617,20 +635,23 @@ private:
                 if (rc) { inner = l; factor = rc; }
                 else if (lc) { inner = r; factor = lc; }
                 else return R::done(std::nullopt);
-                if (factor->dtype != DType::F32 || !can_fuse(inner) || map.count(inner)) return R::done(std::nullopt);
+                if (factor->dtype != dt || !can_fuse(inner) || map.count(inner)) return R::done(std::nullopt);
                 scale = op.binary == BinaryOp::Mul ? (float) factor->f : 1.0f / (float) factor->f;
-                if (!(scale > 0.0f) || !std::isfinite(scale)) return R::done(std::nullopt);
+                // the f32 kernel folds the scale into Q and takes the maximum of the scaled scores
+                if (!std::isfinite(scale) || (!f16 && !(scale > 0.0f))) return R::done(std::nullopt);
+                has_scale = true;
                 scores = inner;
             }
         }
         const Operation &mop = graph[scores].operation;
-        if (mop.kind != OpKind::MatMul || graph[scores].dtype != DType::F32) return R::done(std::nullopt);
+        if (mop.kind != OpKind::MatMul || graph[scores].dtype != dt) return R::done(std::nullopt);
         const Value q_v = mop.inputs[0], kt_v = mop.inputs[1];
         const ConcreteShape q_shape = graph[q_v].shape.eval(batch_size), kt_shape = graph[kt_v].shape.eval(batch_size);
         const ConcreteShape v_shape = graph[v_v].shape.eval(batch_size);
         const size_t b = q_shape[0], lq = q_shape[1], dk = q_shape[2], lk = kt_shape[2], dv = v_shape[2];
         if (b == 0 || lq == 0 || lk == 0 || b > 65535 || lq > INT32_MAX || lk > INT32_MAX) return R::done(std::nullopt);
-        if (dk > 1024 || dv > 1024 || !attention_supported((int) dk, (int) dv)) return R::done(std::nullopt);
+        if (dk > 1024 || dv > 1024) return R::done(std::nullopt);
+        if (!(f16 ? attention_f16_supported((int) dk, (int) dv) : attention_supported((int) dk, (int) dv))) return R::done(std::nullopt);
 
         auto q = visit(q_v);
         if (!q.ok) return R::missing(q.need);
@@ -638,32 +659,60 @@ private:
         if (!kt.ok) return R::missing(kt.need);
         auto v = visit(v_v);
         if (!v.ok) return R::missing(v.need);
-        // the kernel addresses a block of 64 keys with 32 bit offsets from the block's base
-        auto fits = [](const PlanTensor &t) {
-            for (size_t a = 1; a < 3; a++) {
-                const long long s = t.shape.strides()[a];
-                if (s < 0 || s > (1ll << 20)) return false;
-            }
-            return true;
-        };
-        if (!fits(kt.value) || !fits(v.value)) return R::done(std::nullopt);
+        std::optional<PlanTensor> mask;
+        if (mask_v) {
+            auto m = visit(*mask_v);
+            if (!m.ok) return R::missing(m.need);
+            mask = m.value;
+        }
+        const auto &qs = q.value.shape.strides(), &ks = kt.value.shape.strides(), &vs = v.value.shape.strides();
+        if (f16) {
+            // rows of Q, K and V are read as 128 bit vectors
+            auto rows_ok = [](const PlanTensor &t, long long batch_stride, long long row_stride, long long inner_stride) {
+                return inner_stride == 1 && row_stride % 8 == 0 && batch_stride % 8 == 0 && t.ptr.offset_bytes % 16 == 0;
+            };
+            if (!rows_ok(q.value, qs[0], qs[1], qs[2]) || !rows_ok(kt.value, ks[0], ks[2], ks[1]) ||
+                !rows_ok(v.value, vs[0], vs[1], vs[2]))
+                return R::done(std::nullopt);
+            // a block of 64 keys is addressed with 32 bit offsets from the block's base
+            if (ks[2] < 0 || ks[2] > (1 << 20) || vs[1] < 0 || vs[1] > (1 << 20)) return R::done(std::nullopt);
+        } else {
+            // the kernel addresses a block of 64 keys with 32 bit offsets from the block's base
+            auto fits = [](const PlanTensor &t) {
+                for (size_t a = 1; a < 3; a++) {
+                    const long long s = t.shape.strides()[a];
+                    if (s < 0 || s > (1ll << 20)) return false;
+                }
+                return true;
+            };
+            if (!fits(kt.value) || !fits(v.value)) return R::done(std::nullopt);
+        }
 
-        PlanTensor result = batch_first ? alloc_tensor_shared({b, lq, dv}, DType::F32)
-                                        : alloc_tensor_shared({lq, b, dv}, DType::F32).permute({1, 0, 2});
+        PlanTensor result = batch_first ? alloc_tensor_shared({b, lq, dv}, dt)
+                                        : alloc_tensor_shared({lq, b, dv}, dt).permute({1, 0, 2});
         Step step;
         step.kind = StepKind::MatMul;
         step.attention = true;
+        step.gemm_f16 = f16;
         AttentionParams &a = step.attn;
         a.batch = (int) b; a.lq = (int) lq; a.lk = (int) lk; a.dk = (int) dk; a.dv = (int) dv;
         a.scale = scale;
-        const auto &qs = q.value.shape.strides(), &ks = kt.value.shape.strides(), &vs = v.value.shape.strides();
+        a.has_scale = has_scale ? 1 : 0;
         const auto &os = result.shape.strides();
         a.q_sb = qs[0]; a.q_sm = qs[1]; a.q_sk = qs[2];
         a.k_sb = ks[0]; a.k_sk = ks[1]; a.k_sn = ks[2];  // the operand is K^T: [b, dk, lk]
         a.v_sb = vs[0]; a.v_sk = vs[1]; a.v_sn = vs[2];
         a.o_sb = os[0]; a.o_sm = os[1]; a.o_sn = os[2];
-        step.operands = {{q.value, OperandKind::In}, {kt.value, OperandKind::In}, {v.value, OperandKind::In},
-                         {result, OperandKind::Out}};
+        step.operands = {{q.value, OperandKind::In}, {kt.value, OperandKind::In}, {v.value, OperandKind::In}};
+        if (mask) {
+            KN_ASSERT(mask->shape.shape() == ConcreteShape({b, lq, lk}));
+            const auto &ms = mask->shape.strides();
+            a.m_sb = ms[0]; a.m_sq = ms[1]; a.m_sk = ms[2];
+            a.mask_vec = ms[2] == 1 && ms[1] % 4 == 0 && ms[0] % 4 == 0 && mask->ptr.offset_bytes % 8 == 0;
+            step.attention_has_mask = true;
+            step.operands.push_back({*mask, OperandKind::In});
+        }
+        step.operands.push_back({result, OperandKind::Out});
         push(std::move(step), value);
         return R::done(result);
     }

@@ -37,8 +37,9 @@ struct Step {
     GemmParams gemm{};
     bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
     bool gemm_has_addend = false;  // operand 3 is the tensor added in the epilogue
-    // a MatMul step that is a whole softmax(scale * Q K^T) V chain in one launch; operands Q, K, V, O
+    // a MatMul step that is a whole softmax(scale * Q K^T [+ mask]) V chain in one launch; operands Q, K, V, [mask,] O
     bool attention = false;
+    bool attention_has_mask = false;  // operand 3 is the additive mask, the result comes last
     AttentionParams attn{};
     ConvParams conv{};
     bool conv_has_bias = false, conv_has_res = false;

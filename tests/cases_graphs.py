@@ -975,7 +975,7 @@ def f16_norms():
 @case
 def config_llama_small():
     from kyanite_amd.configs import build_llama
-    g, make_inputs, _ = build_llama(seed=1, layers=2, seq=24, d_model=64, heads=4, ffn=176)
+    g, make_inputs, _ = build_llama(seed=1, layers=2, seq=24, d_model=256, heads=4, ffn=352)
     return g, 0, make_inputs(), None
 
 
@@ -1309,3 +1309,61 @@ def softmax_scale_and_mask_prologue():
         outs.append(g.softmax(g.add(g.mul(s, g.scalar(0.125, dtype)), m), 2))
     g.output_all(outs)
     return g, 0, [rng.standard_normal((6, 40, 40)).astype(np.float32) * 4, (rng.standard_normal((6, 40, 40)) * 4).astype(np.float16)], None
+
+
+def _attention_f16_case(seed, b, lq, lk, dk, dv, scale, mask, layout="dense"):
+    """f16 softmax(scale * Q K^T + mask) V; mask: None, 'causal' (a [1, lq, lk] constant of 0 / -inf, broadcast over the
+    batch), 'full' (a [b, lq, lk] input of finite values), 'left' (the constant on the left of the sum)"""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    inputs = []
+
+    def inp(shape):
+        inputs.append(rng.standard_normal(shape).astype(np.float16))
+        return g.input(list(shape), DType.F16)
+
+    if layout == "heads":
+        q = g.permute(inp((lq, b, dk)), [1, 0, 2])
+        kt = g.permute(inp((lk, b, dk)), [1, 2, 0])
+        v = g.permute(inp((lk, b, dv)), [1, 0, 2])
+    else:
+        q = inp((b, lq, dk))
+        kt = g.permute(inp((b, lk, dk)), [0, 2, 1])
+        v = inp((b, lk, dv))
+    scores = g.batched_mat_mul(q, kt)
+    if scale:
+        scores = g.mul(scores, g.scalar(1.0 / np.sqrt(dk), DType.F16))
+    if mask in ("causal", "left"):
+        m = np.where(np.tril(np.ones((lq, lk), bool), k=lk - lq), 0.0, -np.inf).astype(np.float16)
+        mc = g.broadcast(g.constant([1, lq, lk], m[None], DType.F16), [b, lq, lk])
+        scores = g.add(mc, scores) if mask == "left" else g.add(scores, mc)
+    elif mask == "full":
+        scores = g.add(scores, inp((b, lq, lk)))
+    out = g.batched_mat_mul(g.softmax(scores, 2), v)
+    if layout == "heads":
+        out = g.view(g.permute(out, [1, 0, 2]), [lq, b * dv])
+    g.output(out)
+    return g, 0, inputs, None
+
+
+@case
+def attention_f16_causal_heads():
+    """the decoder's attention: width 128, causal mask constant, operands that are permuted views"""
+    return _attention_f16_case(130, 4, 96, 96, 128, 128, True, "causal", "heads")
+
+
+@case
+def attention_f16_ragged_full_mask():
+    """70 queries against 150 keys (partial blocks), width 64, V 40 wide, a mask tensor per batch entry"""
+    return _attention_f16_case(131, 3, 70, 150, 64, 40, True, "full")
+
+
+@case
+def attention_f16_plain():
+    """no scale, no mask; many queries (four waves per workgroup would need 256 workgroups: two here)"""
+    return _attention_f16_case(132, 2, 200, 130, 64, 64, False, None)
+
+
+@case
+def attention_f16_mask_on_the_left_no_scale():
+    return _attention_f16_case(133, 2, 40, 72, 128, 96, False, "left")
