@@ -22,3 +22,12 @@ def test_help_lists_the_workloads():
     assert r.returncode == 0
     for name in ("bandwidth", "mlp", "resnet", "llama", "unet"):
         assert name in r.stdout
+
+
+def test_build_check_graph_still_covers_every_kernel_family():
+    # the graph that `__graft_entry__.build()` plans after compiling; new fusions must not silently remove a family
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+
+    steps, kinds = __graft_entry__.check_kernel_families()
+    assert steps >= 7 and len(kinds) == 7
