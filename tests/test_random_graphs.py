@@ -10,16 +10,18 @@ import numpy as np
 import pytest
 
 from kyanite_amd import BinaryOp, DType, Graph, ReduceOp, UnaryOp
-from runner import check_cpu, check_gpu
+from runner import F16_MAX_REL, check_cpu, check_gpu
 
 SEEDS = list(range(48))
 DIMS = [1, 2, 3, 5, 8, 17, 32, 40, 64]
 
 
 class Builder:
-    def __init__(self, seed):
+    def __init__(self, seed, dtype=DType.F32):
         self.rng = np.random.default_rng(1000 + seed)
         self.g = Graph()
+        self.dtype = dtype
+        self.np_dtype = np.float16 if dtype == DType.F16 else np.float32
         self.inputs = []
         self.values = []  # (value, shape)
 
@@ -27,14 +29,17 @@ class Builder:
         return options[int(self.rng.integers(len(options)))]
 
     def new_input(self, shape):
-        v = self.g.input(list(shape))
-        self.inputs.append(self.rng.standard_normal(shape).astype(np.float32))
+        v = self.g.input(list(shape), self.dtype)
+        self.inputs.append(self.rng.standard_normal(shape).astype(self.np_dtype))
         self.values.append((v, tuple(shape)))
         return v
 
     def const(self, shape, scale=1.0):
-        data = (self.rng.standard_normal(shape) * scale).astype(np.float32)
-        return self.g.constant(list(shape), data)
+        data = (self.rng.standard_normal(shape) * scale).astype(self.np_dtype)
+        return self.g.constant(list(shape), data, self.dtype)
+
+    def scalar(self, x):
+        return self.g.scalar(float(x), self.dtype)
 
     def some_value(self, rank=None):
         candidates = [x for x in self.values if rank is None or len(x[1]) == rank]
@@ -78,7 +83,7 @@ class Builder:
 
     def op_scalar(self):
         v, shape = self.some_value()
-        c = self.g.scalar(float(self.pick([0.5, -1.25, 2.0, 0.125])))
+        c = self.scalar(self.pick([0.5, -1.25, 2.0, 0.125]))
         self.push(self.g.binary(self.pick([BinaryOp.MUL, BinaryOp.ADD]), v, c), shape)
 
     def op_relu(self):
@@ -127,7 +132,7 @@ class Builder:
         axes = sorted(int(a) for a in self.rng.choice(len(shape), n_axes, replace=False))
         op = self.pick([ReduceOp.SUM, ReduceOp.MEAN, ReduceOp.MAX, ReduceOp.MIN])
         if op == ReduceOp.SUM:
-            v = self.g.binary(BinaryOp.MUL, v, self.g.scalar(1.0 / 16))
+            v = self.g.binary(BinaryOp.MUL, v, self.scalar(1.0 / 16))
         out_shape = tuple(d for a, d in enumerate(shape) if a not in axes)
         out = self.g.reduce(v, axes, op)
         self.push(out, out_shape)
@@ -143,7 +148,7 @@ class Builder:
             return
         axis = int(self.rng.integers(len(shape)))
         if self.rng.integers(2):
-            v = self.g.binary(BinaryOp.MUL, v, self.g.scalar(0.5))
+            v = self.g.binary(BinaryOp.MUL, v, self.scalar(0.5))
         if self.rng.integers(3) == 0:
             small = tuple(1 if a == 0 else d for a, d in enumerate(shape))
             v = self.g.add(v, self.g.broadcast(self.const(small), list(shape)))
@@ -188,18 +193,23 @@ class Builder:
         n = self.pick(DIMS[1:])
         w = self.new_input((b, k, n)) if self.rng.integers(2) else self.g.broadcast(self.const((1, k, n)), [b, k, n])
         out = self.g.batched_mat_mul(v, w)
-        out = self.g.binary(BinaryOp.MUL, out, self.g.scalar(1.0 / np.sqrt(k)))
+        out = self.g.binary(BinaryOp.MUL, out, self.scalar(1.0 / np.sqrt(k)))
         self.push(out, (b, m, n))
 
     def op_attention(self):
         b, lq, lk = self.pick([1, 2, 3]), self.pick([5, 17, 40, 130]), self.pick([3, 33, 64, 150])
-        dk, dv = self.pick([32, 40, 64]), self.pick([8, 32, 40, 64])
+        f16 = self.dtype == DType.F16
+        dk, dv = self.pick([64, 128] if f16 else [32, 40, 64]), self.pick([8, 32, 40, 64] + ([96, 128] if f16 else []))
         q = self.new_input((b, lq, dk))
         k = self.new_input((b, lk, dk))
         v = self.new_input((b, lk, dv))
         scores = self.g.batched_mat_mul(q, self.g.permute(k, [0, 2, 1]))
         if self.rng.integers(3):
-            scores = self.g.binary(BinaryOp.MUL, scores, self.g.scalar(1.0 / np.sqrt(dk)))
+            scores = self.g.binary(BinaryOp.MUL, scores, self.scalar(1.0 / np.sqrt(dk)))
+        if f16 and self.rng.integers(2):
+            keep = np.tril(np.ones((lq, lk), bool), k=max(lk - lq, 0))
+            mask = self.g.constant([1, lq, lk], np.where(keep, 0.0, -np.inf).astype(np.float16)[None], DType.F16)
+            scores = self.g.add(scores, self.g.broadcast(mask, [b, lq, lk]))
         probs = self.g.softmax(scores, 2)
         self.push(self.g.batched_mat_mul(probs, v), (b, lq, dv))
         if self.rng.integers(4) == 0:
@@ -225,6 +235,8 @@ class Builder:
         ops = [self.op_unary, self.op_binary_same, self.op_binary_broadcast, self.op_scalar, self.op_relu, self.op_permute,
                self.op_slice, self.op_flip, self.op_view, self.op_reduce, self.op_softmax, self.op_layernorm,
                self.op_linear, self.op_linear, self.op_batched_matmul, self.op_attention, self.op_conv]
+        if self.dtype == DType.F16:
+            ops.remove(self.op_conv)  # convolutions are f32 only
         for _ in range(int(self.rng.integers(6, 16))):
             self.pick(ops)()
         # outputs: the last value and a few others (values with both a consumer and an output role)
@@ -236,12 +248,31 @@ class Builder:
         return self.g, self.inputs
 
 
+F16_SEEDS = list(range(100, 124))
+
+
 @pytest.mark.parametrize("seed", SEEDS)
 def test_cpu(seed):
     graph, inputs = Builder(seed).build()
     outputs = check_cpu(graph, 0, inputs)
     for o in outputs:
         assert np.all(np.isfinite(o)), "the generator is meant to keep values finite"
+
+
+@pytest.mark.parametrize("seed", F16_SEEDS)
+def test_cpu_f16(seed):
+    graph, inputs = Builder(seed, DType.F16).build()
+    outputs = check_cpu(graph, 0, inputs)
+    for o in outputs:
+        assert np.all(np.isfinite(o.astype(np.float32))), "the generator is meant to keep values finite"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", F16_SEEDS)
+def test_gpu_f16(seed, hip_device):
+    graph, inputs = Builder(seed, DType.F16).build()
+    print(f"random f16 graph seed {seed}: {len(graph)} values", flush=True)
+    check_gpu(hip_device, graph, 0, inputs, max_rel=F16_MAX_REL)
 
 
 @pytest.mark.gpu
