@@ -451,14 +451,19 @@ size_t pick_vec(const std::vector<KernelOperand> &ops, const Collapsed &c, size_
 // ------------------------------------------------------------------------------------------------ scalar kernel
 
 KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const ScalarExpr &expr) {
-    KN_ASSERT(!operands.empty());
+    return make_scalar_kernel_multi(operands, {expr});
+}
+
+KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, const std::vector<ScalarExpr> &exprs) {
+    const size_t n_out = exprs.size();
+    KN_ASSERT(n_out >= 1 && operands.size() >= n_out);
     const std::vector<size_t> &shape = operands[0].shape.shape();
     std::vector<std::vector<int64_t>> strides;
     for (auto &op : operands) {
         KN_ASSERT(op.shape.shape() == shape, "all operands of an elementwise kernel must have the same shape");
         strides.push_back(op.shape.strides());
     }
-    KN_ASSERT(expr.nodes.back().dtype == operands[0].dtype);
+    for (size_t o = 0; o < n_out; o++) KN_ASSERT(exprs[o].nodes.back().dtype == operands[o].dtype);
 
     KernelSpec spec;
     spec.name = "kn_scalar";
@@ -485,12 +490,17 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
         ss << "typedef " << storage_type(operands[k].dtype) << " S" << k << ";\n";
         if (vec > 1) ss << vec_type_decl("V" + std::to_string(k), operands[k].dtype, vec);
     }
-    // the fused expression
-    ss << "KN_DEV " << compute_type(operands[0].dtype) << " kn_op(";
-    for (size_t k = 1; k < operands.size(); k++) ss << (k > 1 ? ", " : "") << compute_type(operands[k].dtype) << " x" << k;
-    ss << ") {\n";
-    std::string res = emit_expr(ss, expr, "y", [&](size_t operand) { return "x" + std::to_string(operand); });
-    ss << "    return " << res << ";\n}\n";
+    // the fused expressions, one per output; every one takes all loaded operands
+    for (size_t o = 0; o < n_out; o++) {
+        ss << "KN_DEV " << compute_type(operands[o].dtype) << " kn_op" << o << "(";
+        for (size_t k = n_out; k < operands.size(); k++) ss << (k > n_out ? ", " : "") << compute_type(operands[k].dtype) << " x" << k;
+        ss << ") {\n";
+        std::string res = emit_expr(ss, exprs[o], "y", [&](size_t operand) {
+            KN_ASSERT(operand >= n_out && operand < operands.size());
+            return "x" + std::to_string(operand);
+        });
+        ss << "    return " << res << ";\n}\n";
+    }
 
     // dims in vector units along the last axis
     std::vector<size_t> dims = c.shape;
@@ -504,7 +514,7 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
     ss << "    const idx_t total = (idx_t) " << total_vecs << ";\n";
     ss << "    const idx_t base = (idx_t) blockIdx.x * (idx_t) (256 * UNROLL) + (idx_t) threadIdx.x;\n";
     ss << "    idx_t off[UNROLL][" << operands.size() << "];\n    bool ok[UNROLL];\n";
-    for (size_t k = 1; k < operands.size(); k++) {
+    for (size_t k = n_out; k < operands.size(); k++) {
         bool vload = vec > 1 && c.strides[k][rank - 1] == 1;
         ss << "    " << (vload ? "V" : "S") << k << " r" << k << "[UNROLL];\n";
     }
@@ -518,7 +528,7 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
         for (size_t k = 0; k < operands.size(); k++) offs.push_back("off[u][" + std::to_string(k) + "]");
         emit_decompose(ss, "            ", "v", dims, vstrides, offs);
     }
-    for (size_t k = 1; k < operands.size(); k++) {
+    for (size_t k = n_out; k < operands.size(); k++) {
         bool vload = vec > 1 && c.strides[k][rank - 1] == 1;
         if (vload)
             ss << "            r" << k << "[u] = "
@@ -528,29 +538,29 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
     ss << "        }\n    }\n";
     // phase 2: arithmetic and stores
     ss << "#pragma unroll\n    for (int u = 0; u < UNROLL; u++) {\n        if (ok[u]) {\n";
-    if (vec > 1) {
-        ss << "            V0 out;\n#pragma unroll\n            for (int j = 0; j < VEC; j++) {\n";
-        ss << "                out[j] = " << to_storage(operands[0].dtype, [&] {
-            std::string call = "kn_op(";
-            for (size_t k = 1; k < operands.size(); k++) {
-                bool vload = c.strides[k][rank - 1] == 1;
-                std::string e = vload ? "r" + std::to_string(k) + "[u][j]" : "r" + std::to_string(k) + "[u]";
-                call += (k > 1 ? ", " : "") + from_storage(operands[k].dtype, e);
+    for (size_t o = 0; o < n_out; o++) {
+        const std::string os_name = std::to_string(o);
+        auto call = [&](const std::string &j) {
+            std::string text = "kn_op" + os_name + "(";
+            for (size_t k = n_out; k < operands.size(); k++) {
+                bool vload = vec > 1 && c.strides[k][rank - 1] == 1;
+                std::string e = vload ? "r" + std::to_string(k) + "[u][" + j + "]" : "r" + std::to_string(k) + "[u]";
+                text += (k > n_out ? ", " : "") + from_storage(operands[k].dtype, e);
             }
-            return call + ")";
-        }()) << ";\n            }\n";
-        int64_t os = c.strides[0][rank - 1];
-        if (os == 1) ss << "            " << store_stmt("V0", "p0 + off[u][0]", "out", is_streaming(operands[0])) << "\n";
-        else {
-            // output is not contiguous along the vector axis (never picked by pick_vec, kept for completeness)
-            ss << "#pragma unroll\n            for (int j = 0; j < VEC; j++) p0[off[u][0] + (idx_t) j * (idx_t) " << os << "] = out[j];\n";
+            return text + ")";
+        };
+        if (vec > 1) {
+            ss << "            V" << o << " out" << o << ";\n#pragma unroll\n            for (int j = 0; j < VEC; j++) {\n";
+            ss << "                out" << o << "[j] = " << to_storage(operands[o].dtype, call("j")) << ";\n            }\n";
+            int64_t os = c.strides[o][rank - 1];
+            if (os == 1) ss << "            " << store_stmt("V" + os_name, "p" + os_name + " + off[u][" + os_name + "]", "out" + os_name, is_streaming(operands[o])) << "\n";
+            else {
+                // output is not contiguous along the vector axis (never picked by pick_vec, kept for completeness)
+                ss << "#pragma unroll\n            for (int j = 0; j < VEC; j++) p" << o << "[off[u][" << o << "] + (idx_t) j * (idx_t) " << os << "] = out" << o << "[j];\n";
+            }
+        } else {
+            ss << "            p" << o << "[off[u][" << o << "]] = " << to_storage(operands[o].dtype, call("0")) << ";\n";
         }
-    } else {
-        std::string call = "kn_op(";
-        for (size_t k = 1; k < operands.size(); k++)
-            call += (k > 1 ? ", " : "") + from_storage(operands[k].dtype, "r" + std::to_string(k) + "[u]");
-        call += ")";
-        ss << "            p0[off[u][0]] = " << to_storage(operands[0].dtype, call) << ";\n";
     }
     ss << "        }\n    }\n}\n";
 
@@ -558,6 +568,7 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
     spec.grid = ceil_div_u32(total_vecs, 256 * unroll);
     std::ostringstream note;
     note << "rank=" << rank << " vec=" << vec << " unroll=" << unroll << " idx=" << (idx64 ? 64 : 32);
+    if (n_out > 1) note << " outputs=" << n_out;
     spec.strategy = note.str();
     return spec;
 }

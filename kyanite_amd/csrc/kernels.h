@@ -47,6 +47,9 @@ struct KernelOperand {
 
 // out = expr(loads...). operands[0] is the output; the rest are the loaded operands, all of the same shape.
 KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const ScalarExpr &expr);
+// Several results from one pass: operands[0 .. exprs.size()) are the outputs, one expression each, the rest are the
+// loaded operands that all expressions share (Load nodes index the whole operand list).
+KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, const std::vector<ScalarExpr> &exprs);
 
 // output[kept] = post(fold(op, pre(input[kept, reduced...]))) (reduce.rs:35-153). `pre`: an optional elementwise
 // expression of the loaded element (its only operand is number 1), e.g. the square in a mean of squares.

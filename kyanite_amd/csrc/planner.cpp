@@ -300,17 +300,59 @@ private:
                 }
                 PlanTensor result = alloc_tensor_shared(result_shape, result_dtype);
                 size_t axis = op.axis(), start = 0;
+                // chains of the same shape (the two halves of a rotary embedding) share one launch and their loads
+                struct Pending {
+                    PlanTensor target;
+                    ScalarBlock *block;
+                    Value value;
+                };
+                std::vector<Pending> pending;
+                auto flush = [&]() {
+                    if (pending.empty()) return;
+                    if (pending.size() == 1) {
+                        pending[0].block->operands[0] = pending[0].target;
+                        plan_scalar_op(pending[0].block->expr, pending[0].block->operands, pending[0].value);
+                    } else {
+                        const size_t n_out = pending.size();
+                        std::vector<PlanTensor> operands;
+                        for (auto &pd : pending) operands.push_back(pd.target);
+                        std::vector<ScalarExpr> exprs;
+                        for (auto &pd : pending) {
+                            ScalarExpr expr = pd.block->expr;
+                            for (auto &node : expr.nodes) {
+                                if (node.kind != ScalarNode::Load) continue;
+                                const PlanTensor &t = pd.block->operands[node.operand];
+                                size_t at = n_out;
+                                while (at < operands.size() && !(operands[at] == t)) at++;
+                                if (at == operands.size()) operands.push_back(t);
+                                node.operand = at;
+                            }
+                            exprs.push_back(std::move(expr));
+                        }
+                        std::vector<KernelOperand> kops;
+                        for (auto &t : operands) kops.push_back(kop(t));
+                        Step step;
+                        step.kind = StepKind::ScalarOp;
+                        step.kernel = make_scalar_kernel_multi(kops, exprs);
+                        for (size_t k = 0; k < operands.size(); k++)
+                            step.operands.push_back({operands[k], k < n_out ? OperandKind::Out : OperandKind::In});
+                        push(std::move(step), pending[0].value);
+                    }
+                    pending.clear();
+                };
                 for (auto &piece : pieces) {
                     size_t len = graph[piece.value].shape.eval(batch_size)[axis];
                     PlanTensor target = result.slice(axis, SliceRange{start, start + len, 1});
                     if (piece.block) {
-                        piece.block->operands[0] = target;
-                        plan_scalar_op(piece.block->expr, piece.block->operands, piece.value);
+                        if (!pending.empty() && (pending[0].target.shape.shape() != target.shape.shape() || pending.size() >= 4)) flush();
+                        pending.push_back({target, &*piece.block, piece.value});
                     } else {
+                        flush();
                         plan_copy_tensor(*piece.tensor, target, value);
                     }
                     start += len;
                 }
+                flush();
                 return VT::done(result);
             }
             case OpKind::Conv: fail("Conv should have been handled by the conv fuser (only rank-4 f32 convolutions are supported)");

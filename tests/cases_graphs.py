@@ -1367,3 +1367,29 @@ def attention_f16_plain():
 @case
 def attention_f16_mask_on_the_left_no_scale():
     return _attention_f16_case(133, 2, 40, 72, 128, 96, False, "left")
+
+
+@case
+def concat_pieces_share_a_launch():
+    """pieces of a concat that are elementwise chains of one shape are computed by ONE kernel with several outputs
+    (a rotary embedding's two halves); a piece of another shape and a plain tensor in between get their own"""
+    g = Graph()
+    rng = np.random.default_rng(140)
+    x1, x2 = g.input([5, 24, 16]), g.input([5, 24, 16])
+    cos = g.broadcast(g.constant([1, 24, 16], np.cos(rng.standard_normal((1, 24, 16))).astype(np.float32)), [5, 24, 16])
+    sin = g.broadcast(g.constant([1, 24, 16], np.sin(rng.standard_normal((1, 24, 16))).astype(np.float32)), [5, 24, 16])
+    def chains(k):  # fresh values every time: a chain that two concats share is materialised instead
+        a = g.sub(g.mul(g.mul(x1, g.scalar(float(k))), cos), g.mul(x2, sin))
+        b = g.add(g.mul(g.mul(x1, g.scalar(float(k))), sin), g.mul(x2, cos))
+        c = g.unary(UnaryOp.TANH, g.add(g.mul(x1, g.scalar(float(k))), x2))
+        return a, b, c
+
+    other = g.unary(UnaryOp.NEG, g.input([5, 24, 3]))
+    a, b, _ = chains(1.5)
+    g.output(g.concat([a, b], 2))
+    a, b, c = chains(2.5)
+    g.output(g.concat([c, other, a, x1, b], 2))
+    a, b, c = chains(3.5)
+    g.output(g.concat([a, b, c], 1))
+    return g, 0, [rng.standard_normal((5, 24, 16)).astype(np.float32), rng.standard_normal((5, 24, 16)).astype(np.float32),
+                  rng.standard_normal((5, 24, 3)).astype(np.float32)], None
