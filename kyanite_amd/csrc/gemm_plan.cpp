@@ -59,8 +59,16 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // 512 x 11008 x 4096 82 / 87, 8192^3 1454 / 1439.
     static const int tall_below = env_int("KNHIP_F16_TALL_BELOW", 128);
     const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch * groups;
-    lp.tall_tile = f16 && groups == 1 && !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8 && can_split &&
-                   p.k >= 2048 && tall_blocks < tall_below;
+    const bool tall_fits = !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8;
+    lp.tall_tile = f16 && groups == 1 && tall_fits && can_split && p.k >= 2048 && tall_blocks < tall_below;
+    // Both operands with K contiguous in whole 16 byte vectors and K in whole slices of 64: given aligned
+    // pointers, the launch takes the kernel that loads global -> LDS directly. There the tall tiles run on a ring
+    // of three stages and also pay without a split, as long as they still fill the chip. Measured with weights
+    // that come from memory, not from cache (us, 128 x 128 on two stages against 256 x 128 on three):
+    // 512 x 22016 x 4096 147 / 133, 512 x 12288 x 4096 93 / 72, 4096^3 152 / 144; 512 x 4096 x 4096 53 / 59.
+    lp.direct = f16 && p.k > 0 && p.k % 64 == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % 8 == 0 && p.b_sn % 8 == 0 &&
+                (p.batch <= 1 || (p.a_sb % 8 == 0 && p.b_sb % 8 == 0));
+    if (lp.direct && tall_fits && tall_blocks >= env_int("KNHIP_F16_TALL_FROM", 128)) lp.tall_tile = true;
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile ? 64 : 128;

@@ -7,6 +7,13 @@
 // K^T of attention) move global -> register -> LDS as 128 bit vectors without being transposed.
 // The slices are double buffered in LDS: while slice s is multiplied, slice s + 1 waits in registers and slice
 // s + 2 is in flight from memory; one barrier per slice. The result is rounded to f16 once, at the store.
+//
+// When both operands have K contiguous, 16 byte aligned rows and K is a multiple of 64, a second kernel moves the
+// slices global -> LDS directly (global_load_lds_dwordx4: every lane names its own 16 source bytes, the wave's 64
+// vectors land side by side in LDS), with no trip through registers and no LDS write instructions. Rows are then
+// exactly 128 bytes with no padding, and bank conflicts are avoided by an XOR swizzle instead: the 16 byte chunk q
+// of row r sits at position q ^ (r % 8), which the loading lane arranges by choosing its source chunk and the
+// reading lane by flipping address bits.
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
@@ -95,15 +102,22 @@ struct Loader {
 // Tiles are numbered in bands of 8 tile rows, column by column within a band, so 8 k consecutive numbers are a patch
 // of 8 x k tiles. Workgroups are handed to the 8 XCDs (each with its own L2) in turn, workgroup i to XCD i % 8;
 // the renumbering below gives every XCD runs of `xcd_chunk` consecutive tile numbers (as many as it runs at a time),
-// so that the workgroups sharing an L2 cover one compact patch and find each other's operand tiles there.
+// so that the workgroups sharing an L2 cover one compact patch and find each other's operand tiles there. With 4
+// tile rows (m = 512) and 96 tile columns, a B tile whose 4 users sit on 4 XCDs is fetched from memory 4 times:
+// 103 us against 61 us for 512 x 12288 x 4096.
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_chunk, int *tm, int *tn) {
     int id = blockIdx.x;
     if (xcd_chunk > 0) {
-        const int per_round = 8 * xcd_chunk;
-        const int full = (int) (gridDim.x / per_round) * per_round;  // the tail keeps its numbers
+        const int total = (int) gridDim.x, per_round = 8 * xcd_chunk;
+        const int full = total / per_round * per_round;
+        const int xcd = id & 7;
         if (id < full) {
-            const int xcd = id & 7, local = id >> 3;
+            const int local = id >> 3;
             id = ((local / xcd_chunk) * 8 + xcd) * xcd_chunk + local % xcd_chunk;
+        } else {
+            // the last, partial round: one run per XCD again, as long as that XCD's share of the rest
+            const int rest = total - full, share = rest >> 3, extra = rest & 7;
+            id = full + xcd * share + min(xcd, extra) + ((id - full) >> 3);
         }
     }
     const int group_rows = 8;
@@ -112,6 +126,62 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_
     const int rows_here = min(group_rows, tiles_m - g * group_rows);
     *tm = g * group_rows + in_g % rows_here;
     *tn = in_g / rows_here;
+}
+
+// Stores the MI x NI MFMA tiles of a wave whose first row / column are row0 / col0. Accumulator layout of a 32 x 32
+// tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32.
+template <int MI, int NI>
+__device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 (&acc)[MI][NI], void *c_base, int bz, int row0, int col0) {
+    const int lane = threadIdx.x & 63, c = lane & 31, half = lane >> 5;
+    half_t *out = (half_t *) c_base + bz * p.c_sb;
+    float *partial = (float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n;
+    const bool split = gridDim.z > 1;
+    // the epilogue of a split launch is applied by the pass that sums the partial products
+    const half_t *addend = p.addend ? (const half_t *) p.addend + bz * p.d_sb : nullptr;
+    // Tiles that lie inside the matrix, with offsets that fit 32 bits, skip the bounds checks and the 64 bit
+    // address arithmetic (which otherwise cost about a tenth of a 512 x 12288 x 4096 launch).
+    const long long reach = (long long) (p.m - 1) * p.c_sm + p.n, d_reach = (long long) (p.m - 1) * p.d_sm + (long long) (p.n - 1) * p.d_sn;
+    const bool fast = !split && p.c_sn == 1 && p.c_sm > 0 && reach < 0x7fffffffll && row0 + 32 * MI <= p.m && col0 + 32 * NI <= p.n &&
+                      (!addend || (p.d_sm >= 0 && p.d_sn >= 0 && d_reach < 0x7fffffffll));
+    if (fast) {
+        const int c_sm = (int) p.c_sm, d_sm = (int) p.d_sm, d_sn = (int) p.d_sn;
+        half_t *tile = out + (row0 + 4 * half) * c_sm + col0 + c;
+        const half_t *d_tile = addend ? addend + (row0 + 4 * half) * d_sm + (col0 + c) * d_sn : nullptr;
+        const bool relu = p.relu != 0;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = 32 * i + 8 * (v >> 2) + (v & 3);
+                    half_t x = (half_t) acc[i][j][v];
+                    if (d_tile) x = (half_t) ((float) x + (float) d_tile[r * d_sm + 32 * j * d_sn]);
+                    if (relu) x = x > (half_t) 0 ? x : (half_t) 0;
+                    tile[r * c_sm + 32 * j] = x;
+                }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NI; j++) {
+            const int col = col0 + 32 * j + c;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = row0 + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+                if (row < p.m && col < p.n) {
+                    if (split) {
+                        partial[(long long) row * p.n + col] = acc[i][j][v];
+                    } else {
+                        half_t r = (half_t) acc[i][j][v];
+                        if (addend) r = (half_t) ((float) r + (float) addend[(long long) row * p.d_sm + (long long) col * p.d_sn]);
+                        if (p.relu) r = r > (half_t) 0 ? r : (half_t) 0;
+                        out[(long long) row * p.c_sm + (long long) col * p.c_sn] = r;
+                    }
+                }
+            }
+        }
 }
 
 // TI: MFMA tiles per wave and axis; WM: waves along M (2 along N), so the workgroup tile is (32 TI WM) x (64 TI):
@@ -190,32 +260,143 @@ __global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_
         }
     }
 
-    // accumulator layout of the 32x32 tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32
-    half_t *out = (half_t *) c_base + bz * p.c_sb;
-    float *partial = (float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n;
-    const bool split = gridDim.z > 1;
-    // the epilogue of a split launch is applied by the pass that sums the partial products
-    const half_t *addend = p.addend ? (const half_t *) p.addend + bz * p.d_sb : nullptr;
+    store_tiles<TI, TI>(p, acc, c_base, bz, m0 + wm * 32 * TI, n0 + wn * 32 * TI);
+}
+
+constexpr int DIRECT_BK = 64;
+
+template <int N>
+__device__ __forceinline__ void wait_for_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// The direct-to-LDS kernel: a workgroup of WM x WN waves owns a (32 MI WM) x (32 NI WN) tile, a wave MI x NI MFMA
+// tiles of it. K is walked in slices of 64 through a ring of NSTAGE LDS stages; every stage holds the rows of A,
+// then those of B, 128 bytes each. One load instruction of a wave fills 8 rows (64 chunks of 16 bytes): lane l fills chunk
+// position l % 8 of row l / 8, so it fetches chunk (l % 8) ^ (l / 8) of that row. Rows past the edge of a matrix
+// repeat its last row; they only feed results that are not stored.
+// Per slice: wait for the own loads of this slice (those of the NSTAGE - 2 slices after it may still be in
+// flight), barrier (now everybody's have landed, and everybody is done reading the stage of the slice before),
+// start the loads of slice s + NSTAGE - 1 into that stage, multiply.
+// One slice of both operands on its way, global -> LDS: load i of the wave fills the 1024 bytes at dst + 1024 i,
+// lane l the 16 bytes at 16 l of them from its own source address, which then moves on by `advance` elements.
+// (The host pass of the compiler does not know the load instruction, hence the guard.)
+template <int A_LD, int B_LD>
+__device__ __forceinline__ void issue_loads(const half_t *(&a_src)[A_LD], const half_t *(&b_src)[B_LD], char *dst_a, char *dst_b, int advance) {
+#if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
-    for (int i = 0; i < TI; i++)
+    for (int i = 0; i < A_LD; i++) {
+        __builtin_amdgcn_global_load_lds(a_src[i], dst_a + i * 1024, 16, 0, 0);
+        a_src[i] += advance;
+    }
 #pragma unroll
-        for (int j = 0; j < TI; j++) {
-            const int col = n0 + wn * 32 * TI + 32 * j + c;
+    for (int i = 0; i < B_LD; i++) {
+        __builtin_amdgcn_global_load_lds(b_src[i], dst_b + i * 1024, 16, 0, 0);
+        b_src[i] += advance;
+    }
+#endif
+}
+
+template <int MI, int NI, int WM, int WN, int NSTAGE>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParams p, int k_chunk, int xcd_chunk) {
+    constexpr int WAVES = WM * WN, TM = 32 * MI * WM, TN = 32 * NI * WN, ROW = 2 * DIRECT_BK;
+    constexpr int A_BYTES = TM * ROW, STAGE = (TM + TN) * ROW;
+    constexpr int A_LD = TM / 8 / WAVES, B_LD = TN / 8 / WAVES;  // load instructions per wave and stage
+    static_assert(A_LD >= 1 && B_LD >= 1 && ROW == 128 && NSTAGE >= 2, "tile too small for the workgroup");
+    static_assert((NSTAGE - 2) * (A_LD + B_LD) < 64, "the counter of loads in flight has 6 bits");
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
+    int tm, tn;
+    tile_of_block(tiles_m, tiles_n * p.groups, xcd_chunk, &tm, &tn);
+    const int group = tn / tiles_n;
+    tn -= group * tiles_n;
+    const void *b_base = p.groups > 1 ? p.b_group[group] : p.b;
+    void *c_base = p.groups > 1 ? p.c_group[group] : p.c;
+    const int bz = blockIdx.y;
+    const int m0 = tm * TM, n0 = tn * TN;
+    const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
+    const int slices = (k_end - k_begin) / DIRECT_BK;
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / WN, wn = wave % WN, c = lane & 31, half = lane >> 5;
+
+    // the source of every load of this lane; all of them move on by one slice per issue
+    const half_t *a_src[A_LD], *b_src[B_LD];
+    {
+        const int lr = lane >> 3, chunk = (lane & 7) ^ lr;
+        const half_t *a0 = (const half_t *) p.a + bz * p.a_sb + k_begin + 8 * chunk;
+        const half_t *b0 = (const half_t *) b_base + bz * p.b_sb + k_begin + 8 * chunk;
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int row = m0 + wm * 32 * TI + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
-                if (row < p.m && col < p.n) {
-                    if (split) {
-                        partial[(long long) row * p.n + col] = acc[i][j][v];
-                    } else {
-                        half_t r = (half_t) acc[i][j][v];
-                        if (addend) r = (half_t) ((float) r + (float) addend[(long long) row * p.d_sm + (long long) col * p.d_sn]);
-                        if (p.relu) r = r > (half_t) 0 ? r : (half_t) 0;
-                        out[(long long) row * p.c_sm + (long long) col * p.c_sn] = r;
-                    }
-                }
-            }
+        for (int i = 0; i < A_LD; i++) a_src[i] = a0 + (long long) min(m0 + (wave * A_LD + i) * 8 + lr, p.m - 1) * p.a_sm;
+#pragma unroll
+        for (int i = 0; i < B_LD; i++) b_src[i] = b0 + (long long) min(n0 + (wave * B_LD + i) * 8 + lr, p.n - 1) * p.b_sn;
+    }
+    // MFMA operand of lane (row c, half h) at step t: chunk 2 t + h of its row, found at (2 t + h) ^ (c % 8), which
+    // is the address of step 0 with bits 5 and 6 flipped by t
+    const unsigned a_rd = (wm * 32 * MI + c) * ROW + ((half ^ (c & 7)) * 16);
+    const unsigned b_rd = A_BYTES + (wn * 32 * NI + c) * ROW + ((half ^ (c & 7)) * 16);
+
+    floatx16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NI; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    // The loop is kept free of branches (which make the compiler shuttle the accumulators between register
+    // files): the stages rotate through address arithmetic, and once no slice is left to fetch, the last one is
+    // fetched again into a stage that nobody reads any more.
+    char *const dst_a = lds + wave * A_LD * 1024, *const dst_b = lds + A_BYTES + wave * B_LD * 1024;
+#pragma unroll
+    for (int j = 0; j < NSTAGE - 1; j++)
+        issue_loads<A_LD, B_LD>(a_src, b_src, dst_a + j * STAGE, dst_b + j * STAGE, j + 1 < slices ? DIRECT_BK : 0);
+    unsigned stage_off = 0, fill_off = (NSTAGE - 1) * STAGE;
+    for (int s = 0; s < slices; s++) {
+        wait_for_loads<(NSTAGE - 2) * (A_LD + B_LD)>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_loads<A_LD, B_LD>(a_src, b_src, dst_a + fill_off, dst_b + fill_off, s + NSTAGE < slices ? DIRECT_BK : 0);
+        const char *st = lds + stage_off;
+#pragma unroll
+        for (int t = 0; t < DIRECT_BK / 16; t++) {
+            halfx8 a[MI], b[NI];
+#pragma unroll
+            for (int i = 0; i < MI; i++) a[i] = *(const halfx8 *) (st + (a_rd ^ (32 * t)) + i * 32 * ROW);
+#pragma unroll
+            for (int j = 0; j < NI; j++) b[j] = *(const halfx8 *) (st + (b_rd ^ (32 * t)) + j * 32 * ROW);
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NI; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
         }
+        fill_off = stage_off;
+        stage_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
+    }
+    wait_for_loads<0>();
+    store_tiles<MI, NI>(p, acc, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
+}
+
+template <int MI, int NI, int WM, int WN, int NSTAGE>
+int launch_direct(dim3 grid, hipStream_t stream, const GemmParams &p, int kc, int xc) {
+    constexpr int LDS_BYTES = NSTAGE * (32 * MI * WM + 32 * NI * WN) * 2 * DIRECT_BK;
+    auto kernel = gemm_f16_direct_kernel<MI, NI, WM, WN, NSTAGE>;
+    // more than 64 KB of dynamic LDS has to be asked for, once per device
+    static bool allowed[64] = {};
+    int device = 0;
+    if (LDS_BYTES > 64 * 1024) {
+        int e = (int) hipGetDevice(&device);
+        if (e == 0 && (device < 0 || device >= 64)) e = (int) hipErrorInvalidDevice;
+        if (e == 0 && !allowed[device]) {
+            e = (int) hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+            if (e == 0) allowed[device] = true;
+        }
+        if (e != 0) return e;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * WM * WN), LDS_BYTES, stream, p, kc, xc);
+    return 0;
 }
 
 // `so` / `sk`: element strides of the outer and the K axis; vectors of 8 halves must be aligned and must not
@@ -272,7 +453,16 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     // workgroups an XCD (32 compute units) runs at a time: 1 per compute unit for the tall tiles, else 2
     static const int xc_env = getenv("KNHIP_XCD_CHUNK") ? atoi(getenv("KNHIP_XCD_CHUNK")) : -1;
     const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile ? 32 : 64);
-    if (lp.small_tile) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
+    // both operands K contiguous and K (and every split of it) whole slices: the direct-to-LDS kernel
+    static const int direct_env = getenv("KNHIP_F16_DIRECT") ? atoi(getenv("KNHIP_F16_DIRECT")) : 1;
+    const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % DIRECT_BK == 0;
+    if (direct) {
+        int e;
+        if (lp.small_tile) e = launch_direct<1, 1, 2, 2, 2>(grid, stream, p, lp.k_chunk, xc);
+        else if (lp.tall_tile) e = launch_direct<2, 2, 4, 2, 3>(grid, stream, p, lp.k_chunk, xc);
+        else e = launch_direct<2, 2, 2, 2, 2>(grid, stream, p, lp.k_chunk, xc);
+        if (e != 0) return e;
+    } else if (lp.small_tile) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     else if (lp.tall_tile) launch_a<2, 64, 1, 4>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     else launch_a<2, 128, 1, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     int e = (int) hipGetLastError();

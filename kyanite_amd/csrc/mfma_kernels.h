@@ -44,6 +44,7 @@ struct GemmLaunchPlan {
     GemmParams p;            // operands swapped where needed so that the contiguous axis of C is the column axis
     bool small_tile;         // 64 x 64 workgroup tiles instead of 128 x 128
     bool tall_tile;          // f16 only: 256 x 128 workgroup tiles (8 waves)
+    bool direct;             // f16 only: shapes and strides allow the kernel that loads global -> LDS directly
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)
     int k_chunk;             // K elements per split, a multiple of bk

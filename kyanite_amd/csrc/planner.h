@@ -87,6 +87,7 @@ struct PlannerOptions {
     bool fuse_row_epilogue = true;  // fold elementwise consumers of a layernorm / softmax into the row kernel
     bool fuse_matmul_epilogue = true;  // fold `+ d` and `max(., 0)` after a matmul into the matmul's store
     bool fuse_attention = true;  // matmul, softmax, matmul chains in f32 run as one launch
+    bool pack_matmul_constants = true;  // constant [k, n] right operands of f16 matmuls are laid out again as [n, k]
     bool group_matmuls = true;   // matmuls that share their left operand and have constant right operands share a launch
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;

@@ -1393,3 +1393,82 @@ def concat_pieces_share_a_launch():
     g.output(g.concat([a, b, c], 1))
     return g, 0, [rng.standard_normal((5, 24, 16)).astype(np.float32), rng.standard_normal((5, 24, 16)).astype(np.float32),
                   rng.standard_normal((5, 24, 3)).astype(np.float32)], None
+
+
+# ---- f16 matmuls whose operands both have K contiguous and a multiple of 64: slices go global -> LDS directly
+
+@case
+def f16_matmul_direct_tiles():
+    """all three tile shapes of the direct kernel: 128 x 128 with ragged rows and columns (the edge rows repeat
+    the last row) and an odd number of slices, over a batch; 64 x 64 with one slice and with two; 256 x 128 with
+    the K axis split"""
+    g = Graph()
+    rng = np.random.default_rng(150)
+    a = g.input([16, 264, 192], DType.F16)
+    b = g.input([16, 328, 192], DType.F16)
+    big = g.batched_mat_mul(a, g.permute(b, [0, 2, 1]))
+    s = g.input([72, 128], DType.F16)
+    w1 = g.constant([200, 64], _f16(rng, 200, 64, scale=0.1))
+    w2 = g.constant([40, 128], _f16(rng, 40, 128, scale=0.1))
+    small_one = g.linear(g.slice(s, 1, 0, 64), w1)
+    small_two = g.linear(s, w2)
+    t = g.input([500, 4096], DType.F16)
+    w3 = g.constant([384, 4096], _f16(rng, 384, 4096, scale=0.05))
+    g.output_all([big, small_one, small_two, g.linear(t, w3)])
+    return g, 0, [_f16(rng, 16, 264, 192, scale=0.2), _f16(rng, 16, 328, 192, scale=0.2), _f16(rng, 72, 128),
+                  _f16(rng, 500, 4096)], None
+
+
+@case
+def f16_matmul_direct_epilogue():
+    """bias and relu in the store of the direct kernel, with and without a split of K"""
+    g = Graph()
+    rng = np.random.default_rng(151)
+    x = g.input([300, 256], DType.F16)
+    w = g.constant([520, 256], _f16(rng, 520, 256, scale=0.1))
+    bias = g.constant([1, 520], _f16(rng, 1, 520))
+    y = g.relu(g.add(g.linear(x, w), bias))
+    long_x = g.input([40, 2048], DType.F16)
+    long_w = g.constant([72, 2048], _f16(rng, 72, 2048, scale=0.05))
+    res = g.input([40, 72], DType.F16)
+    z = g.add(g.linear(long_x, long_w), res)
+    g.output_all([y, z])
+    return g, 0, [_f16(rng, 300, 256), _f16(rng, 40, 2048), _f16(rng, 40, 72)], None
+
+
+@case
+def f16_matmul_constant_weights_laid_out_again():
+    """constant [k, n] right operands (`x @ w`) get a [n, k] copy at planning time: a single product, three that
+    share their left operand (one launch), a weight that an elementwise op reads as well (the original stays), a
+    slice of a bigger constant, and a weight broadcast over a batch"""
+    g = Graph()
+    rng = np.random.default_rng(152)
+    x = g.input([48, 128], DType.F16)
+    w = g.constant([128, 72], _f16(rng, 128, 72, scale=0.1))
+    single = g.mat_mul(g.unary(UnaryOp.TANH, x), w)
+    qkv = [g.mat_mul(x, g.constant([128, 136], _f16(rng, 128, 136, scale=0.1))) for _ in range(3)]
+    shared = g.constant([128, 40], _f16(rng, 128, 40, scale=0.1))
+    both = g.mat_mul(g.unary(UnaryOp.NEG, x), shared)
+    doubled = g.mul(shared, g.scalar(2.0, DType.F16))
+    big = g.constant([192, 100], _f16(rng, 192, 100, scale=0.1))
+    sliced = g.mat_mul(g.unary(UnaryOp.ABS, x), g.slice(g.slice(big, 0, 64, 192), 1, 4, 84))
+    xb = g.input([3, 48, 64], DType.F16)
+    wb = g.constant([1, 64, 24], _f16(rng, 1, 64, 24, scale=0.1))
+    batched = g.batched_mat_mul(xb, g.broadcast(wb, [3, 64, 24]))
+    g.output_all([single] + qkv + [both, doubled, sliced, batched])
+    return g, 0, [_f16(rng, 48, 128), _f16(rng, 3, 48, 64)], None
+
+
+@case
+def f16_matmul_direct_tall_ring():
+    """256 x 128 tiles on the ring of three stages without a split of K: a batch with fewer slices (2) than
+    stages and ragged columns, and three projections of one input in one launch with exactly 3 slices"""
+    g = Graph()
+    rng = np.random.default_rng(153)
+    a = g.input([16, 256, 128], DType.F16)
+    b = g.input([16, 1000, 128], DType.F16)
+    g.output(g.batched_mat_mul(a, g.permute(b, [0, 2, 1])))
+    x = g.input([512, 192], DType.F16)
+    for _ in range(3):
+        g.output(g.linear(x, g.constant([2816, 192], _f16(rng, 2816, 192, scale=0.1))))
+    return g, 0, [_f16(rng, 16, 256, 128, scale=0.2), _f16(rng, 16, 1000, 128, scale=0.2), _f16(rng, 512, 192)], None

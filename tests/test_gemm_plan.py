@@ -4,7 +4,7 @@ import re
 
 import numpy as np
 
-from kyanite_amd import DType, Graph, HipExecutor
+from kyanite_amd import DType, Graph, HipExecutor, UnaryOp
 
 
 def plan(m, n, k, batch=1, dtype=DType.F32):
@@ -120,3 +120,30 @@ def test_projections_of_one_input_share_a_launch():
     # where even the group leaves the chip short of tiles, the products run apart and split K
     ex = HipExecutor(0, _projections(2, 8, 4096, 256), 0, plan_only=True)
     assert ex.step_count() == 2 and all("grouped" not in ex.step_str(i) for i in range(2))
+
+
+def test_constant_weights_are_laid_out_again_for_f16_matmuls(monkeypatch):
+    """A constant [k, n] right operand of an f16 matmul is replaced by a [n, k] copy made at planning time; the
+    original takes no room in the arena unless something else reads it."""
+    def graph(also_elementwise):
+        g = Graph()
+        x = g.input([64, 128], DType.F16)
+        w = g.constant([128, 256], np.ones((128, 256), np.float16), DType.F16)
+        g.output(g.mat_mul(x, w))
+        if also_elementwise:
+            g.output(g.unary(UnaryOp.NEG, w))
+        return g
+
+    weight_bytes = 128 * 256 * 2
+    assert HipExecutor(0, graph(False), 0, plan_only=True).mem_usage["dedicated_bytes"] == weight_bytes
+    assert HipExecutor(0, graph(True), 0, plan_only=True).mem_usage["dedicated_bytes"] == 2 * weight_bytes
+    monkeypatch.setenv("KNHIP_PACK_CONSTANTS", "0")
+    assert HipExecutor(0, graph(True), 0, plan_only=True).mem_usage["dedicated_bytes"] == weight_bytes
+    # f32 matmuls and K axes that are no multiple of 64 keep the operand as it is
+    monkeypatch.delenv("KNHIP_PACK_CONSTANTS")
+    g = Graph()
+    x = g.input([64, 96], DType.F16)
+    w = g.constant([96, 256], np.ones((96, 256), np.float16), DType.F16)
+    g.output(g.mat_mul(x, w))
+    g.output(g.unary(UnaryOp.NEG, w))
+    assert HipExecutor(0, g, 0, plan_only=True).mem_usage["dedicated_bytes"] == 96 * 256 * 2
