@@ -85,7 +85,9 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             step.attn.o = l.ptrs.back();
         } else if (step.kind == StepKind::MatMul && step.gemm.groups > 1) {
             const size_t groups = (size_t) step.gemm.groups;
-            KN_ASSERT(l.ptrs.size() == 1 + 2 * groups);
+            const GemmLaunchPlan lp = plan_gemm_launch(step.gemm, step.gemm_f16);
+            size_t next = 1 + 2 * groups;
+            KN_ASSERT(l.ptrs.size() == next + (lp.workspace_bytes > 0) + (lp.counter_bytes > 0));
             step.gemm.a = l.ptrs[0];
             for (size_t g = 0; g < groups; g++) {
                 step.gemm.b_group[g] = l.ptrs[1 + g];
@@ -93,13 +95,18 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             }
             step.gemm.b = step.gemm.b_group[0];
             step.gemm.c = step.gemm.c_group[0];
+            step.gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;
+            step.gemm.counters = lp.counter_bytes > 0 ? l.ptrs[next++] : nullptr;
         } else if (step.kind == StepKind::MatMul) {
             step.gemm.a = l.ptrs[0];
             step.gemm.b = l.ptrs[1];
             step.gemm.c = l.ptrs[2];
             size_t next = 3;
             step.gemm.addend = step.gemm_has_addend ? l.ptrs[next++] : nullptr;
-            step.gemm.workspace = l.ptrs.size() > next ? l.ptrs[next] : nullptr;
+            const GemmLaunchPlan lp = plan_gemm_launch(step.gemm, step.gemm_f16);
+            KN_ASSERT(l.ptrs.size() == next + (lp.workspace_bytes > 0) + (lp.counter_bytes > 0));
+            step.gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;
+            step.gemm.counters = lp.counter_bytes > 0 ? l.ptrs[next++] : nullptr;
         } else if (step.kind == StepKind::Conv) {
             size_t k = 0;
             step.conv.input = (const float *) l.ptrs[k++];

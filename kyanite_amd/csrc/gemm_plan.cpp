@@ -33,6 +33,8 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     lp.p = p;
     lp.split_k = 1;
     lp.k_chunk = p.k;
+    lp.tail_split = 1;
+    lp.tail_k_chunk = p.k;
     if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return lp;
 
     // 128 x 128 tiles unless there are too few of them to fill the chip. Measured thresholds: f32 344 tiles run
@@ -69,13 +71,52 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     lp.direct = f16 && p.k > 0 && p.k % 64 == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % 8 == 0 && p.b_sn % 8 == 0 &&
                 (p.batch <= 1 || (p.a_sb % 8 == 0 && p.b_sb % 8 == 0));
     if (lp.direct && tall_fits && tall_blocks >= env_int("KNHIP_F16_TALL_FROM", 128)) lp.tall_tile = true;
+    // Direct kernel only: 128 x 64 tiles on a ring of four stages, where 128 x 128 tiles leave compute units
+    // without a workgroup and K is too short for a split to pay (512 x 4096 x 4096: 29 us against 39 us on
+    // 256 x 128 tiles split in four; 512 x 4096 x 11008: 84 us against 69 us).
+    const long long narrow_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 63) / 64) * p.batch * groups;
+    lp.narrow_tile = lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= env_int("KNHIP_F16_NARROW_FROM", 192) &&
+                     p.k < env_int("KNHIP_F16_NARROW_K_BELOW", 8192);
+    if (lp.narrow_tile) lp.small_tile = lp.tall_tile = false;
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
-    if (f16) lp.bk = lp.small_tile || lp.tall_tile ? 64 : 128;
+    if (lp.narrow_tile) blocks = narrow_blocks;
+    if (f16) lp.bk = lp.small_tile || lp.tall_tile || lp.narrow_tile ? 64 : 128;
     else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
 
+    // A tile count that leaves the last round of workgroups mostly idle: the direct kernel splits the tiles of just
+    // that round along K and sums the parts inside the launch, so that the round is short instead of sparse.
+    // 344 tiles on 256 compute units run as one full round and 88 tiles in two halves each, instead of a second
+    // round on a third of the chip (512 x 11008 x 4096 twice in one launch: 137 us -> 119 us). The partial tiles
+    // pass between workgroups with accesses that bypass the L2 caches, which costs more than the second launch
+    // of a plain split; so a launch with less than one round of tiles keeps that (512 x 4096 x 11008: 69 us
+    // against 82 us).
+    static const int tail_enabled = env_int("KNHIP_F16_TAIL_SPLIT", 1);
+    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled) {
+        const long long slots = 256 * (lp.tall_tile || lp.narrow_tile ? 1 : 2);
+        const long long full = blocks / slots * slots, rest = blocks - full;
+        long long s = rest > 0 ? slots / rest : 1;
+        if (s > p.k / 512) s = p.k / 512;
+        if (s > 16) s = 16;
+        if (full > 0 && rest * 100 < slots * env_int("KNHIP_F16_TAIL_BELOW", 85) && s >= 2 && blocks <= 0x3fffffff) {
+            long long chunk = (p.k + s - 1) / s;
+            chunk = (chunk + 63) / 64 * 64;
+            s = (p.k + chunk - 1) / chunk;
+            const int tm = lp.tall_tile ? 256 : (lp.small_tile ? 64 : 128), tn = lp.small_tile || lp.narrow_tile ? 64 : 128;
+            const unsigned long long bytes = (unsigned long long) rest * s * tm * tn * 4ull;
+            if (s >= 2 && bytes <= (256ull << 20)) {
+                lp.head_tiles = (int) full;
+                lp.tail_split = (int) s;
+                lp.tail_k_chunk = (int) chunk;
+                lp.workspace_bytes = (size_t) bytes;
+                lp.counter_bytes = (size_t) rest * 4;
+                return lp;
+            }
+        }
+    }
+
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
-    if (can_split && blocks < split_below && groups == 1) {
+    if (can_split && blocks < split_below && groups == 1 && !lp.narrow_tile) {
         const int min_chunk = few_tiles ? 128 : (f16 ? 512 : 256);  // K elements a split should at least cover
         long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;

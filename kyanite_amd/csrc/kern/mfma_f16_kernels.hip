@@ -26,6 +26,8 @@ namespace {
 
 typedef _Float16 half_t;
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 
@@ -105,10 +107,9 @@ struct Loader {
 // so that the workgroups sharing an L2 cover one compact patch and find each other's operand tiles there. With 4
 // tile rows (m = 512) and 96 tile columns, a B tile whose 4 users sit on 4 XCDs is fetched from memory 4 times:
 // 103 us against 61 us for 512 x 12288 x 4096.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int xcd_chunk, int *tm, int *tn) {
-    int id = blockIdx.x;
+__device__ __forceinline__ void tile_of_block(int id, int total, int tiles_m, int tiles_n, int xcd_chunk, int *tm, int *tn) {
     if (xcd_chunk > 0) {
-        const int total = (int) gridDim.x, per_round = 8 * xcd_chunk;
+        const int per_round = 8 * xcd_chunk;
         const int full = total / per_round * per_round;
         const int xcd = id & 7;
         if (id < full) {
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_
     // a grouped launch lines the tiles of its products up along n
     const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n * p.groups, xcd_chunk, &tm, &tn);
+    tile_of_block((int) blockIdx.x, (int) gridDim.x, tiles_m, tiles_n * p.groups, xcd_chunk, &tm, &tn);
     const int group = tn / tiles_n;
     tn -= group * tiles_n;
     const void *b_base = p.groups > 1 ? p.b_group[group] : p.b;
@@ -270,14 +271,6 @@ __device__ __forceinline__ void wait_for_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// The direct-to-LDS kernel: a workgroup of WM x WN waves owns a (32 MI WM) x (32 NI WN) tile, a wave MI x NI MFMA
-// tiles of it. K is walked in slices of 64 through a ring of NSTAGE LDS stages; every stage holds the rows of A,
-// then those of B, 128 bytes each. One load instruction of a wave fills 8 rows (64 chunks of 16 bytes): lane l fills chunk
-// position l % 8 of row l / 8, so it fetches chunk (l % 8) ^ (l / 8) of that row. Rows past the edge of a matrix
-// repeat its last row; they only feed results that are not stored.
-// Per slice: wait for the own loads of this slice (those of the NSTAGE - 2 slices after it may still be in
-// flight), barrier (now everybody's have landed, and everybody is done reading the stage of the slice before),
-// start the loads of slice s + NSTAGE - 1 into that stage, multiply.
 // One slice of both operands on its way, global -> LDS: load i of the wave fills the 1024 bytes at dst + 1024 i,
 // lane l the 16 bytes at 16 l of them from its own source address, which then moves on by `advance` elements.
 // (The host pass of the compiler does not know the load instruction, hence the guard.)
@@ -297,8 +290,30 @@ __device__ __forceinline__ void issue_loads(const half_t *(&a_src)[A_LD], const 
 #endif
 }
 
+// The direct-to-LDS kernel: a workgroup of WM x WN waves owns a (32 MI WM) x (32 NI WN) tile, a wave MI x NI MFMA
+// tiles of it. K is walked in slices of 64 through a ring of NSTAGE LDS stages; every stage holds the rows of A,
+// then those of B, 128 bytes each. One load instruction of a wave fills 8 rows (64 chunks of 16 bytes): lane l fills chunk
+// position l % 8 of row l / 8, so it fetches chunk (l % 8) ^ (l / 8) of that row. Rows past the edge of a matrix
+// repeat its last row; they only feed results that are not stored.
+// Per slice: wait for the own loads of this slice (those of the NSTAGE - 2 slices after it may still be in
+// flight), barrier (now everybody's have landed, and everybody is done reading the stage of the slice before),
+// start the loads of slice s + NSTAGE - 1 into that stage, multiply.
+//
+// Tiles can share the launch in two ways. The first `head_tiles` tiles (in launch order) are computed by one
+// workgroup each, over all of K. Every further tile is shared by `tail_split` workgroups, which take
+// `tail_k_chunk` of K each, park their f32 partial tile in the workspace and count themselves in on the tile's
+// counter; whoever comes last adds the partial tiles up (always in the order of K, so the result does not depend on
+// who that is), applies the epilogue, stores, and puts the counter back to zero for the next launch. A launch
+// with too few tiles for the chip splits all of them (head_tiles = 0); one whose tile count leaves the last round
+// of workgroups mostly idle splits just that round, so that it is short instead of sparse.
+struct DirectSchedule {
+    int k_chunk;     // split over gridDim.z, partial products summed by a second launch (batched products)
+    int xcd_chunk;
+    int head_tiles, tail_split, tail_k_chunk;
+};
+
 template <int MI, int NI, int WM, int WN, int NSTAGE>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParams p, int k_chunk, int xcd_chunk) {
+__global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParams p, DirectSchedule sched) {
     constexpr int WAVES = WM * WN, TM = 32 * MI * WM, TN = 32 * NI * WN, ROW = 2 * DIRECT_BK;
     constexpr int A_BYTES = TM * ROW, STAGE = (TM + TN) * ROW;
     constexpr int A_LD = TM / 8 / WAVES, B_LD = TN / 8 / WAVES;  // load instructions per wave and stage
@@ -307,15 +322,29 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
     const int tiles_m = (p.m + TM - 1) / TM, tiles_n = (p.n + TN - 1) / TN;
+    const int tiles = tiles_m * tiles_n * p.groups;
+    // which tile, and which part of K
+    int tile_id = (int) blockIdx.x, chunk = 0;
+    const bool shared_tile = tile_id >= sched.head_tiles;
+    if (shared_tile) {
+        const int t = tile_id - sched.head_tiles;
+        tile_id = sched.head_tiles + t / sched.tail_split;
+        chunk = t % sched.tail_split;
+    }
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n * p.groups, xcd_chunk, &tm, &tn);
+    if (shared_tile) tile_of_block(tile_id, tiles, tiles_m, tiles_n * p.groups, 0, &tm, &tn);
+    else tile_of_block(tile_id, sched.head_tiles, tiles_m, tiles_n * p.groups, sched.xcd_chunk, &tm, &tn);
     const int group = tn / tiles_n;
     tn -= group * tiles_n;
     const void *b_base = p.groups > 1 ? p.b_group[group] : p.b;
     void *c_base = p.groups > 1 ? p.c_group[group] : p.c;
     const int bz = blockIdx.y;
     const int m0 = tm * TM, n0 = tn * TN;
-    const int k_begin = blockIdx.z * k_chunk, k_end = min(p.k, k_begin + k_chunk);
+    int k_begin = blockIdx.z * sched.k_chunk, k_end = min(p.k, k_begin + sched.k_chunk);
+    if (shared_tile) {
+        k_begin = chunk * sched.tail_k_chunk;
+        k_end = min(p.k, k_begin + sched.tail_k_chunk);
+    }
     const int slices = (k_end - k_begin) / DIRECT_BK;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -376,11 +405,60 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
         stage_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
     }
     wait_for_loads<0>();
+
+    if (shared_tile && sched.tail_split > 1) {
+        // park the partial tile: [workgroup of the tile][wave][MFMA tile][register / 4][lane][register % 4], so that
+        // a wave moves 1 KB per instruction
+        const int shared_index = tile_id - sched.head_tiles;
+        // The partial tiles travel between workgroups that may sit on different XCDs, each with an L2 of its own:
+        // they are written and read with device scope accesses (sc1), which go past those caches, instead of
+        // fences that would write back and invalidate a whole L2 (measured: 163 us instead of 69 us for
+        // 512 x 4096 x 11008).
+        constexpr int SC1 = 16;  // auxiliary bits of the buffer instructions: device scope
+        float *tile_slots = (float *) p.workspace + (size_t) shared_index * sched.tail_split * (TM * TN);
+        const __amdgpu_buffer_rsrc_t slots = __builtin_amdgcn_make_buffer_rsrc(tile_slots, 0, sched.tail_split * (TM * TN) * 4, 0x00020000);
+        const int thread_off = (wave * (MI * NI * 16 * 64) + lane * 4) * 4;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NI; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const floatx4 x = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, x), slots,
+                                                           chunk * (TM * TN * 4) + thread_off + ((i * NI + j) * 4 + q) * 1024, 0, SC1);
+                }
+        // the stores have been acknowledged before the workgroup counts itself in
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // (also: every wave is done with the LDS stages)
+        int *counter = (int *) p.counters + shared_index, *arrived = (int *) lds;
+        if (threadIdx.x == 0) *arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*(volatile int *) arrived != sched.tail_split - 1) return;
+        // the last one in: sum over the parts of K in their order
+        floatx16 sum[MI][NI];
+        for (int part = 0; part < sched.tail_split; part++) {
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NI; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const floatx4 x = __builtin_bit_cast(
+                            floatx4, __builtin_amdgcn_raw_buffer_load_b128(slots, part * (TM * TN * 4) + thread_off + ((i * NI + j) * 4 + q) * 1024, 0, SC1));
+#pragma unroll
+                        for (int u = 0; u < 4; u++) sum[i][j][4 * q + u] = part == 0 ? x[u] : sum[i][j][4 * q + u] + x[u];
+                    }
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        store_tiles<MI, NI>(p, sum, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
+        return;
+    }
     store_tiles<MI, NI>(p, acc, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
 }
 
 template <int MI, int NI, int WM, int WN, int NSTAGE>
-int launch_direct(dim3 grid, hipStream_t stream, const GemmParams &p, int kc, int xc) {
+int launch_direct(dim3 grid, hipStream_t stream, const GemmParams &p, const DirectSchedule &sched) {
     constexpr int LDS_BYTES = NSTAGE * (32 * MI * WM + 32 * NI * WN) * 2 * DIRECT_BK;
     auto kernel = gemm_f16_direct_kernel<MI, NI, WM, WN, NSTAGE>;
     // more than 64 KB of dynamic LDS has to be asked for, once per device
@@ -395,7 +473,7 @@ int launch_direct(dim3 grid, hipStream_t stream, const GemmParams &p, int kc, in
         }
         if (e != 0) return e;
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(64 * WM * WN), LDS_BYTES, stream, p, kc, xc);
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * WM * WN), LDS_BYTES, stream, p, sched);
     return 0;
 }
 
@@ -434,35 +512,46 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
     const GemmLaunchPlan lp = plan_gemm_launch(params, true);
     const GemmParams &p = lp.p;
-    const int t = lp.small_tile ? 64 : 128, t_m = lp.tall_tile ? 256 : t;
     const int groups = p.groups > 1 ? p.groups : 1;
     if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
-    const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t - 1) / t) * groups;
-    if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
+    if (p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
-    dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);
     int b_mode = pick_mode(groups > 1 ? p.b_group[0] : p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
     for (int g = 1; g < groups; g++) {  // the loader that every operand of the group allows
         const int mode = pick_mode(p.b_group[g], p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
         if (mode != b_mode) b_mode = Scalar;
     }
-    // Measured on 128 x 128 tiles (TFLOP/s at 4096^3 / 8192^3): BK 64 single buffered 594 / 757, BK 64 double
-    // buffered 643 / 718, BK 128 single buffered 672 / 744. All of them sit at the rate at which the L2 can feed
-    // the compute units at this tile size (64 flop per byte fetched from L2, about 12 TB/s -> 770 TFLOP/s).
-    // workgroups an XCD (32 compute units) runs at a time: 1 per compute unit for the tall tiles, else 2
-    static const int xc_env = getenv("KNHIP_XCD_CHUNK") ? atoi(getenv("KNHIP_XCD_CHUNK")) : -1;
-    const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile ? 32 : 64);
     // both operands K contiguous and K (and every split of it) whole slices: the direct-to-LDS kernel
     static const int direct_env = getenv("KNHIP_F16_DIRECT") ? atoi(getenv("KNHIP_F16_DIRECT")) : 1;
     const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % DIRECT_BK == 0;
+    // (128 x 64 tiles exist in the direct kernel only; without it they run as 64 x 64)
+    const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct);
+    const int t_n = small || narrow ? 64 : 128, t_m = lp.tall_tile ? 256 : (small ? 64 : 128);
+    const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t_n - 1) / t_n) * groups;
+    if (tiles > 0x7fffffffll) return (int) hipErrorInvalidConfiguration;
+    dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
+    // Measured on 128 x 128 tiles of the kernel that stages through registers (TFLOP/s at 4096^3 / 8192^3): BK 64
+    // single buffered 594 / 757, BK 64 double buffered 643 / 718, BK 128 single buffered 672 / 744.
+    // workgroups an XCD (32 compute units) runs at a time: 1 per compute unit for the tall tiles, else 2
+    static const int xc_env = getenv("KNHIP_XCD_CHUNK") ? atoi(getenv("KNHIP_XCD_CHUNK")) : -1;
+    const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile || narrow ? 32 : 64);
     if (direct) {
+        DirectSchedule sched{lp.k_chunk, xc, (int) tiles, 1, p.k};
+        if (lp.tail_split > 1) {
+            if (p.workspace == nullptr || p.counters == nullptr) return (int) hipErrorInvalidValue;
+            sched.head_tiles = lp.head_tiles;
+            sched.tail_split = lp.tail_split;
+            sched.tail_k_chunk = lp.tail_k_chunk;
+            grid.x = (unsigned) (lp.head_tiles + (tiles - lp.head_tiles) * lp.tail_split);
+        }
         int e;
-        if (lp.small_tile) e = launch_direct<1, 1, 2, 2, 2>(grid, stream, p, lp.k_chunk, xc);
-        else if (lp.tall_tile) e = launch_direct<2, 2, 4, 2, 3>(grid, stream, p, lp.k_chunk, xc);
-        else e = launch_direct<2, 2, 2, 2, 2>(grid, stream, p, lp.k_chunk, xc);
+        if (small) e = launch_direct<1, 1, 2, 2, 4>(grid, stream, p, sched);
+        else if (narrow) e = launch_direct<2, 1, 2, 2, 4>(grid, stream, p, sched);
+        else if (lp.tall_tile) e = launch_direct<2, 2, 4, 2, 3>(grid, stream, p, sched);
+        else e = launch_direct<2, 2, 2, 2, 2>(grid, stream, p, sched);
         if (e != 0) return e;
-    } else if (lp.small_tile) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
+    } else if (small) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     else if (lp.tall_tile) launch_a<2, 64, 1, 4>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     else launch_a<2, 128, 1, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     int e = (int) hipGetLastError();

@@ -36,6 +36,9 @@ struct GemmParams {
     // f32 scratch for partial products when the launch splits the K axis (`GemmLaunchPlan::workspace_bytes`
     // bytes, 256 byte aligned); may be null otherwise
     void *workspace = nullptr;
+    // zero-filled ints that the launch hands back zero-filled (`GemmLaunchPlan::counter_bytes` bytes) when tiles
+    // are shared between workgroups; may be null otherwise
+    void *counters = nullptr;
 };
 
 // How a matrix multiply is launched; a pure function of the shapes, strides and alignments, so the planner can ask
@@ -44,11 +47,16 @@ struct GemmLaunchPlan {
     GemmParams p;            // operands swapped where needed so that the contiguous axis of C is the column axis
     bool small_tile;         // 64 x 64 workgroup tiles instead of 128 x 128
     bool tall_tile;          // f16 only: 256 x 128 workgroup tiles (8 waves)
+    bool narrow_tile;        // f16 direct kernel only: 128 x 64 workgroup tiles
     bool direct;             // f16 only: shapes and strides allow the kernel that loads global -> LDS directly
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)
     int k_chunk;             // K elements per split, a multiple of bk
-    size_t workspace_bytes;  // split_k * batch * m * n * 4 when split_k > 1, else 0
+    // f16 direct kernel, one batch entry: the first `head_tiles` tiles are computed by one workgroup each, every
+    // further tile by `tail_split` workgroups that take `tail_k_chunk` of K each and sum up inside the launch
+    int head_tiles, tail_split, tail_k_chunk;
+    size_t workspace_bytes;  // f32 scratch: split_k * batch * m * n * 4 when split_k > 1; one tile per sharing workgroup
+    size_t counter_bytes;    // one int per shared tile
 };
 GemmLaunchPlan plan_gemm_launch(const GemmParams &p, bool f16);
 // whether `p.groups` products may share one launch: no operand swap, no K split, no epilogue

@@ -43,7 +43,8 @@ double Step::flops() const {
 double Step::bytes() const {
     double total = 0.0;
     for (size_t i = 0; i < operands.size(); i++) {
-        if (kind == StepKind::MatMul && !attention && gemm.groups <= 1 && i >= (gemm_has_addend ? 4u : 3u)) break;  // split-K scratch is not algorithmic traffic
+        // split-K scratch is not algorithmic traffic
+        if (kind == StepKind::MatMul && !attention && i >= (gemm.groups > 1 ? 1u + 2u * (unsigned) gemm.groups : (gemm_has_addend ? 4u : 3u))) break;
         auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
@@ -870,6 +871,7 @@ private:
             results.push_back(alloc_tensor_shared({b, m, n}, dt));
             step.operands.push_back({results.back(), OperandKind::Out});
         }
+        push_gemm_scratch(step);
         push(std::move(step), value);
         for (size_t i = 1; i < kept.size(); i++) insert_mapping(kept[i], results[i]);
         return R::done(results[0]);
@@ -927,6 +929,23 @@ private:
         return t;
     }
 
+    // A launch that splits the K axis needs scratch for its f32 partial products: a shared buffer that is live for
+    // this step only. Where workgroups share tiles inside one launch they also need counters, which start at zero
+    // and which every launch leaves at zero again: a zero-filled constant of the step's own.
+    void push_gemm_scratch(Step &step) {
+        const GemmLaunchPlan lp = plan_gemm_launch(step.gemm, step.gemm_f16);
+        if (lp.workspace_bytes > 0)
+            step.operands.push_back({alloc_tensor_shared({lp.workspace_bytes / 4}, DType::F32), OperandKind::Out});
+        if (lp.counter_bytes > 0) {
+            constants.push_back(HostTensor(DType::I32, {lp.counter_bytes / 4}));
+            PlanTensor t;
+            t.ptr = PlanPtr{BufferKind::Constant, constants.size() - 1, 0};
+            t.dtype = DType::I32;
+            t.shape = StridedShape::simple({lp.counter_bytes / 4});
+            step.operands.push_back({t, OperandKind::Out});
+        }
+    }
+
     VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first,
                     const std::optional<PlanTensor> &addend = std::nullopt, bool relu = false) {
         const DType dt = graph[value].dtype;
@@ -956,11 +975,7 @@ private:
                 step.operands.push_back({*addend, OperandKind::In});
             }
             g.relu = relu ? 1 : 0;
-            // a launch that splits the K axis needs scratch for its f32 partial products: a shared buffer that is
-            // live for this step only
-            const GemmLaunchPlan lp = plan_gemm_launch(g, step.gemm_f16);
-            if (lp.workspace_bytes > 0)
-                step.operands.push_back({alloc_tensor_shared({lp.workspace_bytes / 4}, DType::F32), OperandKind::Out});
+            push_gemm_scratch(step);
             push(std::move(step), value);
         }
         return VT::done(result);

@@ -1472,3 +1472,16 @@ def f16_matmul_direct_tall_ring():
     for _ in range(3):
         g.output(g.linear(x, g.constant([2816, 192], _f16(rng, 2816, 192, scale=0.1))))
     return g, 0, [_f16(rng, 16, 256, 128, scale=0.2), _f16(rng, 16, 1000, 128, scale=0.2), _f16(rng, 512, 192)], None
+
+
+@case
+def f16_matmul_shared_tail_tiles():
+    """520 tiles of 64 x 64 on 512 places: the first 512 tiles get a workgroup each, the last 8 are shared by two
+    workgroups each, which split K and sum up inside the launch; the result also gets a bias and a relu"""
+    g = Graph()
+    rng = np.random.default_rng(154)
+    a = g.input([33, 1024], DType.F16)
+    b = g.input([33280, 1024], DType.F16)
+    bias = g.input([1, 33280], DType.F16)
+    g.output(g.relu(g.add(g.linear(a, b), bias)))
+    return g, 0, [_f16(rng, 33, 1024, scale=0.2), _f16(rng, 33280, 1024, scale=0.2), _f16(rng, 1, 33280)], None
