@@ -136,8 +136,11 @@ def run_bandwidth(args, device):
         log(f"copy probe launched: {probe.step_str(0)}")
         del probe
 
-    steps = args.steps if args.steps is not None else 50
-    elapsed = timed_steps(ex, steps, args.warmup)
+    # (defaults long enough for the clocks to settle: the first few milliseconds of work on an idle chip run a few
+    # percent slower)
+    steps = args.steps if args.steps is not None else 200
+    warmup = args.warmup if args.warmup is not None else 100
+    elapsed = timed_steps(ex, steps, warmup)
     ms_per_step = elapsed / steps * 1e3
     evals_per_s = len(parts) * steps / elapsed
 
@@ -179,7 +182,7 @@ def run_bandwidth(args, device):
         "unit": "graph evals/s",
         "n_gpus": 1,
         "steps": steps,
-        "warmup": args.warmup,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -253,14 +256,14 @@ def run_model(args, device, workload):
         graph, inputs = configs.build_tiny_mlp(seed=0, batch=batch)
         flops = 2 * batch * (16 * 32 + 32 * 10)
         desc = "BASELINE configs[0]: tiny MLP 16->32->10 with softmax, f32, batch 8"
-        default_steps = 5000
+        default_steps, default_warmup = 5000, 2000
     elif workload == "resnet":
         batch = 1024
         graph, make_inputs, flop_per_pos = configs.build_resnet_tower(seed=0)
         inputs = make_inputs(batch)
         flops = flop_per_pos * batch
         desc = "BASELINE configs[2]: AlphaZero style ResNet tower (10 blocks x 128 channels on 8x8, policy + value heads), f32, batch 1024"
-        default_steps = 20
+        default_steps, default_warmup = 50, 20
     elif workload == "llama":
         batch = 0
         graph, make_inputs, flops = configs.build_llama(seed=0)
@@ -268,14 +271,14 @@ def run_model(args, device, workload):
         dtype, tol = "f16", 2e-2
         desc = ("BASELINE configs[3]: 2 layer LLaMA style decoder, d_model 4096, 32 heads, FFN 11008, f16 weights and "
                 "activations with f32 accumulation, batch 1, prefill of 512 tokens")
-        default_steps = 20
+        default_steps, default_warmup = 100, 60
     elif workload == "unet":
         batch = 0
         graph, make_inputs, flops = configs.build_unet_block(seed=0)
         inputs = make_inputs()
         desc = ("BASELINE configs[4]: Stable-Diffusion style UNet block (ResBlock 320 channels at 64x64 + spatial "
                 "transformer with self / cross attention and GEGLU), f32, batch 2")
-        default_steps = 10
+        default_steps, default_warmup = 60, 30
     else:
         raise SystemExit(f"unknown workload {workload}")
     log(f"graph built in {time.time() - t_setup:.1f} s")
@@ -285,8 +288,11 @@ def run_model(args, device, workload):
         ex.upload_input(k, x)
     log(f"setup took {time.time() - t_setup:.1f} s, {ex.step_count()} steps, arena {ex.mem_usage['arena_bytes'] / 2**20:.0f} MiB")
 
+    # (defaults long enough for the clocks to settle: the first few milliseconds of work on an idle chip run up to a
+    # tenth slower)
     steps = args.steps if args.steps is not None else default_steps
-    elapsed = timed_steps(ex, steps, args.warmup)
+    warmup = args.warmup if args.warmup is not None else default_warmup
+    elapsed = timed_steps(ex, steps, warmup)
     ms_per_step = elapsed / steps * 1e3
     evals_per_s = steps / elapsed
 
@@ -355,7 +361,7 @@ def run_model(args, device, workload):
     if workload == "mlp":
         # one HIP graph launch per evaluation instead of one launch per step
         ex.set_graph_mode(True)
-        dt = timed_steps(ex, steps, args.warmup) / steps
+        dt = timed_steps(ex, steps, warmup) / steps
         extra["hip_graph_replay"] = {"ms_per_step": round(dt * 1e3, 5), "evals_per_s": round(1.0 / dt, 1)}
         ex.set_graph_mode(False)
         # the reference's executor contract includes the copies: time `evaluate` (H2D, launches, D2H) as well
@@ -381,7 +387,7 @@ def run_model(args, device, workload):
         "unit": "graph evals/s",
         "n_gpus": 1,
         "steps": steps,
-        "warmup": args.warmup,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -402,8 +408,8 @@ def run_model(args, device, workload):
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=None, help="timed steps (default: 50 for the bandwidth graphs)")
-    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--steps", type=int, default=None, help="timed steps (default: 200 for the bandwidth graphs)")
+    parser.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: 100 for the bandwidth graphs)")
     parser.add_argument("--workload", default="bandwidth", choices=["bandwidth", "mlp", "resnet", "llama", "unet"])
     parser.add_argument("--no-cpu-baseline", action="store_true", help="skip the timed CPU oracle leg and parity check")
     parser.add_argument("--copy-probe", action="store_true",
