@@ -388,19 +388,29 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
         asm volatile("" ::: "memory");
         issue_loads<A_LD, B_LD>(a_src, b_src, dst_a + fill_off, dst_b + fill_off, s + NSTAGE < slices ? DIRECT_BK : 0);
         const char *st = lds + stage_off;
+        // All LDS reads of the slice are requested before its first MFMA: with one or two waves per SIMD nobody
+        // else would cover their latency step by step (512 x 12288 x 4096: 72 -> 67 us). The LDS is what bounds
+        // this kernel: it moves about 64 bytes per clock and compute unit, reads and direct loads together, and a
+        // 256 x 128 tile of 8 waves needs 176 KB of that per slice, 2750 clocks against 1024 clocks of MFMA work.
+        // Fewer waves with bigger tiles each (4 waves of 128 x 64) need less LDS traffic but measured slower, with
+        // one wave per SIMD left to cover every wait by itself (133 us against 120 us for 512 x 22016 x 4096).
+        constexpr int STEPS = DIRECT_BK / 16;
+        halfx8 a[STEPS][MI], b[STEPS][NI];
 #pragma unroll
-        for (int t = 0; t < DIRECT_BK / 16; t++) {
-            halfx8 a[MI], b[NI];
+        for (int t = 0; t < STEPS; t++) {
 #pragma unroll
-            for (int i = 0; i < MI; i++) a[i] = *(const halfx8 *) (st + (a_rd ^ (32 * t)) + i * 32 * ROW);
+            for (int i = 0; i < MI; i++) a[t][i] = *(const halfx8 *) (st + (a_rd ^ (32 * t)) + i * 32 * ROW);
 #pragma unroll
-            for (int j = 0; j < NI; j++) b[j] = *(const halfx8 *) (st + (b_rd ^ (32 * t)) + j * 32 * ROW);
+            for (int j = 0; j < NI; j++) b[t][j] = *(const halfx8 *) (st + (b_rd ^ (32 * t)) + j * 32 * ROW);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < STEPS; t++)
 #pragma unroll
             for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < NI; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
         fill_off = stage_off;
         stage_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
     }
