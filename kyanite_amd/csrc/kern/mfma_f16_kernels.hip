@@ -12,8 +12,11 @@
 // slices global -> LDS directly (global_load_lds_dwordx4: every lane names its own 16 source bytes, the wave's 64
 // vectors land side by side in LDS), with no trip through registers and no LDS write instructions. Rows are then
 // exactly 128 bytes with no padding, and bank conflicts are avoided by an XOR swizzle instead: the 16 byte chunk q
-// of row r sits at position q ^ (r % 8), which the loading lane arranges by choosing its source chunk and the
-// reading lane by flipping address bits.
+// of row r sits at position q ^ swz(r), swz(r) = (r / 2) % 8, which the loading lane arranges by choosing its source
+// chunk and the reading lane by flipping address bits. A 128 bit read is served 16 lanes at a time from 64 banks
+// (256 bytes, two rows): the 16 rows r .. r + 15 of such a group then hit 16 different (row parity, position)
+// pairs. (With swz(r) = r % 8, which would do for 32 banks, the counters showed every second LDS cycle as a
+// conflict.)
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
@@ -293,7 +296,7 @@ __device__ __forceinline__ void issue_loads(const half_t *(&a_src)[A_LD], const 
 // The direct-to-LDS kernel: a workgroup of WM x WN waves owns a (32 MI WM) x (32 NI WN) tile, a wave MI x NI MFMA
 // tiles of it. K is walked in slices of 64 through a ring of NSTAGE LDS stages; every stage holds the rows of A,
 // then those of B, 128 bytes each. One load instruction of a wave fills 8 rows (64 chunks of 16 bytes): lane l fills chunk
-// position l % 8 of row l / 8, so it fetches chunk (l % 8) ^ (l / 8) of that row. Rows past the edge of a matrix
+// position l % 8 of row l / 8, so it fetches chunk (l % 8) ^ swz(row) of that row. Rows past the edge of a matrix
 // repeat its last row; they only feed results that are not stored.
 // Per slice: wait for the own loads of this slice (those of the NSTAGE - 2 slices after it may still be in
 // flight), barrier (now everybody's have landed, and everybody is done reading the stage of the slice before),
@@ -353,18 +356,25 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
     // the source of every load of this lane; all of them move on by one slice per issue
     const half_t *a_src[A_LD], *b_src[B_LD];
     {
-        const int lr = lane >> 3, chunk = (lane & 7) ^ lr;
-        const half_t *a0 = (const half_t *) p.a + bz * p.a_sb + k_begin + 8 * chunk;
-        const half_t *b0 = (const half_t *) b_base + bz * p.b_sb + k_begin + 8 * chunk;
+        // lane l fills chunk position l % 8 of row l / 8 of the 8 rows of its load, with chunk (l % 8) ^ swz(row)
+        const int lr = lane >> 3, pos = lane & 7;
+        const half_t *a0 = (const half_t *) p.a + bz * p.a_sb + k_begin;
+        const half_t *b0 = (const half_t *) b_base + bz * p.b_sb + k_begin;
 #pragma unroll
-        for (int i = 0; i < A_LD; i++) a_src[i] = a0 + (long long) min(m0 + (wave * A_LD + i) * 8 + lr, p.m - 1) * p.a_sm;
+        for (int i = 0; i < A_LD; i++) {
+            const int row = (wave * A_LD + i) * 8 + lr;
+            a_src[i] = a0 + (long long) min(m0 + row, p.m - 1) * p.a_sm + 8 * (pos ^ ((row >> 1) & 7));
+        }
 #pragma unroll
-        for (int i = 0; i < B_LD; i++) b_src[i] = b0 + (long long) min(n0 + (wave * B_LD + i) * 8 + lr, p.n - 1) * p.b_sn;
+        for (int i = 0; i < B_LD; i++) {
+            const int row = (wave * B_LD + i) * 8 + lr;
+            b_src[i] = b0 + (long long) min(n0 + row, p.n - 1) * p.b_sn + 8 * (pos ^ ((row >> 1) & 7));
+        }
     }
-    // MFMA operand of lane (row c, half h) at step t: chunk 2 t + h of its row, found at (2 t + h) ^ (c % 8), which
-    // is the address of step 0 with bits 5 and 6 flipped by t
-    const unsigned a_rd = (wm * 32 * MI + c) * ROW + ((half ^ (c & 7)) * 16);
-    const unsigned b_rd = A_BYTES + (wn * 32 * NI + c) * ROW + ((half ^ (c & 7)) * 16);
+    // MFMA operand of lane (row c, half h) at step t: chunk 2 t + h of its row, found at (2 t + h) ^ swz(c), which is
+    // the address of step 0 with bits 5 and 6 flipped by t
+    const unsigned a_rd = (wm * 32 * MI + c) * ROW + ((half ^ ((c >> 1) & 7)) * 16);
+    const unsigned b_rd = A_BYTES + (wn * 32 * NI + c) * ROW + ((half ^ ((c >> 1) & 7)) * 16);
 
     floatx16 acc[MI][NI];
 #pragma unroll
