@@ -78,9 +78,16 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     lp.narrow_tile = lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= env_int("KNHIP_F16_NARROW_FROM", 192) &&
                      p.k < env_int("KNHIP_F16_NARROW_K_BELOW", 8192);
     if (lp.narrow_tile) lp.small_tile = lp.tall_tile = false;
+    // Direct kernel only: 256 x 256 tiles (8 waves of 128 x 64) where they still give every compute unit a
+    // workgroup. The LDS bounds this kernel, and they need the least LDS traffic per flop: 256 KB per slice of 64
+    // for twice the work of a 256 x 128 tile with its 176 KB (8192^3: 1191 -> 1030 us, 4096^3: 166 -> 139 us).
+    const long long wide_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 255) / 256) * p.batch * groups;
+    lp.wide_tile = lp.direct && lp.tall_tile && p.n >= 256 && (p.n + 255) / 256 * 256 - p.n <= p.n / 8 &&
+                   wide_blocks >= env_int("KNHIP_F16_WIDE_FROM", 256);
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
     if (lp.narrow_tile) blocks = narrow_blocks;
+    if (lp.wide_tile) blocks = wide_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile || lp.narrow_tile ? 64 : 128;
     else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
 
@@ -102,7 +109,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
             long long chunk = (p.k + s - 1) / s;
             chunk = (chunk + 63) / 64 * 64;
             s = (p.k + chunk - 1) / chunk;
-            const int tm = lp.tall_tile ? 256 : (lp.small_tile ? 64 : 128), tn = lp.small_tile || lp.narrow_tile ? 64 : 128;
+            const int tm = lp.tall_tile ? 256 : (lp.small_tile ? 64 : 128), tn = lp.small_tile || lp.narrow_tile ? 64 : (lp.wide_tile ? 256 : 128);
             const unsigned long long bytes = (unsigned long long) rest * s * tm * tn * 4ull;
             if (s >= 2 && bytes <= (256ull << 20)) {
                 lp.head_tiles = (int) full;

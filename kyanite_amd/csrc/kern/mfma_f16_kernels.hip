@@ -404,23 +404,26 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
         // 256 x 128 tile of 8 waves needs 176 KB of that per slice, 2750 clocks against 1024 clocks of MFMA work.
         // Fewer waves with bigger tiles each (4 waves of 128 x 64) need less LDS traffic but measured slower, with
         // one wave per SIMD left to cover every wait by itself (133 us against 120 us for 512 x 22016 x 4096).
-        constexpr int STEPS = DIRECT_BK / 16;
-        halfx8 a[STEPS][MI], b[STEPS][NI];
+        constexpr int STEPS = DIRECT_BK / 16, HOIST = (MI + NI) * STEPS > 16 ? 2 : STEPS;  // (registers permitting)
 #pragma unroll
-        for (int t = 0; t < STEPS; t++) {
+        for (int t0 = 0; t0 < STEPS; t0 += HOIST) {
+            halfx8 a[HOIST][MI], b[HOIST][NI];
 #pragma unroll
-            for (int i = 0; i < MI; i++) a[t][i] = *(const halfx8 *) (st + (a_rd ^ (32 * t)) + i * 32 * ROW);
+            for (int t = 0; t < HOIST; t++) {
 #pragma unroll
-            for (int j = 0; j < NI; j++) b[t][j] = *(const halfx8 *) (st + (b_rd ^ (32 * t)) + j * 32 * ROW);
+                for (int i = 0; i < MI; i++) a[t][i] = *(const halfx8 *) (st + (a_rd ^ (32 * (t0 + t))) + i * 32 * ROW);
+#pragma unroll
+                for (int j = 0; j < NI; j++) b[t][j] = *(const halfx8 *) (st + (b_rd ^ (32 * (t0 + t))) + j * 32 * ROW);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < HOIST; t++)
+#pragma unroll
+                for (int i = 0; i < MI; i++)
+#pragma unroll
+                    for (int j = 0; j < NI; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int t = 0; t < STEPS; t++)
-#pragma unroll
-            for (int i = 0; i < MI; i++)
-#pragma unroll
-                for (int j = 0; j < NI; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
         fill_off = stage_off;
         stage_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
     }
@@ -546,8 +549,9 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     static const int direct_env = getenv("KNHIP_F16_DIRECT") ? atoi(getenv("KNHIP_F16_DIRECT")) : 1;
     const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % DIRECT_BK == 0;
     // (128 x 64 tiles exist in the direct kernel only; without it they run as 64 x 64)
-    const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct);
-    const int t_n = small || narrow ? 64 : 128, t_m = lp.tall_tile ? 256 : (small ? 64 : 128);
+    // (so do 256 x 256 tiles, which otherwise run as 256 x 128)
+    const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct), wide = lp.wide_tile && direct;
+    const int t_n = small || narrow ? 64 : (wide ? 256 : 128), t_m = lp.tall_tile ? 256 : (small ? 64 : 128);
     const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t_n - 1) / t_n) * groups;
     if (tiles > 0x7fffffffll) return (int) hipErrorInvalidConfiguration;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
@@ -555,7 +559,7 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     // single buffered 594 / 757, BK 64 double buffered 643 / 718, BK 128 single buffered 672 / 744.
     // workgroups an XCD (32 compute units) runs at a time: 1 per compute unit for the tall tiles, else 2
     static const int xc_env = getenv("KNHIP_XCD_CHUNK") ? atoi(getenv("KNHIP_XCD_CHUNK")) : -1;
-    const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile || narrow ? 32 : 64);
+    const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile || narrow ? 32 : 64);  // (also for the 256 x 256 tiles)
     if (direct) {
         DirectSchedule sched{lp.k_chunk, xc, (int) tiles, 1, p.k};
         if (lp.tail_split > 1) {
@@ -568,6 +572,7 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
         int e;
         if (small) e = launch_direct<1, 1, 2, 2, 4>(grid, stream, p, sched);
         else if (narrow) e = launch_direct<2, 1, 2, 2, 4>(grid, stream, p, sched);
+        else if (wide) e = launch_direct<4, 2, 2, 4, 2>(grid, stream, p, sched);
         else if (lp.tall_tile) e = launch_direct<2, 2, 4, 2, 3>(grid, stream, p, sched);
         else e = launch_direct<2, 2, 2, 2, 2>(grid, stream, p, sched);
         if (e != 0) return e;

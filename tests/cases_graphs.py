@@ -1485,3 +1485,14 @@ def f16_matmul_shared_tail_tiles():
     bias = g.input([1, 33280], DType.F16)
     g.output(g.relu(g.add(g.linear(a, b), bias)))
     return g, 0, [_f16(rng, 33, 1024, scale=0.2), _f16(rng, 33280, 1024, scale=0.2), _f16(rng, 1, 33280)], None
+
+
+@case
+def f16_matmul_direct_wide_tiles():
+    """256 x 256 tiles (8 waves of 128 x 64), 256 of them over a batch, ragged on both axes"""
+    g = Graph()
+    rng = np.random.default_rng(155)
+    a = g.input([16, 1000, 128], DType.F16)
+    b = g.input([16, 1016, 128], DType.F16)
+    g.output(g.batched_mat_mul(a, g.permute(b, [0, 2, 1])))
+    return g, 0, [_f16(rng, 16, 1000, 128, scale=0.2), _f16(rng, 16, 1016, 128, scale=0.2)], None
