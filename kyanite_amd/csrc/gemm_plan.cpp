@@ -68,27 +68,30 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // of three stages and also pay without a split, as long as they still fill the chip. Measured with weights
     // that come from memory, not from cache (us, 128 x 128 on two stages against 256 x 128 on three):
     // 512 x 22016 x 4096 147 / 133, 512 x 12288 x 4096 93 / 72, 4096^3 152 / 144; 512 x 4096 x 4096 53 / 59.
-    lp.direct = f16 && p.k > 0 && p.k % 64 == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % 8 == 0 && p.b_sn % 8 == 0 &&
-                (p.batch <= 1 || (p.a_sb % 8 == 0 && p.b_sb % 8 == 0));
-    if (lp.direct && tall_fits && tall_blocks >= env_int("KNHIP_F16_TALL_FROM", 128)) lp.tall_tile = true;
+    // (In f32 the same kernel walks K in slices of 32 and has 128 x 128 and 64 x 64 tiles.)
+    const int vec = f16 ? 8 : 4;
+    lp.direct = p.k > 0 && p.k % (8 * vec) == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % vec == 0 && p.b_sn % vec == 0 &&
+                (p.batch <= 1 || (p.a_sb % vec == 0 && p.b_sb % vec == 0));
+    if (f16 && lp.direct && tall_fits && tall_blocks >= env_int("KNHIP_F16_TALL_FROM", 128)) lp.tall_tile = true;
     // Direct kernel only: 128 x 64 tiles on a ring of four stages, where 128 x 128 tiles leave compute units
     // without a workgroup and K is too short for a split to pay (512 x 4096 x 4096: 29 us against 39 us on
     // 256 x 128 tiles split in four; 512 x 4096 x 11008: 84 us against 69 us).
     const long long narrow_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 63) / 64) * p.batch * groups;
-    lp.narrow_tile = lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= env_int("KNHIP_F16_NARROW_FROM", 192) &&
+    lp.narrow_tile = f16 && lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= env_int("KNHIP_F16_NARROW_FROM", 192) &&
                      p.k < env_int("KNHIP_F16_NARROW_K_BELOW", 8192);
     if (lp.narrow_tile) lp.small_tile = lp.tall_tile = false;
     // Direct kernel only: 256 x 256 tiles (8 waves of 128 x 64) where they still give every compute unit a
     // workgroup. The LDS bounds this kernel, and they need the least LDS traffic per flop: 256 KB per slice of 64
     // for twice the work of a 256 x 128 tile with its 176 KB (8192^3: 1191 -> 1030 us, 4096^3: 166 -> 139 us).
     const long long wide_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 255) / 256) * p.batch * groups;
-    lp.wide_tile = lp.direct && lp.tall_tile && p.n >= 256 && (p.n + 255) / 256 * 256 - p.n <= p.n / 8 &&
+    lp.wide_tile = f16 && lp.direct && lp.tall_tile && p.n >= 256 && (p.n + 255) / 256 * 256 - p.n <= p.n / 8 &&
                    wide_blocks >= env_int("KNHIP_F16_WIDE_FROM", 256);
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
     if (lp.narrow_tile) blocks = narrow_blocks;
     if (lp.wide_tile) blocks = wide_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile || lp.narrow_tile ? 64 : 128;
+    else if (lp.direct) lp.bk = 32;
     else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
 
     // A tile count that leaves the last round of workgroups mostly idle: the direct kernel splits the tiles of just

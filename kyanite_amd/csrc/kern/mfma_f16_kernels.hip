@@ -134,14 +134,14 @@ __device__ __forceinline__ void tile_of_block(int id, int total, int tiles_m, in
 
 // Stores the MI x NI MFMA tiles of a wave whose first row / column are row0 / col0. Accumulator layout of a 32 x 32
 // tile: register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32.
-template <int MI, int NI>
+template <typename T, int MI, int NI>
 __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 (&acc)[MI][NI], void *c_base, int bz, int row0, int col0) {
     const int lane = threadIdx.x & 63, c = lane & 31, half = lane >> 5;
-    half_t *out = (half_t *) c_base + bz * p.c_sb;
+    T *out = (T *) c_base + bz * p.c_sb;
     float *partial = (float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n;
     const bool split = gridDim.z > 1;
     // the epilogue of a split launch is applied by the pass that sums the partial products
-    const half_t *addend = p.addend ? (const half_t *) p.addend + bz * p.d_sb : nullptr;
+    const T *addend = p.addend ? (const T *) p.addend + bz * p.d_sb : nullptr;
     // Tiles that lie inside the matrix, with offsets that fit 32 bits, skip the bounds checks and the 64 bit
     // address arithmetic (which otherwise cost about a tenth of a 512 x 12288 x 4096 launch).
     const long long reach = (long long) (p.m - 1) * p.c_sm + p.n, d_reach = (long long) (p.m - 1) * p.d_sm + (long long) (p.n - 1) * p.d_sn;
@@ -149,8 +149,8 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
                       (!addend || (p.d_sm >= 0 && p.d_sn >= 0 && d_reach < 0x7fffffffll));
     if (fast) {
         const int c_sm = (int) p.c_sm, d_sm = (int) p.d_sm, d_sn = (int) p.d_sn;
-        half_t *tile = out + (row0 + 4 * half) * c_sm + col0 + c;
-        const half_t *d_tile = addend ? addend + (row0 + 4 * half) * d_sm + (col0 + c) * d_sn : nullptr;
+        T *tile = out + (row0 + 4 * half) * c_sm + col0 + c;
+        const T *d_tile = addend ? addend + (row0 + 4 * half) * d_sm + (col0 + c) * d_sn : nullptr;
         const bool relu = p.relu != 0;
 #pragma unroll
         for (int i = 0; i < MI; i++)
@@ -159,9 +159,9 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int r = 32 * i + 8 * (v >> 2) + (v & 3);
-                    half_t x = (half_t) acc[i][j][v];
-                    if (d_tile) x = (half_t) ((float) x + (float) d_tile[r * d_sm + 32 * j * d_sn]);
-                    if (relu) x = x > (half_t) 0 ? x : (half_t) 0;
+                    T x = (T) acc[i][j][v];
+                    if (d_tile) x = (T) ((float) x + (float) d_tile[r * d_sm + 32 * j * d_sn]);
+                    if (relu) x = x > (T) 0 ? x : (T) 0;
                     tile[r * c_sm + 32 * j] = x;
                 }
         return;
@@ -178,9 +178,9 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
                     if (split) {
                         partial[(long long) row * p.n + col] = acc[i][j][v];
                     } else {
-                        half_t r = (half_t) acc[i][j][v];
-                        if (addend) r = (half_t) ((float) r + (float) addend[(long long) row * p.d_sm + (long long) col * p.d_sn]);
-                        if (p.relu) r = r > (half_t) 0 ? r : (half_t) 0;
+                        T r = (T) acc[i][j][v];
+                        if (addend) r = (T) ((float) r + (float) addend[(long long) row * p.d_sm + (long long) col * p.d_sn]);
+                        if (p.relu) r = r > (T) 0 ? r : (T) 0;
                         out[(long long) row * p.c_sm + (long long) col * p.c_sn] = r;
                     }
                 }
@@ -264,10 +264,10 @@ __global__ __launch_bounds__(128 * WM) void gemm_f16_kernel(GemmParams p, int k_
         }
     }
 
-    store_tiles<TI, TI>(p, acc, c_base, bz, m0 + wm * 32 * TI, n0 + wn * 32 * TI);
+    store_tiles<half_t, TI, TI>(p, acc, c_base, bz, m0 + wm * 32 * TI, n0 + wn * 32 * TI);
 }
 
-constexpr int DIRECT_BK = 64;
+constexpr int DIRECT_ROW = 128;  // bytes of a row of a slice: 64 halves or 32 floats
 
 template <int N>
 __device__ __forceinline__ void wait_for_loads() {
@@ -277,8 +277,8 @@ __device__ __forceinline__ void wait_for_loads() {
 // One slice of both operands on its way, global -> LDS: load i of the wave fills the 1024 bytes at dst + 1024 i,
 // lane l the 16 bytes at 16 l of them from its own source address, which then moves on by `advance` elements.
 // (The host pass of the compiler does not know the load instruction, hence the guard.)
-template <int A_LD, int B_LD>
-__device__ __forceinline__ void issue_loads(const half_t *(&a_src)[A_LD], const half_t *(&b_src)[B_LD], char *dst_a, char *dst_b, int advance) {
+template <typename T, int A_LD, int B_LD>
+__device__ __forceinline__ void issue_loads(const T *(&a_src)[A_LD], const T *(&b_src)[B_LD], char *dst_a, char *dst_b, int advance) {
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int i = 0; i < A_LD; i++) {
@@ -315,9 +315,9 @@ struct DirectSchedule {
     int head_tiles, tail_split, tail_k_chunk;
 };
 
-template <int MI, int NI, int WM, int WN, int NSTAGE>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParams p, DirectSchedule sched) {
-    constexpr int WAVES = WM * WN, TM = 32 * MI * WM, TN = 32 * NI * WN, ROW = 2 * DIRECT_BK;
+template <typename T, int MI, int NI, int WM, int WN, int NSTAGE>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p, DirectSchedule sched) {
+    constexpr int WAVES = WM * WN, TM = 32 * MI * WM, TN = 32 * NI * WN, ROW = DIRECT_ROW, BK = ROW / (int) sizeof(T), VEC = 16 / (int) sizeof(T);
     constexpr int A_BYTES = TM * ROW, STAGE = (TM + TN) * ROW;
     constexpr int A_LD = TM / 8 / WAVES, B_LD = TN / 8 / WAVES;  // load instructions per wave and stage
     static_assert(A_LD >= 1 && B_LD >= 1 && ROW == 128 && NSTAGE >= 2, "tile too small for the workgroup");
@@ -348,27 +348,27 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
         k_begin = chunk * sched.tail_k_chunk;
         k_end = min(p.k, k_begin + sched.tail_k_chunk);
     }
-    const int slices = (k_end - k_begin) / DIRECT_BK;
+    const int slices = (k_end - k_begin) / BK;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WN, wn = wave % WN, c = lane & 31, half = lane >> 5;
 
     // the source of every load of this lane; all of them move on by one slice per issue
-    const half_t *a_src[A_LD], *b_src[B_LD];
+    const T *a_src[A_LD], *b_src[B_LD];
     {
         // lane l fills chunk position l % 8 of row l / 8 of the 8 rows of its load, with chunk (l % 8) ^ swz(row)
         const int lr = lane >> 3, pos = lane & 7;
-        const half_t *a0 = (const half_t *) p.a + bz * p.a_sb + k_begin;
-        const half_t *b0 = (const half_t *) b_base + bz * p.b_sb + k_begin;
+        const T *a0 = (const T *) p.a + bz * p.a_sb + k_begin;
+        const T *b0 = (const T *) b_base + bz * p.b_sb + k_begin;
 #pragma unroll
         for (int i = 0; i < A_LD; i++) {
             const int row = (wave * A_LD + i) * 8 + lr;
-            a_src[i] = a0 + (long long) min(m0 + row, p.m - 1) * p.a_sm + 8 * (pos ^ ((row >> 1) & 7));
+            a_src[i] = a0 + (long long) min(m0 + row, p.m - 1) * p.a_sm + VEC * (pos ^ ((row >> 1) & 7));
         }
 #pragma unroll
         for (int i = 0; i < B_LD; i++) {
             const int row = (wave * B_LD + i) * 8 + lr;
-            b_src[i] = b0 + (long long) min(n0 + row, p.n - 1) * p.b_sn + 8 * (pos ^ ((row >> 1) & 7));
+            b_src[i] = b0 + (long long) min(n0 + row, p.n - 1) * p.b_sn + VEC * (pos ^ ((row >> 1) & 7));
         }
     }
     // MFMA operand of lane (row c, half h) at step t: chunk 2 t + h of its row, found at (2 t + h) ^ swz(c), which is
@@ -390,13 +390,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
     char *const dst_a = lds + wave * A_LD * 1024, *const dst_b = lds + A_BYTES + wave * B_LD * 1024;
 #pragma unroll
     for (int j = 0; j < NSTAGE - 1; j++)
-        issue_loads<A_LD, B_LD>(a_src, b_src, dst_a + j * STAGE, dst_b + j * STAGE, j + 1 < slices ? DIRECT_BK : 0);
+        issue_loads<T, A_LD, B_LD>(a_src, b_src, dst_a + j * STAGE, dst_b + j * STAGE, j + 1 < slices ? BK : 0);
     unsigned stage_off = 0, fill_off = (NSTAGE - 1) * STAGE;
     for (int s = 0; s < slices; s++) {
         wait_for_loads<(NSTAGE - 2) * (A_LD + B_LD)>();
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        issue_loads<A_LD, B_LD>(a_src, b_src, dst_a + fill_off, dst_b + fill_off, s + NSTAGE < slices ? DIRECT_BK : 0);
+        issue_loads<T, A_LD, B_LD>(a_src, b_src, dst_a + fill_off, dst_b + fill_off, s + NSTAGE < slices ? BK : 0);
         const char *st = lds + stage_off;
         // All LDS reads of the slice are requested before its first MFMA: with one or two waves per SIMD nobody
         // else would cover their latency step by step (512 x 12288 x 4096: 72 -> 67 us). The LDS is what bounds
@@ -404,25 +404,46 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
         // 256 x 128 tile of 8 waves needs 176 KB of that per slice, 2750 clocks against 1024 clocks of MFMA work.
         // Fewer waves with bigger tiles each (4 waves of 128 x 64) need less LDS traffic but measured slower, with
         // one wave per SIMD left to cover every wait by itself (133 us against 120 us for 512 x 22016 x 4096).
-        constexpr int STEPS = DIRECT_BK / 16, HOIST = (MI + NI) * STEPS > 16 ? 2 : STEPS;  // (registers permitting)
+        if constexpr (sizeof(T) == 2) {
+            constexpr int STEPS = 4, HOIST = (MI + NI) * STEPS > 16 ? 2 : STEPS;  // (registers permitting)
 #pragma unroll
-        for (int t0 = 0; t0 < STEPS; t0 += HOIST) {
-            halfx8 a[HOIST][MI], b[HOIST][NI];
+            for (int t0 = 0; t0 < STEPS; t0 += HOIST) {
+                halfx8 a[HOIST][MI], b[HOIST][NI];
 #pragma unroll
-            for (int t = 0; t < HOIST; t++) {
+                for (int t = 0; t < HOIST; t++) {
 #pragma unroll
-                for (int i = 0; i < MI; i++) a[t][i] = *(const halfx8 *) (st + (a_rd ^ (32 * (t0 + t))) + i * 32 * ROW);
+                    for (int i = 0; i < MI; i++) a[t][i] = *(const halfx8 *) (st + (a_rd ^ (32 * (t0 + t))) + i * 32 * ROW);
 #pragma unroll
-                for (int j = 0; j < NI; j++) b[t][j] = *(const halfx8 *) (st + (b_rd ^ (32 * (t0 + t))) + j * 32 * ROW);
+                    for (int j = 0; j < NI; j++) b[t][j] = *(const halfx8 *) (st + (b_rd ^ (32 * (t0 + t))) + j * 32 * ROW);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < HOIST; t++)
+#pragma unroll
+                    for (int i = 0; i < MI; i++)
+#pragma unroll
+                        for (int j = 0; j < NI; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            // f32: a lane's 16 bytes are 4 consecutive k of its row, which feed 4 steps of v_mfma_f32_32x32x2_f32:
+            // step u of group t multiplies k = 8 t + u (lower half of the wave) and k = 8 t + 4 + u (upper half),
+            // in A and B alike
 #pragma unroll
-            for (int t = 0; t < HOIST; t++)
+            for (int t = 0; t < 4; t++) {
+                floatx4 a[MI], b[NI];
 #pragma unroll
-                for (int i = 0; i < MI; i++)
+                for (int i = 0; i < MI; i++) a[i] = *(const floatx4 *) (st + (a_rd ^ (32 * t)) + i * 32 * ROW);
 #pragma unroll
-                    for (int j = 0; j < NI; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NI; j++) b[j] = *(const floatx4 *) (st + (b_rd ^ (32 * t)) + j * 32 * ROW);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int i = 0; i < MI; i++)
+#pragma unroll
+                        for (int j = 0; j < NI; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][u], b[j][u], acc[i][j], 0, 0, 0);
+            }
         }
         fill_off = stage_off;
         stage_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
@@ -474,16 +495,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_f16_direct_kernel(GemmParam
                     }
         }
         if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        store_tiles<MI, NI>(p, sum, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
+        store_tiles<T, MI, NI>(p, sum, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
         return;
     }
-    store_tiles<MI, NI>(p, acc, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
+    store_tiles<T, MI, NI>(p, acc, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
 }
 
-template <int MI, int NI, int WM, int WN, int NSTAGE>
+template <typename T, int MI, int NI, int WM, int WN, int NSTAGE>
 int launch_direct(dim3 grid, hipStream_t stream, const GemmParams &p, const DirectSchedule &sched) {
-    constexpr int LDS_BYTES = NSTAGE * (32 * MI * WM + 32 * NI * WN) * 2 * DIRECT_BK;
-    auto kernel = gemm_f16_direct_kernel<MI, NI, WM, WN, NSTAGE>;
+    constexpr int LDS_BYTES = NSTAGE * (32 * MI * WM + 32 * NI * WN) * DIRECT_ROW;
+    auto kernel = gemm_direct_kernel<T, MI, NI, WM, WN, NSTAGE>;
     // more than 64 KB of dynamic LDS has to be asked for, once per device
     static bool allowed[64] = {};
     int device = 0;
@@ -531,6 +552,33 @@ void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmP
 
 }  // namespace
 
+int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool *launched) {
+    *launched = false;
+    const GemmParams &p = lp.p;
+    static const int direct_env = getenv("KNHIP_F32_DIRECT") ? atoi(getenv("KNHIP_F32_DIRECT")) : 1;
+    if (!direct_env || !lp.direct || lp.k_chunk % 32 != 0) return 0;
+    const int groups = p.groups > 1 ? p.groups : 1;
+    bool aligned = (uintptr_t) p.a % 16 == 0;
+    for (int g = 0; g < groups; g++) aligned = aligned && (uintptr_t) (groups > 1 ? p.b_group[g] : p.b) % 16 == 0;
+    if (!aligned) return 0;
+    const int t = lp.small_tile ? 64 : 128;
+    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * groups;
+    if (tiles > 0x7fffffffll) return (int) hipErrorInvalidConfiguration;
+    dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
+    DirectSchedule sched{lp.k_chunk, 64, (int) tiles, 1, p.k};
+    if (lp.tail_split > 1) {
+        if (p.workspace == nullptr || p.counters == nullptr) return (int) hipErrorInvalidValue;
+        sched.head_tiles = lp.head_tiles;
+        sched.tail_split = lp.tail_split;
+        sched.tail_k_chunk = lp.tail_k_chunk;
+        grid.x = (unsigned) (lp.head_tiles + (tiles - lp.head_tiles) * lp.tail_split);
+    }
+    const int e = lp.small_tile ? launch_direct<float, 1, 1, 2, 2, 4>(grid, stream, p, sched) : launch_direct<float, 2, 2, 2, 2, 2>(grid, stream, p, sched);
+    if (e != 0) return e;
+    *launched = true;
+    return (int) hipGetLastError();
+}
+
 int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
     const GemmLaunchPlan lp = plan_gemm_launch(params, true);
@@ -547,7 +595,7 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     }
     // both operands K contiguous and K (and every split of it) whole slices: the direct-to-LDS kernel
     static const int direct_env = getenv("KNHIP_F16_DIRECT") ? atoi(getenv("KNHIP_F16_DIRECT")) : 1;
-    const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % DIRECT_BK == 0;
+    const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % 64 == 0;
     // (128 x 64 tiles exist in the direct kernel only; without it they run as 64 x 64)
     // (so do 256 x 256 tiles, which otherwise run as 256 x 128)
     const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct), wide = lp.wide_tile && direct;
@@ -570,11 +618,11 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
             grid.x = (unsigned) (lp.head_tiles + (tiles - lp.head_tiles) * lp.tail_split);
         }
         int e;
-        if (small) e = launch_direct<1, 1, 2, 2, 4>(grid, stream, p, sched);
-        else if (narrow) e = launch_direct<2, 1, 2, 2, 4>(grid, stream, p, sched);
-        else if (wide) e = launch_direct<4, 2, 2, 4, 2>(grid, stream, p, sched);
-        else if (lp.tall_tile) e = launch_direct<2, 2, 4, 2, 3>(grid, stream, p, sched);
-        else e = launch_direct<2, 2, 2, 2, 2>(grid, stream, p, sched);
+        if (small) e = launch_direct<half_t, 1, 1, 2, 2, 4>(grid, stream, p, sched);
+        else if (narrow) e = launch_direct<half_t, 2, 1, 2, 2, 4>(grid, stream, p, sched);
+        else if (wide) e = launch_direct<half_t, 4, 2, 2, 4, 2>(grid, stream, p, sched);
+        else if (lp.tall_tile) e = launch_direct<half_t, 2, 2, 4, 2, 3>(grid, stream, p, sched);
+        else e = launch_direct<half_t, 2, 2, 2, 2, 2>(grid, stream, p, sched);
         if (e != 0) return e;
     } else if (small) launch_a<1, 64, 2, 2>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);
     else if (lp.tall_tile) launch_a<2, 64, 1, 4>(a_mode, b_mode, grid, stream, p, lp.k_chunk, xc);

@@ -712,10 +712,14 @@ int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
         const int mode = pick_mode(p.b_group[g], p.b_sn, p.b_sk, p.b_sb, p.batch);
         if (mode != b_mode) b_mode = Scalar;
     }
-    if (lp.small_tile && lp.bk == 64) launch_gemm_a<1, 64>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
+    bool direct = false;
+    int e = launch_gemm_f32_direct(lp, stream, &direct);
+    if (e != 0) return e;
+    if (direct) {
+    } else if (lp.small_tile && lp.bk == 64) launch_gemm_a<1, 64>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
     else if (lp.small_tile) launch_gemm_a<1, 16>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
     else launch_gemm_a<2, 16>(a_mode, b_mode, grid, stream, p, lp.k_chunk);
-    int e = (int) hipGetLastError();
+    e = (int) hipGetLastError();
     if (e == 0 && lp.split_k > 1) e = launch_gemm_reduce_partials(p, lp.split_k, false, stream);
     return e;
 }

@@ -49,7 +49,7 @@ struct GemmLaunchPlan {
     bool tall_tile;          // f16 only: 256 x 128 workgroup tiles (8 waves)
     bool narrow_tile;        // f16 direct kernel only: 128 x 64 workgroup tiles
     bool wide_tile;          // f16 direct kernel only, together with tall_tile: 256 x 256 workgroup tiles
-    bool direct;             // f16 only: shapes and strides allow the kernel that loads global -> LDS directly
+    bool direct;             // shapes and strides allow the kernel that loads global -> LDS directly
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)
     int k_chunk;             // K elements per split, a multiple of bk
@@ -108,6 +108,9 @@ bool attention_f16_supported(int dk, int dv);
 int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream);
 int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream);
 int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
+// the kernel that loads global -> LDS directly, where `lp` (of an f32 product) and the alignment of the pointers allow
+// it; `launched` tells whether it ran (the sum of split-K partial products is left to the caller)
+int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool *launched);
 // f16 operands and result, f32 accumulation, one rounding (to nearest even) at the store
 int launch_gemm_f16(const GemmParams &p, ihipStream_t *stream);
 // second pass of a split-K launch: C = sum of the f32 partial products in the workspace (`p` already oriented)
