@@ -1,0 +1,99 @@
+"""Differential test on seeded random matrix products: shapes, layouts and epilogues drawn so that every launch
+variant of the matmul kernels meets ragged edges (rows and columns that are no multiple of any tile, K with one slice
+or an odd number of slices, long K that is split over workgroups, batches, operands that are slices or permuted views
+of bigger tensors, constant [k, n] weights, bias / residual / relu in the store, projections that share an input).
+K is a multiple of 64 in two cases out of three, so that most products run on the kernel that loads global -> LDS
+directly and the rest on the kernels that stage through registers.
+
+CPU half: the graph evaluates in the oracle and plans for gfx950. GPU half: `check_gpu` (f32 within 1e-4, f16 within
+2e-2 of the oracle).
+"""
+import numpy as np
+import pytest
+
+from kyanite_amd import DType, Graph
+from runner import F16_MAX_REL, check_cpu, check_gpu
+
+SEEDS = list(range(40))
+
+
+def build(seed):
+    rng = np.random.default_rng(7000 + seed)
+    dtype = DType.F16 if seed % 2 else DType.F32
+    np_dtype = np.float16 if dtype == DType.F16 else np.float32
+    pick = lambda options: options[int(rng.integers(len(options)))]
+    g = Graph()
+    inputs = []
+
+    def tensor(shape, scale, constant=False):
+        data = (rng.standard_normal(shape) * scale).astype(np_dtype)
+        if constant:
+            return g.constant(list(shape), data, dtype)
+        inputs.append(data)
+        return g.input(list(shape), dtype)
+
+    m = pick([1, 7, 33, 64, 100, 130, 257, 300, 520])
+    n = pick([1, 8, 40, 72, 128, 200, 264, 392])
+    k = pick([64, 128, 192, 320, 1024, 2112, 4096, 24, 100, 264])
+    if m * n * k > 2.2e8:  # keep the oracle's share of the test run in seconds
+        k = pick([64, 128, 192, 320])
+    batch = pick([1, 1, 1, 2, 5]) if m * n * k < 3e7 else 1
+    scale = 1.0 / np.sqrt(k)
+    layout = pick(["linear", "linear", "matmul_const", "matmul_input", "sliced", "permuted_result"])
+
+    if batch > 1:
+        a = tensor((batch, m, k), 1.0)
+        if layout in ("matmul_input", "matmul_const"):
+            b = tensor((batch, k, n), scale)
+        else:
+            b = g.permute(tensor((batch, n, k), scale), [0, 2, 1])
+        y = g.batched_mat_mul(a, b)
+        if layout == "permuted_result":
+            y = g.permute(y, [0, 2, 1])
+        g.output(y)
+        return g, inputs, dtype
+
+    if layout == "sliced":
+        # both operands are windows of wider tensors: rows start at unaligned-looking offsets, strides exceed K
+        pad = pick([64, 8, 128])
+        a = g.slice(tensor((m, k + pad), 1.0), 1, pad, k + pad) if pad % 8 == 0 else tensor((m, k), 1.0)
+        w = g.slice(tensor((n + 3, k + pad), scale, constant=pick([True, False])), 0, 3, n + 3)
+        w = g.slice(w, 1, 0, k)
+        y = g.linear(a, w)
+    elif layout == "matmul_const":
+        a = tensor((m, k), 1.0)
+        y = g.mat_mul(a, tensor((k, n), scale, constant=True))
+    elif layout == "matmul_input":
+        a = tensor((m, k), 1.0)
+        y = g.mat_mul(a, tensor((k, n), scale))
+    else:
+        a = tensor((m, k), 1.0)
+        y = g.linear(a, tensor((n, k), scale, constant=pick([True, False])))
+    epilogue = pick(["none", "none", "bias", "bias_relu", "residual", "relu"])
+    if epilogue in ("bias", "bias_relu"):
+        y = g.add(y, tensor((1, n), 1.0, constant=True))
+    if epilogue == "residual":
+        y = g.add(y, tensor((m, n), 1.0))
+    if epilogue in ("bias_relu", "relu"):
+        y = g.relu(y)
+    if layout == "permuted_result":
+        y = g.permute(y, [1, 0])
+    g.output(y)
+    # now and then: two more projections of the same input, which may share its launch
+    if pick([True, False, False]):
+        for _ in range(2):
+            g.output(g.linear(a, tensor((n, k), scale, constant=True)))
+    return g, inputs, dtype
+
+
+@pytest.mark.parametrize("seed", SEEDS)
+def test_cpu(seed):
+    g, inputs, dtype = build(seed)
+    check_cpu(g, 0, inputs, None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", SEEDS)
+def test_gpu(seed, hip_device):
+    g, inputs, dtype = build(seed)
+    check_gpu(hip_device, g, 0, inputs, None, max_rel=F16_MAX_REL if dtype == DType.F16 else 1e-4)
