@@ -83,13 +83,32 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // Direct kernel only: 256 x 256 tiles (8 waves of 128 x 64) where they still give every compute unit a
     // workgroup. The LDS bounds this kernel, and they need the least LDS traffic per flop: 256 KB per slice of 64
     // for twice the work of a 256 x 128 tile with its 176 KB (8192^3: 1191 -> 1030 us, 4096^3: 166 -> 139 us).
+    // Between the two sit 256 x 192 tiles (216 KB per slice for one and a half times the work). Among the three
+    // the plan takes the one with the least estimated LDS time: rounds of workgroups on 256 compute units (a last
+    // sparse round counts as one split in two) x LDS clocks per slice. 2 x 512 x 11008 x 4096 in one launch:
+    // 344 tiles of 256 x 128 are 1.6 rounds of 2750 clocks, 232 tiles of 256 x 192 one round of 3375.
     const long long wide_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 255) / 256) * p.batch * groups;
-    lp.wide_tile = f16 && lp.direct && lp.tall_tile && p.n >= 256 && (p.n + 255) / 256 * 256 - p.n <= p.n / 8 &&
-                   wide_blocks >= env_int("KNHIP_F16_WIDE_FROM", 256);
+    const long long mid_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 191) / 192) * p.batch * groups;
+    if (f16 && lp.direct && lp.tall_tile) {
+        auto lds_time = [&](long long tiles, double clocks) {
+            const long long full = tiles / 256, rest = tiles % 256;
+            double rounds = (double) full;
+            if (rest > 0) rounds += full > 0 && rest <= 128 && p.batch == 1 && p.k >= 1024 ? 0.6 : 1.0;
+            return rounds * clocks;
+        };
+        auto fits = [&](int width) { return p.n >= width && (p.n + width - 1) / width * width - p.n <= p.n / 8; };
+        const double t_tall = lds_time(tall_blocks, 2750.0);
+        const double t_mid = fits(192) ? lds_time(mid_blocks, 3375.0) : 1e30;
+        const double t_wide = fits(256) && wide_blocks >= env_int("KNHIP_F16_WIDE_FROM", 256) ? lds_time(wide_blocks, 4000.0) : 1e30;
+        static const int mid_enabled = env_int("KNHIP_F16_MID_TILE", 1);
+        lp.wide_tile = t_wide <= t_tall && t_wide <= t_mid;
+        lp.mid_tile = !lp.wide_tile && mid_enabled && t_mid < t_tall;
+    }
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
     if (lp.narrow_tile) blocks = narrow_blocks;
     if (lp.wide_tile) blocks = wide_blocks;
+    if (lp.mid_tile) blocks = mid_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile || lp.narrow_tile ? 64 : 128;
     else if (lp.direct) lp.bk = 32;
     else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
@@ -112,7 +131,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
             long long chunk = (p.k + s - 1) / s;
             chunk = (chunk + 63) / 64 * 64;
             s = (p.k + chunk - 1) / chunk;
-            const int tm = lp.tall_tile ? 256 : (lp.small_tile ? 64 : 128), tn = lp.small_tile || lp.narrow_tile ? 64 : (lp.wide_tile ? 256 : 128);
+            const int tm = lp.tall_tile ? 256 : (lp.small_tile ? 64 : 128), tn = lp.small_tile || lp.narrow_tile ? 64 : (lp.wide_tile ? 256 : (lp.mid_tile ? 192 : 128));
             const unsigned long long bytes = (unsigned long long) rest * s * tm * tn * 4ull;
             if (s >= 2 && bytes <= (256ull << 20)) {
                 lp.head_tiles = (int) full;

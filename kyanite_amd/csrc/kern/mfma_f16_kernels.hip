@@ -597,9 +597,10 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     static const int direct_env = getenv("KNHIP_F16_DIRECT") ? atoi(getenv("KNHIP_F16_DIRECT")) : 1;
     const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % 64 == 0;
     // (128 x 64 tiles exist in the direct kernel only; without it they run as 64 x 64)
-    // (so do 256 x 256 tiles, which otherwise run as 256 x 128)
-    const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct), wide = lp.wide_tile && direct;
-    const int t_n = small || narrow ? 64 : (wide ? 256 : 128), t_m = lp.tall_tile ? 256 : (small ? 64 : 128);
+    // (so do 256 x 256 and 256 x 192 tiles, which otherwise run as 256 x 128)
+    const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct);
+    const bool wide = lp.wide_tile && direct, mid = lp.mid_tile && direct;
+    const int t_n = small || narrow ? 64 : (wide ? 256 : (mid ? 192 : 128)), t_m = lp.tall_tile ? 256 : (small ? 64 : 128);
     const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t_n - 1) / t_n) * groups;
     if (tiles > 0x7fffffffll) return (int) hipErrorInvalidConfiguration;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
@@ -621,6 +622,7 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
         if (small) e = launch_direct<half_t, 1, 1, 2, 2, 4>(grid, stream, p, sched);
         else if (narrow) e = launch_direct<half_t, 2, 1, 2, 2, 4>(grid, stream, p, sched);
         else if (wide) e = launch_direct<half_t, 4, 2, 2, 4, 2>(grid, stream, p, sched);
+        else if (mid) e = launch_direct<half_t, 2, 3, 4, 2, 2>(grid, stream, p, sched);
         else if (lp.tall_tile) e = launch_direct<half_t, 2, 2, 4, 2, 3>(grid, stream, p, sched);
         else e = launch_direct<half_t, 2, 2, 2, 2, 2>(grid, stream, p, sched);
         if (e != 0) return e;

@@ -1496,3 +1496,15 @@ def f16_matmul_direct_wide_tiles():
     b = g.input([16, 1016, 128], DType.F16)
     g.output(g.batched_mat_mul(a, g.permute(b, [0, 2, 1])))
     return g, 0, [_f16(rng, 16, 1000, 128, scale=0.2), _f16(rng, 16, 1016, 128, scale=0.2)], None
+
+
+@case
+def f16_matmul_direct_mid_tiles():
+    """256 x 192 tiles (8 waves of 64 x 96): 200 of them fill one round of workgroups where 300 tiles of 256 x 128
+    would need two; ragged columns, one slice of K"""
+    g = Graph()
+    rng = np.random.default_rng(156)
+    a = g.input([100, 256, 64], DType.F16)
+    b = g.input([100, 380, 64], DType.F16)
+    g.output(g.batched_mat_mul(a, g.permute(b, [0, 2, 1])))
+    return g, 0, [_f16(rng, 100, 256, 64, scale=0.3), _f16(rng, 100, 380, 64, scale=0.3)], None
