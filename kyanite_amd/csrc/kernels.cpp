@@ -788,9 +788,15 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         for (size_t k = 0; k < ops.size(); k++) static_strides[k].push_back(ops[k].shape.strides()[a]);
     }
 
-    bool softmax = desc.kind == RowKernelDesc::Softmax;
+    const bool softmax = desc.kind == RowKernelDesc::Softmax, rowred = desc.kind == RowKernelDesc::Reduce;
+    const ReduceOp rop = desc.reduce_op;
+    KN_ASSERT(!rowred || rop == ReduceOp::Sum || rop == ReduceOp::Mean || rop == ReduceOp::Max || rop == ReduceOp::Min);
+    // identity and fold of the first reduction over the row
+    const bool fold_max = softmax || (rowred && rop == ReduceOp::Max), fold_min = rowred && rop == ReduceOp::Min;
+    const char *identity = fold_max ? "-KN_INF" : (fold_min ? "KN_INF" : "0.0f");
+    const char *fold_fn = fold_max ? "kn_max" : (fold_min ? "kn_min" : "kn_add");
     KernelSpec spec;
-    spec.name = softmax ? "kn_softmax" : "kn_layernorm";
+    spec.name = softmax ? "kn_softmax" : (rowred ? "kn_rowreduce" : "kn_layernorm");
     spec.n_ptrs = ops.size();
     size_t static_size = concrete_size(static_shape);
     if (static_size == 0 || size == 0) return spec;
@@ -908,6 +914,14 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
 
     ss << "#define VEC " << vec << "\n#define ITEMS " << items << "\n#define G " << G << "\n";
     ss << "KN_DEV float kn_max(float a, float b) { return fmaxf(a, b); }\nKN_DEV float kn_add(float a, float b) { return a + b; }\n";
+    ss << "KN_DEV float kn_min(float a, float b) { return fminf(a, b); }\n";
+    auto emit_fold = [&](const std::string &indent, const std::string &src) {
+        if (fold_max) ss << indent << "for (int j = 0; j < VEC; j++) m = fmaxf(m, " << src << "[j]);\n";
+        else if (fold_min) ss << indent << "for (int j = 0; j < VEC; j++) m = fminf(m, " << src << "[j]);\n";
+        else ss << indent << "for (int j = 0; j < VEC; j++) m += " << src << "[j];\n";
+    };
+    // the row statistic of kind Reduce from the folded value `m` (like the post step of the reduce kernel)
+    const std::string stat_expr = rowred && rop == ReduceOp::Mean ? "m / (float) " + std::to_string(size) + ".0f" : std::string("m");
     // Holding the epilogue operands across rows costs a few registers more than the 64 per lane that full
     // occupancy allows; the compiler is told to stay within them (it has the slack: at most one spill was seen).
     ss << "extern \"C\" __global__ " << (seq > 1 ? "__attribute__((amdgpu_waves_per_eu(8, 8))) " : "") << "__launch_bounds__("
@@ -1025,22 +1039,24 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         if (prefetch_post && seq == 1) emit_post_loads("        ", "ic", "it");
         ss << "    }\n";
         ss << "    float x[ITEMS][VEC];\n";
-        ss << "    float m = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
+        ss << "    float m = " << identity << ";\n";
         ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
         emit_pre_apply("        ", "x[it]", "it");
         if (check_i)
-            ss << "        if (!(i < (idx_t) " << nv << ")) for (int j = 0; j < VEC; j++) x[it][j] = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
-        if (softmax) ss << "        for (int j = 0; j < VEC; j++) m = fmaxf(m, x[it][j]);\n";
-        else ss << "        for (int j = 0; j < VEC; j++) m += x[it][j];\n";
+            ss << "        if (!(i < (idx_t) " << nv << ")) for (int j = 0; j < VEC; j++) x[it][j] = " << identity << ";\n";
+        emit_fold("        ", "x[it]");
         ss << "    }\n";
         // layernorm with the same number of elements in every lane: per-lane mean and centred sum of squares,
         // combined pairwise in a single pass over the lanes instead of one pass for the mean and one for the
         // variance (one barrier instead of two when a row spans several waves)
         static const bool one_pass_env = !(getenv("KNHIP_ROW_ONE_PASS") && !atoi(getenv("KNHIP_ROW_ONE_PASS")));
-        const bool one_pass = !softmax && !check_i && G > 1 && one_pass_env;
-        if (!one_pass) reduce("m", softmax ? "kn_max" : "kn_add");
-        ss << "    float s = 0.0f;\n";
-        if (softmax) {
+        const bool one_pass = !softmax && !rowred && !check_i && G > 1 && one_pass_env;
+        if (!one_pass) reduce("m", fold_fn);
+        if (!rowred) ss << "    float s = 0.0f;\n";
+        if (rowred) {
+            ss << "    const float stat = " << stat_expr << ";\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = stat;\n    }\n";
+        } else if (softmax) {
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
             ss << "        for (int j = 0; j < VEC; j++) {\n            const float e = (i < (idx_t) " << nv << ") ? expf(x[it][j] - m) : 0.0f;\n";
             ss << "            x[it][j] = e;\n            s += e;\n        }\n    }\n";
@@ -1061,7 +1077,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "            x[it][j] = d;\n            s += d * d;\n        }\n    }\n";
             reduce("s", "kn_add");
         }
-        if (!softmax) {
+        if (!softmax && !rowred) {
             ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
             if (use_rcp) ss << "    const float rdenom = 1.0f / denom;\n#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] * rdenom;\n    }\n";
             else ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / denom;\n    }\n";
@@ -1076,35 +1092,42 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     } else {
         // rows too long for registers: stream the row three times (the re-reads come from cache)
         ss << "    float t[VEC];\n";
-        ss << "    float m = " << (softmax ? "-KN_INF" : "0.0f") << ";\n";
+        ss << "    float m = " << identity << ";\n";
         ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
         emit_load_pre("        ", "i", "t");
-        if (softmax) ss << "        for (int j = 0; j < VEC; j++) m = fmaxf(m, t[j]);\n";
-        else ss << "        for (int j = 0; j < VEC; j++) m += t[j];\n";
+        emit_fold("        ", "t");
         ss << "    }\n";
-        reduce("m", softmax ? "kn_max" : "kn_add");
-        if (!softmax) ss << "    const float mean = m / (float) " << size << ".0f;\n";
-        ss << "    float s = 0.0f;\n";
-        ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
-        emit_load_pre("        ", "i", "t");
-        if (softmax) ss << "        for (int j = 0; j < VEC; j++) s += expf(t[j] - m);\n";
-        else ss << "        for (int j = 0; j < VEC; j++) { const float d = t[j] - mean; s += d * d; }\n";
-        ss << "    }\n";
-        reduce("s", "kn_add");
-        if (!softmax) ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
-        ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
-        emit_load_pre("        ", "i", "t");
-        if (softmax) ss << "        for (int j = 0; j < VEC; j++) t[j] = expf(t[j] - m) / s;\n";
-        else ss << "        for (int j = 0; j < VEC; j++) t[j] = (t[j] - mean) / denom;\n";
-        emit_post_store("        ", "i", "t", "");
-        ss << "    }\n}\n";
+        reduce("m", fold_fn);
+        if (rowred) {
+            ss << "    const float stat = " << stat_expr << ";\n";
+            ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
+            ss << "        for (int j = 0; j < VEC; j++) t[j] = stat;\n";
+            emit_post_store("        ", "i", "t", "");
+            ss << "    }\n}\n";
+        } else {
+            if (!softmax) ss << "    const float mean = m / (float) " << size << ".0f;\n";
+            ss << "    float s = 0.0f;\n";
+            ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
+            emit_load_pre("        ", "i", "t");
+            if (softmax) ss << "        for (int j = 0; j < VEC; j++) s += expf(t[j] - m);\n";
+            else ss << "        for (int j = 0; j < VEC; j++) { const float d = t[j] - mean; s += d * d; }\n";
+            ss << "    }\n";
+            reduce("s", "kn_add");
+            if (!softmax) ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << DScalar::f32(desc.eps).to_c_str() << ");\n";
+            ss << "    if (" << valid << ") for (idx_t i = lane; i < (idx_t) " << nv << "; i += (idx_t) G) {\n";
+            emit_load_pre("        ", "i", "t");
+            if (softmax) ss << "        for (int j = 0; j < VEC; j++) t[j] = expf(t[j] - m) / s;\n";
+            else ss << "        for (int j = 0; j < VEC; j++) t[j] = (t[j] - mean) / denom;\n";
+            emit_post_store("        ", "i", "t", "");
+            ss << "    }\n}\n";
+        }
     }
 
     spec.source = ss.str();
     spec.block = (uint32_t) block;
     spec.grid = ceil_div_u32(static_size, rows_per_block * seq);
     std::ostringstream note;
-    note << (softmax ? "softmax" : "layernorm") << " G=" << G << " vec=" << vec << " items=" << items << (cached ? " cached" : " streamed");
+    note << (softmax ? "softmax" : (rowred ? "row statistic + elementwise" : "layernorm")) << " G=" << G << " vec=" << vec << " items=" << items << (cached ? " cached" : " streamed");
     if (seq > 1) note << " rows=" << seq;
     spec.strategy = note.str();
     return spec;

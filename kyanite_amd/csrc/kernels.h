@@ -59,8 +59,11 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
 // Row kernels. The value that gets normalised is `pre(load operands...)`, the value stored is
 // `post(normalised, load operands...)`: this is how a preceding scale / residual add and a following affine
 // (gamma, beta) or activation are fused into the single pass over the row.
+// Kind Reduce: the row statistic `fold(reduce_op, pre(...))` takes the place of the normalised value, the same for
+// every element of the row (an RMS norm: pre = x * x, mean, post = x * rsqrt(stat + eps) * w).
 struct RowKernelDesc {
-    enum Kind { Softmax, Layernorm } kind = Softmax;
+    enum Kind { Softmax, Layernorm, Reduce } kind = Softmax;
+    ReduceOp reduce_op = ReduceOp::Sum;  // Sum, Mean, Max or Min
     size_t axis = 0;
     float eps = 0;
     // operands[0] is the output, operands[1..] are inputs; every operand has the full (output) shape

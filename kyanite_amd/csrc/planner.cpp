@@ -94,7 +94,9 @@ struct ScalarBlock {
     ScalarExpr expr;
     std::map<Value, size_t> value_nodes;
     std::vector<std::optional<size_t>> loaded;  // per operand: the node that holds its loaded value
-    std::optional<Value> row_value;             // the layernorm / softmax whose result this block post-processes
+    // the layernorm / softmax whose result this block post-processes, or the reduction over the last axis whose
+    // result it reads back broadcast along that axis (a mean of squares in an RMS norm)
+    std::optional<Value> row_value;
     size_t row_node = 0;
 
     size_t load_operand(const PlanTensor &t) {
@@ -114,6 +116,7 @@ struct ScalarBlock {
 
 struct FusedRow {
     RowKernelDesc::Kind kind;
+    ReduceOp reduce_op = ReduceOp::Sum;
     size_t axis;
     float eps;
     std::vector<PlanTensor> inputs;  // 1 or 2 tensors
@@ -544,6 +547,7 @@ private:
         PlanTensor output = alloc_tensor_shared(info.shape.eval(batch_size), info.dtype);
         RowKernelDesc desc;
         desc.kind = row.kind;
+        desc.reduce_op = row.reduce_op;
         desc.axis = row.axis;
         desc.eps = row.eps;
         // operand order: output, row inputs, epilogue operands
@@ -558,7 +562,8 @@ private:
             if (n.kind == ScalarNode::Load && n.operand != SIZE_MAX) n.operand = extra_base + n.operand - 1;
 
         Step step;
-        step.kind = row.kind == RowKernelDesc::Softmax ? StepKind::SoftmaxOp : StepKind::LayernormOp;
+        step.kind = row.kind == RowKernelDesc::Softmax ? StepKind::SoftmaxOp
+                                                      : (row.kind == RowKernelDesc::Reduce ? StepKind::ReduceOp : StepKind::LayernormOp);
         step.kernel = make_row_kernel(desc);
         step.operands.push_back({output, OperandKind::Out});
         for (size_t k = 1; k < all.size(); k++) step.operands.push_back({all[k], OperandKind::In});
@@ -1086,8 +1091,10 @@ private:
         KN_ASSERT(root.value == block.expr.result());
 
         if (block.row_value) {
-            // the chain hangs off a layernorm / softmax: it becomes the epilogue of that row kernel
-            auto row = visit_row_inputs(*block.row_value);
+            // the chain hangs off a layernorm / softmax (or reads a statistic of its own rows): it becomes the
+            // epilogue of that row kernel
+            auto row = graph[*block.row_value].operation.kind == OpKind::Reduce ? visit_reduce_row_inputs(*block.row_value)
+                                                                                 : visit_row_inputs(*block.row_value);
             if (!row.ok) return VT::missing(row.need);
             return VT::done(push_row_kernel(*block.row_value, value, row.value, block.expr, block.operands));
         }
@@ -1201,6 +1208,12 @@ private:
         } else if (auto c = graph.as_single_const(value)) {
             n.kind = ScalarNode::Const;
             n.constant = *c;
+        } else if (auto reduce = row_reduce_under(value, target, block)) {
+            // A statistic of the very rows this kernel writes (the mean of squares of an RMS norm): the kernel
+            // becomes a row kernel that computes it itself, instead of a reduce launch in front of it.
+            block.row_value = *reduce;
+            n.kind = ScalarNode::Load;
+            n.operand = SIZE_MAX;
         } else {
             auto t = visit(value);
             if (!t.ok) return R::missing(t.need);
@@ -1211,6 +1224,64 @@ private:
         block.expr.nodes.push_back(n);
         block.value_nodes[value] = block.expr.nodes.size() - 1;
         return R::done(block.expr.nodes.size() - 1);
+    }
+
+    // `value`, seen through views that only it uses, is a Sum / Mean / Max / Min over the last axis of a tensor of
+    // shape `target`, kept as a column ([..., 1]) that the caller broadcasts back along that axis
+    std::optional<Value> row_reduce_under(Value value, const ConcreteShape &target, const ScalarBlock &block) const {
+        if (!options.fuse_row_epilogue || block.row_value || target.empty() || target.back() < 2) return std::nullopt;
+        ConcreteShape column = target;
+        column.back() = 1;
+        if (graph[value].shape.eval(batch_size) != column) return std::nullopt;
+        Value v = value;
+        while (graph[v].operation.kind == OpKind::View) {
+            if (!can_fuse(v) || map.count(v)) return std::nullopt;
+            v = graph[v].operation.inputs[0];
+        }
+        const Operation &op = graph[v].operation;
+        if (op.kind != OpKind::Reduce || !can_fuse(v) || map.count(v)) return std::nullopt;
+        if (op.reduce != ReduceOp::Sum && op.reduce != ReduceOp::Mean && op.reduce != ReduceOp::Max && op.reduce != ReduceOp::Min)
+            return std::nullopt;
+        if (op.axes != std::vector<size_t>{target.size() - 1}) return std::nullopt;
+        if (graph[op.inputs[0]].shape.eval(batch_size) != target) return std::nullopt;
+        const DType dt = graph[v].dtype;
+        if ((dt != DType::F32 && dt != DType::F16) || graph[op.inputs[0]].dtype != dt) return std::nullopt;
+        return v;
+    }
+
+    // The operands and prologue of a reduction that a row kernel computes for itself: an elementwise chain that
+    // only the reduction uses is evaluated on the loaded elements (like in the reduce kernel).
+    Visit<FusedRow> visit_reduce_row_inputs(Value reduce) {
+        using R = Visit<FusedRow>;
+        const Operation &op = graph[reduce].operation;
+        FusedRow row;
+        row.kind = RowKernelDesc::Reduce;
+        row.reduce_op = op.reduce;
+        row.axis = op.axes[0];
+        row.eps = 0;
+        const Value in_v = op.inputs[0];
+        const OpKind in_kind = graph[in_v].operation.kind;
+        if (!map.count(in_v) && can_fuse(in_v) && (in_kind == OpKind::Unary || in_kind == OpKind::Binary)) {
+            ScalarBlock pre;
+            pre.operands.push_back(PlanTensor());
+            pre.loaded.push_back(std::nullopt);
+            auto root = visit_fused_scalar_recurse(in_v, pre, true);
+            if (!root.ok) return R::missing(root.need);
+            if (!pre.row_value) {
+                row.inputs.assign(pre.operands.begin() + 1, pre.operands.end());
+                row.pre = pre.expr;
+                return R::done(row);
+            }
+        }
+        auto t = visit(in_v);
+        if (!t.ok) return R::missing(t.need);
+        row.inputs = {t.value};
+        ScalarNode n;
+        n.kind = ScalarNode::Load;
+        n.dtype = t.value.dtype;
+        n.operand = 1;
+        row.pre.nodes.push_back(n);
+        return R::done(row);
     }
 
     // planner.rs:926-931

@@ -1280,9 +1280,9 @@ def reduce_with_elementwise_prologue():
 
 
 @case
-def rms_norm_two_launches():
-    """x * rsqrt(mean(x^2) + eps) * w: the square folds into the reduction, the rsqrt of the broadcast mean into the
-    scaling kernel; f32 and f16"""
+def rms_norm_one_launch():
+    """x * rsqrt(mean(x^2) + eps) * w: ONE row kernel that computes the mean of squares of its own rows (the square
+    as its prologue) and scales them (the rsqrt of the mean as part of its epilogue); f32 and f16"""
     g = Graph()
     rng = np.random.default_rng(121)
     outs = []
@@ -1508,3 +1508,31 @@ def f16_matmul_direct_mid_tiles():
     b = g.input([100, 380, 64], DType.F16)
     g.output(g.batched_mat_mul(a, g.permute(b, [0, 2, 1])))
     return g, 0, [_f16(rng, 100, 256, 64, scale=0.3), _f16(rng, 100, 380, 64, scale=0.3)], None
+
+
+@case
+def row_statistics_in_the_elementwise_kernel():
+    """more statistics of the very rows an elementwise kernel writes, each computed inside it: x - max(x),
+    |x| / sum(|x|) (with the abs shared by the prologue and the epilogue), x * min(x) on rows too long for registers
+    (streamed), in f16 as well; and the cases that stay separate launches: a statistic that something else reads
+    too, and one over another axis"""
+    g = Graph()
+    rng = np.random.default_rng(160)
+    x = g.input([37, 200])
+    col = lambda v, rows: g.view(v, [rows, 1])
+    g.output(g.sub(x, g.broadcast(col(g.reduce(x, [1], ReduceOp.MAX), 37), [37, 200])))
+    a = g.unary(UnaryOp.ABS, x)
+    g.output(g.binary(BinaryOp.DIV, a, g.broadcast(col(g.reduce(a, [1], ReduceOp.SUM), 37), [37, 200])))
+    long_x = g.input([3, 70000])
+    g.output(g.mul(long_x, g.broadcast(col(g.reduce(long_x, [1], ReduceOp.MIN), 3), [3, 70000])))
+    h = g.input([20, 136], DType.F16)
+    hm = col(g.reduce(g.mul(h, h), [1], ReduceOp.MEAN), 20)
+    g.output(g.mul(h, g.broadcast(g.unary(UnaryOp.SQRT, g.add(hm, g.scalar(0.5, DType.F16))), [20, 136])))
+    # read twice: stays a reduce launch
+    shared = g.reduce(x, [1], ReduceOp.SUM)
+    g.output(shared)
+    g.output(g.add(x, g.broadcast(col(shared, 37), [37, 200])))
+    # over the rows, not along them
+    g.output(g.sub(x, g.broadcast(g.view(g.reduce(x, [0], ReduceOp.MEAN), [1, 200]), [37, 200])))
+    return g, 0, [rng.standard_normal((37, 200)).astype(np.float32), rng.standard_normal((3, 70000)).astype(np.float32),
+                  rng.standard_normal((20, 136)).astype(np.float16)], None

@@ -147,3 +147,16 @@ def test_constant_weights_are_laid_out_again_for_f16_matmuls(monkeypatch):
     g.output(g.mat_mul(x, w))
     g.output(g.unary(UnaryOp.NEG, w))
     assert HipExecutor(0, g, 0, plan_only=True).mem_usage["dedicated_bytes"] == 96 * 256 * 2
+
+
+def test_rms_norm_is_one_row_kernel():
+    """x * rsqrt(mean(x^2) + eps) * w plans as ONE launch: a row kernel that computes the statistic of its own rows."""
+    from kyanite_amd import BinaryOp, ReduceOp
+    g = Graph()
+    x = g.input([512, 4096], DType.F16)
+    w = g.constant([1, 4096], np.ones((1, 4096), np.float16), DType.F16)
+    ms = g.view(g.reduce(g.mul(x, x), [1], ReduceOp.MEAN), [512, 1])
+    r = g.binary(BinaryOp.DIV, g.scalar(1.0, DType.F16), g.unary(UnaryOp.SQRT, g.add(ms, g.scalar(1e-5, DType.F16))))
+    g.output(g.mul(g.mul(x, g.broadcast(r, [512, 4096])), g.broadcast(w, [512, 4096])))
+    ex = HipExecutor(0, g, 0, plan_only=True)
+    assert ex.step_kinds() == ["reduce_op"] and "row statistic" in ex.step_str(0)
