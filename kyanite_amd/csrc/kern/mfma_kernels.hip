@@ -392,7 +392,8 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     constexpr int KS = CB * KH * KW;      // K slice
     constexpr int A_VEC = KS / 4;         // 128 bit loads per filter row and slice
     constexpr int A_ITERS = (BM * A_VEC + THREADS - 1) / THREADS;
-    constexpr int A_STRIDE = BM + 5;      // odd, spreads the transposing stores over the banks
+    // rows k and k + 1, which the two halves of a wave read together, lie 32 of the 64 LDS banks apart
+    constexpr int A_STRIDE = BM + 32;
     static_assert(KS % 4 == 0 && KS % 2 == 0, "slice shape");
     __shared__ float As[KS][A_STRIDE];
     __shared__ __attribute__((aligned(16))) float Bs[PLANE_LDS];
@@ -437,9 +438,10 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     int a_dst[A_ITERS];
 #pragma unroll
     for (int i = 0; i < A_ITERS; i++) {
-        const int e = t + THREADS * i, row = e / A_VEC, q = e - row * A_VEC;
-        a_src[i] = row < BM && (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
-        a_dst[i] = row < BM ? 4 * q * A_STRIDE + row : -1;
+        // (consecutive lanes take consecutive filter rows, so that their transposing stores hit different banks)
+        const int e = t + THREADS * i, q = e / BM, row = e - q * BM;
+        a_src[i] = q < A_VEC && (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
+        a_dst[i] = q < A_VEC ? 4 * q * A_STRIDE + row : -1;
     }
     // ---- where this lane's output positions sit inside a plane, and which taps stay inside the image
     int lane_base[NJ];
