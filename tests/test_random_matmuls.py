@@ -14,7 +14,7 @@ import pytest
 from kyanite_amd import DType, Graph
 from runner import F16_MAX_REL, check_cpu, check_gpu
 
-SEEDS = list(range(40))
+SEEDS = list(range(96))
 
 
 def build(seed):
