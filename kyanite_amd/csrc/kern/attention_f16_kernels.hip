@@ -60,13 +60,14 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     const int query_c = min(query, p.lq - 1);
     half_t (*Ks)[KS] = (half_t (*)[KS]) &lds[wave][0];
     half_t (*Vt)[VS] = (half_t (*)[VS]) &lds[wave][BKEYS * KS * 2];
-    const half_t *kp = (const half_t *) p.k + bz * p.k_sb, *vp = (const half_t *) p.v + bz * p.v_sb;
+    const int bz1 = bz / p.batch_inner, bz2 = bz - bz1 * p.batch_inner;
+    const half_t *kp = (const half_t *) p.k + bz1 * p.k_sb + bz2 * p.k_sb2, *vp = (const half_t *) p.v + bz1 * p.v_sb + bz2 * p.v_sb2;
     const half_t *mp = p.mask ? (const half_t *) p.mask + bz * p.m_sb + (long long) query_c * p.m_sq : nullptr;
 
     // Q^T operand: lane (query c, half h) holds k = 16 t + 8 h .. + 7 for step t
     halfx8 qf[DK / 16];
     {
-        const half_t *qp = (const half_t *) p.q + bz * p.q_sb + (long long) query_c * p.q_sm;
+        const half_t *qp = (const half_t *) p.q + bz1 * p.q_sb + bz2 * p.q_sb2 + (long long) query_c * p.q_sm;
 #pragma unroll
         for (int t = 0; t < DK / 16; t++) {
             qf[t] = *(const halfx8 *) (qp + 16 * t + 8 * h);
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     }
     if (query < p.lq) {
         const float inv = 1.0f / total_sum;
-        half_t *op = (half_t *) p.o + bz * p.o_sb + (long long) query * p.o_sm;
+        half_t *op = (half_t *) p.o + bz1 * p.o_sb + bz2 * p.o_sb2 + (long long) query * p.o_sm;
         // wave w, half h: dims (2 w + h) * DV / 8 ... + DV / 8
         constexpr int PER = DV / 8;
 #pragma unroll
@@ -288,7 +289,8 @@ bool attention_f16_supported(int dk, int dv) {
 
 int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream) {
     if (p.batch <= 0 || p.lq <= 0 || p.dv <= 0) return 0;
-    if (!attention_f16_supported(p.dk, p.dv) || p.lk <= 0 || p.batch > 65535) return (int) hipErrorInvalidValue;
+    if (!attention_f16_supported(p.dk, p.dv) || p.lk <= 0 || p.batch > 65535 || p.batch_inner <= 0) return (int) hipErrorInvalidValue;
+    if (p.q_sb2 % 8 != 0 || p.k_sb2 % 8 != 0 || p.v_sb2 % 8 != 0) return (int) hipErrorInvalidValue;
     // the vector loads need contiguous, 16 byte aligned rows
     auto aligned = [](const void *ptr, long long batch_stride, long long row_stride) {
         return (uintptr_t) ptr % 16 == 0 && batch_stride % 8 == 0 && row_stride % 8 == 0;

@@ -42,14 +42,15 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
     const int c = lane & 31, h = lane >> 5;
     const int bz = blockIdx.y;
     const int query = blockIdx.x * BQ + wave * 32 + c;
-    const float *kp = (const float *) p.k + bz * p.k_sb, *vp = (const float *) p.v + bz * p.v_sb;
+    const int bz1 = bz / p.batch_inner, bz2 = bz - bz1 * p.batch_inner;
+    const float *kp = (const float *) p.k + bz1 * p.k_sb + bz2 * p.k_sb2, *vp = (const float *) p.v + bz1 * p.v_sb + bz2 * p.v_sb2;
 
     // Q^T operand: lane (query c, half h) holds k = h * HALF + t for step t, pre-multiplied by scale * log2(e) so
     // that the exponentials are plain exp2
     float qf[HALF];
     {
         const float factor = p.scale * 1.44269504088896340736f;
-        const float *qp = (const float *) p.q + bz * p.q_sb + (long long) query * p.q_sm;
+        const float *qp = (const float *) p.q + bz1 * p.q_sb + bz2 * p.q_sb2 + (long long) query * p.q_sm;
 #pragma unroll
         for (int t = 0; t < HALF; t++) qf[t] = query < p.lq ? qp[(long long) (h * HALF + t) * p.q_sk] * factor : 0.0f;
     }
@@ -190,7 +191,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
     row_sum += __shfl_xor(row_sum, 32);
     if (query < p.lq) {
         const float inv = 1.0f / row_sum;
-        float *op = (float *) p.o + bz * p.o_sb + (long long) query * p.o_sm;
+        float *op = (float *) p.o + bz1 * p.o_sb + bz2 * p.o_sb2 + (long long) query * p.o_sm;
 #pragma unroll
         for (int t = 0; t < DVT; t++)
 #pragma unroll
@@ -209,7 +210,7 @@ bool attention_supported(int dk, int dv) {
 
 int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream) {
     if (p.batch <= 0 || p.lq <= 0 || p.dv <= 0) return 0;
-    if (!attention_supported(p.dk, p.dv) || p.lk <= 0 || p.batch > 65535) return (int) hipErrorInvalidValue;
+    if (!attention_supported(p.dk, p.dv) || p.lk <= 0 || p.batch > 65535 || p.batch_inner <= 0) return (int) hipErrorInvalidValue;
     const dim3 grid((unsigned) ((p.lq + BQ - 1) / BQ), (unsigned) p.batch), block(THREADS);
     const bool wide = p.dv > 32;
     switch (p.dk) {

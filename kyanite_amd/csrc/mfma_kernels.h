@@ -91,6 +91,10 @@ struct AttentionParams {
     const void *v;
     void *o;
     int batch, lq, lk, dk, dv;
+    // batch entry z is (z / batch_inner, z % batch_inner); the `_sb` strides are those of the first index, the
+    // `_sb2` strides those of the second (the mask is indexed by z itself)
+    int batch_inner = 1;
+    long long q_sb2 = 0, k_sb2 = 0, v_sb2 = 0, o_sb2 = 0;
     long long q_sb, q_sm, q_sk;
     long long k_sb, k_sn, k_sk;  // k_sn: between keys, k_sk: along dk
     long long v_sb, v_sk, v_sn;  // v_sk: between keys, v_sn: along dv

@@ -437,6 +437,23 @@ private:
                 return VT::done(mm.permute(permutation));
             }
         }
+        if (options.fuse_attention && can_fuse(input) && permutation == std::vector<size_t>{0, 2, 1, 3} && !map.count(input)) {
+            // attention over [batch, heads] whose result goes back to [batch, tokens, heads, width] order: the
+            // kernel stores in that order itself instead of a copy after it
+            const Operation &vop = graph[input].operation;
+            const Value mm = vop.kind == OpKind::View ? vop.inputs[0] : input;
+            if (vop.kind == OpKind::View && graph[mm].operation.kind == OpKind::MatMul && can_fuse(mm) && !map.count(mm)) {
+                const ConcreteShape split = graph[input].shape.eval(batch_size), flat = graph[mm].shape.eval(batch_size);
+                if (split.size() == 4 && flat.size() == 3 && split[0] * split[1] == flat[0] && split[2] == flat[1] && split[3] == flat[2]) {
+                    auto fused = try_visit_fused_attention(mm, true, split[1]);
+                    if (!fused.ok) return VT::missing(fused.need);
+                    if (fused.value) {
+                        insert_mapping(input, *fused.value);
+                        return VT::done(fused.value->permute(permutation));
+                    }
+                }
+            }
+        }
         KN_TRY(t, visit(input));
         return VT::done(t.permute(permutation));
     }
@@ -644,7 +661,31 @@ private:
     // matmul(softmax(matmul(q, kt) [* or / constant] [+ mask], last axis), v) in f32 (no mask) or f16, every
     // intermediate value hidden and used once: the scores stay on the compute unit instead of passing through memory
     // between three or more launches (planner.rs:606-648, :418-476 plan them separately).
-    Visit<std::optional<PlanTensor>> try_visit_fused_attention(Value value, bool batch_first = true) {
+    // An operand [b, rows, cols] of the fused attention as [b1, b2, rows, cols] with b1 * b2 = b. The batch of an
+    // attention is usually (batch, heads) flattened, and the flattening of a permuted [batch, tokens, heads, width]
+    // tensor is no stride edit: the kernel takes two batch strides instead of a dense copy of the operand.
+    VT visit_split_batch(Value v) {
+        const Operation &op = graph[v].operation;
+        const ConcreteShape flat = graph[v].shape.eval(batch_size);
+        if (op.kind == OpKind::View && !map.count(v)) {
+            KN_TRY(inner, visit(op.inputs[0]));
+            const auto &shape = inner.shape.shape();
+            if (shape.size() == 4 && shape[0] * shape[1] == flat[0] && shape[2] == flat[1] && shape[3] == flat[2]) return VT::done(inner);
+        }
+        if (op.kind == OpKind::Permute && op.axes == std::vector<size_t>{0, 2, 1} && !map.count(v)) {
+            // K^T: the transposition commutes with the split of the batch
+            KN_TRY(inner, visit_split_batch(op.inputs[0]));
+            return VT::done(inner.permute({0, 1, 3, 2}));
+        }
+        KN_TRY(t, visit(v));
+        auto split = t.view({1, flat[0], flat[1], flat[2]});
+        KN_ASSERT(split.has_value(), "a leading axis of size 1 is a stride edit");
+        return VT::done(*split);
+    }
+
+    // `split_inner` > 0: the result is wanted as [b / split_inner, split_inner, lq, dv], laid out in memory as
+    // [b / split_inner, lq, split_inner, dv] (what `permute [0, 2, 1, 3]` of it turns into a dense tensor)
+    Visit<std::optional<PlanTensor>> try_visit_fused_attention(Value value, bool batch_first = true, size_t split_inner = 0) {
         using R = Visit<std::optional<PlanTensor>>;
         const ValueInfo &info = graph[value];
         const DType dt = info.dtype;
@@ -701,33 +742,56 @@ private:
         if (dk > 1024 || dv > 1024) return R::done(std::nullopt);
         if (!(f16 ? attention_f16_supported((int) dk, (int) dv) : attention_supported((int) dk, (int) dv))) return R::done(std::nullopt);
 
-        auto q = visit(q_v);
+        auto q = visit_split_batch(q_v);
         if (!q.ok) return R::missing(q.need);
-        auto kt = visit(kt_v);
+        auto kt = visit_split_batch(kt_v);
         if (!kt.ok) return R::missing(kt.need);
-        auto v = visit(v_v);
+        auto v = visit_split_batch(v_v);
         if (!v.ok) return R::missing(v.need);
+        // one split of the batch for the whole launch: the one the result asks for, else that of the operands
+        size_t inner_batch = split_inner > 0 ? split_inner : 1;
+        if (split_inner == 0)
+            for (const PlanTensor *t : {&q.value, &kt.value, &v.value})
+                if (t->shape.shape()[0] > 1) inner_batch = std::max(inner_batch, t->shape.shape()[1]);
+        if (b % inner_batch != 0) return R::done(std::nullopt);
+        {
+            const Value from[3] = {q_v, kt_v, v_v};
+            PlanTensor *operand[3] = {&q.value, &kt.value, &v.value};
+            for (int i = 0; i < 3; i++) {
+                const auto &shape = operand[i]->shape.shape();
+                auto again = operand[i]->view({b / inner_batch, inner_batch, shape[2], shape[3]});
+                if (!again) {
+                    // split in another way: the flat operand (a dense copy), whose batch axis splits in any way
+                    auto flat = visit(from[i]);
+                    if (!flat.ok) return R::missing(flat.need);
+                    again = flat.value.view({b / inner_batch, inner_batch, shape[2], shape[3]});
+                    KN_ASSERT(again.has_value(), "splitting an axis is a stride edit");
+                }
+                *operand[i] = *again;
+            }
+        }
         std::optional<PlanTensor> mask;
         if (mask_v) {
             auto m = visit(*mask_v);
             if (!m.ok) return R::missing(m.need);
             mask = m.value;
         }
+        // strides of [b1, b2, rows, cols]
         const auto &qs = q.value.shape.strides(), &ks = kt.value.shape.strides(), &vs = v.value.shape.strides();
         if (f16) {
             // rows of Q, K and V are read as 128 bit vectors
-            auto rows_ok = [](const PlanTensor &t, long long batch_stride, long long row_stride, long long inner_stride) {
-                return inner_stride == 1 && row_stride % 8 == 0 && batch_stride % 8 == 0 && t.ptr.offset_bytes % 16 == 0;
+            auto rows_ok = [](const PlanTensor &t, long long row_stride, long long inner_stride) {
+                const auto &st = t.shape.strides();
+                return inner_stride == 1 && row_stride % 8 == 0 && st[0] % 8 == 0 && st[1] % 8 == 0 && t.ptr.offset_bytes % 16 == 0;
             };
-            if (!rows_ok(q.value, qs[0], qs[1], qs[2]) || !rows_ok(kt.value, ks[0], ks[2], ks[1]) ||
-                !rows_ok(v.value, vs[0], vs[1], vs[2]))
+            if (!rows_ok(q.value, qs[2], qs[3]) || !rows_ok(kt.value, ks[3], ks[2]) || !rows_ok(v.value, vs[2], vs[3]))
                 return R::done(std::nullopt);
             // a block of 64 keys is addressed with 32 bit offsets from the block's base
-            if (ks[2] < 0 || ks[2] > (1 << 20) || vs[1] < 0 || vs[1] > (1 << 20)) return R::done(std::nullopt);
+            if (ks[3] < 0 || ks[3] > (1 << 20) || vs[2] < 0 || vs[2] > (1 << 20)) return R::done(std::nullopt);
         } else {
             // the kernel addresses a block of 64 keys with 32 bit offsets from the block's base
             auto fits = [](const PlanTensor &t) {
-                for (size_t a = 1; a < 3; a++) {
+                for (size_t a = 2; a < 4; a++) {
                     const long long s = t.shape.strides()[a];
                     if (s < 0 || s > (1ll << 20)) return false;
                 }
@@ -736,8 +800,17 @@ private:
             if (!fits(kt.value) || !fits(v.value)) return R::done(std::nullopt);
         }
 
-        PlanTensor result = batch_first ? alloc_tensor_shared({b, lq, dv}, dt)
-                                        : alloc_tensor_shared({lq, b, dv}, dt).permute({1, 0, 2});
+        // the result as the caller sees it, and as [b1, b2, lq, dv] for the kernel
+        PlanTensor result, result_split;
+        if (split_inner > 0) {
+            result = alloc_tensor_shared({b / inner_batch, lq, inner_batch, dv}, dt).permute({0, 2, 1, 3});
+            result_split = result;
+        } else {
+            result = batch_first ? alloc_tensor_shared({b, lq, dv}, dt) : alloc_tensor_shared({lq, b, dv}, dt).permute({1, 0, 2});
+            auto split = result.view({b / inner_batch, inner_batch, lq, dv});
+            KN_ASSERT(split.has_value(), "splitting an axis is a stride edit");
+            result_split = *split;
+        }
         Step step;
         step.kind = StepKind::MatMul;
         step.attention = true;
@@ -746,11 +819,12 @@ private:
         a.batch = (int) b; a.lq = (int) lq; a.lk = (int) lk; a.dk = (int) dk; a.dv = (int) dv;
         a.scale = scale;
         a.has_scale = has_scale ? 1 : 0;
-        const auto &os = result.shape.strides();
-        a.q_sb = qs[0]; a.q_sm = qs[1]; a.q_sk = qs[2];
-        a.k_sb = ks[0]; a.k_sk = ks[1]; a.k_sn = ks[2];  // the operand is K^T: [b, dk, lk]
-        a.v_sb = vs[0]; a.v_sk = vs[1]; a.v_sn = vs[2];
-        a.o_sb = os[0]; a.o_sm = os[1]; a.o_sn = os[2];
+        a.batch_inner = (int) inner_batch;
+        const auto &os = result_split.shape.strides();
+        a.q_sb = qs[0]; a.q_sb2 = qs[1]; a.q_sm = qs[2]; a.q_sk = qs[3];
+        a.k_sb = ks[0]; a.k_sb2 = ks[1]; a.k_sk = ks[2]; a.k_sn = ks[3];  // the operand is K^T: [b, dk, lk]
+        a.v_sb = vs[0]; a.v_sb2 = vs[1]; a.v_sk = vs[2]; a.v_sn = vs[3];
+        a.o_sb = os[0]; a.o_sb2 = os[1]; a.o_sm = os[2]; a.o_sn = os[3];
         step.operands = {{q.value, OperandKind::In}, {kt.value, OperandKind::In}, {v.value, OperandKind::In}};
         if (mask) {
             KN_ASSERT(mask->shape.shape() == ConcreteShape({b, lq, lk}));

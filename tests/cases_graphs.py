@@ -1199,6 +1199,54 @@ def attention_fused_many_blocks():
     return g, b, inputs, None
 
 
+def _attention_split_heads_case(seed, batch, heads, lq, lk, dk, dv, dtype=DType.F32, kv_split=None):
+    """attention over (batch, heads) as a transformer block writes it: q, k, v are [batch * tokens, heads * width]
+    projections, viewed as [batch, tokens, heads, width], permuted to [batch, heads, tokens, width] and flattened to
+    [batch * heads, tokens, width] (no stride edit: a dense copy unless the kernel takes two batch strides); the result
+    goes back the same way. `kv_split`: K and V arrive flattened and dense instead (another split of the batch)."""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    np_dtype = np.float16 if dtype == DType.F16 else np.float32
+    inputs = []
+
+    def inp(shape):
+        inputs.append(rng.standard_normal(shape).astype(np_dtype))
+        return g.input(list(shape), dtype)
+
+    def heads_of(x, tokens, width):
+        x = g.permute(g.view(x, [batch, tokens, heads, width]), [0, 2, 1, 3])
+        return g.view(x, [batch * heads, tokens, width])
+
+    q = heads_of(inp((batch * lq, heads * dk)), lq, dk)
+    if kv_split == "dense":
+        k, v = inp((batch * heads, lk, dk)), inp((batch * heads, lk, dv))
+    else:
+        k, v = heads_of(inp((batch * lk, heads * dk)), lk, dk), heads_of(inp((batch * lk, heads * dv)), lk, dv)
+    scores = g.mul(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), g.scalar(1.0 / np.sqrt(dk), dtype))
+    out = g.batched_mat_mul(g.softmax(scores, 2), v)
+    out = g.permute(g.view(out, [batch, heads, lq, dv]), [0, 2, 1, 3])
+    g.output(g.view(out, [batch * lq, heads * dv]))
+    return g, 0, inputs, None
+
+
+@case
+def attention_split_heads_no_copies():
+    """f32, 2 x 3 heads of width 40: operands and result in [batch, tokens, heads, width] order, ragged lengths"""
+    return _attention_split_heads_case(105, 2, 3, 150, 77, 40, 40)
+
+
+@case
+def attention_split_heads_mixed_operands():
+    """Q and the result split as (batch, heads), K and V dense over the flat batch"""
+    return _attention_split_heads_case(106, 3, 2, 70, 130, 64, 32, kv_split="dense")
+
+
+@case
+def attention_f16_split_heads_no_copies():
+    """f16, 2 x 4 heads of width 64 in [batch, tokens, heads, width] order"""
+    return _attention_split_heads_case(107, 2, 4, 100, 100, 64, 64, DType.F16)
+
+
 @case
 def attention_chain_not_fused():
     """the scores are an output as well, so the chain has to stay three launches"""

@@ -87,6 +87,20 @@ def test_attention_chain_is_one_launch():
     assert nbytes == 4 * 2 * (50 * 40 + 60 * 40 + 60 * 40 + 50 * 40)
 
 
+def test_attention_over_batch_and_heads_needs_no_copies():
+    # q, k, v in [batch, tokens, heads, width] order, flattened to [batch * heads, tokens, width] through a permute
+    # (no stride edit), result permuted back: the kernel takes two batch strides, so the plan is the one launch
+    from cases_graphs import CASES
+    for name in ("attention_split_heads_no_copies", "attention_f16_split_heads_no_copies"):
+        g, batch, _, _ = CASES[name]()
+        ex = HipExecutor(0, g, batch, plan_only=True)
+        assert ex.step_kinds() == ["mat_mul"], name
+        assert "attention" in ex.step_str(0)
+    # K and V split in another way than Q: still one launch, over the flat batch of K and V
+    g, batch, _, _ = CASES["attention_split_heads_mixed_operands"]()
+    assert HipExecutor(0, g, batch, plan_only=True).step_kinds() == ["mat_mul"]
+
+
 def test_attention_chain_stays_apart_when_it_must():
     three = ["mat_mul", "softmax_op", "mat_mul"]
     # the probabilities are needed elsewhere
