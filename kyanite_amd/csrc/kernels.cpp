@@ -454,6 +454,130 @@ KernelSpec make_scalar_kernel(const std::vector<KernelOperand> &operands, const 
     return make_scalar_kernel_multi(operands, {expr});
 }
 
+namespace {
+
+// Elementwise kernels with a transposed operand. When an input is contiguous along another axis than the outputs
+// (a permuted view: NCHW -> tokens, a [k, n] weight read as [n, k]), neither order of the plain kernel's index
+// space gives both sides wide accesses: lanes that run along the outputs' rows read the input with a stride, 4 or
+// 2 useful bytes per cache line touched. Here a workgroup owns a tile of 64 x 64 elements (input axis x output axis): it
+// reads the transposed operands with lanes along THEIR contiguous axis into LDS, then computes and stores with
+// lanes along the outputs' axis, taking those operands from LDS. Rows of the LDS tile are padded so that both
+// directions are free of bank conflicts.
+std::optional<KernelSpec> make_transposed_tile_kernel(const std::vector<KernelOperand> &operands, const std::vector<ScalarExpr> &exprs,
+                                                      const Collapsed &c, size_t total) {
+    static const bool enabled = [] {
+        const char *env = getenv("KNHIP_TILED_TRANSPOSE");
+        return !(env && *env == '0');
+    }();
+    const size_t n_out = exprs.size(), n_ops = operands.size(), rank = c.rank();
+    if (!enabled || rank < 2 || total < (1u << 16)) return std::nullopt;
+    const size_t last = rank - 1;
+    for (size_t o = 0; o < n_out; o++)
+        if (c.strides[o][last] != 1) return std::nullopt;
+    // the transposed operands, and the axis they all are contiguous along
+    std::vector<bool> transposed(n_ops, false);
+    std::optional<size_t> axis;
+    size_t lds_bytes = 0;
+    constexpr size_t TILE = 64;
+    auto pitch_of = [](DType t) { return TILE + std::max<size_t>(1, 4 / dtype_bytes(t)); };
+    for (size_t k = n_out; k < n_ops; k++) {
+        const int64_t inner = c.strides[k][last];
+        if (inner == 0 || inner == 1) continue;
+        std::optional<size_t> mine;
+        for (size_t a = 0; a < last; a++)
+            if (c.strides[k][a] == 1) mine = a;
+        if (!mine || (axis && *axis != *mine)) return std::nullopt;
+        axis = mine;
+        transposed[k] = true;
+        lds_bytes += TILE * pitch_of(operands[k].dtype) * dtype_bytes(operands[k].dtype);
+    }
+    if (!axis || lds_bytes > 48 * 1024 || c.shape[*axis] < 16 || c.shape[last] < 16) return std::nullopt;
+    const size_t A = *axis, dim_a = c.shape[A], dim_l = c.shape[last];
+    const size_t tiles_a = (dim_a + TILE - 1) / TILE, tiles_l = (dim_l + TILE - 1) / TILE;
+    std::vector<size_t> rest_dims;
+    std::vector<std::vector<int64_t>> rest_strides(n_ops);
+    size_t rest = 1;
+    for (size_t a = 0; a < last; a++) {
+        if (a == A) continue;
+        rest_dims.push_back(c.shape[a]);
+        rest *= c.shape[a];
+        for (size_t k = 0; k < n_ops; k++) rest_strides[k].push_back(c.strides[k][a]);
+    }
+    const size_t blocks = rest * tiles_a * tiles_l;
+    if (blocks > 0x7fffffffull) return std::nullopt;
+    const bool idx64 = !fits_i32(operands, total + TILE * TILE);
+
+    KernelSpec spec;
+    spec.name = "kn_scalar";
+    spec.n_ptrs = n_ops;
+    spec.block = 256;
+    std::ostringstream ss;
+    emit_header(ss, idx64, n_ops);
+    for (size_t k = 0; k < n_ops; k++) ss << "typedef " << storage_type(operands[k].dtype) << " S" << k << ";\n";
+    for (size_t o = 0; o < n_out; o++) {
+        ss << "KN_DEV " << compute_type(operands[o].dtype) << " kn_op" << o << "(";
+        for (size_t k = n_out; k < n_ops; k++) ss << (k > n_out ? ", " : "") << compute_type(operands[k].dtype) << " x" << k;
+        ss << ") {\n";
+        std::string res = emit_expr(ss, exprs[o], "y", [&](size_t operand) {
+            KN_ASSERT(operand >= n_out && operand < n_ops);
+            return "x" + std::to_string(operand);
+        });
+        ss << "    return " << res << ";\n}\n";
+    }
+    ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_scalar(KnPtrs ptrs) {\n";
+    for (size_t k = 0; k < n_ops; k++) {
+        ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
+        if (transposed[k]) ss << "    __shared__ S" << k << " tile" << k << "[" << TILE << "][" << pitch_of(operands[k].dtype) << "];\n";
+    }
+    // which tile: the output axis fastest, then the operands' axis, then everything else
+    ss << "    idx_t blk = (idx_t) blockIdx.x;\n";
+    ss << "    const idx_t l0 = (blk % (idx_t) " << tiles_l << ") * " << TILE << "; blk /= (idx_t) " << tiles_l << ";\n";
+    ss << "    const idx_t a0 = (blk % (idx_t) " << tiles_a << ") * " << TILE << "; blk /= (idx_t) " << tiles_a << ";\n";
+    for (size_t k = 0; k < n_ops; k++) ss << "    idx_t off" << k << " = 0;\n";
+    {
+        std::vector<std::string> offs;
+        for (size_t k = 0; k < n_ops; k++) offs.push_back("off" + std::to_string(k));
+        emit_decompose(ss, "    ", "blk", rest_dims, rest_strides, offs);
+    }
+    auto offset_of = [&](size_t k, const std::string &a, const std::string &l) {
+        std::string text = "off" + std::to_string(k);
+        if (c.strides[k][A] != 0) text += " + (a0 + " + a + ") * (idx_t) " + std::to_string(c.strides[k][A]);
+        if (c.strides[k][last] != 0) text += " + (l0 + " + l + ") * (idx_t) " + std::to_string(c.strides[k][last]);
+        return text;
+    };
+    ss << "    const int lane = threadIdx.x & 63, row = threadIdx.x >> 6;\n";
+    // phase 1: lanes along the transposed operands' contiguous axis
+    ss << "    if (a0 + lane < (idx_t) " << dim_a << ") {\n#pragma unroll\n        for (int i = 0; i < 16; i++) {\n";
+    ss << "            const int l = row + 4 * i;\n            if (l0 + l < (idx_t) " << dim_l << ") {\n";
+    for (size_t k = n_out; k < n_ops; k++)
+        if (transposed[k]) ss << "                tile" << k << "[l][lane] = p" << k << "[" << offset_of(k, "lane", "l") << "];\n";
+    ss << "            }\n        }\n    }\n    __syncthreads();\n";
+    // phase 2: lanes along the outputs' contiguous axis
+    ss << "    if (l0 + lane < (idx_t) " << dim_l << ") {\n#pragma unroll\n        for (int i = 0; i < 16; i++) {\n";
+    ss << "            const int a = row + 4 * i;\n            if (a0 + a < (idx_t) " << dim_a << ") {\n";
+    for (size_t k = n_out; k < n_ops; k++) {
+        ss << "                const S" << k << " r" << k << " = ";
+        if (transposed[k]) ss << "tile" << k << "[lane][a];\n";
+        else ss << "p" << k << "[" << offset_of(k, "a", "lane") << "];\n";
+    }
+    for (size_t o = 0; o < n_out; o++) {
+        std::string call = "kn_op" + std::to_string(o) + "(";
+        for (size_t k = n_out; k < n_ops; k++) call += (k > n_out ? ", " : "") + from_storage(operands[k].dtype, "r" + std::to_string(k));
+        call += ")";
+        ss << "                p" << o << "[" << offset_of(o, "a", "lane") << "] = " << to_storage(operands[o].dtype, call) << ";\n";
+    }
+    ss << "            }\n        }\n    }\n}\n";
+    spec.source = ss.str();
+    spec.grid = (uint32_t) blocks;
+    std::ostringstream note;
+    note << "rank=" << rank << " transposed tiles " << TILE << "x" << TILE << " idx=" << (idx64 ? 64 : 32);
+    if (n_out > 1) note << " outputs=" << n_out;
+    spec.strategy = note.str();
+    return spec;
+}
+
+}  // namespace
+
 KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, const std::vector<ScalarExpr> &exprs) {
     const size_t n_out = exprs.size();
     KN_ASSERT(n_out >= 1 && operands.size() >= n_out);
@@ -480,6 +604,8 @@ KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, 
     size_t rank = c.rank();
     size_t inner = c.shape[rank - 1];
     size_t vec = pick_vec(operands, c, inner);
+    if (vec == 1)
+        if (auto tiled = make_transposed_tile_kernel(operands, exprs, c, total)) return *tiled;
     size_t total_vecs = total / vec;
     size_t unroll = total_vecs >= 256 * 4 * 1024 ? 4 : (total_vecs >= 256 * 2 * 512 ? 2 : 1);
     bool idx64 = !fits_i32(operands, total + 256 * unroll);

@@ -1199,6 +1199,46 @@ def attention_fused_many_blocks():
     return g, b, inputs, None
 
 
+@case
+def transposed_copy_through_tiles():
+    """[3, 200, 330] read as its [0, 2, 1] permutation and stored densely (NCHW -> tokens): big enough for the kernel
+    that turns tiles of 64 x 64 through LDS; neither 200 nor 330 is a multiple of the tile"""
+    g = Graph()
+    rng = np.random.default_rng(140)
+    x = g.input([3, 200, 330])
+    # the view cannot be a stride edit, so the permuted tensor is copied
+    g.output(g.view(g.permute(x, [0, 2, 1]), [3 * 330, 200]))
+    return g, 0, [rng.standard_normal((3, 200, 330)).astype(np.float32)], None
+
+
+@case
+def transposed_operands_in_elementwise_chain():
+    """f16: two transposed operands, one straight operand, one broadcast row and a flipped axis in one chain"""
+    g = Graph()
+    rng = np.random.default_rng(141)
+    shapes = [(2, 300, 136), (2, 300, 136), (2, 136, 300), (1, 1, 300)]
+    a, b, c, d = [g.input(list(shape), DType.F16) for shape in shapes]
+    at, bt = g.permute(a, [0, 2, 1]), g.flip(g.permute(b, [0, 2, 1]), 2)
+    y = g.add(g.mul(at, c), g.mul(bt, g.broadcast(d, [2, 136, 300])))
+    g.output(y)
+    return g, 0, [rng.standard_normal(shape).astype(np.float16) for shape in shapes], None
+
+
+@case
+def transposed_operand_two_outputs_and_wide_types():
+    """one transposed f64 operand feeding two outputs (tiles of 8 byte elements), and a bool one (1 byte elements)"""
+    g = Graph()
+    rng = np.random.default_rng(142)
+    x = g.input([260, 300], DType.F64)
+    w = g.input([300, 260], DType.F64)
+    xt = g.permute(x, [1, 0])
+    g.output_all([g.add(xt, w), g.mul(xt, w)])
+    m = g.input([300, 260], DType.BOOL)
+    g.output(g.view(g.permute(m, [1, 0]), [260 * 300]))
+    inputs = [rng.standard_normal((260, 300)), rng.standard_normal((300, 260)), rng.random((300, 260)) < 0.5]
+    return g, 0, inputs, None
+
+
 def _attention_split_heads_case(seed, batch, heads, lq, lk, dk, dv, dtype=DType.F32, kv_split=None):
     """attention over (batch, heads) as a transformer block writes it: q, k, v are [batch * tokens, heads * width]
     projections, viewed as [batch, tokens, heads, width], permuted to [batch, heads, tokens, width] and flattened to
