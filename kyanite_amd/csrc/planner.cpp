@@ -524,8 +524,10 @@ private:
         row.kind = op.kind == OpKind::Softmax ? RowKernelDesc::Softmax : RowKernelDesc::Layernorm;
         // `a0 * x0 + a1 * x1` in front of the row operation (planner.rs:522-604 for layernorm; here for softmax as
         // well, which covers `scale * scores + mask`); the operands may be laid out differently (a broadcast mask)
+        // (a sum that something else uses as well is stored for that user anyway, bias or residual in the store of
+        // the matmul that feeds it where that applies: the row kernel then reads the one tensor)
         const Operation &iop = graph[input].operation;
-        if (iop.kind == OpKind::Binary && iop.binary == BinaryOp::Add && !map.count(input)) {
+        if (iop.kind == OpKind::Binary && iop.binary == BinaryOp::Add && !map.count(input) && can_fuse(input)) {
             auto l = visit_scalable_value(iop.inputs[0]);
             if (!l.ok) return R::missing(l.need);
             auto r = visit_scalable_value(iop.inputs[1]);
@@ -658,9 +660,6 @@ private:
         return R::done(*viewed);
     }
 
-    // matmul(softmax(matmul(q, kt) [* or / constant] [+ mask], last axis), v) in f32 (no mask) or f16, every
-    // intermediate value hidden and used once: the scores stay on the compute unit instead of passing through memory
-    // between three or more launches (planner.rs:606-648, :418-476 plan them separately).
     // An operand [b, rows, cols] of the fused attention as [b1, b2, rows, cols] with b1 * b2 = b. The batch of an
     // attention is usually (batch, heads) flattened, and the flattening of a permuted [batch, tokens, heads, width]
     // tensor is no stride edit: the kernel takes two batch strides instead of a dense copy of the operand.
@@ -683,6 +682,9 @@ private:
         return VT::done(*split);
     }
 
+    // matmul(softmax(matmul(q, kt) [* or / constant] [+ mask], last axis), v) in f32 (no mask) or f16, every
+    // intermediate value hidden and used once: the scores stay on the compute unit instead of passing through memory
+    // between three or more launches (planner.rs:606-648, :418-476 plan them separately).
     // `split_inner` > 0: the result is wanted as [b / split_inner, split_inner, lq, dv], laid out in memory as
     // [b / split_inner, lq, split_inner, dv] (what `permute [0, 2, 1, 3]` of it turns into a dense tensor)
     Visit<std::optional<PlanTensor>> try_visit_fused_attention(Value value, bool batch_first = true, size_t split_inner = 0) {
@@ -1213,6 +1215,12 @@ private:
             // give the conv fuser the first shot, so that this chain does not steal its relu, add or bias
             auto fused = try_visit_fused_conv(value);
             if (!fused.ok) return R::missing(fused.need);
+            // `matmul + bias` or `matmul + residual` that more than this chain uses: stored by the matmul itself and
+            // loaded here, instead of computed again in every chain that uses it
+            if (!fused.value && !is_root && options.fuse_matmul_epilogue && !can_fuse(value)) {
+                fused = try_visit_fused_matmul(value);
+                if (!fused.ok) return R::missing(fused.need);
+            }
             if (fused.value) {
                 if (!map.count(value)) insert_mapping(value, *fused.value);
                 node = block.load_operand(*fused.value);

@@ -101,6 +101,20 @@ def test_attention_over_batch_and_heads_needs_no_copies():
     assert HipExecutor(0, g, batch, plan_only=True).step_kinds() == ["mat_mul"]
 
 
+def test_sum_with_two_users_is_stored_by_the_matmul():
+    # y = x @ w + bias feeds a layernorm AND a residual sum: the matmul stores y (bias in its epilogue), the row kernel
+    # and the elementwise kernel load it; neither computes `x @ w + bias` again
+    g = Graph()
+    x, w, bias, z = g.input([256, 64]), g.input([64, 128]), g.input([1, 128]), g.input([256, 128])
+    y = g.add(g.mat_mul(x, w), g.broadcast(bias, [256, 128]))
+    g.output(g.add(g.layernorm(y, 1, 1e-5), g.add(y, z)))
+    ex = HipExecutor(0, g, 0, plan_only=True)
+    assert ex.step_kinds() == ["mat_mul", "layernorm_op"], [ex.step_str(i) for i in range(ex.step_count())]
+    assert "+add" in ex.step_str(0)
+    # the row kernel reads y (as the row and again in its epilogue, where the residual sum rides), z and writes the result
+    assert ex.step_str(1).count("f32[256, 128]") == 4
+
+
 def test_attention_chain_stays_apart_when_it_must():
     three = ["mat_mul", "softmax_op", "mat_mul"]
     # the probabilities are needed elsewhere
