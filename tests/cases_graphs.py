@@ -1239,6 +1239,19 @@ def transposed_operand_two_outputs_and_wide_types():
     return g, 0, inputs, None
 
 
+@case
+def matmul_sum_with_two_users():
+    """y = x @ w + bias feeds a layernorm and a residual sum (a transformer block's skip connection): y is stored by
+    the matmul, and both users load it"""
+    g = Graph()
+    rng = np.random.default_rng(143)
+    shapes = [(200, 96), (96, 136), (1, 136), (200, 136)]
+    x, w, bias, z = [g.input(list(shape)) for shape in shapes]
+    y = g.add(g.mat_mul(x, w), g.broadcast(bias, [200, 136]))
+    g.output_all([g.add(g.layernorm(y, 1, 1e-5), g.add(y, z)), g.mul(y, z)])
+    return g, 0, [rng.standard_normal(shape).astype(np.float32) for shape in shapes], None
+
+
 def _attention_split_heads_case(seed, batch, heads, lq, lk, dk, dv, dtype=DType.F32, kv_split=None):
     """attention over (batch, heads) as a transformer block writes it: q, k, v are [batch * tokens, heads * width]
     projections, viewed as [batch, tokens, heads, width], permuted to [batch, heads, tokens, width] and flattened to
