@@ -573,7 +573,9 @@ int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool 
         sched.tail_k_chunk = lp.tail_k_chunk;
         grid.x = (unsigned) (lp.head_tiles + (tiles - lp.head_tiles) * lp.tail_split);
     }
-    const int e = lp.small_tile ? launch_direct<float, 1, 1, 2, 2, 4>(grid, stream, p, sched) : launch_direct<float, 2, 2, 2, 2, 2>(grid, stream, p, sched);
+    // (64 x 64 tiles on three stages: 48 KB of LDS, so three workgroups share a compute unit; on four stages and two
+    // workgroups the 8192 x 320 x 320 projections of a transformer block took 26.7 us instead of 24.9 us)
+    const int e = lp.small_tile ? launch_direct<float, 1, 1, 2, 2, 3>(grid, stream, p, sched) : launch_direct<float, 2, 2, 2, 2, 2>(grid, stream, p, sched);
     if (e != 0) return e;
     *launched = true;
     return (int) hipGetLastError();
