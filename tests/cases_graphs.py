@@ -1295,6 +1295,12 @@ def attention_split_heads_mixed_operands():
 
 
 @case
+def attention_split_heads_unsupported_width():
+    """width 24 is none the fused kernel is built for: the same graph runs as copies, matmul, softmax, matmul"""
+    return _attention_split_heads_case(108, 2, 3, 50, 60, 24, 24)
+
+
+@case
 def attention_f16_split_heads_no_copies():
     """f16, 2 x 4 heads of width 64 in [batch, tokens, heads, width] order"""
     return _attention_split_heads_case(107, 2, 4, 100, 100, 64, 64, DType.F16)
