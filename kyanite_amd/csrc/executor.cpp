@@ -103,6 +103,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             step.gemm.c = l.ptrs[2];
             size_t next = 3;
             step.gemm.addend = step.gemm_has_addend ? l.ptrs[next++] : nullptr;
+            step.gemm.addend2 = step.gemm_has_addend2 ? l.ptrs[next++] : nullptr;
             const GemmLaunchPlan lp = plan_gemm_launch(step.gemm, step.gemm_f16);
             KN_ASSERT(l.ptrs.size() == next + (lp.workspace_bytes > 0) + (lp.counter_bytes > 0));
             step.gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;

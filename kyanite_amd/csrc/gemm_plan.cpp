@@ -28,6 +28,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         q.b_sb = p.a_sb; q.b_sk = p.a_sk; q.b_sn = p.a_sm;
         q.c_sm = p.c_sn; q.c_sn = p.c_sm;
         q.d_sm = p.d_sn; q.d_sn = p.d_sm;
+        q.d2_sm = p.d2_sn; q.d2_sn = p.d2_sm;
         p = q;
     }
     lp.p = p;

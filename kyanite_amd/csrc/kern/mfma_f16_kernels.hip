@@ -142,28 +142,43 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
     const bool split = gridDim.z > 1;
     // the epilogue of a split launch is applied by the pass that sums the partial products
     const T *addend = p.addend ? (const T *) p.addend + bz * p.d_sb : nullptr;
+    const T *addend2 = p.addend2 ? (const T *) p.addend2 + bz * p.d2_sb : nullptr;
     // Tiles that lie inside the matrix, with offsets that fit 32 bits, skip the bounds checks and the 64 bit
     // address arithmetic (which otherwise cost about a tenth of a 512 x 12288 x 4096 launch).
     const long long reach = (long long) (p.m - 1) * p.c_sm + p.n, d_reach = (long long) (p.m - 1) * p.d_sm + (long long) (p.n - 1) * p.d_sn;
+    const long long d2_reach = (long long) (p.m - 1) * p.d2_sm + (long long) (p.n - 1) * p.d2_sn;
     const bool fast = !split && p.c_sn == 1 && p.c_sm > 0 && reach < 0x7fffffffll && row0 + 32 * MI <= p.m && col0 + 32 * NI <= p.n &&
-                      (!addend || (p.d_sm >= 0 && p.d_sn >= 0 && d_reach < 0x7fffffffll));
+                      (!addend || (p.d_sm >= 0 && p.d_sn >= 0 && d_reach < 0x7fffffffll)) &&
+                      (!addend2 || (p.d2_sm >= 0 && p.d2_sn >= 0 && d2_reach < 0x7fffffffll));
     if (fast) {
-        const int c_sm = (int) p.c_sm, d_sm = (int) p.d_sm, d_sn = (int) p.d_sn;
+        const int c_sm = (int) p.c_sm, d_sm = (int) p.d_sm, d_sn = (int) p.d_sn, d2_sm = (int) p.d2_sm, d2_sn = (int) p.d2_sn;
         T *tile = out + (row0 + 4 * half) * c_sm + col0 + c;
         const T *d_tile = addend ? addend + (row0 + 4 * half) * d_sm + (col0 + c) * d_sn : nullptr;
+        const T *d2_tile = addend2 ? addend2 + (row0 + 4 * half) * d2_sm + (col0 + c) * d2_sn : nullptr;
         const bool relu = p.relu != 0;
 #pragma unroll
         for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int j = 0; j < NI; j++)
+            for (int j = 0; j < NI; j++) {
+                // every addend of the MFMA tile is requested before its first store: the compiler cannot move a
+                // load over a store that might alias it, and one round trip per element is the tail of the workgroup
+                T d[16], d2[16];
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = 32 * i + 8 * (v >> 2) + (v & 3);
+                    d[v] = d_tile ? d_tile[r * d_sm + 32 * j * d_sn] : (T) 0;
+                    d2[v] = d2_tile ? d2_tile[r * d2_sm + 32 * j * d2_sn] : (T) 0;
+                }
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int r = 32 * i + 8 * (v >> 2) + (v & 3);
                     T x = (T) acc[i][j][v];
-                    if (d_tile) x = (T) ((float) x + (float) d_tile[r * d_sm + 32 * j * d_sn]);
+                    if (d_tile) x = (T) ((float) x + (float) d[v]);
+                    if (d2_tile) x = (T) ((float) x + (float) d2[v]);
                     if (relu) x = x > (T) 0 ? x : (T) 0;
                     tile[r * c_sm + 32 * j] = x;
                 }
+            }
         return;
     }
 #pragma unroll
@@ -180,6 +195,7 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
                     } else {
                         T r = (T) acc[i][j][v];
                         if (addend) r = (T) ((float) r + (float) addend[(long long) row * p.d_sm + (long long) col * p.d_sn]);
+                        if (addend2) r = (T) ((float) r + (float) addend2[(long long) row * p.d2_sm + (long long) col * p.d2_sn]);
                         if (p.relu) r = r > (T) 0 ? r : (T) 0;
                         out[(long long) row * p.c_sm + (long long) col * p.c_sn] = r;
                     }
@@ -587,6 +603,7 @@ int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
     const GemmParams &p = lp.p;
     const int groups = p.groups > 1 ? p.groups : 1;
     if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
+    if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;
     if (p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);

@@ -187,6 +187,8 @@ struct GemmStore {
     int M, N;
     const float *addend;  // optional epilogue operand (null = none), with its own strides
     long long dm, dn;
+    const float *addend2;  // a second one, added after the first
+    long long d2m, d2n;
     int relu;
     // what `prepare` derives for the two columns this lane owns
     const float *d_col[2];  // addend at (row 0, column), or null
@@ -205,6 +207,7 @@ struct GemmStore {
     __device__ __forceinline__ void store(int m, int n, int j, float v) const {
         if (m < M && n < N) {
             if (addend) v += row_invariant ? d_bias[j] : d_col[j][(long long) m * dm];
+            if (addend2) v += addend2[(long long) m * d2m + (long long) n * d2n];
             if (relu) v = fmaxf(v, 0.0f);
             p[(long long) m * sm + (long long) n * sn] = v;
         }
@@ -335,9 +338,10 @@ __global__ __launch_bounds__(THREADS) void gemm_f32_kernel(GemmParams p, int k_c
     // the epilogue of a split launch is applied by the pass that sums the partial products
     GemmStore s = gridDim.z > 1
         ? GemmStore{(float *) p.workspace + ((long long) bz * gridDim.z + blockIdx.z) * p.m * p.n, p.n, 1, p.m, p.n,
-                    nullptr, 0, 0, 0, {nullptr, nullptr}, {0.0f, 0.0f}, false}
+                    nullptr, 0, 0, nullptr, 0, 0, 0, {nullptr, nullptr}, {0.0f, 0.0f}, false}
         : GemmStore{(float *) c_base + bz * p.c_sb, p.c_sm, p.c_sn, p.m, p.n,
-                    p.addend ? (const float *) p.addend + bz * p.d_sb : nullptr, p.d_sm, p.d_sn, p.relu,
+                    p.addend ? (const float *) p.addend + bz * p.d_sb : nullptr, p.d_sm, p.d_sn,
+                    p.addend2 ? (const float *) p.addend2 + bz * p.d2_sb : nullptr, p.d2_sm, p.d2_sn, p.relu,
                     {nullptr, nullptr}, {0.0f, 0.0f}, false};
     mfma_tile_loop<TI, TI>(la, lb, s, k_begin, k_end, m0, n0);
 }
@@ -651,11 +655,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p,
     const long long row = e / p.n, col = e - row * p.n;
     OutT *out = (OutT *) p.c + bz * p.c_sb + row * p.c_sm + col * p.c_sn;
     const OutT *addend = p.addend ? (const OutT *) p.addend + bz * p.d_sb + row * p.d_sm + col * p.d_sn : nullptr;
+    const OutT *addend2 = p.addend2 ? (const OutT *) p.addend2 + bz * p.d2_sb + row * p.d2_sm + col * p.d2_sn : nullptr;
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
         // rounding to the output type after the product and after the sum, like separate operations would
         float v = (float) (OutT) total[j];
         if (addend) v = (float) (OutT) (v + (float) addend[j * p.d_sn]);
+        if (addend2) v = (float) (OutT) (v + (float) addend2[j * p.d2_sn]);
         if (p.relu) v = fmaxf(v, 0.0f);
         out[j * p.c_sn] = (OutT) v;
     }
@@ -704,6 +710,7 @@ int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
     const int t = lp.small_tile ? 64 : 128;
     const int groups = p.groups > 1 ? p.groups : 1;
     if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
+    if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;
     const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * groups;
     if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;

@@ -26,6 +26,10 @@ struct GemmParams {
     // operations would
     const void *addend = nullptr;
     long long d_sb = 0, d_sm = 0, d_sn = 0;
+    // a second operand of the same kind, added after the first (bias, then residual): C = act((A * B + D) + D2),
+    // for f16 with a rounding after either sum; only together with `addend`
+    const void *addend2 = nullptr;
+    long long d2_sb = 0, d2_sm = 0, d2_sn = 0;
     int relu = 0;
     // Grouped launch: `groups` (up to GEMM_MAX_GROUPS) products A * B_g = C_g that share A, all shapes and all
     // strides, in one launch; b / c are then ignored in favour of b_group / c_group. Not combined with an addend

@@ -19,7 +19,7 @@ std::string Step::str() const {
         ss << " attention " << (gemm_f16 ? "f16" : "f32") << (attention_has_mask ? " +mask" : "") << " b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
     else if (kind == StepKind::MatMul) {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
-           << (gemm_has_addend ? " +add" : "") << (gemm.relu ? " relu" : "");
+           << (gemm_has_addend ? " +add" : "") << (gemm_has_addend2 ? " +add" : "") << (gemm.relu ? " relu" : "");
         if (gemm.groups > 1) ss << " x" << gemm.groups << " grouped";
     }
     else if (kind == StepKind::Conv)
@@ -44,7 +44,7 @@ double Step::bytes() const {
     double total = 0.0;
     for (size_t i = 0; i < operands.size(); i++) {
         // split-K scratch is not algorithmic traffic
-        if (kind == StepKind::MatMul && !attention && i >= (gemm.groups > 1 ? 1u + 2u * (unsigned) gemm.groups : (gemm_has_addend ? 4u : 3u))) break;
+        if (kind == StepKind::MatMul && !attention && i >= (gemm.groups > 1 ? 1u + 2u * (unsigned) gemm.groups : 3u + (gemm_has_addend ? 1u : 0u) + (gemm_has_addend2 ? 1u : 0u))) break;
         auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
@@ -624,15 +624,33 @@ private:
             if (graph[v].operation.kind != OpKind::MatMul) return std::nullopt;
             return v;
         };
-        std::optional<Value> addend;
+        // `(matmul + d) + d2` (a bias, then the skip connection of a transformer block): the sum next to the matmul
+        // and its shape, then optionally the sum above it, each hidden and used once except for `curr` itself
+        std::optional<Value> addend, addend2;
         std::optional<Value> mm;
         {
+            auto sum_over_matmul = [&](Value sum, std::optional<Value> &other) -> std::optional<Value> {
+                const Operation &op = graph[sum].operation;
+                if (op.kind != OpKind::Binary || op.binary != BinaryOp::Add) return std::nullopt;
+                const Value l = op.inputs[0], r = op.inputs[1];
+                std::optional<Value> found;
+                if (can_fuse(l)) found = matmul_under(l);
+                if (found) other = r;
+                else if (can_fuse(r) && (found = matmul_under(r))) other = l;
+                return found;
+            };
             const Operation &op = graph[curr].operation;
             if (op.kind == OpKind::Binary && op.binary == BinaryOp::Add) {
-                Value l = op.inputs[0], r = op.inputs[1];
-                if (can_fuse(l)) mm = matmul_under(l);
-                if (mm) addend = r;
-                else if (can_fuse(r) && (mm = matmul_under(r))) addend = l;
+                mm = sum_over_matmul(curr, addend);
+                if (!mm) {
+                    // one more sum in between, of the same shape (views between the two sums are not followed)
+                    for (int side = 0; side < 2 && !mm; side++) {
+                        const Value inner = op.inputs[side], outer = op.inputs[1 - side];
+                        if (!can_fuse(inner) || map.count(inner) || graph[inner].shape != graph[curr].shape) continue;
+                        mm = sum_over_matmul(inner, addend);
+                        if (mm) addend2 = outer;
+                    }
+                }
             } else if (relu) {
                 mm = matmul_under(curr);
             }
@@ -642,18 +660,21 @@ private:
 
         const ConcreteShape final_shape = graph[value].shape.eval(batch_size);
         const ConcreteShape mm_shape = graph[*mm].shape.eval(batch_size);
-        std::optional<PlanTensor> addend_t;
-        if (addend) {
-            auto at = visit(*addend);
+        std::optional<PlanTensor> addend_t, addend2_t;
+        for (int which = 0; which < 2; which++) {
+            const std::optional<Value> &from = which == 0 ? addend : addend2;
+            if (!from) continue;
+            auto at = visit(*from);
             if (!at.ok) return R::missing(at.need);
             // the operand in the matmul's own [b, m, n] shape; an operand whose layout cannot follow the views
             // between the matmul and the sum is not fused
             KN_ASSERT(at.value.shape.shape() == final_shape);
-            addend_t = at.value.view(mm_shape);
-            if (!addend_t) return R::done(std::nullopt);
+            auto viewed = at.value.view(mm_shape);
+            if (!viewed) return R::done(std::nullopt);
+            (which == 0 ? addend_t : addend2_t) = viewed;
         }
         const Operation &mop = graph[*mm].operation;
-        auto result = visit_matmul(value, mop.inputs[0], mop.inputs[1], true, addend_t, relu);
+        auto result = visit_matmul(value, mop.inputs[0], mop.inputs[1], true, addend_t, relu, addend2_t);
         if (!result.ok) return R::missing(result.need);
         auto viewed = result.value.view(final_shape);
         KN_ASSERT(viewed.has_value(), "a dense matmul result can always be viewed");
@@ -1048,7 +1069,8 @@ private:
     }
 
     VT visit_matmul(Value value, Value left_v, Value right_v, bool batch_first,
-                    const std::optional<PlanTensor> &addend = std::nullopt, bool relu = false) {
+                    const std::optional<PlanTensor> &addend = std::nullopt, bool relu = false,
+                    const std::optional<PlanTensor> &addend2 = std::nullopt) {
         const DType dt = graph[value].dtype;
         if (dt != DType::F32 && dt != DType::F16) fail("GPU matmul only supports f32 and f16, got ", dtype_name(dt));
         KN_TRY(left, visit(left_v));
@@ -1074,6 +1096,12 @@ private:
                 g.d_sb = addend->shape.strides()[0]; g.d_sm = addend->shape.strides()[1]; g.d_sn = addend->shape.strides()[2];
                 step.gemm_has_addend = true;
                 step.operands.push_back({*addend, OperandKind::In});
+            }
+            if (addend2) {
+                KN_ASSERT(addend.has_value() && addend2->dtype == dt && addend2->shape.shape() == ConcreteShape({b, m, n}));
+                g.d2_sb = addend2->shape.strides()[0]; g.d2_sm = addend2->shape.strides()[1]; g.d2_sn = addend2->shape.strides()[2];
+                step.gemm_has_addend2 = true;
+                step.operands.push_back({*addend2, OperandKind::In});
             }
             g.relu = relu ? 1 : 0;
             push_gemm_scratch(step);

@@ -37,6 +37,7 @@ struct Step {
     GemmParams gemm{};
     bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
     bool gemm_has_addend = false;  // operand 3 is the tensor added in the epilogue
+    bool gemm_has_addend2 = false;  // operand 4 is a second one, added after the first
     // a MatMul step that is a whole softmax(scale * Q K^T [+ mask]) V chain in one launch; operands Q, K, V, [mask,] O
     bool attention = false;
     bool attention_has_mask = false;  // operand 3 is the additive mask, the result comes last

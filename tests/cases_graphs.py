@@ -1252,6 +1252,62 @@ def matmul_sum_with_two_users():
     return g, 0, [rng.standard_normal(shape).astype(np.float32) for shape in shapes], None
 
 
+def _two_addend_case(seed, m, n, k, dtype=DType.F32, relu=False, residual_first=False, permuted=False):
+    """`(x @ w + bias) + residual` (the output projection of a transformer block with its skip connection), which the
+    matmul stores in one go; `residual_first`: the skip connection on the left of the outer sum; `permuted`: the
+    result is handed out transposed"""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    np_dtype = np.float16 if dtype == DType.F16 else np.float32
+    shapes = [(m, k), (n, k), (1, n), (m, n)]
+    x, w, bias, res = [g.input(list(shape), dtype) for shape in shapes]
+    y = g.add(g.linear(x, w), g.broadcast(bias, [m, n]))
+    y = g.add(res, y) if residual_first else g.add(y, res)
+    if relu:
+        y = g.relu(y)
+    if permuted:
+        y = g.permute(y, [1, 0])
+    g.output(y)
+    scale = [1.0, 1.0 / np.sqrt(k), 1.0, 1.0]
+    return g, 0, [(rng.standard_normal(shape) * sc).astype(np_dtype) for shape, sc in zip(shapes, scale)], None
+
+
+@case
+def matmul_bias_and_residual_f32():
+    """f32 on the direct kernel (K a multiple of 32), ragged tiles"""
+    return _two_addend_case(150, 200, 136, 96)
+
+
+@case
+def matmul_bias_and_residual_f32_staged_relu():
+    """K = 100 is no multiple of 32: the kernel that stages through registers; relu on top, residual on the left"""
+    return _two_addend_case(151, 130, 72, 100, relu=True, residual_first=True)
+
+
+@case
+def matmul_bias_and_residual_split_k():
+    """few tiles and a long K: the partial products are summed by a pass of its own, which adds both operands"""
+    return _two_addend_case(152, 40, 64, 4096)
+
+
+@case
+def matmul_bias_and_residual_f16():
+    """f16: a rounding after the product and after either sum, like the three separate operations"""
+    return _two_addend_case(153, 300, 264, 320, DType.F16)
+
+
+@case
+def matmul_bias_and_residual_f16_permuted():
+    """f16 with relu on top, the result handed out transposed"""
+    return _two_addend_case(154, 257, 130, 128, DType.F16, relu=True, permuted=True)
+
+
+@case
+def matmul_bias_and_residual_f16_split_k():
+    """f16 with K split over workgroups (summing pass)"""
+    return _two_addend_case(155, 64, 128, 8192, DType.F16, residual_first=True)
+
+
 def _attention_split_heads_case(seed, batch, heads, lq, lk, dk, dv, dtype=DType.F32, kv_split=None):
     """attention over (batch, heads) as a transformer block writes it: q, k, v are [batch * tokens, heads * width]
     projections, viewed as [batch, tokens, heads, width], permuted to [batch, heads, tokens, width] and flattened to

@@ -115,6 +115,17 @@ def test_sum_with_two_users_is_stored_by_the_matmul():
     assert ex.step_str(1).count("f32[256, 128]") == 4
 
 
+def test_bias_and_residual_ride_in_the_matmul_store():
+    from cases_graphs import CASES
+    for name in ("matmul_bias_and_residual_f32", "matmul_bias_and_residual_f32_staged_relu", "matmul_bias_and_residual_split_k",
+                 "matmul_bias_and_residual_f16", "matmul_bias_and_residual_f16_permuted", "matmul_bias_and_residual_f16_split_k"):
+        g, batch, _, _ = CASES[name]()
+        ex = HipExecutor(0, g, batch, plan_only=True)
+        # (the transposed graph output is a dense copy after the matmul)
+        assert ex.step_kinds() == (["mat_mul", "scalar_op"] if name.endswith("permuted") else ["mat_mul"]), (name, ex.step_kinds())
+        assert "+add +add" in ex.step_str(0), ex.step_str(0)
+
+
 def test_attention_chain_stays_apart_when_it_must():
     three = ["mat_mul", "softmax_op", "mat_mul"]
     # the probabilities are needed elsewhere
