@@ -552,13 +552,28 @@ std::optional<KernelSpec> make_transposed_tile_kernel(const std::vector<KernelOp
     for (size_t k = n_out; k < n_ops; k++)
         if (transposed[k]) ss << "                tile" << k << "[l][lane] = p" << k << "[" << offset_of(k, "lane", "l") << "];\n";
     ss << "            }\n        }\n    }\n    __syncthreads();\n";
-    // phase 2: lanes along the outputs' contiguous axis
-    ss << "    if (l0 + lane < (idx_t) " << dim_l << ") {\n#pragma unroll\n        for (int i = 0; i < 16; i++) {\n";
+    // phase 2: lanes along the outputs' contiguous axis. The operands that are read straight from global memory
+    // are all requested before the first store (a load may not pass a store that might alias it).
+    ss << "    if (l0 + lane < (idx_t) " << dim_l << ") {\n";
+    bool any_straight = false;
+    for (size_t k = n_out; k < n_ops; k++) {
+        if (transposed[k]) continue;
+        any_straight = true;
+        ss << "        S" << k << " g" << k << "[16];\n";
+    }
+    if (any_straight) {
+        ss << "#pragma unroll\n        for (int i = 0; i < 16; i++) {\n            const int a = row + 4 * i;\n";
+        ss << "            if (a0 + a < (idx_t) " << dim_a << ") {\n";
+        for (size_t k = n_out; k < n_ops; k++)
+            if (!transposed[k]) ss << "                g" << k << "[i] = p" << k << "[" << offset_of(k, "a", "lane") << "];\n";
+        ss << "            }\n        }\n";
+    }
+    ss << "#pragma unroll\n        for (int i = 0; i < 16; i++) {\n";
     ss << "            const int a = row + 4 * i;\n            if (a0 + a < (idx_t) " << dim_a << ") {\n";
     for (size_t k = n_out; k < n_ops; k++) {
         ss << "                const S" << k << " r" << k << " = ";
         if (transposed[k]) ss << "tile" << k << "[lane][a];\n";
-        else ss << "p" << k << "[" << offset_of(k, "a", "lane") << "];\n";
+        else ss << "g" << k << "[i];\n";
     }
     for (size_t o = 0; o < n_out; o++) {
         std::string call = "kn_op" + std::to_string(o) + "(";
