@@ -656,12 +656,19 @@ __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p,
     OutT *out = (OutT *) p.c + bz * p.c_sb + row * p.c_sm + col * p.c_sn;
     const OutT *addend = p.addend ? (const OutT *) p.addend + bz * p.d_sb + row * p.d_sm + col * p.d_sn : nullptr;
     const OutT *addend2 = p.addend2 ? (const OutT *) p.addend2 + bz * p.d2_sb + row * p.d2_sm + col * p.d2_sn : nullptr;
+    // (the addends are requested before the first store: a load may not pass a store that might alias it)
+    OutT d[VEC], d2[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        d[j] = addend ? addend[j * p.d_sn] : (OutT) 0;
+        d2[j] = addend2 ? addend2[j * p.d2_sn] : (OutT) 0;
+    }
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
         // rounding to the output type after the product and after the sum, like separate operations would
         float v = (float) (OutT) total[j];
-        if (addend) v = (float) (OutT) (v + (float) addend[j * p.d_sn]);
-        if (addend2) v = (float) (OutT) (v + (float) addend2[j * p.d2_sn]);
+        if (addend) v = (float) (OutT) (v + (float) d[j]);
+        if (addend2) v = (float) (OutT) (v + (float) d2[j]);
         if (p.relu) v = fmaxf(v, 0.0f);
         out[j * p.c_sn] = (OutT) v;
     }
