@@ -1303,6 +1303,12 @@ def matmul_bias_and_residual_f16_permuted():
 
 
 @case
+def matmul_bias_and_residual_f16_staged():
+    """f16 with K = 200, no multiple of 64: the kernel that stages through registers"""
+    return _two_addend_case(156, 130, 72, 200, DType.F16, relu=True)
+
+
+@case
 def matmul_bias_and_residual_f16_split_k():
     """f16 with K split over workgroups (summing pass)"""
     return _two_addend_case(155, 64, 128, 8192, DType.F16, residual_first=True)
