@@ -135,7 +135,7 @@ typedef struct {
     int cast_dtype;   /* for casts, else -1 */
     size_t rank;
     size_t operand_count;
-    size_t axis_count; /* permutation / axis / axes */
+    size_t axis_count; /* permutation / axis / axes; for a conv: stride_y, stride_x, padding_y, padding_x */
     size_t non_output_uses;
     size_t slice_start, slice_end, slice_step;
     float eps;

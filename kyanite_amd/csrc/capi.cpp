@@ -388,7 +388,7 @@ int knhip_graph_value_info(const knhip_graph *g, knhip_value value, knhip_value_
         info->cast_dtype = is_cast ? (int) op.cast_to : -1;
         info->rank = vi.shape.rank();
         info->operand_count = op.inputs.size();
-        info->axis_count = op.axes.size();
+        info->axis_count = op.kind == OpKind::Conv ? 4 : op.axes.size();
         info->non_output_uses = vi.non_output_uses;
         info->slice_start = op.range.start;
         info->slice_end = op.range.end;
@@ -419,7 +419,12 @@ int knhip_graph_value_operands(const knhip_graph *g, knhip_value value, knhip_va
 int knhip_graph_value_axes(const knhip_graph *g, knhip_value value, size_t *buf, size_t cap) {
     return guarded([&] {
         KN_REQUIRE(g != nullptr);
-        return copy_list(g->graph[value].operation.axes, buf, cap, (size_t *) nullptr);
+        const Operation &op = g->graph[value].operation;
+        if (op.kind == OpKind::Conv) {
+            std::vector<size_t> geometry = {op.conv.stride_y, op.conv.stride_x, op.conv.padding_y, op.conv.padding_x};
+            return copy_list(geometry, buf, cap, (size_t *) nullptr);
+        }
+        return copy_list(op.axes, buf, cap, (size_t *) nullptr);
     });
 }
 int knhip_graph_value_constant(const knhip_graph *g, knhip_value value, const void **data, size_t *bytes) {

@@ -1,6 +1,7 @@
 // Launch decisions for the MFMA matrix multiply kernels: operand orientation, tile size, slice depth and the split
 // of the K axis. Kept apart from the kernels so that the planner can reserve the split-K workspace in the arena.
 #include <cstdlib>
+#include <sstream>
 
 #include "mfma_kernels.h"
 
@@ -163,6 +164,23 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         }
     }
     return lp;
+}
+
+std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16) {
+    std::ostringstream ss;
+    int tm = lp.small_tile ? 64 : 128, tn = tm;
+    if (lp.tall_tile) tm = 256;
+    if (lp.narrow_tile) tn = 64;
+    if (lp.direct && f16) {
+        if (lp.wide_tile) tn = 256;
+        if (lp.mid_tile) tn = 192;
+    } else if (lp.narrow_tile) {
+        tm = tn = 64;
+    }
+    ss << (lp.direct ? "direct " : "staged ") << tm << "x" << tn << " bk" << lp.bk;
+    if (lp.split_k > 1) ss << " split_k=" << lp.split_k << "x" << lp.k_chunk;
+    if (lp.tail_split > 1) ss << " head=" << lp.head_tiles << " tail_split=" << lp.tail_split << "x" << lp.tail_k_chunk;
+    return ss.str();
 }
 
 bool gemm_group_ok(const GemmParams &p, bool f16) {

@@ -4,6 +4,7 @@
 #pragma once
 
 #include <cstdint>
+#include <string>
 
 struct ihipStream_t;
 
@@ -65,6 +66,8 @@ struct GemmLaunchPlan {
     size_t counter_bytes;    // one int per shared tile
 };
 GemmLaunchPlan plan_gemm_launch(const GemmParams &p, bool f16);
+// "direct 256x128 bk64 head=256 tail_split=2x2048": kernel family, workgroup tile, slice depth and the splits
+std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16);
 // whether `p.groups` products may share one launch: no operand swap, no K split, no epilogue
 bool gemm_group_ok(const GemmParams &p, bool f16);
 

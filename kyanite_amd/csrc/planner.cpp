@@ -21,6 +21,7 @@ std::string Step::str() const {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm_has_addend2 ? " +add" : "") << (gemm.relu ? " relu" : "");
         if (gemm.groups > 1) ss << " x" << gemm.groups << " grouped";
+        ss << " [" << describe_gemm_plan(plan_gemm_launch(gemm, gemm_f16), gemm_f16) << "]";
     }
     else if (kind == StepKind::Conv)
         ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="

@@ -988,6 +988,56 @@ def config_llama_f32_small():
 
 
 @case
+def config_bandwidth_fused_chain_small():
+    """configs[1] (a) through its own builder: the last axis has the benchmark's length (1024), so the same
+    vectorised kernel variant with the broadcast a, b is generated"""
+    from kyanite_amd.configs import build_fused_chain
+    g, inputs, _ = build_fused_chain(seed=11, shape=(4, 128, 1024))
+    return g, 0, inputs(), None
+
+
+@case
+def config_bandwidth_softmax_small():
+    """configs[1] (b): rows of 512 like the benchmark's"""
+    from kyanite_amd.configs import build_softmax
+    g, inputs, _ = build_softmax(seed=12, shape=(2, 4, 64, 512))
+    return g, 0, inputs(), None
+
+
+@case
+def config_bandwidth_layernorm_small():
+    """configs[1] (c): rows of 4096 with the fused gamma / beta epilogue"""
+    from kyanite_amd.configs import build_layernorm
+    g, inputs, _ = build_layernorm(seed=13, shape=(64, 4096))
+    return g, 0, inputs(), None
+
+
+@case
+def config_bandwidth_reduce_small():
+    """configs[1] (d): sums over 8192 elements"""
+    from kyanite_amd.configs import build_reduce
+    g, inputs, _ = build_reduce(seed=14, shape=(64, 8192))
+    return g, 0, inputs(), None
+
+
+@case
+def config_resnet_small():
+    """configs[2] through its own builder: 128 channels like the benchmark (the same conv tiles), two blocks,
+    batch 6"""
+    from kyanite_amd.configs import build_resnet_tower
+    g, make_inputs, _ = build_resnet_tower(seed=15, channels=128, blocks=2)
+    return g, 6, make_inputs(6), None
+
+
+@case
+def config_tiny_mlp():
+    """configs[0] as the benchmark and the smoke check build it"""
+    from kyanite_amd.configs import build_tiny_mlp
+    g, inputs = build_tiny_mlp(seed=16, batch=8)
+    return g, 8, inputs, None
+
+
+@case
 def config_unet_block_small():
     from kyanite_amd.configs import build_unet_block
     g, make_inputs, _ = build_unet_block(seed=2, batch=2, channels=64, size=8, groups=4, heads=2, time_dim=48, ctx_len=5,

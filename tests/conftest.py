@@ -19,3 +19,20 @@ def hip_device():
 
     assert HipDevice.count() >= 1, "no HIP device visible: GPU tests need the MI355X"
     return HipDevice(0)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """Write the measured parity errors of every GPU comparison of the session next to the other run outputs, so
+    that a regression of a case shows as a number and not only as a pass that became a failure."""
+    try:
+        from runner import PARITY_RECORDS
+    except Exception:
+        return
+    if not PARITY_RECORDS:
+        return
+    import json
+
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "parity_report.json"), "w") as f:
+        json.dump(PARITY_RECORDS, f, indent=0)

@@ -13,19 +13,14 @@ from oracle import cpu_eval_graph
 TOLERANCE_ABS_DIFF = 0.001
 TOLERANCE_REL_DIFF = 0.001
 
-# The tighter bar this project states for its own GPU path against the oracle:
-#   max over elements of |actual - expected| / max(|expected|, FLOOR_FRACTION * rms(expected)) <= F32_MAX_REL.
-# The floor is needed because sums that cancel to (almost) zero carry the rounding of their large terms. Two f32
-# evaluations of one K-term contraction that differ only in summation order differ by about
-# sqrt(2) * (eps / 2) * sqrt(K) * rms per element (one sigma), and the largest of millions of elements sits near
-# five sigma: 7e-6 * rms for K = 1152 and 1.1e-5 * rms for K = 2880 (both measured on the ResNet and UNet
-# configurations at full size, where they match this estimate), 2.2e-5 * rms for K = 11008. A floor of half the
-# tensor's rms keeps that noise a factor of two under the 1e-4 bar for the longest contraction of any configuration;
-# a real defect (wrong index, dropped term) shows up as an error of the order of the rms itself.
-F32_MAX_REL = 1e-4
-FLOOR_FRACTION = 0.5
-# f16 tensors (f16 storage, f32 arithmetic, one rounding per operation; not part of the reference IR): 2e-2
-F16_MAX_REL = 2e-2
+# The tighter bars this project states for its own GPU path against the oracle live in oracle/parity.py:
+# bit-exact for data movement and IEEE-fixed arithmetic, 1e-4 (f32) / 2e-2 (f16) with a floor of 1e-3 rms for
+# everything else, and for sums of K terms an f64-referenced rule that asks the GPU result to be no further
+# from the exact value than the oracle is.
+from oracle.parity import F16_MAX_REL, F32_MAX_REL, SMALL_FLOOR, check_outputs, rel_error
+
+# one dict per compared output of every GPU check of the session (conftest.py writes them out at the end)
+PARITY_RECORDS = []
 
 
 def assert_tensors_match(expected, actual, what=""):
@@ -57,29 +52,19 @@ def assert_tensors_match(expected, actual, what=""):
                 raise AssertionError(f"{what}: output {i} mismatch in {bad.sum()}/{bad.size} values:\n" + "\n".join(lines))
 
 
-def max_rel_error(expected, actual):
-    """max |a - e| / max(|e|, floor) with floor = FLOOR_FRACTION * rms(e); infinities and NaN must agree exactly."""
-    e = np.asarray(expected, dtype=np.float64)
-    a = np.asarray(actual, dtype=np.float64)
-    special = ~np.isfinite(e)
-    if special.any():
-        assert np.array_equal(e[special], a[special], equal_nan=True), "non-finite values differ"
-    e, a = e[~special], a[~special]
-    if e.size == 0:
-        return 0.0
-    assert np.isfinite(a).all(), "actual holds non-finite values where expected is finite"
-    floor = FLOOR_FRACTION * np.sqrt(np.mean(e * e))
-    denom = np.maximum(np.abs(e), max(floor, 1e-30))
-    return float(np.max(np.abs(a - e) / denom))
+# Golden vectors were written by another f32 implementation (the exporter's runtime), so both sides of a comparison
+# with them carry rounding noise of their own; the reference accepts abs 1e-3 and rel 1e-3 for them.
+GOLDEN_FLOOR = 0.1
 
 
-def assert_close(expected, actual, what="", max_rel=F32_MAX_REL):
-    """Project bar: bit-exact for ints / bools, `max_rel` for floats."""
+def assert_close(expected, actual, what="", max_rel=F32_MAX_REL, floor=GOLDEN_FLOOR):
+    """Against vectors that come without an oracle run (golden files): bit-exact for ints / bools, `max_rel` with
+    `floor` (a fraction of the tensor's rms) for floats."""
     assert len(expected) == len(actual)
     for i, (e, a) in enumerate(zip(expected, actual)):
         assert list(e.shape) == list(a.shape) and e.dtype == a.dtype, f"{what}: output {i} shape/dtype mismatch"
         if e.dtype.kind == "f":
-            err = max_rel_error(e, a)
+            err = rel_error(e, a, floor)
             bar = F16_MAX_REL if e.dtype == np.float16 else max_rel
             assert err <= bar, f"{what}: output {i} max relative error {err:.3e} exceeds {bar:.1e}"
         else:
@@ -101,9 +86,10 @@ def check_cpu(graph, batch_size, inputs, expected=None):
     return cpu_outputs
 
 
-def check_gpu(device, graph, batch_size, inputs, expected=None, max_rel=F32_MAX_REL):
+def check_gpu(device, graph, batch_size, inputs, expected=None, what=""):
     """GPU half of `test_all`: the HIP executor on the graph and on its optimized form against
-    expected-or-oracle, with the reference's tolerance and with this project's tighter bar vs the oracle."""
+    expected-or-oracle with the reference's tolerance, and against the oracle on the same graph with this
+    project's own rules (oracle/parity.py)."""
     cpu_outputs = cpu_eval_graph(graph, batch_size, inputs)
     reference = expected if expected is not None else cpu_outputs
     results = []
@@ -112,7 +98,7 @@ def check_gpu(device, graph, batch_size, inputs, expected=None, max_rel=F32_MAX_
         gpu_outputs = ex.evaluate(inputs)
         assert_tensors_match(reference, gpu_outputs, f"gpu, {name}")
         cpu_same_graph = cpu_outputs if name == "unoptimized" else cpu_eval_graph(g, batch_size, inputs)
-        assert_close(cpu_same_graph, gpu_outputs, f"gpu vs oracle, {name}", max_rel)
+        check_outputs(g, batch_size, inputs, cpu_same_graph, gpu_outputs, f"{what} {name}".strip(), PARITY_RECORDS)
         # a second evaluation must give the same answer (buffers are reused between calls)
         again = ex.evaluate(inputs)
         for x, y in zip(gpu_outputs, again):

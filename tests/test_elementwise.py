@@ -159,7 +159,7 @@ def test_cpu(name):
 def test_gpu(name, hip_device):
     graph, batch, inputs, expected = CASES[name]()
     print(f"case {name}", flush=True)
-    check_gpu(hip_device, graph, batch, inputs, expected)
+    check_gpu(hip_device, graph, batch, inputs, expected, what=f"elementwise {name}")
 
 
 def test_cast_to_same_type_is_identity():

@@ -1,5 +1,6 @@
-"""HIP graph replay of the launch list against step-by-step launches: several replays with different inputs, with
-eager work and synchronisations of the same executor (and of a second one) in between, every replay checked."""
+"""HIP graph replay of the launch list: several replays with different inputs, with eager work and
+synchronisations of the same executor (and of a second one) in between; every replay is checked against the CPU
+oracle (the parity rules of the other GPU tests) and has to equal the step-by-step launches bit for bit."""
 import os
 
 import numpy as np
@@ -8,6 +9,8 @@ import pytest
 from kyanite_amd import HipExecutor, optimize_graph
 from kyanite_amd.configs import build_resnet_tower, build_tiny_mlp, uniform
 from kyanite_amd.onnx import load_check_data, load_graph_from_onnx_bytes
+from oracle import cpu_eval_graph
+from runner import PARITY_RECORDS, check_outputs
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
@@ -44,6 +47,8 @@ def test_graph_replay_matches_eager(build, hip_device):
                for x in inputs]
         want = eager.evaluate(ins)
         got = replay.evaluate(ins)
+        check_outputs(graph, batch, ins, cpu_eval_graph(graph, batch, ins), got, f"graph replay {build.__name__} round {round_}",
+                      PARITY_RECORDS)
         for w, g in zip(want, got):
             assert np.array_equal(w, g, equal_nan=True), f"round {round_}: graph replay differs from eager launches"
         # device-only replays between the checked ones

@@ -6,13 +6,7 @@ graph, and both graphs must plan and compile for gfx950. GPU: the HIP executor a
 import pytest
 
 from cases_graphs import CASES
-from runner import F32_MAX_REL, check_cpu, check_gpu
-
-# Cases whose f32 rounding differences compound over several chained contractions with cancelling terms get a
-# wider (still stated) bound against the oracle; everything else has to meet F32_MAX_REL.
-MAX_REL_OVERRIDES = {
-}
-
+from runner import check_cpu, check_gpu
 
 @pytest.mark.parametrize("name", list(CASES))
 def test_cpu(name):
@@ -25,4 +19,4 @@ def test_cpu(name):
 def test_gpu(name, hip_device):
     graph, batch, inputs, expected = CASES[name]()
     print(f"case {name} batch {batch}", flush=True)
-    check_gpu(hip_device, graph, batch, inputs, expected, MAX_REL_OVERRIDES.get(name, F32_MAX_REL))
+    check_gpu(hip_device, graph, batch, inputs, expected, what=name)

@@ -36,7 +36,7 @@ def test_fixture_cpu(name):
 @pytest.mark.parametrize("name", FIXTURES)
 def test_fixture_gpu(name, hip_device):
     graph, batch, inputs, expected = load(name)
-    outputs = check_gpu(hip_device, graph, batch, inputs, expected)
+    outputs = check_gpu(hip_device, graph, batch, inputs, expected, what=f"onnx {name}")
     assert_close(expected, outputs, f"{name}: gpu vs golden vectors")
 
 

@@ -42,7 +42,7 @@ def test_scalar_fusion_cpu(kind):
 @pytest.mark.parametrize("kind", KINDS)
 def test_scalar_fusion_gpu(kind, hip_device):
     print(f"case {kind}", flush=True)
-    check_gpu(hip_device, *_scalar_graph(kind))
+    check_gpu(hip_device, *_scalar_graph(kind), what=f"scalar fusion {kind}")
 
 
 def test_scalar_fusion_plans():

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 from kyanite_amd import BinaryOp, DType, Graph, ReduceOp, UnaryOp
-from runner import F16_MAX_REL, check_cpu, check_gpu
+from runner import check_cpu, check_gpu
 
 SEEDS = list(range(48))
 DIMS = [1, 2, 3, 5, 8, 17, 32, 40, 64]
@@ -272,7 +272,7 @@ def test_cpu_f16(seed):
 def test_gpu_f16(seed, hip_device):
     graph, inputs = Builder(seed, DType.F16).build()
     print(f"random f16 graph seed {seed}: {len(graph)} values", flush=True)
-    check_gpu(hip_device, graph, 0, inputs, max_rel=F16_MAX_REL)
+    check_gpu(hip_device, graph, 0, inputs, what=f"random f16 graph {seed}")
 
 
 @pytest.mark.gpu
@@ -280,4 +280,4 @@ def test_gpu_f16(seed, hip_device):
 def test_gpu(seed, hip_device):
     graph, inputs = Builder(seed).build()
     print(f"random graph seed {seed}: {len(graph)} values", flush=True)
-    check_gpu(hip_device, graph, 0, inputs)
+    check_gpu(hip_device, graph, 0, inputs, what=f"random graph {seed}")

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 
 from kyanite_amd import DType, Graph
-from runner import F16_MAX_REL, check_cpu, check_gpu
+from runner import check_cpu, check_gpu
 
 SEEDS = list(range(96))
 
@@ -96,4 +96,4 @@ def test_cpu(seed):
 @pytest.mark.parametrize("seed", SEEDS)
 def test_gpu(seed, hip_device):
     g, inputs, dtype = build(seed)
-    check_gpu(hip_device, g, 0, inputs, None, max_rel=F16_MAX_REL if dtype == DType.F16 else 1e-4)
+    check_gpu(hip_device, g, 0, inputs, None, what=f"random matmul {seed}")
