@@ -71,6 +71,25 @@ int knhip_host_alloc(size_t bytes, void **ptr);
 int knhip_host_free(void *ptr);
 int knhip_device_synchronize(int device);
 
+/* streams and events (replaces CudaStream, kn-cuda-sys/src/wrapper/handle.rs:105-174, and CudaEvent, event.rs:7-45).
+ * Handles are the HIP objects themselves (hipStream_t / hipEvent_t behind void *); a NULL stream is the device's
+ * default stream. Every stream has the default priority. An event belongs to the device it was created on. */
+int knhip_stream_create(int device, void **stream);                      /* CudaStream::new, handle.rs:124-131 */
+int knhip_stream_destroy(int device, void *stream);                      /* Drop, handle.rs:115-121 */
+int knhip_stream_synchronize(int device, void *stream);                  /* handle.rs:133-135 */
+int knhip_stream_wait_event(int device, void *stream, void *event);      /* wait_for_event, handle.rs:155-159 */
+int knhip_event_create(int device, void **event);                        /* CudaEvent::new, event.rs:10-16 */
+int knhip_event_destroy(int device, void *event);                        /* Drop, event.rs:40-44 */
+int knhip_event_record(int device, void *event, void *stream);           /* record_existing_event, handle.rs:151-153 */
+int knhip_event_synchronize(int device, void *event);                    /* event.rs:28-30 */
+/* seconds between two recorded events, like CudaEvent::time_elapsed_since (event.rs:19-26) */
+int knhip_event_elapsed_seconds(int device, void *start, void *end, float *seconds);
+/* copies that return once queued on `stream` (copy_linear_{from,to}_host_async, mem/device.rs:114-153): the host
+ * side must be pinned memory (knhip_host_alloc) that stays untouched until the stream has passed the copy */
+int knhip_memcpy_h2d_async(int device, void *dst, const void *src, size_t bytes, void *stream);
+int knhip_memcpy_d2h_async(int device, void *dst, const void *src, size_t bytes, void *stream);
+int knhip_memcpy_d2d_async(int device, void *dst, const void *src, size_t bytes, void *stream);
+
 /* ---- graph (kn-graph/src/graph.rs) ------------------------------------------------------------------------- */
 typedef struct knhip_graph knhip_graph;
 typedef uint32_t knhip_value; /* index of a value inside its graph; values are append-only (graph.rs:86-91) */

@@ -128,6 +128,94 @@ int knhip_memcpy_h2d(int device, void *dst, const void *src, size_t bytes) { ret
 int knhip_memcpy_d2h(int device, void *dst, const void *src, size_t bytes) { return do_memcpy(device, dst, src, bytes, hipMemcpyDeviceToHost); }
 int knhip_memcpy_d2d(int device, void *dst, const void *src, size_t bytes) { return do_memcpy(device, dst, src, bytes, hipMemcpyDeviceToDevice); }
 
+static int do_memcpy_async(int device, void *dst, const void *src, size_t bytes, hipMemcpyKind kind, void *stream) {
+    return guarded([&] {
+        HipDevice::check(device);
+        KN_REQUIRE(bytes == 0 || (dst != nullptr && src != nullptr));
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        if (bytes) hip_check(hipMemcpyAsync(dst, src, bytes, kind, (hipStream_t) stream), "hipMemcpyAsync");
+        return KNHIP_OK;
+    });
+}
+int knhip_memcpy_h2d_async(int device, void *dst, const void *src, size_t bytes, void *stream) {
+    return do_memcpy_async(device, dst, src, bytes, hipMemcpyHostToDevice, stream);
+}
+int knhip_memcpy_d2h_async(int device, void *dst, const void *src, size_t bytes, void *stream) {
+    return do_memcpy_async(device, dst, src, bytes, hipMemcpyDeviceToHost, stream);
+}
+int knhip_memcpy_d2d_async(int device, void *dst, const void *src, size_t bytes, void *stream) {
+    return do_memcpy_async(device, dst, src, bytes, hipMemcpyDeviceToDevice, stream);
+}
+
+// Every call names its device and selects it first (handle.rs:60-64): the caller's thread may have switched.
+template <typename F>
+static int on_device(int device, F f) {
+    return guarded([&] {
+        HipDevice::check(device);
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        f();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_stream_create(int device, void **stream) {
+    return on_device(device, [&] {
+        KN_REQUIRE(stream != nullptr);
+        hipStream_t s = nullptr;
+        hip_check(hipStreamCreate(&s), "hipStreamCreate");  // default priority
+        *stream = s;
+    });
+}
+int knhip_stream_destroy(int device, void *stream) {
+    return on_device(device, [&] {
+        KN_REQUIRE(stream != nullptr);
+        hip_check(hipStreamDestroy((hipStream_t) stream), "hipStreamDestroy");
+    });
+}
+int knhip_stream_synchronize(int device, void *stream) {
+    return on_device(device, [&] { hip_check(hipStreamSynchronize((hipStream_t) stream), "hipStreamSynchronize"); });
+}
+int knhip_stream_wait_event(int device, void *stream, void *event) {
+    return on_device(device, [&] {
+        KN_REQUIRE(event != nullptr);
+        hip_check(hipStreamWaitEvent((hipStream_t) stream, (hipEvent_t) event, 0), "hipStreamWaitEvent");
+    });
+}
+int knhip_event_create(int device, void **event) {
+    return on_device(device, [&] {
+        KN_REQUIRE(event != nullptr);
+        hipEvent_t e = nullptr;
+        hip_check(hipEventCreate(&e), "hipEventCreate");
+        *event = e;
+    });
+}
+int knhip_event_destroy(int device, void *event) {
+    return on_device(device, [&] {
+        KN_REQUIRE(event != nullptr);
+        hip_check(hipEventDestroy((hipEvent_t) event), "hipEventDestroy");
+    });
+}
+int knhip_event_record(int device, void *event, void *stream) {
+    return on_device(device, [&] {
+        KN_REQUIRE(event != nullptr);
+        hip_check(hipEventRecord((hipEvent_t) event, (hipStream_t) stream), "hipEventRecord");
+    });
+}
+int knhip_event_synchronize(int device, void *event) {
+    return on_device(device, [&] {
+        KN_REQUIRE(event != nullptr);
+        hip_check(hipEventSynchronize((hipEvent_t) event), "hipEventSynchronize");
+    });
+}
+int knhip_event_elapsed_seconds(int device, void *start, void *end, float *seconds) {
+    return on_device(device, [&] {
+        KN_REQUIRE(start != nullptr && end != nullptr && seconds != nullptr);
+        float ms = 0;
+        hip_check(hipEventElapsedTime(&ms, (hipEvent_t) start, (hipEvent_t) end), "hipEventElapsedTime");
+        *seconds = ms / 1000.0f;
+    });
+}
+
 int knhip_host_alloc(size_t bytes, void **ptr) {
     return guarded([&] {
         KN_REQUIRE(ptr != nullptr);

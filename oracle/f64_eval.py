@@ -144,8 +144,16 @@ def eval_graph_f64(graph, batch_size, inputs, storage_rounding=False):
     which is the sharper comparison when only the MEANING of the operations is in question."""
     values = {}
     input_index = {int(v): i for i, v in enumerate(graph.inputs())}
-    for v in graph.values():
-        info = graph[v]
+    # intermediate values are dropped after their last use (full-size graphs hold gigabytes in f64)
+    all_values = list(graph.values())
+    infos = {int(v): graph[v] for v in all_values}
+    last_use = {}
+    for v in all_values:
+        for o in infos[int(v)].operands:
+            last_use[int(o)] = int(v)
+    keep = {int(o) for o in graph.outputs()}
+    for v in all_values:
+        info = infos[int(v)]
         shape = [d.eval(batch_size) for d in info.shape]
         is_float = _is_float(info.dtype)
         ops = [values[int(o)] for o in info.operands]
@@ -170,7 +178,7 @@ def eval_graph_f64(graph, batch_size, inputs, storage_rounding=False):
         elif kind == OpKind.FLIP:
             out = np.flip(ops[0], info.axes[0])
         elif kind == OpKind.GATHER:
-            src = graph[info.operands[1]]
+            src = infos[int(info.operands[1])]
             if src.op not in (OpKind.INPUT, OpKind.CONSTANT):
                 raise Unsupported("gather through computed indices")
             out = np.take(ops[0], ops[1].astype(np.int64), axis=info.axes[0])
@@ -185,7 +193,7 @@ def eval_graph_f64(graph, batch_size, inputs, storage_rounding=False):
             out = np.matmul(ops[0], ops[1])
         elif kind == OpKind.UNARY:
             op = UnaryOp(info.sub_op)
-            src_dtype = graph[info.operands[0]].dtype
+            src_dtype = infos[int(info.operands[0])].dtype
             if op == UnaryOp.VALUE_CAST:
                 if _is_float(src_dtype) and is_float:
                     out = ops[0]
@@ -261,4 +269,7 @@ def eval_graph_f64(graph, batch_size, inputs, storage_rounding=False):
             with np.errstate(all="ignore"):
                 out = out.astype(_NUMPY[int(info.dtype)]).astype(np.float64)
         values[int(v)] = out
+        for o in info.operands:
+            if last_use.get(int(o)) == int(v) and int(o) not in keep:
+                values.pop(int(o), None)
     return [np.array(values[int(o)], order="C") for o in graph.outputs()]

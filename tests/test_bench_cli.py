@@ -20,7 +20,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 def test_help_lists_the_workloads():
     r = run("--help")
     assert r.returncode == 0
-    for name in ("bandwidth", "mlp", "resnet", "llama", "unet"):
+    for name in ("all", "bandwidth", "mlp", "resnet", "llama", "unet"):
         assert name in r.stdout
 
 
