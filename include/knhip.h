@@ -90,6 +90,29 @@ int knhip_memcpy_h2d_async(int device, void *dst, const void *src, size_t bytes,
 int knhip_memcpy_d2h_async(int device, void *dst, const void *src, size_t bytes, void *stream);
 int knhip_memcpy_d2d_async(int device, void *dst, const void *src, size_t bytes, void *stream);
 
+/* ---- one batched matrix product on device memory, outside any executor ---------------------------------------
+ * The role of BatchedMatMulArgs::run (kn-cuda-sys/src/wrapper/group.rs:107-171, cublasSgemm[StridedBatched]):
+ * C[b] = A[b] B[b] for b < batch, A [m, k], B [k, n], C [m, n], every matrix addressed by element strides (batch, row,
+ * column; a zero batch stride broadcasts the matrix). cuBLAS operands map onto this directly: a column-major operand
+ * with leading dimension ld has row stride 1 and column stride ld, a transposed one the other way round, and
+ * MatMulOperand::stride is the batch stride. alpha = 1 and beta = 0, the only values the reference passes
+ * (kn-cuda-eval/src/planner.rs:606-648). Elements are f32, or f16 with f32 accumulation and one rounding at the store.
+ * Launches that split the K axis between workgroups keep f32 partial products and tile counters in `workspace`
+ * (device memory, 256 byte aligned, knhip_batched_mat_mul_workspace_bytes(args) bytes; may be NULL when that is 0);
+ * the call returns once the work is queued on `stream`, and the workspace must stay untouched until it has run. */
+typedef struct {
+    int dtype; /* KNHIP_F32 or KNHIP_F16 */
+    int batch, m, n, k;
+    const void *a;
+    int64_t a_batch_stride, a_row_stride, a_col_stride;
+    const void *b;
+    int64_t b_batch_stride, b_row_stride, b_col_stride;
+    void *c;
+    int64_t c_batch_stride, c_row_stride, c_col_stride;
+} knhip_matmul_args;
+int knhip_batched_mat_mul_workspace_bytes(const knhip_matmul_args *args, size_t *bytes);
+int knhip_batched_mat_mul(int device, void *stream, const knhip_matmul_args *args, void *workspace, size_t workspace_bytes);
+
 /* ---- graph (kn-graph/src/graph.rs) ------------------------------------------------------------------------- */
 typedef struct knhip_graph knhip_graph;
 typedef uint32_t knhip_value; /* index of a value inside its graph; values are append-only (graph.rs:86-91) */

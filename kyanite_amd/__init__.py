@@ -5,6 +5,8 @@ shaped like the reference's `kn-graph` builder and `CudaExecutor`.
 """
 from ._lib import KnError, LIB_PATH
 from .executor import Device, HipDevice, HipExecutor, PreparedGraph, Profile, compile_stats
+from .runtime import (DeviceBuffer, HipEvent, HipStream, PinnedMem, batched_mat_mul, batched_mat_mul_workspace_bytes,
+                      matmul_args)
 from .graph import (BATCH, BINARY_ALL, REDUCE_ALL, UNARY_ALL, BinaryOp, DType, Graph, OpKind, OptimizerSettings,
                     ReduceOp, Size, UnaryOp, Value, optimize_graph, shape)
 
@@ -12,4 +14,5 @@ __all__ = [
     "KnError", "LIB_PATH", "Device", "HipDevice", "HipExecutor", "PreparedGraph", "Profile", "compile_stats",
     "BATCH", "BINARY_ALL", "REDUCE_ALL", "UNARY_ALL", "BinaryOp", "DType", "Graph", "OpKind", "OptimizerSettings",
     "ReduceOp", "Size", "UnaryOp", "Value", "optimize_graph", "shape",
+    "DeviceBuffer", "HipEvent", "HipStream", "PinnedMem", "batched_mat_mul", "batched_mat_mul_workspace_bytes", "matmul_args",
 ]

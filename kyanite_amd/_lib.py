@@ -36,6 +36,13 @@ class ProfileT(Structure):
                 ("step_count", c_size_t)]
 
 
+class MatmulArgsT(Structure):
+    _fields_ = [("dtype", c_int), ("batch", c_int), ("m", c_int), ("n", c_int), ("k", c_int),
+                ("a", c_void_p), ("a_batch_stride", c_int64), ("a_row_stride", c_int64), ("a_col_stride", c_int64),
+                ("b", c_void_p), ("b_batch_stride", c_int64), ("b_row_stride", c_int64), ("b_col_stride", c_int64),
+                ("c", c_void_p), ("c_batch_stride", c_int64), ("c_row_stride", c_int64), ("c_col_stride", c_int64)]
+
+
 class MemUsageT(Structure):
     _fields_ = [("dedicated_bytes", c_size_t), ("shared_bytes", c_size_t), ("zero_bytes", c_size_t),
                 ("hypo_shared_bytes_peak", c_size_t), ("hypo_shared_bytes_total", c_size_t), ("arena_bytes", c_size_t)]
@@ -60,6 +67,20 @@ SIGNATURES = {
     "knhip_host_alloc": [c_size_t, POINTER(c_void_p)],
     "knhip_host_free": [c_void_p],
     "knhip_device_synchronize": [c_int],
+    "knhip_stream_create": [c_int, POINTER(c_void_p)],
+    "knhip_stream_destroy": [c_int, c_void_p],
+    "knhip_stream_synchronize": [c_int, c_void_p],
+    "knhip_stream_wait_event": [c_int, c_void_p, c_void_p],
+    "knhip_event_create": [c_int, POINTER(c_void_p)],
+    "knhip_event_destroy": [c_int, c_void_p],
+    "knhip_event_record": [c_int, c_void_p, c_void_p],
+    "knhip_event_synchronize": [c_int, c_void_p],
+    "knhip_event_elapsed_seconds": [c_int, c_void_p, c_void_p, POINTER(c_float)],
+    "knhip_memcpy_h2d_async": [c_int, c_void_p, c_void_p, c_size_t, c_void_p],
+    "knhip_memcpy_d2h_async": [c_int, c_void_p, c_void_p, c_size_t, c_void_p],
+    "knhip_memcpy_d2d_async": [c_int, c_void_p, c_void_p, c_size_t, c_void_p],
+    "knhip_batched_mat_mul_workspace_bytes": [POINTER(MatmulArgsT), PZ],
+    "knhip_batched_mat_mul": [c_int, c_void_p, POINTER(MatmulArgsT), c_void_p, c_size_t],
     "knhip_graph_new": [POINTER(G)],
     "knhip_graph_clone": [G, POINTER(G)],
     "knhip_graph_deserialize": [POINTER(c_uint8), c_size_t, POINTER(G)],

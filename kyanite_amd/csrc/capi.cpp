@@ -6,6 +6,7 @@
 #include <new>
 
 #include "executor.h"
+#include "matmul_api.h"
 #include "optimizer.h"
 
 using namespace kn;
@@ -76,7 +77,66 @@ int copy_list(const std::vector<T> &v, U *buf, size_t cap, size_t *count) {
     return KNHIP_OK;
 }
 
+// Every call names its device and selects it first (handle.rs:60-64): the caller's thread may have switched.
+template <typename F>
+int on_device(int device, F f) {
+    return guarded([&] {
+        HipDevice::check(device);
+        hip_check(hipSetDevice(device), "hipSetDevice");
+        f();
+        return KNHIP_OK;
+    });
+}
+
 }  // namespace
+
+namespace kn {
+
+void set_last_error(const std::string &message) { g_last_error = message; }
+
+GemmLaunchPlan matmul_api_plan(const knhip_matmul_args &a, MatmulWorkspace *ws) {
+    if (a.dtype != KNHIP_F32 && a.dtype != KNHIP_F16) fail("batched_mat_mul: dtype must be f32 or f16, got code ", a.dtype);
+    if (a.batch < 0 || a.m < 0 || a.n < 0 || a.k < 0) fail("batched_mat_mul: negative size");
+    const bool empty = a.batch == 0 || a.m == 0 || a.n == 0;
+    if (!empty && (a.c == nullptr || (a.k > 0 && (a.a == nullptr || a.b == nullptr)))) fail("batched_mat_mul: null operand");
+    if (a.batch > 65535) fail("batched_mat_mul: at most 65535 batch entries per call, got ", a.batch);
+    GemmParams p{};
+    p.a = a.a;
+    p.b = a.b;
+    p.c = a.c;
+    p.batch = a.batch;
+    p.m = a.m;
+    p.n = a.n;
+    p.k = a.k;
+    p.a_sb = a.a_batch_stride; p.a_sm = a.a_row_stride; p.a_sk = a.a_col_stride;
+    p.b_sb = a.b_batch_stride; p.b_sk = a.b_row_stride; p.b_sn = a.b_col_stride;
+    p.c_sb = a.c_batch_stride; p.c_sm = a.c_row_stride; p.c_sn = a.c_col_stride;
+    GemmLaunchPlan lp = plan_gemm_launch(p, a.dtype == KNHIP_F16);
+    ws->counter_bytes = lp.counter_bytes;
+    ws->partial_bytes = lp.workspace_bytes;
+    return lp;
+}
+
+void matmul_api_launch(const knhip_matmul_args &args, void *workspace, size_t workspace_bytes, ihipStream_t *stream) {
+    MatmulWorkspace ws;
+    GemmLaunchPlan lp = matmul_api_plan(args, &ws);
+    if (args.batch == 0 || args.m == 0 || args.n == 0) return;
+    if (ws.total() > 0) {
+        if (workspace == nullptr || workspace_bytes < ws.total())
+            fail("batched_mat_mul: this product needs ", ws.total(), " bytes of workspace, got ", workspace_bytes);
+        if ((uintptr_t) workspace % 256 != 0) fail("batched_mat_mul: the workspace must be 256 byte aligned");
+        if (ws.counter_bytes > 0) {
+            // the tile counters start at zero (a fill kernel, not a memset: the call may be under stream capture)
+            hip_check((hipError_t) launch_fill_zero(workspace, ws.counter_bytes, stream), "counter fill launch");
+            lp.p.counters = workspace;
+        }
+        if (ws.partial_bytes > 0) lp.p.workspace = (char *) workspace + ws.partial_offset();
+    }
+    const bool f16 = args.dtype == KNHIP_F16;
+    hip_check((hipError_t) (f16 ? launch_gemm_f16(lp, stream) : launch_gemm_f32(lp, stream)), "matmul launch");
+}
+
+}  // namespace kn
 
 extern "C" {
 
@@ -147,17 +207,6 @@ int knhip_memcpy_d2d_async(int device, void *dst, const void *src, size_t bytes,
     return do_memcpy_async(device, dst, src, bytes, hipMemcpyDeviceToDevice, stream);
 }
 
-// Every call names its device and selects it first (handle.rs:60-64): the caller's thread may have switched.
-template <typename F>
-static int on_device(int device, F f) {
-    return guarded([&] {
-        HipDevice::check(device);
-        hip_check(hipSetDevice(device), "hipSetDevice");
-        f();
-        return KNHIP_OK;
-    });
-}
-
 int knhip_stream_create(int device, void **stream) {
     return on_device(device, [&] {
         KN_REQUIRE(stream != nullptr);
@@ -213,6 +262,23 @@ int knhip_event_elapsed_seconds(int device, void *start, void *end, float *secon
         float ms = 0;
         hip_check(hipEventElapsedTime(&ms, (hipEvent_t) start, (hipEvent_t) end), "hipEventElapsedTime");
         *seconds = ms / 1000.0f;
+    });
+}
+
+int knhip_batched_mat_mul_workspace_bytes(const knhip_matmul_args *args, size_t *bytes) {
+    return guarded([&] {
+        KN_REQUIRE(args != nullptr && bytes != nullptr);
+        MatmulWorkspace ws;
+        (void) matmul_api_plan(*args, &ws);
+        *bytes = ws.total();
+        return KNHIP_OK;
+    });
+}
+
+int knhip_batched_mat_mul(int device, void *stream, const knhip_matmul_args *args, void *workspace, size_t workspace_bytes) {
+    return on_device(device, [&] {
+        KN_REQUIRE(args != nullptr);
+        matmul_api_launch(*args, workspace, workspace_bytes, (ihipStream_t *) stream);
     });
 }
 

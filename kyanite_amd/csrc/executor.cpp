@@ -97,6 +97,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             step.gemm.c = step.gemm.c_group[0];
             step.gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;
             step.gemm.counters = lp.counter_bytes > 0 ? l.ptrs[next++] : nullptr;
+            step.gemm_plan = plan_gemm_launch(step.gemm, step.gemm_f16);
         } else if (step.kind == StepKind::MatMul) {
             step.gemm.a = l.ptrs[0];
             step.gemm.b = l.ptrs[1];
@@ -108,6 +109,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             KN_ASSERT(l.ptrs.size() == next + (lp.workspace_bytes > 0) + (lp.counter_bytes > 0));
             step.gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;
             step.gemm.counters = lp.counter_bytes > 0 ? l.ptrs[next++] : nullptr;
+            step.gemm_plan = plan_gemm_launch(step.gemm, step.gemm_f16);
         } else if (step.kind == StepKind::Conv) {
             size_t k = 0;
             step.conv.input = (const float *) l.ptrs[k++];
@@ -209,7 +211,7 @@ void HipExecutor::launch_step(size_t index, hipEvent_t start, hipEvent_t stop) {
                           "attention launch");
                 break;
             }
-            hip_check((hipError_t) (step.gemm_f16 ? launch_gemm_f16(step.gemm, stream_) : launch_gemm_f32(step.gemm, stream_)),
+            hip_check((hipError_t) (step.gemm_f16 ? launch_gemm_f16(step.gemm_plan, stream_) : launch_gemm_f32(step.gemm_plan, stream_)),
                       "matmul launch");
             break;
         case StepKind::Conv: hip_check((hipError_t) launch_conv_f32(step.conv, stream_), "conv launch"); break;
@@ -299,8 +301,8 @@ const std::vector<HostTensor> &HipExecutor::evaluate(const std::vector<HostTenso
             fail("Wrong dtype for input ", i, ": expected ", dtype_name(plan_.inputs[i].dtype), ", got ", dtype_name(inputs[i].dtype));
     }
     hip_check(hipSetDevice(device_), "hipSetDevice");
-    // make sure nothing else is still using the staging buffers
-    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    // The staging buffers are free: every evaluate ends with a synchronisation, and run_async never touches them.
+    // Device work a caller queued through run_async is ordered before the copies below by the stream itself.
     for (size_t i = 0; i < inputs.size(); i++) {
         size_t bytes = inputs[i].nbytes();
         if (bytes == 0) continue;

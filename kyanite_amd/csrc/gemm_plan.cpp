@@ -31,6 +31,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         q.d_sm = p.d_sn; q.d_sn = p.d_sm;
         q.d2_sm = p.d2_sn; q.d2_sn = p.d2_sm;
         p = q;
+        lp.swapped = true;
     }
     lp.p = p;
     lp.split_k = 1;

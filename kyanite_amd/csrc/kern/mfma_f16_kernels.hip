@@ -597,12 +597,11 @@ int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool 
     return (int) hipGetLastError();
 }
 
-int launch_gemm_f16(const GemmParams &params, ihipStream_t *stream) {
-    if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
-    const GemmLaunchPlan lp = plan_gemm_launch(params, true);
+int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     const GemmParams &p = lp.p;
+    if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
     const int groups = p.groups > 1 ? p.groups : 1;
-    if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
+    if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || lp.swapped))) return (int) hipErrorInvalidValue;
     if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;
     if (p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;

@@ -698,6 +698,19 @@ int small_tile_threshold() {
 
 }  // namespace
 
+__global__ __launch_bounds__(256) void fill_zero_kernel(unsigned *p, size_t words) {
+    const size_t i = (size_t) blockIdx.x * 256 + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+int launch_fill_zero(void *ptr, size_t bytes, ihipStream_t *stream) {
+    if (bytes == 0) return 0;
+    if (bytes % 4 != 0 || (uintptr_t) ptr % 4 != 0 || bytes / 4 > 0x7fffffffull * 256) return (int) hipErrorInvalidValue;
+    const size_t words = bytes / 4;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned) ((words + 255) / 256)), dim3(256), 0, stream, (unsigned *) ptr, words);
+    return (int) hipGetLastError();
+}
+
 int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipStream_t *stream) {
     const long long mn = (long long) p.m * p.n;
     const bool vec = p.n % 4 == 0 && p.c_sn == 1 && (uintptr_t) p.workspace % 16 == 0;
@@ -710,13 +723,12 @@ int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipSt
     return (int) hipGetLastError();
 }
 
-int launch_gemm_f32(const GemmParams &params, ihipStream_t *stream) {
-    if (params.batch <= 0 || params.m <= 0 || params.n <= 0) return 0;
-    const GemmLaunchPlan lp = plan_gemm_launch(params, false);
+int launch_gemm_f32(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     const GemmParams &p = lp.p;
+    if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
     const int t = lp.small_tile ? 64 : 128;
     const int groups = p.groups > 1 ? p.groups : 1;
-    if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || p.a != params.a))) return (int) hipErrorInvalidValue;
+    if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || lp.swapped))) return (int) hipErrorInvalidValue;
     if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;
     const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * groups;
     if (tiles > 0x7fffffffll || p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;

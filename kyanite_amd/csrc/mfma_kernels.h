@@ -50,6 +50,7 @@ struct GemmParams {
 // for it ahead of time (to reserve the workspace) and the launch reproduces it.
 struct GemmLaunchPlan {
     GemmParams p;            // operands swapped where needed so that the contiguous axis of C is the column axis
+    bool swapped;            // whether they were
     bool small_tile;         // 64 x 64 workgroup tiles instead of 128 x 128
     bool tall_tile;          // f16 only: 256 x 128 workgroup tiles (8 waves)
     bool narrow_tile;        // f16 direct kernel only: 128 x 64 workgroup tiles
@@ -119,14 +120,17 @@ bool attention_f16_supported(int dk, int dv);
 // All return a hipError_t value (0 = success).
 int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream);
 int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream);
-int launch_gemm_f32(const GemmParams &p, ihipStream_t *stream);
+// (the plan is computed once per step, when the executor is built, from the operands at their final addresses)
+int launch_gemm_f32(const GemmLaunchPlan &lp, ihipStream_t *stream);
 // the kernel that loads global -> LDS directly, where `lp` (of an f32 product) and the alignment of the pointers allow
 // it; `launched` tells whether it ran (the sum of split-K partial products is left to the caller)
 int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool *launched);
 // f16 operands and result, f32 accumulation, one rounding (to nearest even) at the store
-int launch_gemm_f16(const GemmParams &p, ihipStream_t *stream);
+int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream);
 // second pass of a split-K launch: C = sum of the f32 partial products in the workspace (`p` already oriented)
 int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipStream_t *stream);
 int launch_conv_f32(const ConvParams &p, ihipStream_t *stream);
+// zero `bytes` bytes (a multiple of 4, 4 byte aligned) with a kernel on `stream`
+int launch_fill_zero(void *ptr, size_t bytes, ihipStream_t *stream);
 
 }  // namespace kn

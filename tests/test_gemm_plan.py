@@ -159,7 +159,7 @@ def test_projections_of_one_input_share_a_launch():
     assert [("x4" in ex.step_str(i), "x2" in ex.step_str(i)) for i in range(ex.step_count())] == [(True, False), (False, True)]
     # a product whose bias is folded into its store keeps its own launch
     ex = HipExecutor(0, _projections(3, 256, 64, 128, bias_on=(1,)), 0, plan_only=True)
-    texts = sorted(ex.step_str(i).split(" operands")[0].split("k=64")[1].strip() for i in range(ex.step_count()))
+    texts = sorted(ex.step_str(i).split(" [")[0].split("k=64")[1].strip() for i in range(ex.step_count()))
     assert texts == ["+add", "x2 grouped"]
     # where even the group leaves the chip short of tiles, the products run apart and split K
     ex = HipExecutor(0, _projections(2, 8, 4096, 256), 0, plan_only=True)
