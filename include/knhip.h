@@ -113,6 +113,14 @@ typedef struct {
 int knhip_batched_mat_mul_workspace_bytes(const knhip_matmul_args *args, size_t *bytes);
 int knhip_batched_mat_mul(int device, void *stream, const knhip_matmul_args *args, void *workspace, size_t workspace_bytes);
 
+/* No counterpart in the reference. For callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): knhip_batched_mat_mul with the workspace taken from a static
+ * device array of KNHIP_STATIC_SCRATCH_BYTES per GPU instead of an argument. The call allocates nothing and fails
+ * with a message when the product needs more scratch than that. All calls on one GPU share the array: calls whose
+ * work overlaps on one GPU (two streams, two threads) race, the caller orders them. */
+#define KNHIP_STATIC_SCRATCH_BYTES (32u << 20)
+int knhip_batched_mat_mul_static(int device, void *stream, const knhip_matmul_args *args);
+
 /* ---- graph (kn-graph/src/graph.rs) ------------------------------------------------------------------------- */
 typedef struct knhip_graph knhip_graph;
 typedef uint32_t knhip_value; /* index of a value inside its graph; values are append-only (graph.rs:86-91) */

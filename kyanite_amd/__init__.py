@@ -5,8 +5,8 @@ shaped like the reference's `kn-graph` builder and `CudaExecutor`.
 """
 from ._lib import KnError, LIB_PATH
 from .executor import Device, HipDevice, HipExecutor, PreparedGraph, Profile, compile_stats
-from .runtime import (DeviceBuffer, HipEvent, HipStream, PinnedMem, batched_mat_mul, batched_mat_mul_workspace_bytes,
-                      matmul_args)
+from .runtime import (STATIC_SCRATCH_BYTES, DeviceBuffer, HipEvent, HipStream, PinnedMem, batched_mat_mul,
+                      batched_mat_mul_static, batched_mat_mul_workspace_bytes, matmul_args)
 from .graph import (BATCH, BINARY_ALL, REDUCE_ALL, UNARY_ALL, BinaryOp, DType, Graph, OpKind, OptimizerSettings,
                     ReduceOp, Size, UnaryOp, Value, optimize_graph, shape)
 
@@ -15,4 +15,5 @@ __all__ = [
     "BATCH", "BINARY_ALL", "REDUCE_ALL", "UNARY_ALL", "BinaryOp", "DType", "Graph", "OpKind", "OptimizerSettings",
     "ReduceOp", "Size", "UnaryOp", "Value", "optimize_graph", "shape",
     "DeviceBuffer", "HipEvent", "HipStream", "PinnedMem", "batched_mat_mul", "batched_mat_mul_workspace_bytes", "matmul_args",
+    "STATIC_SCRATCH_BYTES", "batched_mat_mul_static",
 ]

@@ -81,6 +81,7 @@ SIGNATURES = {
     "knhip_memcpy_d2d_async": [c_int, c_void_p, c_void_p, c_size_t, c_void_p],
     "knhip_batched_mat_mul_workspace_bytes": [POINTER(MatmulArgsT), PZ],
     "knhip_batched_mat_mul": [c_int, c_void_p, POINTER(MatmulArgsT), c_void_p, c_size_t],
+    "knhip_batched_mat_mul_static": [c_int, c_void_p, POINTER(MatmulArgsT)],
     "knhip_graph_new": [POINTER(G)],
     "knhip_graph_clone": [G, POINTER(G)],
     "knhip_graph_deserialize": [POINTER(c_uint8), c_size_t, POINTER(G)],

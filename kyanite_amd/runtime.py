@@ -153,3 +153,12 @@ def batched_mat_mul(device, stream, args, workspace=None):
     handle = stream._h if isinstance(stream, HipStream) else c_void_p(stream)
     ptr, size = (c_void_p(workspace.ptr), workspace.nbytes) if workspace is not None else (None, 0)
     check(lib.knhip_batched_mat_mul(_index(device), handle, byref(args), ptr, size))
+
+
+STATIC_SCRATCH_BYTES = 32 << 20
+
+
+def batched_mat_mul_static(device, stream, args):
+    """`batched_mat_mul` on the library's static scratch (at most STATIC_SCRATCH_BYTES): allocates nothing."""
+    handle = stream._h if isinstance(stream, HipStream) else c_void_p(stream)
+    check(lib.knhip_batched_mat_mul_static(_index(device), handle, byref(args)))
