@@ -73,7 +73,10 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // 512 x 22016 x 4096 147 / 133, 512 x 12288 x 4096 93 / 72, 4096^3 152 / 144; 512 x 4096 x 4096 53 / 59.
     // (In f32 the same kernel walks K in slices of 32 and has 128 x 128 and 64 x 64 tiles.)
     const int vec = f16 ? 8 : 4;
+    // (row strides: positive and small enough for the 32 bit byte offsets that the kernel keeps per lane within a tile)
+    constexpr long long max_row_stride = 1ll << 21;
     lp.direct = p.k > 0 && p.k % (8 * vec) == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % vec == 0 && p.b_sn % vec == 0 &&
+                p.a_sm > 0 && p.b_sn > 0 && p.a_sm < max_row_stride && p.b_sn < max_row_stride &&
                 (p.batch <= 1 || (p.a_sb % vec == 0 && p.b_sb % vec == 0));
     if (f16 && lp.direct && tall_fits && tall_blocks >= env_int("KNHIP_F16_TALL_FROM", 128)) lp.tall_tile = true;
     // Direct kernel only: 128 x 64 tiles on a ring of four stages, where 128 x 128 tiles leave compute units

@@ -20,6 +20,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "../mfma_kernels.h"
 
@@ -309,6 +310,46 @@ __device__ __forceinline__ void issue_loads(const T *(&a_src)[A_LD], const T *(&
 #endif
 }
 
+// compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// One K step of a wave's MI x NI MFMA tiles from the operands in `ca` / `cb`, 16 bytes per lane and tile row: 8 halves
+// for one v_mfma_f32_32x32x16_f16 per tile, or 4 floats for four v_mfma_f32_32x32x2_f32 (element u of the vector
+// multiplies k = 8 t + u in the lower half of the wave and 8 t + 4 + u in the upper, in A and B alike). Other work is
+// slotted in between the MFMAs so that the matrix cores never wait for it: `pre(m)` runs right in front of MFMA m,
+// and the scheduling barriers keep the compiler from moving it. The operands of the following step are read during
+// this one (read r goes in front of MFMA r, the operands the next step needs first are read first), so a wave
+// needs no second wave on its SIMD to cover LDS latency.
+template <typename T, int MI, int NI, int ROW, typename V, typename Pre>
+__device__ __forceinline__ void mfma_step(floatx16 (&acc)[MI][NI], const V (&ca)[MI], const V (&cb)[NI], V (&na)[MI], V (&nb)[NI],
+                                          const char *src_a, const char *src_b, Pre &&pre) {
+    constexpr int U = sizeof(T) == 2 ? 1 : 4, R = MI + NI, M = MI * NI * U;
+    auto read_next = [&](auto rc) {
+        constexpr int r = decltype(rc)::value;
+        // order of need in the next step (i-major MFMAs): a[0], b[0 .. NI - 1], a[1 ..]
+        if constexpr (r == 0) na[0] = *(const V *) src_a;
+        else if constexpr (r <= NI) nb[r - 1] = *(const V *) (src_b + (r - 1) * 32 * ROW);
+        else na[r - NI] = *(const V *) (src_a + (r - NI) * 32 * ROW);
+    };
+    // with fewer MFMAs than reads, the surplus reads go first
+    static_for<0, (R > M ? R - M : 0)>([&](auto rc) { read_next(rc); });
+    static_for<0, M>([&](auto mc) {
+        constexpr int m = decltype(mc)::value, r = m + (R > M ? R - M : 0);
+        constexpr int u = m / (MI * NI), i = (m % (MI * NI)) / NI, j = m % NI;
+        pre(mc);
+        if constexpr (r < R) read_next(std::integral_constant<int, r>{});
+        if constexpr (sizeof(T) == 2) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ca[i], cb[j], acc[i][j], 0, 0, 0);
+        else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[i][u], cb[j][u], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
 // The direct-to-LDS kernel: a workgroup of WM x WN waves owns a (32 MI WM) x (32 NI WN) tile, a wave MI x NI MFMA
 // tiles of it. K is walked in slices of 64 through a ring of NSTAGE LDS stages; every stage holds the rows of A,
 // then those of B, 128 bytes each. One load instruction of a wave fills 8 rows (64 chunks of 16 bytes): lane l fills chunk
@@ -335,8 +376,10 @@ template <typename T, int MI, int NI, int WM, int WN, int NSTAGE>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p, DirectSchedule sched) {
     constexpr int WAVES = WM * WN, TM = 32 * MI * WM, TN = 32 * NI * WN, ROW = DIRECT_ROW, BK = ROW / (int) sizeof(T), VEC = 16 / (int) sizeof(T);
     constexpr int A_BYTES = TM * ROW, STAGE = (TM + TN) * ROW;
-    constexpr int A_LD = TM / 8 / WAVES, B_LD = TN / 8 / WAVES;  // load instructions per wave and stage
-    static_assert(A_LD >= 1 && B_LD >= 1 && ROW == 128 && NSTAGE >= 2, "tile too small for the workgroup");
+    constexpr int ROWS_PER_LOAD = 1024 / ROW, CHUNKS = ROW / 16;  // one load instruction of a wave moves 1024 bytes
+    constexpr int A_LD = TM / ROWS_PER_LOAD / WAVES, B_LD = TN / ROWS_PER_LOAD / WAVES;  // load instructions per wave and stage
+    static_assert(A_LD >= 1 && B_LD >= 1 && NSTAGE >= 2, "tile too small for the workgroup");
+    static_assert(TM % (ROWS_PER_LOAD * WAVES) == 0 && TN % (ROWS_PER_LOAD * WAVES) == 0, "rows of a stage do not divide over the waves");
     static_assert((NSTAGE - 2) * (A_LD + B_LD) < 64, "the counter of loads in flight has 6 bits");
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -369,29 +412,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wm = wave / WN, wn = wave % WN, c = lane & 31, half = lane >> 5;
 
-    // the source of every load of this lane; all of them move on by one slice per issue
-    const T *a_src[A_LD], *b_src[B_LD];
-    {
-        // lane l fills chunk position l % 8 of row l / 8 of the 8 rows of its load, with chunk (l % 8) ^ swz(row)
-        const int lr = lane >> 3, pos = lane & 7;
-        const T *a0 = (const T *) p.a + bz * p.a_sb + k_begin;
-        const T *b0 = (const T *) b_base + bz * p.b_sb + k_begin;
-#pragma unroll
-        for (int i = 0; i < A_LD; i++) {
-            const int row = (wave * A_LD + i) * 8 + lr;
-            a_src[i] = a0 + (long long) min(m0 + row, p.m - 1) * p.a_sm + VEC * (pos ^ ((row >> 1) & 7));
-        }
-#pragma unroll
-        for (int i = 0; i < B_LD; i++) {
-            const int row = (wave * B_LD + i) * 8 + lr;
-            b_src[i] = b0 + (long long) min(n0 + row, p.n - 1) * p.b_sn + VEC * (pos ^ ((row >> 1) & 7));
-        }
-    }
-    // MFMA operand of lane (row c, half h) at step t: chunk 2 t + h of its row, found at (2 t + h) ^ swz(c), which is
-    // the address of step 0 with bits 5 and 6 flipped by t
-    const unsigned a_rd = (wm * 32 * MI + c) * ROW + ((half ^ ((c >> 1) & 7)) * 16);
-    const unsigned b_rd = A_BYTES + (wn * 32 * NI + c) * ROW + ((half ^ ((c >> 1) & 7)) * 16);
-
     floatx16 acc[MI][NI];
 #pragma unroll
     for (int i = 0; i < MI; i++)
@@ -400,69 +420,102 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    // The loop is kept free of branches (which make the compiler shuttle the accumulators between register
-    // files): the stages rotate through address arithmetic, and once no slice is left to fetch, the last one is
-    // fetched again into a stage that nobody reads any more.
-    char *const dst_a = lds + wave * A_LD * 1024, *const dst_b = lds + A_BYTES + wave * B_LD * 1024;
+    // MFMA operand of lane (row c, half h) at step t: chunk 2 t + h of its row, found at (2 t + h) ^ swz(c), which is
+    // the address of step 0 with bits 5 and 6 flipped by t
+    auto swz = [](int row) { return (row >> 1) & 7; };
+    const unsigned a_rd = (wm * 32 * MI + c) * ROW + ((half ^ swz(c)) * 16);
+    const unsigned b_rd = A_BYTES + (wn * 32 * NI + c) * ROW + ((half ^ swz(c)) * 16);
+
+    // Software pipelined main loop. Every lane keeps 32 bit byte offsets from the tile's uniform base
+    // pointers, which move on by one slice per issue on the scalar unit. A slice is walked in 4 steps of 16 k; the
+    // operands of step t + 1 are read from LDS between the MFMAs of step t. In the last step of a slice the wave
+    // waits for its own loads of the next slice, meets the others at the barrier (everybody's loads have landed,
+    // and everybody has read the last operands of this slice), sends the loads of the slice NSTAGE further on into
+    // the stage just read, and reads the first operands of the next slice, all between the MFMAs of that step.
+    constexpr int LD = A_LD + B_LD;
+    const int lr = lane / CHUNKS, pos = lane % CHUNKS;
+    const char *a_tile = (const char *) ((const T *) p.a + bz * p.a_sb + k_begin + (long long) m0 * p.a_sm);
+    const char *b_tile = (const char *) ((const T *) b_base + bz * p.b_sb + k_begin + (long long) n0 * p.b_sn);
+    unsigned a_off[A_LD], b_off[B_LD];
 #pragma unroll
-    for (int j = 0; j < NSTAGE - 1; j++)
-        issue_loads<T, A_LD, B_LD>(a_src, b_src, dst_a + j * STAGE, dst_b + j * STAGE, j + 1 < slices ? BK : 0);
-    unsigned stage_off = 0, fill_off = (NSTAGE - 1) * STAGE;
+    for (int i = 0; i < A_LD; i++) {
+        const int row = (wave * A_LD + i) * ROWS_PER_LOAD + lr;
+        a_off[i] = (unsigned) (((long long) (min(m0 + row, p.m - 1) - m0) * p.a_sm + VEC * (pos ^ swz(row))) * (long long) sizeof(T));
+    }
+#pragma unroll
+    for (int i = 0; i < B_LD; i++) {
+        const int row = (wave * B_LD + i) * ROWS_PER_LOAD + lr;
+        b_off[i] = (unsigned) (((long long) (min(n0 + row, p.n - 1) - n0) * p.b_sn + VEC * (pos ^ swz(row))) * (long long) sizeof(T));
+    }
+    char *const dst_a = lds + wave * A_LD * 1024, *const dst_b = lds + A_BYTES + wave * B_LD * 1024;
+    // load l of a slice: the first A_LD fill rows of A, the others rows of B
+    auto issue_load = [&](auto lc, unsigned stage) {
+        constexpr int l = decltype(lc)::value;
+#if defined(__HIP_DEVICE_COMPILE__)
+        if constexpr (l < A_LD) __builtin_amdgcn_global_load_lds((const void *) (a_tile + a_off[l]), dst_a + stage + l * 1024, 16, 0, 0);
+        else __builtin_amdgcn_global_load_lds((const void *) (b_tile + b_off[l - A_LD]), dst_b + stage + (l - A_LD) * 1024, 16, 0, 0);
+#endif
+    };
+    int fetched = 0;  // slices whose loads have been issued
+    auto advance = [&]() {
+        // once no slice is left, the last one is fetched again, into a stage nobody reads any more
+        fetched++;
+        if (fetched < slices) {
+            a_tile += ROW;
+            b_tile += ROW;
+        }
+    };
+#pragma unroll
+    for (int j = 0; j < NSTAGE - 1; j++) {
+        static_for<0, LD>([&](auto lc) { issue_load(lc, (unsigned) (j * STAGE)); });
+        advance();
+    }
+    // operand addresses of the steps within a stage
+    constexpr int STEPS = ROW / 32;
+    unsigned a_rd_t[STEPS], b_rd_t[STEPS];
+#pragma unroll
+    for (int t = 0; t < STEPS; t++) {
+        a_rd_t[t] = a_rd ^ (32 * t);
+        b_rd_t[t] = b_rd ^ (32 * t);
+    }
+    typedef typename std::conditional<sizeof(T) == 2, halfx8, floatx4>::type V;
+    V ra[2][MI], rb[2][NI];
+    wait_for_loads<(NSTAGE - 2) * LD>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    static_for<0, LD>([&](auto lc) { issue_load(lc, (unsigned) ((NSTAGE - 1) * STAGE)); });
+    advance();
+#pragma unroll
+    for (int i = 0; i < MI; i++) ra[0][i] = *(const V *) (lds + a_rd_t[0] + i * 32 * ROW);
+#pragma unroll
+    for (int j = 0; j < NI; j++) rb[0][j] = *(const V *) (lds + b_rd_t[0] + j * 32 * ROW);
+    unsigned stage_off = 0;
+    auto nothing = [](auto) {};
     for (int s = 0; s < slices; s++) {
-        wait_for_loads<(NSTAGE - 2) * (A_LD + B_LD)>();
+        const char *st = lds + stage_off;
+        const unsigned next_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
+        // (STEPS is even: the operand registers alternate, step t multiplies set t % 2 and fills the other)
+        static_for<0, STEPS - 1>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            mfma_step<T, MI, NI, ROW>(acc, ra[t & 1], rb[t & 1], ra[(t + 1) & 1], rb[(t + 1) & 1], st + a_rd_t[t + 1], st + b_rd_t[t + 1], nothing);
+        });
+        // the turn of the ring: the own loads of slice s + 1 have landed, the own reads of slice s are complete
+        wait_for_loads<(NSTAGE - 2) * LD>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        issue_loads<T, A_LD, B_LD>(a_src, b_src, dst_a + fill_off, dst_b + fill_off, s + NSTAGE < slices ? BK : 0);
-        const char *st = lds + stage_off;
-        // All LDS reads of the slice are requested before its first MFMA: with one or two waves per SIMD nobody
-        // else would cover their latency step by step (512 x 12288 x 4096: 72 -> 67 us). The LDS is what bounds
-        // this kernel: it moves about 64 bytes per clock and compute unit, reads and direct loads together, and a
-        // 256 x 128 tile of 8 waves needs 176 KB of that per slice, 2750 clocks against 1024 clocks of MFMA work.
-        // Fewer waves with bigger tiles each (4 waves of 128 x 64) need less LDS traffic but measured slower, with
-        // one wave per SIMD left to cover every wait by itself (133 us against 120 us for 512 x 22016 x 4096).
-        if constexpr (sizeof(T) == 2) {
-            constexpr int STEPS = 4, HOIST = (MI + NI) * STEPS > 16 ? 2 : STEPS;  // (registers permitting)
-#pragma unroll
-            for (int t0 = 0; t0 < STEPS; t0 += HOIST) {
-                halfx8 a[HOIST][MI], b[HOIST][NI];
-#pragma unroll
-                for (int t = 0; t < HOIST; t++) {
-#pragma unroll
-                    for (int i = 0; i < MI; i++) a[t][i] = *(const halfx8 *) (st + (a_rd ^ (32 * (t0 + t))) + i * 32 * ROW);
-#pragma unroll
-                    for (int j = 0; j < NI; j++) b[t][j] = *(const halfx8 *) (st + (b_rd ^ (32 * (t0 + t))) + j * 32 * ROW);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < HOIST; t++)
-#pragma unroll
-                    for (int i = 0; i < MI; i++)
-#pragma unroll
-                        for (int j = 0; j < NI; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t][i], b[t][j], acc[i][j], 0, 0, 0);
-            }
-        } else {
-            // f32: a lane's 16 bytes are 4 consecutive k of its row, which feed 4 steps of v_mfma_f32_32x32x2_f32:
-            // step u of group t multiplies k = 8 t + u (lower half of the wave) and k = 8 t + 4 + u (upper half),
-            // in A and B alike
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                floatx4 a[MI], b[NI];
-#pragma unroll
-                for (int i = 0; i < MI; i++) a[i] = *(const floatx4 *) (st + (a_rd ^ (32 * t)) + i * 32 * ROW);
-#pragma unroll
-                for (int j = 0; j < NI; j++) b[j] = *(const floatx4 *) (st + (b_rd ^ (32 * t)) + j * 32 * ROW);
-#pragma unroll
-                for (int u = 0; u < 4; u++)
-#pragma unroll
-                    for (int i = 0; i < MI; i++)
-#pragma unroll
-                        for (int j = 0; j < NI; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][u], b[j][u], acc[i][j], 0, 0, 0);
-            }
-        }
-        fill_off = stage_off;
-        stage_off = stage_off + STAGE == NSTAGE * STAGE ? 0 : stage_off + STAGE;
+        __builtin_amdgcn_sched_barrier(0);
+        const char *nx = lds + next_off;
+        constexpr int M = MI * NI * (sizeof(T) == 2 ? 1 : 4), PER = (LD + M - 1) / M;
+        mfma_step<T, MI, NI, ROW>(acc, ra[1], rb[1], ra[0], rb[0], nx + a_rd_t[0], nx + b_rd_t[0], [&](auto mc) {
+            constexpr int m = decltype(mc)::value;
+            static_for<0, PER>([&](auto uc) {
+                constexpr int l = m * PER + decltype(uc)::value;
+                if constexpr (l < LD) issue_load(std::integral_constant<int, l>{}, stage_off);
+            });
+        });
+        advance();
+        stage_off = next_off;
     }
     wait_for_loads<0>();
 
