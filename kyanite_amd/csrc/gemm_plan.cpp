@@ -126,14 +126,14 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // pass between workgroups with accesses that bypass the L2 caches, which costs more than the second launch
     // of a plain split; so a launch with less than one round of tiles keeps that (512 x 4096 x 11008: 69 us
     // against 82 us).
-    static const int tail_enabled = env_int("KNHIP_F16_TAIL_SPLIT", 1);
+    static const int tail_enabled = env_int("KNHIP_TAIL_SPLIT", 1);
     if (lp.direct && p.batch == 1 && tail_enabled && split_enabled) {
         const long long slots = 256 * (lp.tall_tile || lp.narrow_tile ? 1 : 2);
         const long long full = blocks / slots * slots, rest = blocks - full;
         long long s = rest > 0 ? slots / rest : 1;
         if (s > p.k / 512) s = p.k / 512;
         if (s > 16) s = 16;
-        if (full > 0 && rest * 100 < slots * env_int("KNHIP_F16_TAIL_BELOW", 85) && s >= 2 && blocks <= 0x3fffffff) {
+        if (full > 0 && rest * 100 < slots * env_int("KNHIP_TAIL_BELOW", 85) && s >= 2 && blocks <= 0x3fffffff) {
             long long chunk = (p.k + s - 1) / s;
             chunk = (chunk + 63) / 64 * 64;
             s = (p.k + chunk - 1) / chunk;

@@ -60,8 +60,8 @@ struct GemmLaunchPlan {
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)
     int k_chunk;             // K elements per split, a multiple of bk
-    // f16 direct kernel, one batch entry: the first `head_tiles` tiles are computed by one workgroup each, every
-    // further tile by `tail_split` workgroups that take `tail_k_chunk` of K each and sum up inside the launch
+    // direct kernel (f16 and f32), one batch entry: the first `head_tiles` tiles are computed by one workgroup each,
+    // every further tile by `tail_split` workgroups that take `tail_k_chunk` of K each and sum up inside the launch
     int head_tiles, tail_split, tail_k_chunk;
     size_t workspace_bytes;  // f32 scratch: split_k * batch * m * n * 4 when split_k > 1; one tile per sharing workgroup
     size_t counter_bytes;    // one int per shared tile
