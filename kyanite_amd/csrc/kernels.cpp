@@ -661,9 +661,14 @@ KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, 
     }
     // phase 1: addresses and loads, all issued before any arithmetic
     ss << "#pragma unroll\n    for (int u = 0; u < UNROLL; u++) {\n";
-    ss << "        const idx_t v = base + (idx_t) (u * 256);\n        ok[u] = v < total;\n";
+    // Vectors past the end are clamped for addressing and only their stores are masked, so that the loads are
+    // straight-line code that the compiler issues back to back (a branch per load makes every load wait for the one
+    // before it); a grid that covers the tensor exactly needs no check at all.
+    const bool exact = total_vecs % (256 * unroll) == 0;
+    if (exact) ss << "        const idx_t v = base + (idx_t) (u * 256);\n        ok[u] = true;\n";
+    else ss << "        const idx_t v_raw = base + (idx_t) (u * 256);\n        ok[u] = v_raw < total;\n        const idx_t v = ok[u] ? v_raw : total - 1;\n";
     ss << "        for (int k = 0; k < " << operands.size() << "; k++) off[u][k] = 0;\n";
-    ss << "        if (ok[u]) {\n";
+    ss << "        {\n";
     {
         std::vector<std::string> offs;
         for (size_t k = 0; k < operands.size(); k++) offs.push_back("off[u][" + std::to_string(k) + "]");
@@ -1027,25 +1032,50 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     // Epilogue operands (gamma, beta, ...) are requested together with the row itself when they fit in registers,
     // so that their latency overlaps with the reductions instead of following them.
     size_t n_post = 0;
-    bool post_row_invariant = true;  // the epilogue operands only vary along the normalised axis
     for (size_t k = 1; k < ops.size(); k++) {
         if (!in_post[k]) continue;
         n_post++;
-        for (size_t a = 0; a < sc.rank(); a++) post_row_invariant &= sc.strides[k][a] == 0;
     }
     bool prefetch_post = cached && n_post > 0 && n_post * items * vec <= 64;
-    // When they are the same for every row, a group of lanes walks over `seq` rows one after another and loads
-    // them once, as long as enough workgroups remain to fill the chip.
-    size_t seq = 1;
-    if (prefetch_post && post_row_invariant) {
-        // measured on [8192, 4096] with gamma / beta: 2 or 4 rows per group are no faster than 1 (49.5 us against
-        // 54.6 / 55.9 us), so this stays off unless asked for
-        static const size_t max_seq = getenv("KNHIP_ROW_SEQ") ? (size_t) atoi(getenv("KNHIP_ROW_SEQ")) : 1;
-        for (size_t c = max_seq; c > 1; c /= 2)
-            if (static_size / (rows_per_block * c) >= 2048) {
-                seq = c;
-                break;
+    // Which of them: the row and the operands requested with it should stay within 32 values per lane, or the
+    // kernel needs more than the 64 registers that full occupancy allows ([8192, 4096] with gamma and beta: 47.1 us
+    // with both held from the start, one wave per SIMD less; 43.2 us with gamma alone, 42.6 us without either).
+    // The others are loaded where the epilogue uses them, after the statistics, into registers that are free by then.
+    std::vector<bool> early(ops.size(), false);
+    if (prefetch_post) {
+        size_t held = items * vec;
+        for (size_t k = 1; k < ops.size(); k++) {
+            if (!in_post[k]) continue;
+            const size_t need = axis_strides[k] == 1 ? items * vec * std::max<size_t>(dtype_bytes(ops[k].dtype), 4) / 4 : items;
+            if (held + need <= 32) {
+                early[k] = true;
+                held += need;
             }
+        }
+    }
+    // Epilogue operands that are the same for every row (gamma, beta) and together as large as the L1 cache: every
+    // row would fetch them from L2 again, and those fetches queue up with the row itself ([8192, 4096]: 42.6 us without
+    // them, 43.0 us with gamma, 47.3 us with gamma and beta). A workgroup then stages them in LDS once and walks over
+    // `seq` rows, as long as enough workgroups remain to fill the chip.
+    std::vector<bool> staged(ops.size(), false);
+    size_t seq = 1, staged_bytes = 0;
+    if (cached && vec > 1) {
+        for (size_t k = 1; k < ops.size(); k++) {
+            if (!in_post[k] || in_pre[k] || axis_strides[k] != 1) continue;
+            bool invariant = true;
+            for (size_t a = 0; a < sc.rank(); a++) invariant &= sc.strides[k][a] == 0;
+            if (invariant) {
+                staged[k] = true;
+                staged_bytes += size * dtype_bytes(ops[k].dtype);
+            }
+        }
+        // (measured with gamma and beta, the loads of the next row requested ahead: 43.4 us with 2 rows per workgroup,
+        // 45.8 us with 4, 49.0 us with 8; 47.3 us with one row and the operands from L2)
+        if (staged_bytes >= 24 * 1024 && staged_bytes <= 40 * 1024 && static_size % (rows_per_block * 2) == 0 &&
+            static_size / (rows_per_block * 2) >= 1024)
+            seq = 2;
+        if (seq == 1) staged.assign(ops.size(), false);
+        else prefetch_post = false;  // (registers that hold operands of the epilogue would be refilled for the next row too early)
     }
     // Rows and vector positions past the end are clamped for addressing and masked afterwards, so that the loads of
     // a row are straight-line code that the compiler can issue back to back (a branch per load would make every
@@ -1063,18 +1093,18 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     };
     // the row statistic of kind Reduce from the folded value `m` (like the post step of the reduce kernel)
     const std::string stat_expr = rowred && rop == ReduceOp::Mean ? "m / (float) " + std::to_string(size) + ".0f" : std::string("m");
-    // Holding the epilogue operands across rows costs a few registers more than the 64 per lane that full
-    // occupancy allows; the compiler is told to stay within them (it has the slack: at most one spill was seen).
-    ss << "extern \"C\" __global__ " << (seq > 1 ? "__attribute__((amdgpu_waves_per_eu(8, 8))) " : "") << "__launch_bounds__("
-       << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
+    ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
     for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
-    if (nw > 1) ss << "    __shared__ float lds_m[" << nw << "], lds_s[" << nw << "], lds_st[" << 2 * nw << "];\n";
+    // (statistics of consecutive rows of a workgroup alternate between two sets of slots: one barrier per exchange)
+    if (nw > 1) ss << "    __shared__ float lds_m[" << nw << "], lds_s[" << nw << "], lds_st[" << 2 * nw * (seq > 1 ? 2 : 1) << "];\n";
+    for (size_t k = 1; k < ops.size(); k++)
+        if (staged[k]) ss << "    __shared__ V" << k << " lds_b" << k << "[" << nv << "];\n";
     ss << "    const idx_t lane = (idx_t) (threadIdx.x % G);\n";
     ss << "    idx_t base[" << ops.size() << "];\n    for (int k = 0; k < " << ops.size() << "; k++) base[k] = 0;\n";
     const std::string row0 = "((idx_t) blockIdx.x * (idx_t) " + std::to_string(rows_per_block) + " + (idx_t) (threadIdx.x / G))";
-    auto emit_row_setup = [&]() {
+    auto emit_row_setup = [&](const std::string &into = "base") {
         std::vector<std::string> offs;
-        for (size_t k = 0; k < ops.size(); k++) offs.push_back("base[" + std::to_string(k) + "]");
+        for (size_t k = 0; k < ops.size(); k++) offs.push_back(into + "[" + std::to_string(k) + "]");
         if (check_row) ss << "    const idx_t rowc = row < (idx_t) " << static_size << " ? row : (idx_t) " << (static_size - 1) << ";\n";
         emit_decompose(ss, "    ", check_row ? "rowc" : "row", sc.shape, sc.strides, offs);
     };
@@ -1090,10 +1120,11 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     };
     // the prologue operands of vector position `i` (in vector units along the axis): loaded into `a<k>`, either
     // declared on the spot or assigned to an element of a register array that was declared earlier (`slot`)
+    std::string pre_base = "base";  // the row offsets that the prologue loads start from
     auto emit_pre_loads = [&](const std::string &indent, const std::string &i, const std::string &slot) {
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_pre[k]) continue;
-            std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
+            std::string o = "(" + pre_base + "[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
             bool v = vec > 1 && axis_strides[k] == 1;
             std::string lhs = slot.empty() ? std::string("const ") + (v ? "V" : "S") + std::to_string(k) + " a" + std::to_string(k)
                                            : "a" + std::to_string(k) + "[" + slot + "]";
@@ -1124,7 +1155,11 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     // assigned to an element of a register array that was declared earlier (`slot`)
     auto emit_post_loads = [&](const std::string &indent, const std::string &i, const std::string &slot) {
         for (size_t k = 1; k < ops.size(); k++) {
-            if (!in_post[k]) continue;
+            if (!in_post[k] || (prefetch_post && early[k] == slot.empty())) continue;
+            if (staged[k]) {
+                ss << indent << "const V" << k << " b" << k << " = lds_b" << k << "[" << i << "];\n";
+                continue;
+            }
             std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
             bool v = vec > 1 && axis_strides[k] == 1;
             std::string lhs = slot.empty() ? std::string("const ") + (v ? "V" : "S") + std::to_string(k) + " b" + std::to_string(k)
@@ -1134,14 +1169,14 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         }
     };
     auto emit_post_store = [&](const std::string &indent, const std::string &i, const std::string &src, const std::string &slot) {
-        if (slot.empty()) emit_post_loads(indent, i, "");
+        emit_post_loads(indent, i, "");  // (those not requested ahead)
         const std::string pick = slot.empty() ? std::string() : "[" + slot + "]";
         std::string o0 = "(base[0] + " + i + " * (idx_t) " + i64_str(axis_strides[0] * (int64_t) vec) + ")";
         auto call = [&](const std::string &j) {
             std::string c = row_dtype == DType::F16 ? "kn_post(kn_r16(" + src + "[" + j + "])" : "kn_post(" + src + "[" + j + "]";
             for (size_t k = 1; k < ops.size(); k++) {
                 if (!in_post[k]) continue;
-                std::string e = "b" + std::to_string(k) + pick + ((vec > 1 && axis_strides[k] == 1) ? "[" + j + "]" : "");
+                std::string e = "b" + std::to_string(k) + (early[k] ? pick : std::string()) + ((vec > 1 && axis_strides[k] == 1) ? "[" + j + "]" : "");
                 c += ", " + from_storage(ops[k].dtype, e);
             }
             return to_storage(ops[0].dtype, c + ")");
@@ -1162,23 +1197,37 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         for (size_t k = 1; k < ops.size(); k++) {
             const char *t = (vec > 1 && axis_strides[k] == 1) ? "V" : "S";
             if (in_pre[k]) ss << "    " << t << k << " a" << k << "[ITEMS];\n";
-            if (in_post[k] && prefetch_post) ss << "    " << t << k << " b" << k << "[ITEMS];\n";
+            if (in_post[k] && prefetch_post && early[k]) ss << "    " << t << k << " b" << k << "[ITEMS];\n";
         }
-        if (seq > 1) {
-            // the epilogue operands once, then the rows of this group one after another
+        auto emit_row_loads = [&]() {
+            // every load of the row first, then the arithmetic
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n" << item_index;
-            emit_post_loads("        ", "ic", "it");
+            emit_pre_loads("        ", "ic", "it");
+            if (prefetch_post) emit_post_loads("        ", "ic", "it");
             ss << "    }\n";
+        };
+        const std::string seq_row = "(" + row0 + " / (idx_t) " + std::to_string(rows_per_block) + ") * (idx_t) " +
+                                    std::to_string(rows_per_block * seq) + " + (idx_t) (threadIdx.x / G)";
+        if (seq > 1) {
+            // the rows of this group one after another; the loads of row r + 1 are requested as soon as row r has
+            // left the registers they arrive in, i.e. before its statistics
+            for (size_t k = 1; k < ops.size(); k++)
+                if (staged[k])
+                    ss << "    for (idx_t i = (idx_t) threadIdx.x; i < (idx_t) " << nv << "; i += (idx_t) " << block << ") lds_b" << k
+                       << "[i] = *(const V" << k << " *) (p" << k << " + i * (idx_t) " << vec << ");\n";
+            ss << "    idx_t nbase[" << ops.size() << "];\n    for (int k = 0; k < " << ops.size() << "; k++) nbase[k] = 0;\n";
+            ss << "    {\n    const idx_t row = " << seq_row << ";\n";
+            emit_row_setup("nbase");
+            ss << "    }\n";
+            pre_base = "nbase";
+            emit_row_loads();
+            ss << "    __syncthreads();\n";
             ss << "    for (int rs = 0; rs < " << seq << "; rs++) {\n";
-            ss << "    const idx_t row = " << row0 << " * (idx_t) " << seq << " + (idx_t) rs;\n";
-            ss << "    for (int k = 0; k < " << ops.size() << "; k++) base[k] = 0;\n";
-            emit_row_setup();
+            ss << "    const idx_t row = " << seq_row << " + (idx_t) rs * (idx_t) " << rows_per_block << ";\n";
+            ss << "    for (int k = 0; k < " << ops.size() << "; k++) base[k] = nbase[k];\n";
+        } else {
+            emit_row_loads();
         }
-        // every load of the row first, then the arithmetic
-        ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n" << item_index;
-        emit_pre_loads("        ", "ic", "it");
-        if (prefetch_post && seq == 1) emit_post_loads("        ", "ic", "it");
-        ss << "    }\n";
         ss << "    float x[ITEMS][VEC];\n";
         ss << "    float m = " << identity << ";\n";
         ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
@@ -1187,6 +1236,14 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "        if (!(i < (idx_t) " << nv << ")) for (int j = 0; j < VEC; j++) x[it][j] = " << identity << ";\n";
         emit_fold("        ", "x[it]");
         ss << "    }\n";
+        if (seq > 1) {
+            ss << "    if (rs + 1 < " << seq << ") {\n    const idx_t row = " << seq_row << " + (idx_t) (rs + 1) * (idx_t) " << rows_per_block << ";\n";
+            ss << "    for (int k = 0; k < " << ops.size() << "; k++) nbase[k] = 0;\n";
+            emit_row_setup("nbase");
+            emit_row_loads();
+            ss << "    }\n";
+            pre_base = "base";
+        }
         // layernorm with the same number of elements in every lane: per-lane mean and centred sum of squares,
         // combined pairwise in a single pass over the lanes instead of one pass for the mean and one for the
         // variance (one barrier instead of two when a row spans several waves)
@@ -1208,7 +1265,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "    float mean = m / (float) " << cnt << ".0f;\n";
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n";
             ss << "        for (int j = 0; j < VEC; j++) {\n            const float d = x[it][j] - mean;\n            s += d * d;\n        }\n    }\n";
-            if (nw > 1) ss << "    kn_block_stats<" << nw << ">(mean, s, (float) " << cnt << ".0f, lds_st);\n";
+            if (nw > 1) ss << "    kn_block_stats<" << nw << ">(mean, s, (float) " << cnt << ".0f, lds_st" << (seq > 1 ? " + (rs & 1) * " + std::to_string(2 * nw) : std::string()) << ");\n";
             else ss << "    kn_group_stats<G>(mean, s, (float) " << cnt << ".0f);\n";
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] - mean;\n    }\n";
         } else {
@@ -1229,7 +1286,10 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         if (check_row) guard += (guard.empty() ? "" : " && ") + valid;
         ss << "        " << (guard.empty() ? std::string() : "if (" + guard + ") ") << "{\n";
         emit_post_store("            ", "i", "x[it]", prefetch_post ? "it" : "");
-        ss << "        }\n    }\n" << (seq > 1 ? "    }\n" : "") << "}\n";
+        ss << "        }\n    }\n";
+        // (the slots of the other reductions are reused by the next row: everybody has to be done reading them)
+        if (seq > 1) ss << (nw > 1 && !one_pass ? "    __syncthreads();\n" : "") << "    }\n";
+        ss << "}\n";
     } else {
         // rows too long for registers: stream the row three times (the re-reads come from cache)
         ss << "    float t[VEC];\n";

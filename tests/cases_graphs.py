@@ -1005,6 +1005,17 @@ def config_bandwidth_softmax_small():
 
 
 @case
+def layernorm_affine_rows_share_staged_operands():
+    """enough rows of 4096 that a workgroup stages gamma / beta in LDS and walks over two rows, the loads of the
+    second one requested before the statistics of the first"""
+    from kyanite_amd import HipExecutor
+    from kyanite_amd.configs import build_layernorm
+    g, inputs, _ = build_layernorm(seed=14, shape=(2048, 4096))
+    assert "rows=2" in HipExecutor(0, g, 0, plan_only=True).step_str(0)
+    return g, 0, inputs(), None
+
+
+@case
 def config_bandwidth_layernorm_small():
     """configs[1] (c): rows of 4096 with the fused gamma / beta epilogue"""
     from kyanite_amd.configs import build_layernorm
