@@ -225,9 +225,12 @@ typedef struct knhip_executor knhip_executor;
 /* CudaExecutor::new(device, &graph, batch_size) (executor.rs:61); `flags` is 0 for the reference's behaviour.
  * KNHIP_PLAN_ONLY: nothing touches a device, the graph is planned and its kernels are compiled (works on a machine
  * without a GPU). KNHIP_PRESERVE_INPUTS: input buffers are never reused for later values, for callers that write
- * the inputs on the device once and then call run_async many times (the reference re-uploads them per evaluate). */
+ * the inputs on the device once and then call run_async many times (the reference re-uploads them per evaluate).
+ * KNHIP_STEP_BY_STEP: every run launches the planned steps one by one, also where the whole plan is small enough to
+ * run as one kernel (knhip_executor_fused_source). */
 #define KNHIP_PLAN_ONLY 1
 #define KNHIP_PRESERVE_INPUTS 2
+#define KNHIP_STEP_BY_STEP 4
 int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int flags, knhip_executor **out);
 int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int flags,
                                  knhip_executor **out);
@@ -287,6 +290,10 @@ int knhip_executor_step_str(const knhip_executor *ex, size_t index, char *buf, s
  * flops = 2 * multiply-adds of a conv / mat_mul step (0 for the others), bytes = every distinct operand element once */
 int knhip_executor_step_work(const knhip_executor *ex, size_t index, double *flops, double *bytes);
 int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf, size_t cap, size_t *needed);
+/* No counterpart in the reference. A plan of a few tiny steps (each small enough for a single workgroup) is also
+ * compiled into ONE kernel that runs the steps in launch order; run_async and evaluate launch it instead of the steps
+ * unless the run is profiled. The source of that kernel, or an empty string when the plan is launched step by step. */
+int knhip_executor_fused_source(const knhip_executor *ex, char *buf, size_t cap, size_t *needed);
 int knhip_executor_str(const knhip_executor *ex, char *buf, size_t cap, size_t *needed);
 
 /* Layout algebra hooks for tests (kn-cuda-eval/src/shape.rs:25-285). Strides are in elements.

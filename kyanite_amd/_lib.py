@@ -150,6 +150,7 @@ SIGNATURES = {
     "knhip_executor_set_graph_mode": [E, c_int],
     "knhip_executor_step_work": [E, c_size_t, POINTER(c_double), POINTER(c_double)],
     "knhip_executor_step_source": [E, c_size_t, c_char_p, c_size_t, PZ],
+    "knhip_executor_fused_source": [E, c_char_p, c_size_t, PZ],
     "knhip_executor_str": [E, c_char_p, c_size_t, PZ],
     "knhip_strided_flags": [PZ, POINTER(c_int64), c_size_t, POINTER(c_int), POINTER(c_int)],
     "knhip_strided_view": [PZ, POINTER(c_int64), c_size_t, PZ, c_size_t, POINTER(c_int), POINTER(c_int64)],

@@ -17,7 +17,7 @@ struct knhip_graph {
 struct knhip_executor {
     HipExecutor ex;
     knhip_executor(int device, const Graph &g, size_t batch, int flags)
-        : ex(device, g, batch, (flags & KNHIP_PLAN_ONLY) != 0, (flags & KNHIP_PRESERVE_INPUTS) != 0) {}
+        : ex(device, g, batch, (flags & KNHIP_PLAN_ONLY) != 0, (flags & KNHIP_PRESERVE_INPUTS) != 0, (flags & KNHIP_STEP_BY_STEP) == 0) {}
 };
 
 namespace {
@@ -885,6 +885,13 @@ int knhip_executor_step_source(const knhip_executor *ex, size_t index, char *buf
     return guarded([&] {
         KN_REQUIRE(ex != nullptr);
         return copy_out(ex->ex.plan().steps.at(index).kernel.source, buf, cap, needed);
+    });
+}
+
+int knhip_executor_fused_source(const knhip_executor *ex, char *buf, size_t cap, size_t *needed) {
+    return guarded([&] {
+        KN_REQUIRE(ex != nullptr);
+        return copy_out(ex->ex.fused_source(), buf, cap, needed);
     });
 }
 

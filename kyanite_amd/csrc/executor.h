@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include "fused_graph.h"
 #include "planner.h"
 
 namespace kn {
@@ -29,7 +30,9 @@ public:
     // `plan_only` builds and compiles the plan without touching a device (no allocation, no launches)
     // `preserve_inputs` keeps the input buffers from being reused for later values, for callers that write the
     // inputs on the device once and then call run_async many times
-    HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only = false, bool preserve_inputs = false);
+    // `fuse_small`: a plan of a few tiny steps is launched as one kernel (fused_graph.h)
+    HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only = false, bool preserve_inputs = false,
+                bool fuse_small = true);
     ~HipExecutor();
     HipExecutor(const HipExecutor &) = delete;
     HipExecutor &operator=(const HipExecutor &) = delete;
@@ -59,13 +62,22 @@ public:
     void *input_ptr(size_t i) const;
     void *output_ptr(size_t i) const;
     std::string str() const;
+    // whether the whole plan runs as one generated kernel, and that kernel's source
+    bool fused() const { return fused_spec_.has_value(); }
+    const std::string &fused_source() const;
 
 private:
+    // the launch arguments of one step with every operand at its final address
     struct Launch {
         hipFunction_t function = nullptr;
         std::vector<void *> ptrs;
+        GemmLaunchPlan gemm_plan{};
+        AttentionParams attn{};
+        ConvParams conv{};
     };
-    void launch_step(size_t index, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
+    // `mapped`: the variant of the launch whose inputs and outputs are the page-locked host buffers themselves
+    void launch_step(size_t index, hipEvent_t start = nullptr, hipEvent_t stop = nullptr, bool mapped = false);
+    void realise_launch(size_t index, Launch &l, bool mapped);
 
     int device_;
     size_t batch_size_;
@@ -75,6 +87,20 @@ private:
     hipStream_t stream_ = nullptr;
     std::vector<hipModule_t> modules_;
     std::vector<Launch> launches_;
+    // Small graphs (inputs and outputs of a few KB): `evaluate` runs the steps on launches whose input / output
+    // operands point at the page-locked staging buffers, which the device reads and writes across the bus, so an
+    // evaluation is the launches and one synchronisation, without copy commands in between.
+    std::vector<Launch> mapped_launches_;
+    bool mapped_io_ = false;
+    // A plan of a few tiny steps as ONE generated kernel, one workgroup (fused_graph.h); runs that are not profiled
+    // launch it instead of the steps.
+    std::optional<KernelSpec> fused_spec_;
+    std::shared_ptr<const CodeObject> fused_code_;
+    hipFunction_t fused_function_ = nullptr;
+    std::vector<void *> fused_ptrs_, fused_mapped_ptrs_;
+    uint32_t *fused_done_ = nullptr;  // page-locked word that the fused kernel writes the number of its launch into
+    uint32_t fused_seq_ = 0;
+    void launch_fused(bool mapped);
     std::vector<void *> pinned_inputs_, pinned_outputs_;
     std::vector<HostTensor> tensor_outputs_;
     bool profile_ = false;

@@ -35,7 +35,6 @@ struct Step {
     std::shared_ptr<const CodeObject> code;
     // matrix-core kernels; the pointers are filled in when the plan is realised
     GemmParams gemm{};
-    GemmLaunchPlan gemm_plan{};  // filled in by the executor once the operands have their addresses
     bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
     bool gemm_has_addend = false;  // operand 3 is the tensor added in the epilogue
     bool gemm_has_addend2 = false;  // operand 4 is a second one, added after the first

@@ -54,10 +54,10 @@ class Profile:
 class HipExecutor:
     """`HipExecutor(device, graph, batch_size)` / `evaluate(inputs) -> outputs`."""
 
-    def __init__(self, device, graph, batch_size, plan_only=False, preserve_inputs=False):
+    def __init__(self, device, graph, batch_size, plan_only=False, preserve_inputs=False, step_by_step=False):
         index = device.index if isinstance(device, HipDevice) else int(device)
         h = c_void_p()
-        flags = (1 if plan_only else 0) | (2 if preserve_inputs else 0)
+        flags = (1 if plan_only else 0) | (2 if preserve_inputs else 0) | (4 if step_by_step else 0)
         check(lib.knhip_executor_new(index, graph._h, batch_size, flags, byref(h)))
         self._h = h
         self.device = index
@@ -196,6 +196,10 @@ class HipExecutor:
 
     def step_source(self, i):
         return get_string(lib.knhip_executor_step_source, self._h, i)
+
+    def fused_source(self):
+        """Source of the one kernel that runs the whole plan, "" when the plan is launched step by step."""
+        return get_string(lib.knhip_executor_fused_source, self._h)
 
     def __str__(self):
         return get_string(lib.knhip_executor_str, self._h)

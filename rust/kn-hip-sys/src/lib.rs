@@ -64,6 +64,7 @@ pub const KNHIP_BUFFER_TOO_SMALL: c_int = 2;
 
 pub const KNHIP_PLAN_ONLY: c_int = 1;
 pub const KNHIP_PRESERVE_INPUTS: c_int = 2;
+pub const KNHIP_STEP_BY_STEP: c_int = 4;
 
 pub const KNHIP_F32: c_int = 0;
 pub const KNHIP_F64: c_int = 1;
@@ -141,6 +142,7 @@ extern "C" {
     pub fn knhip_executor_step_kind(ex: *const knhip_executor, index: usize, kind: *mut c_int) -> c_int;
     pub fn knhip_executor_step_str(ex: *const knhip_executor, index: usize, buf: *mut c_char, cap: usize, needed: *mut usize) -> c_int;
     pub fn knhip_executor_step_work(ex: *const knhip_executor, index: usize, flops: *mut f64, bytes: *mut f64) -> c_int;
+    pub fn knhip_executor_fused_source(ex: *const knhip_executor, buf: *mut c_char, cap: usize, needed: *mut usize) -> c_int;
     pub fn knhip_executor_str(ex: *const knhip_executor, buf: *mut c_char, cap: usize, needed: *mut usize) -> c_int;
 
     pub fn knhip_compile_stats(compiled: *mut usize, memory_hits: *mut usize, disk_hits: *mut usize) -> c_int;

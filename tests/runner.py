@@ -94,15 +94,21 @@ def check_gpu(device, graph, batch_size, inputs, expected=None, what=""):
     reference = expected if expected is not None else cpu_outputs
     results = []
     for name, g in (("unoptimized", graph), ("optimized", optimize_graph(graph))):
-        ex = HipExecutor(device, g, batch_size)
-        gpu_outputs = ex.evaluate(inputs)
-        assert_tensors_match(reference, gpu_outputs, f"gpu, {name}")
         cpu_same_graph = cpu_outputs if name == "unoptimized" else cpu_eval_graph(g, batch_size, inputs)
-        check_outputs(g, batch_size, inputs, cpu_same_graph, gpu_outputs, f"{what} {name}".strip(), PARITY_RECORDS)
-        # a second evaluation must give the same answer (buffers are reused between calls)
-        again = ex.evaluate(inputs)
-        for x, y in zip(gpu_outputs, again):
-            assert np.array_equal(x, y, equal_nan=True), f"gpu, {name}: second evaluation differs"
+        ex = HipExecutor(device, g, batch_size)
+        # a plan of a few tiny steps runs as ONE kernel: then the steps are checked launched one by one as well, and
+        # so is the path of callers that write the inputs on the device themselves (run_async on arena addresses)
+        executors = [(name, ex)]
+        if ex.fused_source():
+            executors.append((name + ", step by step", HipExecutor(device, g, batch_size, step_by_step=True)))
+        for label, e in executors:
+            gpu_outputs = e.evaluate(inputs)
+            assert_tensors_match(reference, gpu_outputs, f"gpu, {label}")
+            check_outputs(g, batch_size, inputs, cpu_same_graph, gpu_outputs, f"{what} {label}".strip(), PARITY_RECORDS)
+            # a second evaluation must give the same answer (buffers are reused between calls)
+            again = e.evaluate(inputs)
+            for x, y in zip(gpu_outputs, again):
+                assert np.array_equal(x, y, equal_nan=True), f"gpu, {label}: second evaluation differs"
         results.append(gpu_outputs)
     return results[0]
 

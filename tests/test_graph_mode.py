@@ -38,8 +38,10 @@ def small_tower():
 @pytest.mark.parametrize("build", [tiny_mlp, att_tiny, small_tower])
 def test_graph_replay_matches_eager(build, hip_device):
     graph, batch, inputs = build()
-    eager = HipExecutor(hip_device, graph, batch)
-    replay = HipExecutor(hip_device, graph, batch)
+    # (both launch the planned steps: a plan as small as the MLP's would otherwise run as one fused kernel, whose plain
+    # dot products round differently from the matrix-core kernels of the replayed launch list)
+    eager = HipExecutor(hip_device, graph, batch, step_by_step=True)
+    replay = HipExecutor(hip_device, graph, batch, step_by_step=True)
     replay.set_graph_mode(True)
     for round_ in range(5):
         # new inputs every round: a replay that re-used stale results would show
