@@ -90,6 +90,7 @@ struct PlannerOptions {
     bool fuse_attention = true;  // matmul, softmax, matmul chains in f32 run as one launch
     bool pack_matmul_constants = true;  // constant [k, n] right operands of f16 matmuls are laid out again as [n, k]
     bool group_matmuls = true;   // matmuls that share their left operand and have constant right operands share a launch
+    bool pointwise_conv_as_matmul = true;  // 1 x 1 convolutions with stride 1 run as one matrix product per image
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
 };
