@@ -95,6 +95,9 @@ def per_step_seconds(ex, iters):
     import numpy as np
     ex.set_profile(True)
     per_step = np.zeros(ex.step_count())
+    # (one untimed pass first: a small plan runs as one fused kernel otherwise, so this may be the first launch of its
+    # step kernels, which loads their code)
+    ex.run_async()
     for _ in range(iters):
         ex.run_async()
         per_step += np.asarray(ex.last_profile().step_seconds)

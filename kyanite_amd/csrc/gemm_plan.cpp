@@ -44,8 +44,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // 534 us on 64 x 64 tiles against 597 us, 512 tiles 734 us against 662 us; f16 344 tiles 112 us against 85 us,
     // 128 tiles 47 us against 56 us. An output no wider than 64 would leave most of a 128 wide tile unused
     // (16 x [4096 x 4096] x [4096 x 40] in f32: 450 us on 64 x 64 tiles against 682 us).
-    static const int threshold_env = env_int("KNHIP_SMALL_TILE_BELOW", -1);
-    const long long threshold = threshold_env >= 0 ? threshold_env : (f16 ? 256 : 512);
+    const long long threshold = f16 ? 256 : 512;
     static const int split_enabled = env_int("KNHIP_SPLIT_K", 1);
     const int groups = p.groups > 1 ? p.groups : 1;
     const long long big_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch * groups;
@@ -62,7 +61,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // fewer bytes from L2 per flop and halve the partial products per split. Measured (us, 128 x 128 against
     // 256 x 128): 512 x 4096 x 4096 43 / 38, 512 x 4096 x 11008 89 / 75; without a split they do not pay:
     // 512 x 11008 x 4096 82 / 87, 8192^3 1454 / 1439.
-    static const int tall_below = env_int("KNHIP_F16_TALL_BELOW", 128);
+    constexpr int tall_below = 128;
     const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch * groups;
     const bool tall_fits = !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8;
     lp.tall_tile = f16 && groups == 1 && tall_fits && can_split && p.k >= 2048 && tall_blocks < tall_below;
@@ -78,13 +77,13 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     lp.direct = p.k > 0 && p.k % (8 * vec) == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % vec == 0 && p.b_sn % vec == 0 &&
                 p.a_sm > 0 && p.b_sn > 0 && p.a_sm < max_row_stride && p.b_sn < max_row_stride &&
                 (p.batch <= 1 || (p.a_sb % vec == 0 && p.b_sb % vec == 0));
-    if (f16 && lp.direct && tall_fits && tall_blocks >= env_int("KNHIP_F16_TALL_FROM", 128)) lp.tall_tile = true;
+    if (f16 && lp.direct && tall_fits && tall_blocks >= 128) lp.tall_tile = true;
     // Direct kernel only: 128 x 64 tiles on a ring of four stages, where 128 x 128 tiles leave compute units
     // without a workgroup and K is too short for a split to pay (512 x 4096 x 4096: 29 us against 39 us on
     // 256 x 128 tiles split in four; 512 x 4096 x 11008: 84 us against 69 us).
     const long long narrow_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 63) / 64) * p.batch * groups;
-    lp.narrow_tile = f16 && lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= env_int("KNHIP_F16_NARROW_FROM", 192) &&
-                     p.k < env_int("KNHIP_F16_NARROW_K_BELOW", 8192);
+    lp.narrow_tile = f16 && lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= 192 &&
+                     p.k < 8192;
     if (lp.narrow_tile) lp.small_tile = lp.tall_tile = false;
     // Direct kernel only: 256 x 256 tiles (8 waves of 128 x 64) where they still give every compute unit a
     // workgroup. The LDS bounds this kernel, and they need the least LDS traffic per flop: 256 KB per slice of 64
@@ -105,10 +104,9 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         auto fits = [&](int width) { return p.n >= width && (p.n + width - 1) / width * width - p.n <= p.n / 8; };
         const double t_tall = lds_time(tall_blocks, 2750.0);
         const double t_mid = fits(192) ? lds_time(mid_blocks, 3375.0) : 1e30;
-        const double t_wide = fits(256) && wide_blocks >= env_int("KNHIP_F16_WIDE_FROM", 256) ? lds_time(wide_blocks, 4000.0) : 1e30;
-        static const int mid_enabled = env_int("KNHIP_F16_MID_TILE", 1);
-        lp.wide_tile = t_wide <= t_tall && t_wide <= t_mid;
-        lp.mid_tile = !lp.wide_tile && mid_enabled && t_mid < t_tall;
+        const double t_wide = fits(256) && wide_blocks >= 256 ? lds_time(wide_blocks, 4000.0) : 1e30;
+                lp.wide_tile = t_wide <= t_tall && t_wide <= t_mid;
+        lp.mid_tile = !lp.wide_tile && t_mid < t_tall;
     }
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
@@ -117,7 +115,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     if (lp.mid_tile) blocks = mid_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile || lp.narrow_tile ? 64 : 128;
     else if (lp.direct) lp.bk = 32;
-    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= env_int("KNHIP_BK64_FROM", 256) && small_blocks < env_int("KNHIP_BK64_BLOCKS", 512))) ? 64 : 16;
+    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= 256 && small_blocks < 512)) ? 64 : 16;
 
     // A tile count that leaves the last round of workgroups mostly idle: the direct kernel splits the tiles of just
     // that round along K and sums the parts inside the launch, so that the round is short instead of sparse.
@@ -133,7 +131,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         long long s = rest > 0 ? slots / rest : 1;
         if (s > p.k / 512) s = p.k / 512;
         if (s > 16) s = 16;
-        if (full > 0 && rest * 100 < slots * env_int("KNHIP_TAIL_BELOW", 85) && s >= 2 && blocks <= 0x3fffffff) {
+        if (full > 0 && rest * 100 < slots * 85 && s >= 2 && blocks <= 0x3fffffff) {
             long long chunk = (p.k + s - 1) / s;
             chunk = (chunk + 63) / 64 * 64;
             s = (p.k + chunk - 1) / chunk;

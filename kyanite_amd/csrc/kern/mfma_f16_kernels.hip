@@ -678,8 +678,7 @@ int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     // Measured on 128 x 128 tiles of the kernel that stages through registers (TFLOP/s at 4096^3 / 8192^3): BK 64
     // single buffered 594 / 757, BK 64 double buffered 643 / 718, BK 128 single buffered 672 / 744.
     // workgroups an XCD (32 compute units) runs at a time: 1 per compute unit for the tall tiles, else 2
-    static const int xc_env = getenv("KNHIP_XCD_CHUNK") ? atoi(getenv("KNHIP_XCD_CHUNK")) : -1;
-    const int xc = xc_env >= 0 ? xc_env : (lp.tall_tile || narrow ? 32 : 64);  // (also for the 256 x 256 tiles)
+    const int xc = lp.tall_tile || narrow ? 32 : 64;  // (also for the 256 x 256 tiles)
     if (direct) {
         DirectSchedule sched{lp.k_chunk, xc, (int) tiles, 1, p.k};
         if (lp.tail_split > 1) {

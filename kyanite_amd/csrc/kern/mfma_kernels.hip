@@ -766,13 +766,11 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     // 512 102 / 108, 768 176 / 156, 1024 189 / 206; 320 -> 320 on 2 x 64 x 64 228 / 183; 1280 -> 1280 on
     // 2 x 16 x 16 818 / 291. (128 x 64 tiles never won against both.)
     PlaneGeom geom;
-    static const int variant_env = getenv("KNHIP_CONV_PLANE_VARIANT") ? atoi(getenv("KNHIP_CONV_PLANE_VARIANT")) : 0;
     struct Variant { int bm, tn, id; double unit_cost; };
     static const Variant variants[2] = {{128, 128, 22, 4 * 1.00}, {64, 64, 11, 1 * 1.10}};
     const Variant *best = nullptr;
     double best_cost = 0.0;
     for (const Variant &v : variants) {
-        if (variant_env && variant_env != v.id) continue;
         if (!plane_geometry(p, v.tn, &geom)) continue;
         const long long tiles = ((positions + v.tn - 1) / v.tn) * ((p.out_c + v.bm - 1) / v.bm);
         const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost;

@@ -947,7 +947,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     size_t static_size = concrete_size(static_shape);
     if (static_size == 0 || size == 0) return spec;
     // the normalised value is x * (1 / denom) instead of x / denom: one division per row, at most one ulp apart
-    static const bool use_rcp = !(getenv("KNHIP_ROW_RCP") && !atoi(getenv("KNHIP_ROW_RCP")));
+    constexpr bool use_rcp = true;
 
     Collapsed sc = collapse_axes(static_shape, static_strides, true);
 
@@ -975,8 +975,8 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     size_t G = 1024;
     for (size_t g : {1, 4, 16, 64, 256, 1024}) {
         size_t per_lane = (nv + g - 1) / g;
-        static const size_t wave_items = getenv("KNHIP_ROW_WAVE_ITEMS") ? (size_t) atoi(getenv("KNHIP_ROW_WAVE_ITEMS")) : 4;
-        static const size_t block_items = getenv("KNHIP_ROW_BLOCK_ITEMS") ? (size_t) atoi(getenv("KNHIP_ROW_BLOCK_ITEMS")) : 8;
+        constexpr size_t wave_items = 4;
+        constexpr size_t block_items = 8;
         size_t limit = g == 1024 ? MAX_ITEMS : g == 256 ? block_items : g == 64 ? wave_items : g == 1 ? 2 : 4;
         if (per_lane <= limit) {
             G = g;
@@ -985,7 +985,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     }
     size_t items = (nv + G - 1) / G;
     bool cached = items <= MAX_ITEMS;
-    static const size_t min_block = getenv("KNHIP_ROW_MIN_BLOCK") ? (size_t) atoi(getenv("KNHIP_ROW_MIN_BLOCK")) : 256;
+    constexpr size_t min_block = 256;  // (rows that span several waves get a workgroup each: G is 256 or 1024 then)
     size_t block = std::max<size_t>(G, min_block);
     size_t rows_per_block = block / G;
     size_t nw = G / 64;  // waves per row when a row spans several waves
@@ -1247,8 +1247,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         // layernorm with the same number of elements in every lane: per-lane mean and centred sum of squares,
         // combined pairwise in a single pass over the lanes instead of one pass for the mean and one for the
         // variance (one barrier instead of two when a row spans several waves)
-        static const bool one_pass_env = !(getenv("KNHIP_ROW_ONE_PASS") && !atoi(getenv("KNHIP_ROW_ONE_PASS")));
-        const bool one_pass = !softmax && !rowred && !check_i && G > 1 && one_pass_env;
+        const bool one_pass = !softmax && !rowred && !check_i && G > 1;
         if (!one_pass) reduce("m", fold_fn);
         if (!rowred) ss << "    float s = 0.0f;\n";
         if (rowred) {
