@@ -70,6 +70,11 @@ int knhip_memcpy_d2d(int device, void *dst, const void *src, size_t bytes);
 int knhip_host_alloc(size_t bytes, void **ptr);
 int knhip_host_free(void *ptr);
 int knhip_device_synchronize(int device);
+/* No counterpart in the reference. What the matrix cores of the device sustain when nothing else limits them: a
+ * register-only loop of independent f16 MFMAs on one wave per SIMD, with small integers (normal_data = 0) or N(0, 1)
+ * values (normal_data = 1) in the operands, and the shader clock it ran at. The rate on N(0, 1) data is the ceiling
+ * that matmul / convolution rates on real data should be read against (the clock drops under the power they draw). */
+int knhip_device_mfma_probe(int device, int normal_data, int iterations, double *tflops, double *shader_mhz);
 
 /* streams and events (replaces CudaStream, kn-cuda-sys/src/wrapper/handle.rs:105-174, and CudaEvent, event.rs:7-45).
  * Handles are the HIP objects themselves (hipStream_t / hipEvent_t behind void *); a NULL stream is the device's

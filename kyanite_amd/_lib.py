@@ -67,6 +67,7 @@ SIGNATURES = {
     "knhip_host_alloc": [c_size_t, POINTER(c_void_p)],
     "knhip_host_free": [c_void_p],
     "knhip_device_synchronize": [c_int],
+    "knhip_device_mfma_probe": [c_int, c_int, c_int, POINTER(c_double), POINTER(c_double)],
     "knhip_stream_create": [c_int, POINTER(c_void_p)],
     "knhip_stream_destroy": [c_int, c_void_p],
     "knhip_stream_synchronize": [c_int, c_void_p],

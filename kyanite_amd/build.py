@@ -19,7 +19,7 @@ HOST_SOURCES = [
     "kernels.cpp", "fused_graph.cpp", "rtc.cpp", "gemm_plan.cpp", "planner.cpp", "executor.cpp", "capi.cpp",
 ]
 DEVICE_SOURCES = ["kern/mfma_kernels.hip", "kern/mfma_f16_kernels.hip", "kern/attention_kernels.hip", "kern/attention_f16_kernels.hip",
-                  "kern/static_scratch.hip"]
+                  "kern/static_scratch.hip", "kern/probe_kernels.hip"]
 
 COMMON_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-D__HIP_PLATFORM_AMD__",
                 f"-I{ROCM}/include"]

@@ -95,6 +95,7 @@ extern "C" {
     pub fn knhip_host_alloc(bytes: usize, ptr: *mut *mut c_void) -> c_int;
     pub fn knhip_host_free(ptr: *mut c_void) -> c_int;
     pub fn knhip_device_synchronize(device: c_int) -> c_int;
+    pub fn knhip_device_mfma_probe(device: c_int, normal_data: c_int, iterations: c_int, tflops: *mut f64, shader_mhz: *mut f64) -> c_int;
 
     // streams, events, asynchronous copies
     pub fn knhip_stream_create(device: c_int, stream: *mut *mut c_void) -> c_int;

@@ -111,3 +111,15 @@ def test_batched_mat_mul(case, hip_device):
     if need:
         with pytest.raises(KnError, match="workspace"):
             batched_mat_mul(hip_device, stream, args, None)
+
+
+@pytest.mark.gpu
+def test_mfma_probe_reports_a_plausible_ceiling(hip_device):
+    """the register-only MFMA loop: normally distributed operands cannot be faster than small integers by more than
+    noise, and both sit between a fifth of the published f16 peak and the peak itself"""
+    from kyanite_amd.device_probe import mfma_probe
+    ints, ints_mhz = mfma_probe(hip_device.index, normal_data=False, iterations=20000)
+    normal, normal_mhz = mfma_probe(hip_device.index, normal_data=True, iterations=20000)
+    print(f"mfma probe: {ints:.0f} TFLOP/s at {ints_mhz:.0f} MHz (integers), {normal:.0f} at {normal_mhz:.0f} MHz (normal)", flush=True)
+    assert 500.0 < normal <= ints * 1.05 and ints < 2600.0
+    assert 500.0 < normal_mhz < 3000.0 and 500.0 < ints_mhz < 3000.0
