@@ -45,6 +45,23 @@ std::string Profile::str() const {
     return ss.str();
 }
 
+namespace {
+
+// A code object from the disk cache that the runtime refuses to load is dropped and built again, once.
+hipModule_t load_code_object(std::shared_ptr<const CodeObject> &code, const std::string &source) {
+    hipModule_t module = nullptr;
+    hipError_t e = hipModuleLoadData(&module, code->binary.data());
+    if (e != hipSuccess && code->from_disk) {
+        (void) hipGetLastError();
+        code = recompile_kernel(source);
+        e = hipModuleLoadData(&module, code->binary.data());
+    }
+    hip_check(e, "hipModuleLoadData");
+    return module;
+}
+
+}  // namespace
+
 HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only, bool preserve_inputs, bool fuse_small)
     : device_(device), batch_size_(batch_size), plan_only_(plan_only) {
     if (!plan_only) HipDevice::check(device);
@@ -115,8 +132,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
             KN_ASSERT(l.ptrs.size() == step.kernel.n_ptrs);
             auto it = loaded.find(step.code->key);
             if (it == loaded.end()) {
-                hipModule_t module;
-                hip_check(hipModuleLoadData(&module, step.code->binary.data()), "hipModuleLoadData");
+                hipModule_t module = load_code_object(step.code, step.kernel.source);
                 modules_.push_back(module);
                 it = loaded.emplace(step.code->key, module).first;
             }
@@ -148,8 +164,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     if (fused_spec_) {
         hip_check(hipHostMalloc((void **) &fused_done_, 64, hipHostMallocCoherent), "hipHostMalloc");
         *fused_done_ = 0;
-        hipModule_t module;
-        hip_check(hipModuleLoadData(&module, fused_code_->binary.data()), "hipModuleLoadData");
+        hipModule_t module = load_code_object(fused_code_, fused_spec_->source);
         modules_.push_back(module);
         hip_check(hipModuleGetFunction(&fused_function_, module, fused_spec_->name.c_str()), "hipModuleGetFunction");
         for (auto &l : launches_) fused_ptrs_.insert(fused_ptrs_.end(), l.ptrs.begin(), l.ptrs.end());

@@ -13,15 +13,22 @@ namespace kn {
 struct CodeObject {
     std::vector<char> binary;
     uint64_t key = 0;
+    bool from_disk = false;  // read from the disk cache rather than compiled by this process
 };
 
 // Compile (or fetch from cache) the code object for a kernel source. Works without a GPU.
 // The disk cache lives in $KNHIP_CACHE_DIR, or next to the library in `_kcache/` when that is unset;
 // set KNHIP_CACHE_DIR to an empty string to disable it.
+// A cache file carries a header (layout, key, a second hash of the source, length and hash of the code object); the
+// key covers the source, the compile options and the hipRTC / HIP versions. A file that fails any of these checks is
+// deleted and the kernel compiled again.
 std::shared_ptr<const CodeObject> compile_kernel(const std::string &source);
+// Forget the cached code object of `source` (memory and disk) and compile it again: for a code object from the disk
+// cache that passed the checks above and still does not load.
+std::shared_ptr<const CodeObject> recompile_kernel(const std::string &source);
 
 struct CompileStats {
-    size_t compiled = 0, memory_hits = 0, disk_hits = 0;
+    size_t compiled = 0, memory_hits = 0, disk_hits = 0, discarded = 0;
 };
 CompileStats compile_stats();
 
