@@ -147,6 +147,109 @@ std::vector<uint8_t> Graph::serialize() const {
 
 // Rebuilds the values exactly as written (no builder canonicalisation is re-run), checking every
 // operand index, shape and dtype relation the executor later relies on.
+namespace {
+
+// What the builder methods of Graph guarantee about a value, checked for a value that comes out of a blob instead:
+// the operation's axes and operands are in range and the stored shape and dtype are the ones the operation yields.
+// The planner and the kernels index with these without looking again.
+void check_value(const Graph &g, uint32_t vi, const Shape &shape, DType dtype, const Operation &op) {
+    auto bad = [&](const char *what) { fail("graph blob: value ", vi, ": ", what); };
+    auto in = [&](size_t k) -> const ValueInfo & { return g.values[op.inputs[k]]; };
+    auto is_float = [](DType d) { return d == DType::F32 || d == DType::F16; };
+    switch (op.kind) {
+        case OpKind::Input: case OpKind::Constant: break;
+        case OpKind::View:
+            if (in(0).dtype != dtype || in(0).shape.size() != shape.size()) bad("view changes the dtype or the size");
+            break;
+        case OpKind::Broadcast: {
+            const Shape &is = in(0).shape;
+            if (in(0).dtype != dtype || is.rank() != shape.rank()) bad("broadcast changes the dtype or the rank");
+            for (size_t a = 0; a < shape.rank(); a++)
+                if (!(is.dims[a] == shape.dims[a] || is.dims[a] == Size::one())) bad("broadcast of an axis that is not 1");
+            break;
+        }
+        case OpKind::Permute: {
+            const Shape &is = in(0).shape;
+            if (in(0).dtype != dtype || op.axes.size() != is.rank() || shape.rank() != is.rank()) bad("permutation rank mismatch");
+            std::vector<bool> seen(is.rank(), false);
+            for (size_t a = 0; a < op.axes.size(); a++) {
+                if (op.axes[a] >= is.rank() || seen[op.axes[a]]) bad("not a permutation of the axes");
+                seen[op.axes[a]] = true;
+                if (shape.dims[a] != is.dims[op.axes[a]]) bad("permuted shape mismatch");
+            }
+            break;
+        }
+        case OpKind::Slice: {
+            const Shape &is = in(0).shape;
+            size_t axis = op.axes[0];
+            if (in(0).dtype != dtype || axis >= is.rank() || !is.dims[axis].is_fixed()) bad("slice axis out of range or not fixed");
+            op.range.assert_in_bounds(is.dims[axis].fixed_factor);
+            size_t n = (op.range.end - op.range.start) / op.range.step;
+            if (shape != is.replace(axis, Shape::fixed({n}))) bad("sliced shape mismatch");
+            break;
+        }
+        case OpKind::Flip: case OpKind::Softmax: case OpKind::Layernorm:
+            if (in(0).dtype != dtype || in(0).shape != shape || op.axes[0] >= shape.rank()) bad("axis out of range, or shape or dtype changed");
+            if (op.kind != OpKind::Flip && !is_float(dtype)) bad("softmax and layernorm need f32 or f16");
+            break;
+        case OpKind::Gather: {
+            const Shape &is = in(0).shape;
+            const ValueInfo &idx = in(1);
+            size_t axis = op.axes[0];
+            if (in(0).dtype != dtype || axis >= is.rank()) bad("gather axis out of range or dtype changed");
+            if (idx.shape.rank() != 1 || !dtype_is_int(idx.dtype)) bad("gather indices must be a rank 1 integer value");
+            if (shape != is.replace(axis, idx.shape)) bad("gathered shape mismatch");
+            break;
+        }
+        case OpKind::Concat: {
+            size_t axis = op.axes[0];
+            if (axis >= shape.rank()) bad("concat axis out of range");
+            Shape base = shape.replace(axis, Shape::fixed({0}));
+            Size along = Size::zero();
+            for (size_t k = 0; k < op.inputs.size(); k++) {
+                if (in(k).dtype != dtype || in(k).shape.rank() != shape.rank() || in(k).shape.replace(axis, Shape::fixed({0})) != base)
+                    bad("concat operand does not match the result off the axis");
+                auto sum = along.add(in(k).shape.dims[axis]);
+                if (!sum) bad("concat sizes do not add");
+                along = *sum;
+            }
+            if (along != shape.dims[axis]) bad("concat size along the axis mismatch");
+            break;
+        }
+        case OpKind::Conv: {
+            const ConvDetails &d = op.conv;
+            if (in(0).dtype != dtype || in(1).dtype != dtype) bad("conv operands must have the dtype of the result");
+            if (d.kernel_h % 2 != 1 || d.kernel_w % 2 != 1) bad("conv kernel sizes must be odd");
+            if (shape != Shape({d.batch_size, Size::fixed(d.output_channels), Size::fixed(d.output_h), Size::fixed(d.output_w)}))
+                bad("conv output shape mismatch");
+            break;
+        }
+        case OpKind::MatMul: {
+            const Shape &l = in(0).shape, &r = in(1).shape;
+            if (in(0).dtype != dtype || in(1).dtype != dtype) bad("matmul operands must have the dtype of the result");
+            if (l.rank() != 3 || r.rank() != 3 || l.dims[0] != r.dims[0] || l.dims[2] != r.dims[1]) bad("matmul operand shapes mismatch");
+            if (shape != Shape({l.dims[0], l.dims[1], r.dims[2]})) bad("matmul output shape mismatch");
+            break;
+        }
+        case OpKind::Unary: {
+            auto out = unary_output_dtype(op.unary, in(0).dtype, op.cast_to);
+            if (!out || *out != dtype || in(0).shape != shape) bad("unary operation does not yield this dtype and shape");
+            break;
+        }
+        case OpKind::Binary:
+            if (in(0).dtype != dtype || in(1).dtype != dtype || in(0).shape != shape || in(1).shape != shape)
+                bad("binary operands must have the shape and dtype of the result");
+            break;
+        case OpKind::Reduce:
+            if (in(0).dtype != dtype || op.axes.empty()) bad("reduce changes the dtype or has no axes");
+            if (op.reduce == ReduceOp::Mean && !is_float(dtype)) bad("mean needs f32 or f16");
+            if (shape != in(0).shape.replace_all(op.axes, Shape())) bad("reduced shape mismatch");  // checks range and uniqueness
+            break;
+    }
+}
+
+}  // namespace
+
 Graph Graph::deserialize(const uint8_t *data, size_t len) {
     Reader r{data, len};
     if (r.u32() != MAGIC) fail("graph blob has a wrong magic number");
@@ -287,6 +390,7 @@ Graph Graph::deserialize(const uint8_t *data, size_t len) {
         std::string debug_id((const char *) r.p + r.pos, id_len);
         r.pos += id_len;
 
+        check_value(g, vi, shape, dtype, op);
         bool is_input = op.kind == OpKind::Input;
         size_t before = g.values.size();
         Value v = g.push(shape, dtype, std::move(op));
