@@ -205,6 +205,7 @@ void HipExecutor::realise_launch(size_t index, Launch &l, bool mapped) {
         l.attn.k = l.ptrs[1];
         l.attn.v = l.ptrs[2];
         l.attn.mask = step.attention_has_mask ? l.ptrs[3] : nullptr;
+        l.attn.block_class = step.attention_has_classes ? l.ptrs[4] : nullptr;
         l.attn.o = l.ptrs.back();
     } else if (step.kind == StepKind::MatMul && step.gemm.groups > 1) {
         GemmParams gemm = step.gemm;

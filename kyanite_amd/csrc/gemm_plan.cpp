@@ -5,6 +5,8 @@
 
 #include "mfma_kernels.h"
 
+#include <algorithm>
+
 namespace kn {
 
 namespace {
@@ -183,6 +185,26 @@ std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16) {
     if (lp.split_k > 1) ss << " split_k=" << lp.split_k << "x" << lp.k_chunk;
     if (lp.tail_split > 1) ss << " head=" << lp.head_tiles << " tail_split=" << lp.tail_split << "x" << lp.tail_k_chunk;
     return ss.str();
+}
+
+std::vector<unsigned char> attention_f16_block_classes(const void *mask_f16, int batches, int lq, int lk, long long m_sb, long long m_sq, long long m_sk) {
+    const uint16_t *m = (const uint16_t *) mask_f16;
+    const int q_tiles = (lq + 31) / 32, key_blocks = (lk + ATTENTION_F16_BLOCK - 1) / ATTENTION_F16_BLOCK;
+    std::vector<unsigned char> classes((size_t) batches * q_tiles * key_blocks);
+    for (int b = 0; b < batches; b++)
+        for (int qt = 0; qt < q_tiles; qt++)
+            for (int kb = 0; kb < key_blocks; kb++) {
+                // queries past lq repeat the last query in the kernel and keys past lk are dropped there: neither counts
+                bool all_neg_inf = true, all_zero = true;
+                for (int q = 32 * qt; q < std::min(lq, 32 * qt + 32); q++)
+                    for (int k = ATTENTION_F16_BLOCK * kb; k < std::min(lk, ATTENTION_F16_BLOCK * (kb + 1)); k++) {
+                        const uint16_t bits = m[b * m_sb + q * m_sq + k * m_sk];
+                        all_neg_inf &= bits == 0xfc00;
+                        all_zero &= (bits & 0x7fff) == 0;  // +0 or -0: adding either leaves every score's value
+                    }
+                classes[((size_t) b * q_tiles + qt) * key_blocks + kb] = all_neg_inf ? 1 : all_zero ? 2 : 0;
+            }
+    return classes;
 }
 
 bool gemm_group_ok(const GemmParams &p, bool f16) {

@@ -6,11 +6,17 @@
 //
 // Like the f32 kernel, everything is computed transposed so that a lane owns one query:
 //   S^T = K Q^T      A operand: 8 consecutive k of a key row from LDS, B operand: Q, in registers
-//   O^T += V^T P^T   A operand: 8 keys of one dim of V from LDS, B operand: P^T, straight from the S^T accumulators
+//   O^T += V^T P^T   A operand: 8 keys of one dim of V, B operand: P^T, straight from the S^T accumulators
 // Register v of half h of a lane holds key 8 (v / 4) + 4 h + v % 4 of a 32-key tile, and an MFMA step takes 8 keys
 // per half, so step s of the second product uses registers 8 s .. 8 s + 7, i.e. keys 16 s + 8 a + 4 h + b
-// (a < 2, b < 4). V is stored in LDS transposed, [dim][slot], with slot = 16 s + 8 h + 4 a + b, so that those 8 keys
-// are one 128 bit read.
+// (a < 2, b < 4). K and V are both staged in LDS the way they lie in memory, one row per key; the A operand of the
+// second product, which runs along the keys, is read with the transposing LDS load of gfx950 (ds_read_b64_tr_b16):
+// 16 lanes hand in the addresses of 4 dims of 4 consecutive keys each and every lane gets the 4 keys of one dim.
+//
+// What bounds a prefill of a few hundred tokens is not arithmetic (a microsecond of it) but the number of 128 byte
+// lines a compute unit requests from L2, of which it keeps about 64 in flight. So: rows are fetched whole (every
+// line requested once per block), Q is fetched once per workgroup, blocks of keys that the mask removes are not
+// fetched at all and neither is the mask where it is known to be zero.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -24,20 +30,21 @@ namespace {
 typedef _Float16 half_t;
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 
-constexpr int BKEYS = 32;  // keys per block: one MFMA tile
+constexpr int BKEYS = ATTENTION_F16_BLOCK;  // keys per block: one MFMA tile
 constexpr int WAVES = 4;   // waves per workgroup; they share 32 queries and take every fourth block of keys each
 
-__device__ __forceinline__ float r16(float x) { return (float) (half_t) x; }
-
-// position of a key of a block inside a row of the transposed V tile
-__device__ __forceinline__ int slot_of_key(int key) {
-    // key = 16 s + 8 a + 4 h + b  ->  16 s + 8 h + 4 a + b
-    return (key & ~12) | ((key & 8) >> 1) | ((key & 4) << 1);
+// the 4 keys (consecutive rows of the staged V) of one dim: see the head of the file
+__device__ __forceinline__ halfx4 lds_read_transposed(const half_t *p) {
+    return __builtin_bit_cast(halfx4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4 *) p));
 }
 
-// DK: width of Q and K (a multiple of 16); DVT: 32-wide tiles that cover the width of V.
+// DK: width of Q and K (a multiple of 64); DVT: 32-wide tiles that cover the width of V.
 // A workgroup owns 32 queries of one batch entry. Its 4 waves split the keys: wave w walks blocks w, w + 4, ... of 32
 // keys with a running softmax of its own, staging K and V in a private part of LDS (no workgroup barriers in the
 // loop), and the four partial results (maximum, sum, unnormalised output) are merged through LDS at the end. That
@@ -45,118 +52,197 @@ __device__ __forceinline__ int slot_of_key(int key) {
 // fill the chip, and lets every wave skip its own masked-out blocks.
 template <int DK, int DVT>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_f16_kernel(AttentionParams p) {
-    constexpr int DV = 32 * DVT, KS = DK + 8, VS = BKEYS + 8;
-    constexpr int K_VECS = BKEYS * DK / 8 / 64;          // 128 bit loads of K per lane and block
-    constexpr int V_ITEMS = (BKEYS / 2) * (DV / 8) / 64;  // (key pair, 8 dims) items of V per lane and block
-    constexpr int STAGE_BYTES = (BKEYS * KS + DV * VS) * 2, MERGE_BYTES = (DV * 32 + 64) * 4;
+    // Row strides in LDS. K rows are read 16 bytes per lane by 32 lanes with consecutive rows: 8 extra halves shift
+    // consecutive rows by 4 banks. V rows are read 8 bytes per lane, 4 consecutive rows of 64 bytes at a time: the
+    // stride is 64 or 192 bytes modulo 256, so that those 4 pieces cover all 64 banks once.
+    constexpr int DV = 32 * DVT, KS = DK + 8, VS = (DV + 31) / 64 * 64 + 32;
+    constexpr int KC = DK / 8, VC = DV / 8;      // 16 byte pieces per row
+    constexpr int K_VECS = BKEYS * KC / 64;      // 128 bit loads of K per lane and block
+    constexpr int V_VECS = BKEYS * VC / 64;      // and of V
+    constexpr int Q_VECS = (32 / WAVES) * KC / 64;
+    constexpr int OS = DV + 4;  // floats per query in the merge at the end
+    constexpr int STAGE_BYTES = (BKEYS * KS + BKEYS * VS) * 2, MERGE_BYTES = (32 * OS + 64) * 4;
     constexpr int WAVE_BYTES = ((STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES) + 15) / 16 * 16;
-    static_assert(DK % 16 == 0 && K_VECS >= 1 && V_ITEMS >= 1, "unsupported shape");
+    static_assert(DK % 64 == 0 && K_VECS >= 1 && V_VECS >= 1 && Q_VECS >= 1 && 64 % KC == 0 && 32 * KS * 2 <= WAVE_BYTES, "unsupported shape");
     __shared__ __attribute__((aligned(16))) unsigned char lds[WAVES][WAVE_BYTES];
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // (the wave index as a scalar: block base pointers then stay in scalar registers)
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 31, h = lane >> 5;
-    const int bz = blockIdx.y;
-    const int query = blockIdx.x * 32 + c;
+    // Which 32 queries of which batch entry. Under a causal mask the last tile of queries has the most live key blocks
+    // and the first has one; workgroups start in the order of their linear index and a compute unit holds two of them,
+    // so the first half of the launch takes the later tiles of every batch entry, latest first, and the second half
+    // the earlier ones: the two workgroups of a compute unit then carry about the same work together, and so do the
+    // eight parts of the chip, which take workgroups in turn. Without a mask it is a harmless permutation.
+    int tile = blockIdx.x, bz = blockIdx.y;
+    {
+        const int nt = gridDim.x, pairs = nt >> 1;
+        if ((nt & 1) == 0) {
+            int linear = bz * nt + tile;
+            const int half_launch = pairs * (int) gridDim.y;
+            const bool late = linear < half_launch;
+            if (!late) linear -= half_launch;
+            bz = linear / pairs;
+            const int t = linear - bz * pairs;
+            tile = late ? nt - 1 - t : t;
+        }
+    }
+    const int query = tile * 32 + c;
     const int query_c = min(query, p.lq - 1);
     half_t (*Ks)[KS] = (half_t (*)[KS]) &lds[wave][0];
-    half_t (*Vt)[VS] = (half_t (*)[VS]) &lds[wave][BKEYS * KS * 2];
+    half_t (*Vs)[VS] = (half_t (*)[VS]) &lds[wave][BKEYS * KS * 2];
     const int bz1 = bz / p.batch_inner, bz2 = bz - bz1 * p.batch_inner;
     const half_t *kp = (const half_t *) p.k + bz1 * p.k_sb + bz2 * p.k_sb2, *vp = (const half_t *) p.v + bz1 * p.v_sb + bz2 * p.v_sb2;
     const half_t *mp = p.mask ? (const half_t *) p.mask + bz * p.m_sb + (long long) query_c * p.m_sq : nullptr;
 
-    // Q^T operand: lane (query c, half h) holds k = 16 t + 8 h .. + 7 for step t
-    halfx8 qf[DK / 16];
-    {
-        const half_t *qp = (const half_t *) p.q + bz1 * p.q_sb + bz2 * p.q_sb2 + (long long) query_c * p.q_sm;
+    // ---- the blocks of this wave and what the mask does to each: 0 = added as it is, 1 = removes the whole block
+    // (every entry -inf: nothing to fetch or compute, all its terms are exact zeros), 2 = all zeros (nothing to add).
+    // The launcher passes the classes where the mask is a constant; lane l keeps the class of the wave's block l.
+    const int first = wave * BKEYS, stride = WAVES * BKEYS;
+    const int n_blocks = first < p.lk ? (p.lk - first + stride - 1) / stride : 0;
+    int class_of_block = mp ? 0 : 2;
+    if (p.block_class) {
+        const int key_blocks = (p.lk + BKEYS - 1) / BKEYS, kb = wave + WAVES * lane;
+        const unsigned char *row = (const unsigned char *) p.block_class + ((long long) (p.m_sb ? bz : 0) * gridDim.x + tile) * key_blocks;
+        class_of_block = kb < key_blocks ? row[kb] : 1;
+    }
+    auto block_class = [&](int i) { return __builtin_amdgcn_readlane(class_of_block, i & 63); };
+    auto next_live = [&](int i) {
+        while (i < n_blocks && block_class(i) == 1) i++;
+        return i;
+    };
+
+    // ---- Q: every wave fetches 8 of the 32 rows, whole lines at a time; they go through the part of LDS that wave 0
+    // stages K in later. The loads are issued here and picked up after the first block of keys has been requested,
+    // so that the two round trips to memory overlap.
+    const char *qb = (const char *) ((const half_t *) p.q + bz1 * p.q_sb + bz2 * p.q_sb2);
+    const unsigned q_row = (unsigned) p.q_sm * 2;
+    halfx8 qreg[Q_VECS];
 #pragma unroll
-        for (int t = 0; t < DK / 16; t++) {
-            qf[t] = *(const halfx8 *) (qp + 16 * t + 8 * h);
-            if (query >= p.lq) qf[t] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
-        }
+    for (int i = 0; i < Q_VECS; i++) {
+        const int e = lane + 64 * i, row = (32 / WAVES) * wave + e / KC, part = e % KC;
+        qreg[i] = *(const halfx8 *) (qb + ((unsigned) min(tile * 32 + row, p.lq - 1) * q_row + 16 * part));
     }
 
-    // global -> registers -> LDS. Element offsets inside a block of keys are the same for every block and kept as
-    // 32 bit numbers (the host checks that they fit), the block's base pointer is wave-uniform; in a partial block
-    // rows past the last key are read from the last key and zeroed when staged.
-    halfx8 kreg[K_VECS], vreg[V_ITEMS][2];
-    int koff[K_VECS], voff[V_ITEMS];
+    // ---- global -> registers -> LDS. The block's base pointer is wave-uniform and the lanes' offsets inside a block
+    // are the same for every block, 32 bit numbers (the host checks that they fit); in a partial block rows past
+    // the last key are read from the last key, and the rows of V among them are zeroed when staged.
+    halfx8 kreg[K_VECS], vreg[V_VECS];
+    const unsigned k_row = (unsigned) p.k_sn * 2, v_row = (unsigned) p.v_sk * 2;
+    unsigned koff[K_VECS], voff[V_VECS];  // in bytes
 #pragma unroll
     for (int i = 0; i < K_VECS; i++) {
-        const int e = lane + 64 * i, key = e / (DK / 8), part = e % (DK / 8);
-        koff[i] = key * (int) p.k_sn + 8 * part;
+        const int e = lane + 64 * i;
+        koff[i] = (unsigned) (e / KC) * k_row + 16 * (e % KC);
     }
 #pragma unroll
-    for (int i = 0; i < V_ITEMS; i++) {
-        const int e = lane + 64 * i, pair = e % (BKEYS / 2), part = e / (BKEYS / 2);
-        voff[i] = 2 * pair * (int) p.v_sk + min(8 * part, (p.dv - 1) & ~7);  // dims past dv: any valid vector
+    for (int i = 0; i < V_VECS; i++) {
+        const int e = lane + 64 * i;
+        voff[i] = (unsigned) (e / VC) * v_row + 2 * min(8 * (e % VC), (p.dv - 1) & ~7);  // dims past dv: any valid vector
     }
-    halfx4 mreg[4];  // the mask of this lane's 16 scores
-    auto fetch = [&](int key0) {
-        const half_t *kb = kp + (long long) key0 * p.k_sn, *vb = vp + (long long) key0 * p.v_sk;
+    // the mask of this lane's 16 scores; a whole block with contiguous, aligned rows arrives as keys 16 h .. 16 h + 15
+    // of the lane's query and is put in order later (see `mask_in_order`)
+    uintx4 mraw[2];
+    const unsigned moff = (unsigned) (query_c * (int) p.m_sq + 16 * h) * 2;  // vector loads only (the host checks the range)
+    const char *mbase = p.mask ? (const char *) ((const half_t *) p.mask + bz * p.m_sb) : nullptr;
+    auto mask_as_rows = [&](int key0) { return p.mask_vec == 2 && key0 + BKEYS <= p.lk; };
+    auto fetch = [&](int i) {
+        const int key0 = first + i * stride;
+        const char *kb = (const char *) (kp + (long long) key0 * p.k_sn), *vb = (const char *) (vp + (long long) key0 * p.v_sk);
         if (key0 + BKEYS <= p.lk) {
 #pragma unroll
-            for (int i = 0; i < K_VECS; i++) kreg[i] = *(const halfx8 *) (kb + koff[i]);
+            for (int j = 0; j < K_VECS; j++) kreg[j] = *(const halfx8 *) (kb + koff[j]);
 #pragma unroll
-            for (int i = 0; i < V_ITEMS; i++) {
-                vreg[i][0] = *(const halfx8 *) (vb + voff[i]);
-                vreg[i][1] = *(const halfx8 *) (vb + voff[i] + (int) p.v_sk);
-            }
+            for (int j = 0; j < V_VECS; j++) vreg[j] = *(const halfx8 *) (vb + voff[j]);
         } else {
             const int last = p.lk - 1 - key0;  // last valid row of the block
 #pragma unroll
-            for (int i = 0; i < K_VECS; i++) {
-                const int key = (lane + 64 * i) / (DK / 8);
-                kreg[i] = *(const halfx8 *) (kb + koff[i] - (key - min(key, last)) * (int) p.k_sn);
+            for (int j = 0; j < K_VECS; j++) {
+                const int key = (lane + 64 * j) / KC;
+                kreg[j] = *(const halfx8 *) (kb + (koff[j] - (unsigned) (key - min(key, last)) * k_row));
             }
 #pragma unroll
-            for (int i = 0; i < V_ITEMS; i++) {
-                const int key = 2 * ((lane + 64 * i) % (BKEYS / 2));
-#pragma unroll
-                for (int u = 0; u < 2; u++)
-                    vreg[i][u] = *(const halfx8 *) (vb + voff[i] + (min(key + u, last) - key) * (int) p.v_sk);
+            for (int j = 0; j < V_VECS; j++) {
+                const int key = (lane + 64 * j) / VC;
+                vreg[j] = *(const halfx8 *) (vb + (voff[j] - (unsigned) (key - min(key, last)) * v_row));
             }
         }
-        if (mp) {
-            if (p.mask_vec && key0 + BKEYS <= p.lk) {  // whole block, contiguous aligned rows
-#pragma unroll
-                for (int a = 0; a < 4; a++) mreg[a] = *(const halfx4 *) (mp + key0 + 8 * a + 4 * h);
+        if (block_class(i) == 0) {
+            if (mask_as_rows(key0)) {
+                const char *mb = mbase + 2 * key0;
+                mraw[0] = *(const uintx4 *) (mb + moff);
+                mraw[1] = *(const uintx4 *) (mb + (moff + 16));
             } else {
+                halfx4 m[4];
 #pragma unroll
                 for (int a = 0; a < 4; a++)
 #pragma unroll
                     for (int b = 0; b < 4; b++)
-                        mreg[a][b] = mp[(long long) min(key0 + 8 * a + 4 * h + b, p.lk - 1) * p.m_sk];
+                        m[a][b] = mp[(long long) min(key0 + 8 * a + 4 * h + b, p.lk - 1) * p.m_sk];
+                mraw[0] = uintx4{__builtin_bit_cast(uint2, m[0]).x, __builtin_bit_cast(uint2, m[0]).y, __builtin_bit_cast(uint2, m[1]).x, __builtin_bit_cast(uint2, m[1]).y};
+                mraw[1] = uintx4{__builtin_bit_cast(uint2, m[2]).x, __builtin_bit_cast(uint2, m[2]).y, __builtin_bit_cast(uint2, m[3]).x, __builtin_bit_cast(uint2, m[3]).y};
             }
         }
+    };
+    // Keys 16 h .. 16 h + 15 of the query, as 8 registers d0 .. d7 of two keys each, become the keys of the lane's
+    // scores, 8 a + 4 h + b: half 0 keeps d0 d1 d4 d5 and needs the same four of the other half's, half 1 keeps
+    // d2 d3 d6 d7 and needs those of half 0. v_permlane32_swap(x, y) exchanges the upper half of x with the lower half
+    // of y, so swapping (d0, d2) leaves keys 8 a + 4 h + {0, 1} for a = 0 in the first and for a = 2 in the second.
+    auto mask_in_order = [&](int key0, halfx4 (&mv)[4]) {
+        uint2 m[4];
+        if (mask_as_rows(key0)) {
+            const auto s0 = __builtin_amdgcn_permlane32_swap(mraw[0][0], mraw[0][2], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(mraw[0][1], mraw[0][3], false, false);
+            const auto s2 = __builtin_amdgcn_permlane32_swap(mraw[1][0], mraw[1][2], false, false);
+            const auto s3 = __builtin_amdgcn_permlane32_swap(mraw[1][1], mraw[1][3], false, false);
+            m[0] = uint2{s0[0], s1[0]};
+            m[2] = uint2{s0[1], s1[1]};
+            m[1] = uint2{s2[0], s3[0]};
+            m[3] = uint2{s2[1], s3[1]};
+        } else {
+            m[0] = uint2{mraw[0][0], mraw[0][1]};
+            m[1] = uint2{mraw[0][2], mraw[0][3]};
+            m[2] = uint2{mraw[1][0], mraw[1][1]};
+            m[3] = uint2{mraw[1][2], mraw[1][3]};
+        }
+#pragma unroll
+        for (int a = 0; a < 4; a++) mv[a] = __builtin_bit_cast(halfx4, m[a]);
     };
     auto stage = [&](int key0) {
         const halfx8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-        // a whole block of keys and all DV dims present (wave-uniform): nothing to zero
-        const bool full = key0 + BKEYS <= p.lk && p.dv == DV;
+        const bool full = key0 + BKEYS <= p.lk;  // wave-uniform
 #pragma unroll
-        for (int i = 0; i < K_VECS; i++) {
-            const int e = lane + 64 * i, key = e / (DK / 8), part = e % (DK / 8);
-            *(halfx8 *) &Ks[key][8 * part] = full || key0 + key < p.lk ? kreg[i] : zero;
+        for (int j = 0; j < K_VECS; j++) {
+            const int e = lane + 64 * j;
+            *(halfx8 *) &Ks[e / KC][8 * (e % KC)] = kreg[j];
         }
 #pragma unroll
-        for (int i = 0; i < V_ITEMS; i++) {
-            const int e = lane + 64 * i, pair = e % (BKEYS / 2), part = e / (BKEYS / 2);
-            const int key = 2 * pair, slot = slot_of_key(key);  // the odd key sits in the next slot
-            halfx8 v0 = vreg[i][0], v1 = vreg[i][1];
-            if (!full) {
-                if (!(key0 + key < p.lk && 8 * part < p.dv)) v0 = zero;
-                if (!(key0 + key + 1 < p.lk && 8 * part < p.dv)) v1 = zero;
-            }
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
-                halfx2 two;
-                two[0] = v0[j];
-                two[1] = v1[j];
-                *(halfx2 *) &Vt[8 * part + j][slot] = two;
-            }
+        for (int j = 0; j < V_VECS; j++) {
+            const int e = lane + 64 * j, key = e / VC;
+            *(halfx8 *) &Vs[key][8 * (e % VC)] = full || key0 + key < p.lk ? vreg[j] : zero;
         }
     };
+
+    int i = next_live(0);
+    if (i < n_blocks) fetch(i);
+
+    // ---- Q into LDS, and from there each lane's operand: lane (query c, half h) holds k = 16 t + 8 h .. + 7 for step t
+    halfx8 qf[DK / 16];
+    {
+        half_t (*Qs)[KS] = (half_t (*)[KS]) &lds[0][0];
+#pragma unroll
+        for (int j = 0; j < Q_VECS; j++) {
+            const int e = lane + 64 * j, row = (32 / WAVES) * wave + e / KC, part = e % KC;
+            *(halfx8 *) &Qs[row][8 * part] = qreg[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < DK / 16; t++) {
+            qf[t] = *(const halfx8 *) &Qs[c][16 * t + 8 * h];
+            if (query >= p.lq) qf[t] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+        __syncthreads();
+    }
 
     floatx16 oacc[DVT];
 #pragma unroll
@@ -166,25 +252,29 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     float row_max = -INFINITY, row_sum = 0.0f;  // row_sum: this half's share of the keys only
     const float scale = p.scale;                // already an f16 value
     constexpr float LOG2E = 1.44269504088896340736f;
+    // the lane's corner of the transposed reads of V: 16 lanes cover 4 keys x 16 dims, lane s of them hands in the
+    // address of dims 4 (s % 4) .. + 3 of key s / 4; the groups are (dims 0-15, 16-31) x (keys of half 0, half 1)
+    const half_t *v_corner = &Vs[4 * h + (lane & 15) / 4][16 * ((lane >> 4) & 1) + 4 * (lane & 3)];
 
-    const int first = wave * BKEYS, stride = WAVES * BKEYS;
-    if (first < p.lk) fetch(first);
-    for (int key0 = first; key0 < p.lk; key0 += stride) {
+    while (i < n_blocks) {
+        const int key0 = first + i * stride, cls = block_class(i), i_next = next_live(i + 1);
         halfx4 mv[4];
+        bool skip = false;
+        if (cls == 0) {
+            mask_in_order(key0, mv);
+            // A block whose mask is -inf for every query of the wave (the upper triangle of a causal mask) adds exact
+            // zeros to every sum: nothing to compute. (-inf + a finite score is -inf whatever the score.)
+            unsigned differs = 0;  // from -inf (0xfc00), two values at a time
 #pragma unroll
-        for (int a = 0; a < 4; a++) mv[a] = mreg[a];
-        // A block whose mask is -inf for every query of the wave (the upper triangle of a causal mask) adds exact
-        // zeros to every sum: nothing to compute. (-inf + a finite score is -inf whatever the score.)
-        bool dead = mp != nullptr;
-        if (mp) {
-#pragma unroll
-            for (int a = 0; a < 4; a++)
-#pragma unroll
-                for (int b = 0; b < 4; b++) dead = dead && (float) mv[a][b] == -INFINITY;
+            for (int a = 0; a < 4; a++) {
+                const uint2 bits = __builtin_bit_cast(uint2, mv[a]);
+                differs |= (bits.x ^ 0xfc00fc00u) | (bits.y ^ 0xfc00fc00u);
+            }
+            skip = __all(differs == 0);
         }
-        const bool skip = __all(dead);
         if (!skip) stage(key0);  // (the loaded registers are free again)
-        if (key0 + stride < p.lk) fetch(key0 + stride);
+        if (i_next < n_blocks) fetch(i_next);
+        i = i_next;
         if (skip) continue;
 
         floatx16 st;
@@ -196,16 +286,43 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             st = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[t], st, 0, 0, 0);
         }
 
-        // the roundings of matmul -> * scale -> + mask, then the running softmax in f32
+        // The roundings of matmul -> * scale -> + mask, in f16 arithmetic, two scores per instruction, with the same
+        // results as f32 arithmetic rounded to f16: the product of two f16 values is exact in f32, and so is their sum
+        // unless one is below a quarter of the other's last place, where either way of rounding returns the larger one.
+        halfx2 sh[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            floatx2 two;
+            two[0] = st[2 * j];
+            two[1] = st[2 * j + 1];
+            sh[j] = __builtin_convertvector(two, halfx2);
+        }
+        if (p.has_scale) {
+            halfx2 scale2;
+            scale2[0] = scale2[1] = (half_t) scale;
+#pragma unroll
+            for (int j = 0; j < 8; j++) sh[j] = sh[j] * scale2;
+        }
+        if (cls == 0) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                halfx2 m;
+                m[0] = mv[j >> 1][2 * (j & 1)];
+                m[1] = mv[j >> 1][2 * (j & 1) + 1];
+                sh[j] = sh[j] + m;
+            }
+        }
+        if (key0 + BKEYS > p.lk) {  // the last, partial block of keys
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (key0 + 8 * (v >> 2) + 4 * h + (v & 3) >= p.lk) sh[v >> 1][v & 1] = (half_t) -INFINITY;
+        }
+        // the running softmax in f32
         float block_max = -INFINITY;
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            float s = r16(st[v]);
-            if (p.has_scale) s = r16(s * scale);
-            if (mp) s = r16(s + (float) mv[v >> 2][v & 3]);
-            if (key0 + 8 * (v >> 2) + 4 * h + (v & 3) >= p.lk) s = -INFINITY;
-            st[v] = s;
-            block_max = fmaxf(block_max, s);
+            st[v] = (float) sh[v >> 1][v & 1];
+            block_max = fmaxf(block_max, st[v]);
         }
         block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
         const float new_max = fmaxf(row_max, block_max);
@@ -232,20 +349,27 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         for (int s = 0; s < 2; s++) {
             halfx8 a[DVT];
 #pragma unroll
-            for (int t = 0; t < DVT; t++) a[t] = *(const halfx8 *) &Vt[32 * t + c][16 * s + 8 * h];
+            for (int t = 0; t < DVT; t++) {
+                const halfx4 lo = lds_read_transposed(v_corner + (16 * s) * VS + 32 * t);
+                const halfx4 hi = lds_read_transposed(v_corner + (16 * s + 8) * VS + 32 * t);
+                a[t] = halfx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
 #pragma unroll
             for (int t = 0; t < DVT; t++) oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t], pv[s], oacc[t], 0, 0, 0);
         }
     }
 
-    // ---- merge the four partial results: every wave leaves its maximum, sum and output in its own part of LDS
+    // ---- merge the four partial results: every wave leaves its maximum, sum and output in its own part of LDS, one
+    // row of DV + 4 floats per query (rows 16 bytes apart modulo 256: 128 bit accesses of 16 lanes cover all banks)
     row_sum += __shfl_xor(row_sum, 32);
-    float (*Of)[32] = (float (*)[32]) &lds[wave][0];
-    float *stats = (float *) &lds[wave][DV * 32 * 4];  // [0..31] maxima, [32..63] sums
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+    float (*Of)[OS] = (float (*)[OS]) &lds[wave][0];
+    float *stats = (float *) &lds[wave][32 * OS * 4];  // [0..31] maxima, [32..63] sums
 #pragma unroll
     for (int t = 0; t < DVT; t++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) Of[32 * t + 8 * (v >> 2) + 4 * h + (v & 3)][c] = oacc[t][v];
+        for (int a = 0; a < 4; a++)  // registers 4 a .. 4 a + 3: dims 32 t + 8 a + 4 h + (0 .. 3)
+            *(floatx4 *) &Of[c][32 * t + 8 * a + 4 * h] = floatx4{oacc[t][4 * a], oacc[t][4 * a + 1], oacc[t][4 * a + 2], oacc[t][4 * a + 3]};
     if (h == 0) {
         stats[c] = row_max;
         stats[32 + c] = row_sum;
@@ -253,10 +377,10 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     __syncthreads();
     float weight[WAVES], total_max = -INFINITY, total_sum = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; w++) total_max = fmaxf(total_max, ((const float *) &lds[w][DV * 32 * 4])[c]);
+    for (int w = 0; w < WAVES; w++) total_max = fmaxf(total_max, ((const float *) &lds[w][32 * OS * 4])[c]);
 #pragma unroll
     for (int w = 0; w < WAVES; w++) {
-        const float *st_w = (const float *) &lds[w][DV * 32 * 4];
+        const float *st_w = (const float *) &lds[w][32 * OS * 4];
         weight[w] = __builtin_amdgcn_exp2f((st_w[c] - (total_max == -INFINITY ? 0.0f : total_max)) * LOG2E);
         total_sum += weight[w] * st_w[32 + c];
     }
@@ -265,13 +389,30 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
         half_t *op = (half_t *) p.o + bz1 * p.o_sb + bz2 * p.o_sb2 + (long long) query * p.o_sm;
         // wave w, half h: dims (2 w + h) * DV / 8 ... + DV / 8
         constexpr int PER = DV / 8;
+        const int d0 = (2 * wave + h) * PER;
+        float x[PER];
 #pragma unroll
-        for (int i = 0; i < PER; i++) {
-            const int d = (2 * wave + h) * PER + i;
-            float x = 0.0f;
+        for (int j = 0; j < PER; j++) x[j] = 0.0f;
 #pragma unroll
-            for (int w = 0; w < WAVES; w++) x += weight[w] * ((const float (*)[32]) &lds[w][0])[d][c];
-            if (d < p.dv) op[(long long) d * p.o_sn] = (half_t) (x * inv);
+        for (int w = 0; w < WAVES; w++)
+#pragma unroll
+            for (int j = 0; j < PER; j += 4) {
+                const floatx4 part = *(const floatx4 *) &((const float (*)[OS]) &lds[w][0])[c][d0 + j];
+#pragma unroll
+                for (int u = 0; u < 4; u++) x[j + u] += weight[w] * part[u];
+            }
+        if (PER % 8 == 0 && p.o_sn == 1 && p.o_vec && d0 + PER <= p.dv) {
+#pragma unroll
+            for (int j = 0; j < PER; j += 8) {
+                halfx8 out;
+#pragma unroll
+                for (int u = 0; u < 8; u++) out[u] = (half_t) (x[j + u] * inv);
+                *(halfx8 *) (op + d0 + j) = out;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < PER; j++)
+                if (d0 + j < p.dv) op[(long long) (d0 + j) * p.o_sn] = (half_t) (x[j] * inv);
         }
     }
 }
@@ -298,21 +439,33 @@ int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream) {
     if (p.q_sk != 1 || p.k_sk != 1 || p.v_sn != 1 || !aligned(p.q, p.q_sb, p.q_sm) || !aligned(p.k, p.k_sb, p.k_sn) ||
         !aligned(p.v, p.v_sb, p.v_sk))
         return (int) hipErrorInvalidValue;
+    // rows inside a block of keys, and the queries of a batch entry, are addressed with 32 bit byte offsets
     if (p.k_sn < 0 || p.k_sn > (1 << 20) || p.v_sk < 0 || p.v_sk > (1 << 20)) return (int) hipErrorInvalidValue;
+    if (p.q_sm < 0 || (long long) p.lq * p.q_sm >= (1ll << 30)) return (int) hipErrorInvalidValue;
+    AttentionParams q = p;
+    // whole rows of the mask are loaded 32 bytes per lane, addressed with 32 bit byte offsets inside a batch entry
+    q.mask_vec = 0;
+    if (p.mask && p.mask_vec && p.m_sk == 1 && p.m_sq >= 0 && p.m_sq % 8 == 0 && p.m_sb % 8 == 0 && (uintptr_t) p.mask % 16 == 0 &&
+        (long long) p.lq * p.m_sq + p.lk < (1ll << 30))
+        q.mask_vec = 2;
+    // rows of the result can be stored 16 bytes at a time
+    q.o_vec = p.o_sn == 1 && (uintptr_t) p.o % 16 == 0 && p.o_sb % 8 == 0 && p.o_sb2 % 8 == 0 && p.o_sm % 8 == 0;
+    // block classes are indexed by at most 64 blocks per wave
+    if (!p.mask || p.lk > 64 * 4 * ATTENTION_F16_BLOCK) q.block_class = nullptr;
     const int dvt = (p.dv + 31) / 32;
     if (p.dk == 64) {
         switch (dvt) {
-            case 1: launch_waves<64, 1>(p, stream); break;
-            case 2: launch_waves<64, 2>(p, stream); break;
-            case 3: launch_waves<64, 3>(p, stream); break;
-            default: launch_waves<64, 4>(p, stream); break;
+            case 1: launch_waves<64, 1>(q, stream); break;
+            case 2: launch_waves<64, 2>(q, stream); break;
+            case 3: launch_waves<64, 3>(q, stream); break;
+            default: launch_waves<64, 4>(q, stream); break;
         }
     } else {
         switch (dvt) {
-            case 1: launch_waves<128, 1>(p, stream); break;
-            case 2: launch_waves<128, 2>(p, stream); break;
-            case 3: launch_waves<128, 3>(p, stream); break;
-            default: launch_waves<128, 4>(p, stream); break;
+            case 1: launch_waves<128, 1>(q, stream); break;
+            case 2: launch_waves<128, 2>(q, stream); break;
+            case 3: launch_waves<128, 3>(q, stream); break;
+            default: launch_waves<128, 4>(q, stream); break;
         }
     }
     return (int) hipGetLastError();

@@ -5,6 +5,7 @@
 
 #include <cstdint>
 #include <string>
+#include <vector>
 
 struct ihipStream_t;
 
@@ -112,7 +113,17 @@ struct AttentionParams {
     const void *mask = nullptr;
     long long m_sb = 0, m_sq = 0, m_sk = 0;
     int mask_vec = 0;  // rows of the mask are contiguous and 8 byte aligned
+    // f16 kernel, optional: what the mask does to each block of 32 queries x ATTENTION_F16_BLOCK keys, one byte per
+    // block, [mask batch (1 when m_sb is 0, else batch)][ceil(lq / 32)][ceil(lk / ATTENTION_F16_BLOCK)]:
+    // 0 = has to be read and added, 1 = every entry is -inf (the block is not fetched or computed), 2 = every entry
+    // is zero (the mask is not read). Known ahead of time where the mask is a constant.
+    const void *block_class = nullptr;
+    int o_vec = 0;  // set by the launcher: rows of O are contiguous and 16 byte aligned
 };
+constexpr int ATTENTION_F16_BLOCK = 32;
+// the classes above for a mask given as f16 values on the host with element strides (batch, query, key); `batches` is
+// 1 for a mask shared by all batch entries
+std::vector<unsigned char> attention_f16_block_classes(const void *mask_f16, int batches, int lq, int lk, long long m_sb, long long m_sq, long long m_sk);
 // widths the fused kernel is built for; other chains run as matmul, softmax, matmul
 bool attention_supported(int dk, int dv);
 bool attention_f16_supported(int dk, int dv);

@@ -16,7 +16,7 @@ std::string Step::str() const {
     ss << step_kind_name(kind) << " value=" << debug_value;
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
     if (kind == StepKind::MatMul && attention)
-        ss << " attention " << (gemm_f16 ? "f16" : "f32") << (attention_has_mask ? " +mask" : "") << " b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
+        ss << " attention " << (gemm_f16 ? "f16" : "f32") << (attention_has_mask ? (attention_has_classes ? " +mask (constant, classified by block)" : " +mask") : "") << " b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
     else if (kind == StepKind::MatMul) {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm_has_addend2 ? " +add" : "") << (gemm.relu ? " relu" : "");
@@ -857,6 +857,28 @@ private:
             a.mask_vec = ms[2] == 1 && ms[1] % 4 == 0 && ms[0] % 4 == 0 && mask->ptr.offset_bytes % 8 == 0;
             step.attention_has_mask = true;
             step.operands.push_back({*mask, OperandKind::In});
+            // a constant mask (the causal triangle of a decoder) is looked at once, here: the kernel then neither
+            // fetches nor computes the blocks it removes and does not read it where it is zero
+            if (f16 && mask->ptr.kind == BufferKind::Constant && mask->dtype == DType::F16 && lk <= 64 * 4 * ATTENTION_F16_BLOCK &&
+                ms[0] >= 0 && ms[1] >= 0 && ms[2] >= 0) {
+                const HostTensor &src = constants[mask->ptr.index];
+                const size_t batches = ms[0] == 0 ? 1 : b;
+                const int64_t last = mask->ptr.offset_bytes / 2 + (int64_t) (batches - 1) * ms[0] + (int64_t) (lq - 1) * ms[1] + (int64_t) (lk - 1) * ms[2];
+                KN_ASSERT(mask->ptr.offset_bytes >= 0 && mask->ptr.offset_bytes % 2 == 0 && last < (int64_t) src.len());
+                std::vector<unsigned char> classes = attention_f16_block_classes(src.bytes() + mask->ptr.offset_bytes, (int) batches,
+                                                                                 (int) lq, (int) lk, ms[0], ms[1], ms[2]);
+                bool useful = false;
+                for (unsigned char cl : classes) useful |= cl != 0;
+                if (useful) {
+                    constants.push_back(HostTensor(DType::U8, {classes.size()}, classes.data()));
+                    PlanTensor t;
+                    t.ptr = PlanPtr{BufferKind::Constant, constants.size() - 1, 0};
+                    t.dtype = DType::U8;
+                    t.shape = StridedShape::simple({classes.size()});
+                    step.operands.push_back({t, OperandKind::In});
+                    step.attention_has_classes = true;
+                }
+            }
         }
         step.operands.push_back({result, OperandKind::Out});
         push(std::move(step), value);

@@ -41,6 +41,7 @@ struct Step {
     // a MatMul step that is a whole softmax(scale * Q K^T [+ mask]) V chain in one launch; operands Q, K, V, [mask,] O
     bool attention = false;
     bool attention_has_mask = false;  // operand 3 is the additive mask, the result comes last
+    bool attention_has_classes = false;  // operand 4 is the per-block classification of a constant mask
     AttentionParams attn{};
     ConvParams conv{};
     bool conv_has_bias = false, conv_has_res = false;

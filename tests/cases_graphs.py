@@ -1583,6 +1583,13 @@ def attention_f16_causal_heads():
 
 
 @case
+def attention_f16_causal_even_tiles():
+    """an even number of query tiles (the launch pairs late tiles with early ones), 5 key blocks per wave at most, and
+    a last tile of queries that is partial"""
+    return _attention_f16_case(134, 3, 250, 250, 128, 128, True, "causal")
+
+
+@case
 def attention_f16_ragged_full_mask():
     """70 queries against 150 keys (partial blocks), width 64, V 40 wide, a mask tensor per batch entry"""
     return _attention_f16_case(131, 3, 70, 150, 64, 40, True, "full")
