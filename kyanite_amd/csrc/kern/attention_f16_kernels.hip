@@ -249,7 +249,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     for (int t = 0; t < DVT; t++)
 #pragma unroll
         for (int v = 0; v < 16; v++) oacc[t][v] = 0.0f;
-    float row_max = -INFINITY, row_sum = 0.0f;  // row_sum: this half's share of the keys only
+    float row_max = -INFINITY, row_sum = 0.0f;  // row_max: the reference of the exponentials; row_sum: this half's share of the keys only
     const float scale = p.scale;                // already an f16 value
     constexpr float LOG2E = 1.44269504088896340736f;
     // the lane's corner of the transposed reads of V: 16 lanes cover 4 keys x 16 dims, lane s of them hands in the
@@ -325,26 +325,33 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
             block_max = fmaxf(block_max, st[v]);
         }
         block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
-        const float new_max = fmaxf(row_max, block_max);
-        // a row that is masked out completely so far keeps zero weights instead of exp(-inf + inf)
-        const float safe_max = new_max == -INFINITY ? 0.0f : new_max;
-        const float alpha = __builtin_amdgcn_exp2f((row_max - safe_max) * LOG2E);
-        row_max = new_max;
-        float block_sum = 0.0f;
-        halfx8 pv[2];
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float e = __builtin_amdgcn_exp2f((st[v] - safe_max) * LOG2E);
-            block_sum += e;
-            pv[v >> 3][v & 7] = (half_t) e;
-        }
-        row_sum = row_sum * alpha + block_sum;
-        if (!__all(alpha == 1.0f)) {  // the maximum of some query moved
+        // The reference value of the exponentials follows the maximum lazily: it moves (and the sums so far are
+        // scaled down) only when some query's scores exceed it by more than 2^8 in the exponentials; until then the
+        // weights of this wave are up to 256 instead of up to 1, which f16 weights and f32 sums hold as well, and the
+        // merge at the end is told the reference, not the maximum. (The first live block of a query always moves it,
+        // from -inf.)
+        constexpr float SLACK = 8.0f / LOG2E;
+        if (__any(block_max > row_max + SLACK)) {
+            const float new_max = fmaxf(row_max, block_max);
+            // a row that is masked out completely so far keeps zero weights instead of exp(-inf + inf)
+            const float alpha = __builtin_amdgcn_exp2f((row_max - (new_max == -INFINITY ? 0.0f : new_max)) * LOG2E);
+            row_max = new_max;
+            row_sum *= alpha;
 #pragma unroll
             for (int t = 0; t < DVT; t++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) oacc[t][v] *= alpha;
         }
+        const float minus_ref = (row_max == -INFINITY ? 0.0f : -row_max) * LOG2E;
+        float block_sum = 0.0f;
+        halfx8 pv[2];
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(st[v], LOG2E, minus_ref));
+            block_sum += e;
+            pv[v >> 3][v & 7] = (half_t) e;
+        }
+        row_sum += block_sum;
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             halfx8 a[DVT];

@@ -1590,6 +1590,15 @@ def attention_f16_causal_even_tiles():
 
 
 @case
+def attention_f16_rising_scores():
+    """scores whose spread grows along the keys (later keys are up to 9 times larger): the reference value of the
+    running softmax moves in some blocks and stays behind the maximum, within its slack, in others"""
+    g, batch, inputs, _ = _attention_f16_case(135, 2, 64, 320, 64, 64, True, None)
+    inputs[1] = (inputs[1].astype(np.float32) * (1.0 + np.arange(320, dtype=np.float32)[None, :, None] / 40.0)).astype(np.float16)
+    return g, batch, inputs, None
+
+
+@case
 def attention_f16_ragged_full_mask():
     """70 queries against 150 keys (partial blocks), width 64, V 40 wide, a mask tensor per batch entry"""
     return _attention_f16_case(131, 3, 70, 150, 64, 40, True, "full")

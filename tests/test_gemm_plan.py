@@ -204,3 +204,17 @@ def test_rms_norm_is_one_row_kernel():
     g.output(g.mul(g.mul(x, g.broadcast(r, [512, 4096])), g.broadcast(w, [512, 4096])))
     ex = HipExecutor(0, g, 0, plan_only=True)
     assert ex.step_kinds() == ["reduce_op"] and "row statistic" in ex.step_str(0)
+
+
+def test_constant_attention_masks_are_classified_by_block():
+    """a constant f16 mask (the causal triangle) is classified per block of 32 queries x 32 keys when the plan is made,
+    so the kernel skips the blocks it removes; a mask that is an input cannot be"""
+    from cases_graphs import CASES
+    g, batch, _, _ = CASES["attention_f16_causal_even_tiles"]()
+    ex = HipExecutor(0, g, batch, plan_only=True)
+    steps = [ex.step_str(i) for i in range(ex.step_count())]
+    assert any("attention f16 +mask (constant, classified by block)" in s for s in steps), steps
+    g, batch, _, _ = CASES["attention_f16_ragged_full_mask"]()
+    ex = HipExecutor(0, g, batch, plan_only=True)
+    steps = [ex.step_str(i) for i in range(ex.step_count())]
+    assert any("attention f16 +mask" in s for s in steps) and not any("classified" in s for s in steps), steps
