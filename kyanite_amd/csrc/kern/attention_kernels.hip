@@ -12,7 +12,15 @@
 // per-lane values (plus one exchange between the two halves of the wave), and the accumulator registers of S^T are,
 // as they are, B operands of the second product: register v of half h holds key 8 (v / 4) + 4 h + v % 4 of the
 // tile, and the sum over keys may run in any order, so step v of the second product simply takes that key from V.
-// The softmax is the usual running one: a maximum and a sum per query, the output rescaled when the maximum moves.
+// The softmax is the usual running one: a reference value and a sum per query, the output rescaled when the
+// reference moves.
+//
+// A width of V that is a little over a multiple of 32 (40 for the heads of a diffusion UNet) would leave most of its
+// last 32-wide tile empty. Up to 16 such dims are computed with v_mfma_f32_4x4x1_16B_f32 instead: sixteen independent
+// 4 x 4 outer products per instruction, one per group of 4 lanes, 4 dims of V against the 4 queries of those lanes.
+// The B operand is again the lane's own register of P^T, the A operand one float of V per lane, and the result is
+// the lane's own query: 4 accumulator registers per 4 dims, no exchange between lanes. 8 cycles per 4 dims where a
+// 32 x 32 x 2 instruction takes 64 for 32.
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -30,10 +38,12 @@ constexpr int THREADS = 256;  // 4 waves
 constexpr int BQ = 128;       // queries per workgroup
 constexpr int BKEYS = 64;     // keys per block
 
-// DK: width of Q and K (a multiple of 8); DVT: 32-wide tiles that cover the width of V
-template <int DK, int DVT>
+// DK: width of Q and K (a multiple of 8); DVT: 32-wide tiles of V; R4: groups of 4 more dims of V after those tiles.
+// Group g of them holds dims 32 DVT + R4 i + g, i < 4, so that a lane reads the R4 floats it feeds to the groups
+// (its i is lane % 4) with one load.
+template <int DK, int DVT, int R4>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) void attention_f32_kernel(AttentionParams p) {
-    constexpr int DV = 32 * DVT, KS = DK + 4, VS = DV + 4, HALF = DK / 2;  // row strides that spread the LDS banks
+    constexpr int DV = 32 * DVT + 4 * R4, KS = DK + 4, VS = DV + 4, HALF = DK / 2;  // row strides that spread the LDS banks
     static_assert(DK % 8 == 0 && BKEYS * 4 == THREADS, "unsupported shape");
     __shared__ __attribute__((aligned(16))) float Ks[BKEYS][KS];
     __shared__ __attribute__((aligned(16))) float Vs[BKEYS][VS];
@@ -83,6 +93,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
     for (int t = 0; t < DVT; t++)
 #pragma unroll
         for (int v = 0; v < 16; v++) oacc[t][v] = 0.0f;
+    floatx4 orem[R4 > 0 ? R4 : 1];  // [g][i]: dim 32 DVT + R4 i + g of the lane's own query, this half's share of the keys
+#pragma unroll
+    for (int g = 0; g < R4; g++) orem[g] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float row_max = -INFINITY, row_sum = 0.0f;  // row_sum: this half's share of the keys only
 
     fetch(0);
@@ -138,49 +151,65 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
 #pragma unroll
             for (int v = 0; v < 16; v++) block_max = fmaxf(block_max, st[j][v]);
         block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
-        const float new_max = fmaxf(row_max, block_max);
-        const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);  // 0 for the first block
-        row_max = new_max;
+        // The reference of the exponentials follows the maximum lazily: it moves, and what has been summed so far is
+        // scaled down, only when some query of the wave exceeds it by more than 2^8; until then the weights are up
+        // to 256 instead of up to 1. (The first block always moves it, from -inf.)
+        if (__any(block_max > row_max + 8.0f)) {
+            const float new_max = fmaxf(row_max, block_max);
+            const float alpha = __builtin_amdgcn_exp2f(row_max - new_max);  // 0 for the first block
+            row_max = new_max;
+            row_sum *= alpha;
+#pragma unroll
+            for (int t = 0; t < DVT; t++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) oacc[t][v] *= alpha;
+#pragma unroll
+            for (int g = 0; g < R4; g++) orem[g] *= alpha;
+        }
         float block_sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                st[j][v] = __builtin_amdgcn_exp2f(st[j][v] - new_max);
+                st[j][v] = __builtin_amdgcn_exp2f(st[j][v] - row_max);
                 block_sum += st[j][v];
             }
-        row_sum = row_sum * alpha + block_sum;
-#pragma unroll
-        for (int t = 0; t < DVT; t++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) oacc[t][v] *= alpha;
+        row_sum += block_sum;
 
         {
             // steps of the second product in groups of 4 keys (one per accumulator register v % 4)
             auto key_of = [&](int step) { return 32 * (step >> 4) + 8 * ((step & 15) >> 2) + 4 * h + (step & 3); };
-            float v_next[4][DVT];
+            constexpr int VT = DVT + R4;  // the last R4: the lane's floats of the remaining dims
+            float v_next[4][VT];
             auto read_v = [&](int step0) {
 #pragma unroll
-                for (int u = 0; u < 4; u++)
+                for (int u = 0; u < 4; u++) {
 #pragma unroll
                     for (int t = 0; t < DVT; t++) v_next[u][t] = Vs[key_of(step0 + u)][32 * t + c];
+#pragma unroll
+                    for (int g = 0; g < R4; g++) v_next[u][DVT + g] = Vs[key_of(step0 + u)][32 * DVT + R4 * (lane & 3) + g];
+                }
             };
             read_v(0);
 #pragma unroll
             for (int step0 = 0; step0 < 32; step0 += 4) {
-                float vv[4][DVT];
+                float vv[4][VT];
 #pragma unroll
                 for (int u = 0; u < 4; u++)
 #pragma unroll
-                    for (int t = 0; t < DVT; t++) vv[u][t] = v_next[u][t];
+                    for (int t = 0; t < VT; t++) vv[u][t] = v_next[u][t];
                 if (step0 + 4 < 32) read_v(step0 + 4);
                 __builtin_amdgcn_sched_barrier(0);
                 __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-                for (int u = 0; u < 4; u++)
+                for (int u = 0; u < 4; u++) {
 #pragma unroll
                     for (int t = 0; t < DVT; t++)
                         oacc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(vv[u][t], st[(step0 + u) >> 4][(step0 + u) & 15], oacc[t], 0, 0, 0);
+#pragma unroll
+                    for (int g = 0; g < R4; g++)
+                        orem[g] = __builtin_amdgcn_mfma_f32_4x4x1f32(vv[u][DVT + g], st[(step0 + u) >> 4][(step0 + u) & 15], orem[g], 0, 0, 0);
+                }
                 __builtin_amdgcn_s_setprio(0);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -200,6 +229,25 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) vo
                 if (d < p.dv) op[(long long) d * p.o_sn] = oacc[t][v] * inv;
             }
     }
+    if (R4 > 0) {
+        floatx4 total[R4 > 0 ? R4 : 1];
+#pragma unroll
+        for (int g = 0; g < R4; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) total[g][i] = orem[g][i] + __shfl_xor(orem[g][i], 32);
+        // both halves hold the sums now; half h stores groups g with g % 2 == h
+        if (query < p.lq) {
+            const float inv = 1.0f / row_sum;
+            float *op = (float *) p.o + bz1 * p.o_sb + bz2 * p.o_sb2 + (long long) query * p.o_sm;
+#pragma unroll
+            for (int g = 0; g < R4; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int d = 32 * DVT + R4 * i + g;
+                    if ((g & 1) == h && d < p.dv) op[(long long) d * p.o_sn] = total[g][i] * inv;
+                }
+        }
+    }
 }
 
 }  // namespace
@@ -212,21 +260,24 @@ int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream) {
     if (p.batch <= 0 || p.lq <= 0 || p.dv <= 0) return 0;
     if (!attention_supported(p.dk, p.dv) || p.lk <= 0 || p.batch > 65535 || p.batch_inner <= 0) return (int) hipErrorInvalidValue;
     const dim3 grid((unsigned) ((p.lq + BQ - 1) / BQ), (unsigned) p.batch), block(THREADS);
-    const bool wide = p.dv > 32;
+    // 32-wide tiles of V, and the groups of 4 dims after them (up to 16 dims; a second tile beyond that)
+    const int tiles = p.dv > 48 ? 2 : 1;
+    const int rem = p.dv > 32 && p.dv <= 48 ? (p.dv - 32 + 3) / 4 : 0;
+#define KN_LAUNCH_ATTENTION(DK) \
+    do { \
+        if (tiles == 2) hipLaunchKernelGGL((attention_f32_kernel<DK, 2, 0>), grid, block, 0, stream, p); \
+        else if (rem == 1) hipLaunchKernelGGL((attention_f32_kernel<DK, 1, 1>), grid, block, 0, stream, p); \
+        else if (rem == 2) hipLaunchKernelGGL((attention_f32_kernel<DK, 1, 2>), grid, block, 0, stream, p); \
+        else if (rem == 3) hipLaunchKernelGGL((attention_f32_kernel<DK, 1, 3>), grid, block, 0, stream, p); \
+        else if (rem == 4) hipLaunchKernelGGL((attention_f32_kernel<DK, 1, 4>), grid, block, 0, stream, p); \
+        else hipLaunchKernelGGL((attention_f32_kernel<DK, 1, 0>), grid, block, 0, stream, p); \
+    } while (0)
     switch (p.dk) {
-        case 32:
-            if (wide) hipLaunchKernelGGL((attention_f32_kernel<32, 2>), grid, block, 0, stream, p);
-            else hipLaunchKernelGGL((attention_f32_kernel<32, 1>), grid, block, 0, stream, p);
-            break;
-        case 40:
-            if (wide) hipLaunchKernelGGL((attention_f32_kernel<40, 2>), grid, block, 0, stream, p);
-            else hipLaunchKernelGGL((attention_f32_kernel<40, 1>), grid, block, 0, stream, p);
-            break;
-        default:
-            if (wide) hipLaunchKernelGGL((attention_f32_kernel<64, 2>), grid, block, 0, stream, p);
-            else hipLaunchKernelGGL((attention_f32_kernel<64, 1>), grid, block, 0, stream, p);
-            break;
+        case 32: KN_LAUNCH_ATTENTION(32); break;
+        case 40: KN_LAUNCH_ATTENTION(40); break;
+        default: KN_LAUNCH_ATTENTION(64); break;
     }
+#undef KN_LAUNCH_ATTENTION
     return (int) hipGetLastError();
 }
 

@@ -1253,6 +1253,24 @@ def attention_fused_narrow_v():
 
 
 @case
+def attention_fused_v_width_36():
+    """V four dims wider than a 32-wide tile: one group of four dims on the 4 x 4 matrix instruction; heads layout"""
+    return _attention_case(104, 3, 100, 150, 32, 36, "mul", "heads")
+
+
+@case
+def attention_fused_v_width_42():
+    """42 is 32 + three groups of four with two dims of padding; queries and keys in partial blocks"""
+    return _attention_case(105, 2, 150, 200, 40, 42, "div", "dense")
+
+
+@case
+def attention_fused_v_width_48():
+    """32 + four full groups, V stored transposed"""
+    return _attention_case(106, 2, 64, 128, 64, 48, "mul_left", "v_transposed")
+
+
+@case
 def attention_fused_many_blocks():
     """enough keys that the running maximum and sum are rescaled many times; large score range"""
     g, b, inputs, _ = _attention_case(103, 2, 256, 1000, 40, 40, "mul_left", "dense")
