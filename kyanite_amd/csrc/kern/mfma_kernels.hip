@@ -388,8 +388,10 @@ struct PlaneGeom {
 };
 
 // NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64); MI: the same along
-// the output channels (2 -> 128 channels per tile, 1 -> 64)
-template <int KH, int KW, int NJ, int MI>
+// the output channels (2 -> 128 channels per tile, 1 -> 64); RAGGED: the channel count is not a multiple of CB (the
+// 21 planes of a board game's input): the last slice takes zeros for the channels past the end, and the filter rows,
+// whose length is no multiple of 4 floats then, are read float by float.
+template <int KH, int KW, int NJ, int MI, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, PlaneGeom g) {
     constexpr int TN = 64 * NJ;  // positions per tile
     constexpr int BM = 64 * MI;  // output channels per tile
@@ -426,6 +428,7 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     // ---- B planes: what this thread moves per slice (the same places every slice, only the channel base moves)
     const float *b_src[PLANE_MAX_VEC];
     int b_dst[PLANE_MAX_VEC];  // -1: nothing to move
+    int b_channel[PLANE_MAX_VEC];  // inside the slice
 #pragma unroll
     for (int i = 0; i < PLANE_MAX_VEC; i++) {
         const int e = t + THREADS * i;
@@ -436,16 +439,18 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         const bool ok = e < g.n_vec && iy >= 0 && iy < H && img < p.batch;
         b_dst[i] = e < g.n_vec ? PLANE_SLACK + t1 * RS + PLANE_PAD + 4 * w4 : -1;
         b_src[i] = ok ? p.input + (((long long) img * C + c) * H + iy) * W + 4 * w4 : nullptr;
+        b_channel[i] = c;
     }
     // ---- A (filter) rows: K contiguous
     const float *a_src[A_ITERS];
-    int a_dst[A_ITERS];
+    int a_dst[A_ITERS], a_k[A_ITERS];  // a_k: the first of the 4 floats inside the slice
 #pragma unroll
     for (int i = 0; i < A_ITERS; i++) {
         // (consecutive lanes take consecutive filter rows, so that their transposing stores hit different banks)
         const int e = t + THREADS * i, q = e / BM, row = e - q * BM;
         a_src[i] = q < A_VEC && (m0 + row) < p.out_c ? p.filter + (long long) (m0 + row) * K + 4 * q : nullptr;
         a_dst[i] = q < A_VEC ? 4 * q * A_STRIDE + row : -1;
+        a_k[i] = 4 * q;
     }
     // ---- where this lane's output positions sit inside a plane, and which taps stay inside the image
     int lane_base[NJ];
@@ -459,6 +464,17 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     floatx4 ra[A_ITERS], rb[PLANE_MAX_VEC];
     auto fetch = [&](int c0) {
         const long long a_off = (long long) c0 * KH * KW, b_off = (long long) c0 * ohw;
+        if (RAGGED) {
+#pragma unroll
+            for (int i = 0; i < A_ITERS; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    ra[i][j] = a_src[i] && a_off + a_k[i] + j < K ? (a_src[i] + a_off)[j] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < PLANE_MAX_VEC; i++)
+                rb[i] = b_src[i] && c0 + b_channel[i] < C ? *(const floatx4 *) (b_src[i] + b_off) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < A_ITERS; i++)
             ra[i] = a_src[i] ? *(const floatx4 *) (a_src[i] + a_off) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -578,7 +594,8 @@ int log2_exact(int x) {
 bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     if (p.kernel_h != 3 || p.kernel_w != 3 || p.stride_y != 1 || p.stride_x != 1) return false;
     if (p.pad_y != 1 || p.pad_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
-    if (p.in_c % CB != 0 || (uintptr_t) p.input % 16 != 0 || (uintptr_t) p.filter % 16 != 0) return false;
+    // (a channel count that is no multiple of CB runs on the variant that reads the filter float by float)
+    if (p.in_c <= 0 || (uintptr_t) p.input % 16 != 0 || (p.in_c % CB == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
     const int W = p.in_w, H = p.in_h;
     if (W < 4 || W > tn || log2_exact(W) < 0) return false;
     const long long hw = (long long) H * W;
@@ -780,8 +797,11 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
         plane_geometry(p, best->tn, &geom);
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
         const dim3 grid((unsigned) tiles), block(THREADS);
-        if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2>), grid, block, 0, stream, p, geom);
-        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1>), grid, block, 0, stream, p, geom);
+        const bool ragged = p.in_c % CB != 0;
+        if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true>), grid, block, 0, stream, p, geom);
+        else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false>), grid, block, 0, stream, p, geom);
+        else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true>), grid, block, 0, stream, p, geom);
+        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false>), grid, block, 0, stream, p, geom);
         return (int) hipGetLastError();
     }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
