@@ -660,14 +660,25 @@ __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p,
     float total[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; j++) total[j] = 0.0f;
-    for (int s = 0; s < split; s++) {
-        if (VEC == 4) {
+    if (VEC == 4) {
+        // four parts requested at a time (the order of the sum stays that of K)
+        int s = 0;
+        for (; s + 4 <= split; s += 4) {
+            floatx4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = *(const floatx4 *) (part + (s + u) * mn);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int j = 0; j < VEC; j++) total[j] += v[u][j];
+        }
+        for (; s < split; s++) {
             const floatx4 v = *(const floatx4 *) (part + s * mn);
 #pragma unroll
             for (int j = 0; j < VEC; j++) total[j] += v[j];
-        } else {
-            total[0] += part[s * mn];
         }
+    } else {
+        for (int s = 0; s < split; s++) total[0] += part[s * mn];
     }
     const long long row = e / p.n, col = e - row * p.n;
     OutT *out = (OutT *) p.c + bz * p.c_sb + row * p.c_sm + col * p.c_sn;
@@ -675,11 +686,26 @@ __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p,
     const OutT *addend2 = p.addend2 ? (const OutT *) p.addend2 + bz * p.d2_sb + row * p.d2_sm + col * p.d2_sn : nullptr;
     // (the addends are requested before the first store: a load may not pass a store that might alias it)
     OutT d[VEC], d2[VEC];
+    typedef OutT OutVec __attribute__((ext_vector_type(VEC)));
+    // contiguous, aligned columns move as one vector
+    auto as_vector = [](const OutT *ptr, long long stride) { return VEC > 1 && stride == 1 && (uintptr_t) ptr % (VEC * sizeof(OutT)) == 0; };
+    if (addend && as_vector(addend, p.d_sn)) {
+        const OutVec v = *(const OutVec *) addend;
 #pragma unroll
-    for (int j = 0; j < VEC; j++) {
-        d[j] = addend ? addend[j * p.d_sn] : (OutT) 0;
-        d2[j] = addend2 ? addend2[j * p.d2_sn] : (OutT) 0;
+        for (int j = 0; j < VEC; j++) d[j] = v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) d[j] = addend ? addend[j * p.d_sn] : (OutT) 0;
     }
+    if (addend2 && as_vector(addend2, p.d2_sn)) {
+        const OutVec v = *(const OutVec *) addend2;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) d2[j] = v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) d2[j] = addend2 ? addend2[j * p.d2_sn] : (OutT) 0;
+    }
+    OutVec result;
 #pragma unroll
     for (int j = 0; j < VEC; j++) {
         // rounding to the output type after the product and after the sum, like separate operations would
@@ -687,7 +713,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_partials_kernel(GemmParams p,
         if (addend) v = (float) (OutT) (v + (float) d[j]);
         if (addend2) v = (float) (OutT) (v + (float) d2[j]);
         if (p.relu) v = fmaxf(v, 0.0f);
-        out[j * p.c_sn] = (OutT) v;
+        result[j] = (OutT) v;
+    }
+    if (as_vector(out, p.c_sn)) {
+        *(OutVec *) out = result;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) out[j * p.c_sn] = result[j];
     }
 }
 
