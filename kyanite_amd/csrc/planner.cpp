@@ -812,6 +812,8 @@ private:
                 return R::done(std::nullopt);
             // a block of 64 keys is addressed with 32 bit offsets from the block's base
             if (ks[3] < 0 || ks[3] > (1 << 20) || vs[2] < 0 || vs[2] > (1 << 20)) return R::done(std::nullopt);
+            // the 32 queries of a workgroup are addressed with 32 bit byte offsets from the batch entry's base
+            if (qs[2] < 0 || (long long) lq * qs[2] >= (1ll << 30)) return R::done(std::nullopt);
         } else {
             // the kernel addresses a block of 64 keys with 32 bit offsets from the block's base
             auto fits = [](const PlanTensor &t) {
