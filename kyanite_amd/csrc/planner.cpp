@@ -159,6 +159,13 @@ public:
         return r.value;
     }
 
+    // (kernels are compiled when the whole plan stands: steps may still be joined until then)
+    void compile_steps() {
+        if (!options.compile) return;
+        for (Step &step : steps)
+            if (step.kind != StepKind::Conv && step.kind != StepKind::MatMul) step.code = compile_kernel(step.kernel.source);
+    }
+
 private:
     VT visit(Value value) {
         auto it = map.find(value);
@@ -203,9 +210,57 @@ private:
         step.debug_id = graph[debug_value].debug_id;
         if (step.kind != StepKind::Conv && step.kind != StepKind::MatMul) {
             if (step.kernel.grid == 0) return;  // nothing to compute (empty tensors)
-            if (options.compile) step.code = compile_kernel(step.kernel.source);
+            if (step.kind == StepKind::ScalarOp && !steps.empty() && try_join_elementwise(steps.back(), step)) return;
         }
         steps.push_back(std::move(step));
+    }
+
+    // Two elementwise steps in a row that walk the same shape and do not touch each other's tensors - the rotary
+    // embeddings of q and of k - become one launch with the outputs of both: small kernels cost their launch and one
+    // round trip to memory each, whatever they compute. Large ones, which run at the rate of the memory, stay apart.
+    bool try_join_elementwise(Step &prev, const Step &next) {
+        constexpr size_t max_elements = 1u << 22, max_outputs = 4, max_operands = 12;
+        if (!options.join_elementwise || prev.kind != StepKind::ScalarOp || prev.scalar_exprs.empty() || next.scalar_exprs.empty()) return false;
+        const auto &shape = prev.operands[0].tensor.shape.shape();
+        if (next.operands[0].tensor.shape.shape() != shape || concrete_size(shape) > max_elements) return false;
+        const size_t out_a = prev.scalar_exprs.size(), out_b = next.scalar_exprs.size();
+        if (out_a + out_b > max_outputs) return false;
+        auto same_buffer = [](const PlanTensor &x, const PlanTensor &y) { return x.ptr.kind == y.ptr.kind && x.ptr.index == y.ptr.index; };
+        // neither reads or writes what the other writes
+        for (size_t i = 0; i < prev.operands.size(); i++)
+            for (size_t j = 0; j < next.operands.size(); j++)
+                if ((i < out_a || j < out_b) && same_buffer(prev.operands[i].tensor, next.operands[j].tensor)) return false;
+        std::vector<PlanTensor> operands;
+        for (size_t i = 0; i < out_a; i++) operands.push_back(prev.operands[i].tensor);
+        for (size_t j = 0; j < out_b; j++) operands.push_back(next.operands[j].tensor);
+        const size_t n_out = out_a + out_b;
+        std::vector<ScalarExpr> exprs;
+        auto take = [&](const Step &from, size_t own_outputs) {
+            for (ScalarExpr expr : from.scalar_exprs) {
+                for (auto &node : expr.nodes) {
+                    if (node.kind != ScalarNode::Load) continue;
+                    KN_ASSERT(node.operand >= own_outputs && node.operand < from.operands.size());
+                    const PlanTensor &t = from.operands[node.operand].tensor;
+                    size_t at = n_out;
+                    while (at < operands.size() && !(operands[at] == t)) at++;
+                    if (at == operands.size()) operands.push_back(t);
+                    node.operand = at;
+                }
+                exprs.push_back(std::move(expr));
+            }
+        };
+        take(prev, out_a);
+        take(next, out_b);
+        if (operands.size() > max_operands) return false;
+        std::vector<KernelOperand> kops;
+        for (auto &t : operands) kops.push_back(kop(t));
+        KernelSpec joined = make_scalar_kernel_multi(kops, exprs);
+        if (joined.grid == 0) return false;
+        prev.kernel = std::move(joined);
+        prev.scalar_exprs = std::move(exprs);
+        prev.operands.clear();
+        for (size_t k = 0; k < operands.size(); k++) prev.operands.push_back({operands[k], k < n_out ? OperandKind::Out : OperandKind::In});
+        return true;
     }
 
     static KernelOperand kop(const PlanTensor &t) { return KernelOperand{t.dtype, t.shape, t.ptr.offset_bytes}; }
@@ -339,6 +394,7 @@ private:
                         Step step;
                         step.kind = StepKind::ScalarOp;
                         step.kernel = make_scalar_kernel_multi(kops, exprs);
+                        step.scalar_exprs = exprs;
                         for (size_t k = 0; k < operands.size(); k++)
                             step.operands.push_back({operands[k], k < n_out ? OperandKind::Out : OperandKind::In});
                         push(std::move(step), pending[0].value);
@@ -1492,6 +1548,7 @@ private:
         Step step;
         step.kind = StepKind::ScalarOp;
         step.kernel = make_scalar_kernel(kops, expr);
+        step.scalar_exprs = {expr};
         step.operands.push_back({operands[0], OperandKind::Out});
         for (size_t k = 1; k < operands.size(); k++) step.operands.push_back({operands[k], OperandKind::In});
         push(std::move(step), debug_value);
@@ -1509,6 +1566,8 @@ Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &opt
     // allocate inputs (even if they are not actually used), then plan everything the outputs need
     for (Value in : graph.inputs) plan.inputs.push_back(planner.visit_completely(in));
     for (Value out : graph.outputs) plan.outputs.push_back(planner.visit_completely_ensure_simple_strides(out));
+
+    planner.compile_steps();
 
     size_t buffer_count = planner.shared_sizes.size();
     size_t step_count = planner.steps.size();

@@ -33,6 +33,9 @@ struct Step {
     // run-time compiled kernels
     KernelSpec kernel;
     std::shared_ptr<const CodeObject> code;
+    // ScalarOp steps: the expression of every output (operands: the outputs first, then what is loaded), kept so that
+    // neighbouring elementwise steps of one shape can still be joined into one launch
+    std::vector<ScalarExpr> scalar_exprs;
     // matrix-core kernels; the pointers are filled in when the plan is realised
     GemmParams gemm{};
     bool gemm_f16 = false;  // element type of a MatMul step: f16 (f32 accumulation) instead of f32
@@ -92,6 +95,7 @@ struct PlannerOptions {
     bool pack_matmul_constants = true;  // constant [k, n] right operands of f16 matmuls are laid out again as [n, k]
     bool group_matmuls = true;   // matmuls that share their left operand and have constant right operands share a launch
     bool pointwise_conv_as_matmul = true;  // 1 x 1 convolutions with stride 1 run as one matrix product per image
+    bool join_elementwise = true;  // small elementwise steps of one shape that do not depend on each other share a launch
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
 };

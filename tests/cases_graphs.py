@@ -1634,6 +1634,30 @@ def attention_f16_mask_on_the_left_no_scale():
 
 
 @case
+def rotary_of_two_tensors_is_one_launch():
+    """two rotary embeddings (two concats of two elementwise halves each) over different inputs and the same cos / sin:
+    four results from one launch; a third chain that reads one of the results stays a launch of its own"""
+    g = Graph()
+    rng = np.random.default_rng(141)
+    cos = g.broadcast(g.constant([1, 24, 16], np.cos(rng.standard_normal((1, 24, 16))).astype(np.float32)), [5, 24, 16])
+    sin = g.broadcast(g.constant([1, 24, 16], np.sin(rng.standard_normal((1, 24, 16))).astype(np.float32)), [5, 24, 16])
+
+    def rotary(x1, x2):
+        return g.concat([g.sub(g.mul(x1, cos), g.mul(x2, sin)), g.add(g.mul(x1, sin), g.mul(x2, cos))], 2)
+
+    q = rotary(g.input([5, 24, 16]), g.input([5, 24, 16]))
+    k = rotary(g.input([5, 24, 16]), g.input([5, 24, 16]))
+    g.output(q)
+    g.output(k)
+    g.output(g.unary(UnaryOp.TANH, g.add(q, k)))
+    inputs = [rng.standard_normal((5, 24, 16)).astype(np.float32) for _ in range(4)]
+    from kyanite_amd import HipExecutor
+    ex = HipExecutor(0, g, 0, plan_only=True)
+    assert ex.step_kinds() == ["scalar_op", "scalar_op"] and "outputs=4" in ex.step_str(0), [ex.step_str(i) for i in range(ex.step_count())]
+    return g, 0, inputs, None
+
+
+@case
 def concat_pieces_share_a_launch():
     """pieces of a concat that are elementwise chains of one shape are computed by ONE kernel with several outputs
     (a rotary embedding's two halves); a piece of another shape and a plain tensor in between get their own"""
