@@ -71,10 +71,15 @@ int knhip_host_alloc(size_t bytes, void **ptr);
 int knhip_host_free(void *ptr);
 int knhip_device_synchronize(int device);
 /* No counterpart in the reference. What the matrix cores of the device sustain when nothing else limits them: a
- * register-only loop of independent f16 MFMAs on one wave per SIMD, with small integers (normal_data = 0) or N(0, 1)
- * values (normal_data = 1) in the operands, and the shader clock it ran at. The rate on N(0, 1) data is the ceiling
- * that matmul / convolution rates on real data should be read against (the clock drops under the power they draw). */
-int knhip_device_mfma_probe(int device, int normal_data, int iterations, double *tflops, double *shader_mhz);
+ * register-only loop of independent MFMAs on one wave per SIMD and the shader clock it ran at. `mode` is a sum of
+ * KNHIP_PROBE_NORMAL (operands N(0, 1) instead of small integers), KNHIP_PROBE_F32 (v_mfma_f32_32x32x2_f32 instead
+ * of v_mfma_f32_32x32x16_f16) and KNHIP_PROBE_RECTIFIED (the B operands max(x, 0), like activations after a relu).
+ * The rate on N(0, 1) data is the ceiling that matmul / convolution rates on real data should be read against (the
+ * clock drops under the power they draw). */
+#define KNHIP_PROBE_NORMAL 1
+#define KNHIP_PROBE_F32 2
+#define KNHIP_PROBE_RECTIFIED 4
+int knhip_device_mfma_probe(int device, int mode, int iterations, double *tflops, double *shader_mhz);
 
 /* streams and events (replaces CudaStream, kn-cuda-sys/src/wrapper/handle.rs:105-174, and CudaEvent, event.rs:7-45).
  * Handles are the HIP objects themselves (hipStream_t / hipEvent_t behind void *); a NULL stream is the device's

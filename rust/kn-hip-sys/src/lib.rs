@@ -66,6 +66,10 @@ pub const KNHIP_PLAN_ONLY: c_int = 1;
 pub const KNHIP_PRESERVE_INPUTS: c_int = 2;
 pub const KNHIP_STEP_BY_STEP: c_int = 4;
 
+pub const KNHIP_PROBE_NORMAL: c_int = 1;
+pub const KNHIP_PROBE_F32: c_int = 2;
+pub const KNHIP_PROBE_RECTIFIED: c_int = 4;
+
 pub const KNHIP_F32: c_int = 0;
 pub const KNHIP_F64: c_int = 1;
 pub const KNHIP_I8: c_int = 2;
@@ -95,7 +99,7 @@ extern "C" {
     pub fn knhip_host_alloc(bytes: usize, ptr: *mut *mut c_void) -> c_int;
     pub fn knhip_host_free(ptr: *mut c_void) -> c_int;
     pub fn knhip_device_synchronize(device: c_int) -> c_int;
-    pub fn knhip_device_mfma_probe(device: c_int, normal_data: c_int, iterations: c_int, tflops: *mut f64, shader_mhz: *mut f64) -> c_int;
+    pub fn knhip_device_mfma_probe(device: c_int, mode: c_int, iterations: c_int, tflops: *mut f64, shader_mhz: *mut f64) -> c_int;
 
     // streams, events, asynchronous copies
     pub fn knhip_stream_create(device: c_int, stream: *mut *mut c_void) -> c_int;
