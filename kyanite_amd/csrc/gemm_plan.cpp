@@ -16,6 +16,75 @@ int env_int(const char *name, int fallback) {
     return env && *env ? atoi(env) : fallback;
 }
 
+// ---- Cost model of the f16 kernel that loads global -> LDS directly.
+//
+// What a compute unit can do per slice of 64 along K is bounded by the 128 byte lines it can request - it keeps
+// about 64 of them in flight, so a line costs latency / 64 of its time, whoever asked for it - and by its matrix
+// cores. A workgroup with a TM x TN tile asks for TM + TN lines per slice and issues TM * TN * 64 multiply-adds; a
+// launch is as slow as the busiest compute unit: rounds of workgroups, each round its slices plus a fixed cost
+// (first slice's round trip, epilogue), plus the pass that sums the parts when K is split. The constants were fitted
+// (least squares on log time) to 780 timings of forced tile / split combinations over 38 shapes from 1 x 4096 x 4096
+// to 8192 x 8192 x 1024 with weights that do not stay in cache; the model's choice is within 1.5 % of the best
+// measured combination on average and 15 % at worst, where the thresholds it replaces were 10 % and 53 % off.
+struct F16Tile {
+    int tm, tn;
+    int per_cu;          // workgroups of this tile a compute unit holds at a time
+    double ns_per_line;  // fitted; 1.8 to 2.6 ns = 4.5 to 6 cycles: the 300 to 400 cycles of a request over 64 in flight
+};
+constexpr int F16_TILES = 6;
+const F16Tile f16_tiles[F16_TILES] = {
+    {64, 64, 2, 1.998}, {128, 64, 1, 1.849}, {128, 128, 2, 2.572}, {256, 128, 1, 2.196}, {256, 192, 1, 2.396}, {256, 256, 1, 2.590},
+};
+enum { TILE_SMALL = 0, TILE_NARROW = 1, TILE_PLAIN = 2, TILE_TALL = 3, TILE_MID = 4, TILE_WIDE = 5 };
+constexpr double MFMA_EFFICIENCY = 0.745;    // of 2500 TFLOP/s: what the matrix cores sustain on real data
+constexpr double WORKGROUP_FIXED_US = 3.26;  // per round: first round trip to memory, epilogue ...
+constexpr double WORKGROUP_TILE_US = 1.53;   // ... and the part of it that grows with the tile (per 128 x 128 outputs)
+constexpr double LAUNCH_US = 1.14;
+constexpr double SHARED_CU_FACTOR = 0.87;    // two workgroups on a compute unit overlap a little of each other's waits
+constexpr double SUM_PASS_US = 2.31, SUM_PASS_US_PER_MB = 0.255;  // the pass that sums split-K parts
+constexpr int COMPUTE_UNITS = 256;
+
+// parts of the last, sparse round of tiles (0: the round is not split), see plan_gemm_launch
+int tail_parts(long long blocks, long long slots, int k) {
+    const long long full = blocks / slots * slots, rest = blocks - full;
+    long long s = rest > 0 ? slots / rest : 1;
+    if (s > k / 512) s = k / 512;
+    if (s > 16) s = 16;
+    if (!(full > 0 && rest * 100 < slots * 85 && s >= 2 && blocks <= 0x3fffffff)) return 0;
+    long long chunk = (k + s - 1) / s;
+    chunk = (chunk + 63) / 64 * 64;
+    s = (k + chunk - 1) / chunk;
+    return s >= 2 ? (int) s : 0;
+}
+
+double estimate_f16_direct_us(const GemmParams &p, int groups, int tile, int split, bool tail_allowed) {
+    const F16Tile &t = f16_tiles[tile];
+    const long long tiles = (long long) ((p.m + t.tm - 1) / t.tm) * ((p.n + t.tn - 1) / t.tn) * groups * p.batch;
+    long long chunk = p.k;
+    if (split > 1) chunk = ((p.k + split - 1) / split + 63) / 64 * 64;
+    const long long parts = (p.k + chunk - 1) / chunk, workgroups = tiles * parts;
+    const double slices = (double) chunk / 64.0;
+    const double mfma_us = (double) t.tm * t.tn * 64 * 2 / (2500e12 / COMPUTE_UNITS * MFMA_EFFICIENCY) * 1e6;
+    const double fixed_us = WORKGROUP_FIXED_US + WORKGROUP_TILE_US * t.tm * t.tn / 16384.0;
+    auto round_us = [&](long long per_cu, double slices_here) {
+        double per_slice = std::max((double) per_cu * (t.tm + t.tn) * t.ns_per_line * 1e-3, (double) per_cu * mfma_us);
+        if (per_cu > 1) per_slice *= SHARED_CU_FACTOR;
+        return slices_here * per_slice + fixed_us;
+    };
+    const long long capacity = (long long) COMPUTE_UNITS * t.per_cu;
+    const long long full = workgroups / capacity, rest = workgroups % capacity;
+    double us = LAUNCH_US + (double) full * round_us(t.per_cu, slices);
+    if (rest > 0) {
+        const long long per_cu = (rest + COMPUTE_UNITS - 1) / COMPUTE_UNITS;
+        const int tail = tail_allowed && parts == 1 && p.batch == 1 ? tail_parts(tiles, capacity, p.k) : 0;
+        // a round split into `tail` parts of K: measured at 0.78 of a whole round for two parts (the parts pass
+        // f32 tiles to each other through memory)
+        us += tail ? round_us(per_cu, slices) * (1.0 / tail + 0.28) : round_us(per_cu, slices);
+    }
+    if (parts > 1) us += SUM_PASS_US + SUM_PASS_US_PER_MB * (double) p.batch * p.m * p.n * (4.0 * parts + 4.0) / 1e6;
+    return us;
+}
+
 }  // namespace
 
 GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
@@ -67,48 +136,52 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     const long long tall_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 127) / 128) * p.batch * groups;
     const bool tall_fits = !lp.small_tile && p.m >= 256 && (p.m + 255) / 256 * 256 - p.m <= p.m / 8;
     lp.tall_tile = f16 && groups == 1 && tall_fits && can_split && p.k >= 2048 && tall_blocks < tall_below;
-    // Both operands with K contiguous in whole 16 byte vectors and K in whole slices of 64: given aligned
-    // pointers, the launch takes the kernel that loads global -> LDS directly. There the tall tiles run on a ring
-    // of three stages and also pay without a split, as long as they still fill the chip. Measured with weights
-    // that come from memory, not from cache (us, 128 x 128 on two stages against 256 x 128 on three):
-    // 512 x 22016 x 4096 147 / 133, 512 x 12288 x 4096 93 / 72, 4096^3 152 / 144; 512 x 4096 x 4096 53 / 59.
-    // (In f32 the same kernel walks K in slices of 32 and has 128 x 128 and 64 x 64 tiles.)
+    // Both operands with K contiguous in whole 16 byte vectors and K in whole slices of 64 (f32: 32): given aligned
+    // pointers, the launch takes the kernel that loads global -> LDS directly. In f32 that kernel has the 128 x 128
+    // and 64 x 64 tiles chosen above; in f16 it has six tiles, chosen below.
     const int vec = f16 ? 8 : 4;
     // (row strides: positive and small enough for the 32 bit byte offsets that the kernel keeps per lane within a tile)
     constexpr long long max_row_stride = 1ll << 21;
     lp.direct = p.k > 0 && p.k % (8 * vec) == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % vec == 0 && p.b_sn % vec == 0 &&
                 p.a_sm > 0 && p.b_sn > 0 && p.a_sm < max_row_stride && p.b_sn < max_row_stride &&
                 (p.batch <= 1 || (p.a_sb % vec == 0 && p.b_sb % vec == 0));
-    if (f16 && lp.direct && tall_fits && tall_blocks >= 128) lp.tall_tile = true;
-    // Direct kernel only: 128 x 64 tiles on a ring of four stages, where 128 x 128 tiles leave compute units
-    // without a workgroup and K is too short for a split to pay (512 x 4096 x 4096: 29 us against 39 us on
-    // 256 x 128 tiles split in four; 512 x 4096 x 11008: 84 us against 69 us).
     const long long narrow_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 63) / 64) * p.batch * groups;
-    lp.narrow_tile = f16 && lp.direct && !narrow && p.m > 64 && big_blocks < 256 && narrow_blocks >= 192 &&
-                     p.k < 8192;
-    if (lp.narrow_tile) lp.small_tile = lp.tall_tile = false;
-    // Direct kernel only: 256 x 256 tiles (8 waves of 128 x 64) where they still give every compute unit a
-    // workgroup. The LDS bounds this kernel, and they need the least LDS traffic per flop: 256 KB per slice of 64
-    // for twice the work of a 256 x 128 tile with its 176 KB (8192^3: 1191 -> 1030 us, 4096^3: 166 -> 139 us).
-    // Between the two sit 256 x 192 tiles (216 KB per slice for one and a half times the work). Among the three
-    // the plan takes the one with the least estimated LDS time: rounds of workgroups on 256 compute units (a last
-    // sparse round counts as one split in two) x LDS clocks per slice. 2 x 512 x 11008 x 4096 in one launch:
-    // 344 tiles of 256 x 128 are 1.6 rounds of 2750 clocks, 232 tiles of 256 x 192 one round of 3375.
     const long long wide_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 255) / 256) * p.batch * groups;
     const long long mid_blocks = (long long) ((p.m + 255) / 256) * ((p.n + 191) / 192) * p.batch * groups;
-    if (f16 && lp.direct && lp.tall_tile) {
-        auto lds_time = [&](long long tiles, double clocks) {
-            const long long full = tiles / 256, rest = tiles % 256;
-            double rounds = (double) full;
-            if (rest > 0) rounds += full > 0 && rest <= 128 && p.batch == 1 && p.k >= 1024 ? 0.6 : 1.0;
-            return rounds * clocks;
-        };
-        auto fits = [&](int width) { return p.n >= width && (p.n + width - 1) / width * width - p.n <= p.n / 8; };
-        const double t_tall = lds_time(tall_blocks, 2750.0);
-        const double t_mid = fits(192) ? lds_time(mid_blocks, 3375.0) : 1e30;
-        const double t_wide = fits(256) && wide_blocks >= 256 ? lds_time(wide_blocks, 4000.0) : 1e30;
-                lp.wide_tile = t_wide <= t_tall && t_wide <= t_mid;
-        lp.mid_tile = !lp.wide_tile && t_mid < t_tall;
+    // The direct f16 kernel takes tile and split from the cost model (estimate_f16_direct_us): the cheapest of
+    // 64 x 64, 128 x 64, 128 x 128, 256 x 128, 256 x 192 and 256 x 256 tiles with K in 1 to 16 parts. On the shapes of
+    // a 512 token LLaMA layer that is 256 x 192 for gate + up (232 tiles: one round), 256 x 128 for q + k + v,
+    // 256 x 128 with K in four parts for down, 128 x 64 for o - what sweeps over those shapes had arrived at before -
+    // and on shapes nobody swept it is what the thresholds it replaces were not: 256 x 4096 x 4096 22 us instead of
+    // 30 us, 512 x 512 x 4096 13 / 20, 768 x 768 x 3072 16 / 20, 8192 x 320 x 1280 20 / 25, 512 x 32000 x 4096 166 / 187.
+    static const int tail_enabled = env_int("KNHIP_TAIL_SPLIT", 1);
+    int model_split = 0;
+    if (f16 && lp.direct) {
+        int best_tile = TILE_SMALL, best_split = 1;
+        double best_us = 0.0;
+        static const int split_choices[] = {1, 2, 3, 4, 6, 8, 12, 16};
+        for (int tile = 0; tile < F16_TILES; tile++) {
+            const F16Tile &t = f16_tiles[tile];
+            if ((t.tm == 256 && p.m <= 128) || (tile == TILE_NARROW && p.m <= 64)) continue;
+            for (int split : split_choices) {
+                if (split > 1) {
+                    const unsigned long long bytes = (unsigned long long) split * p.batch * p.m * p.n * 4ull;
+                    if (!split_enabled || groups > 1 || p.k / split < 256 || bytes > (256ull << 20)) continue;
+                }
+                const double us = estimate_f16_direct_us(p, groups, tile, split, tail_enabled && split_enabled);
+                if (best_us == 0.0 || us < best_us) {
+                    best_us = us;
+                    best_tile = tile;
+                    best_split = split;
+                }
+            }
+        }
+        lp.small_tile = best_tile == TILE_SMALL;
+        lp.narrow_tile = best_tile == TILE_NARROW;
+        lp.tall_tile = best_tile >= TILE_TALL;
+        lp.mid_tile = best_tile == TILE_MID;
+        lp.wide_tile = best_tile == TILE_WIDE;
+        model_split = best_split;
     }
     long long blocks = lp.small_tile ? small_blocks : big_blocks;
     if (lp.tall_tile) blocks = tall_blocks;
@@ -126,28 +199,37 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // pass between workgroups with accesses that bypass the L2 caches, which costs more than the second launch
     // of a plain split; so a launch with less than one round of tiles keeps that (512 x 4096 x 11008: 69 us
     // against 82 us).
-    static const int tail_enabled = env_int("KNHIP_TAIL_SPLIT", 1);
-    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled) {
+    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled && model_split <= 1) {
         const long long slots = 256 * (lp.tall_tile || lp.narrow_tile ? 1 : 2);
         const long long full = blocks / slots * slots, rest = blocks - full;
-        long long s = rest > 0 ? slots / rest : 1;
-        if (s > p.k / 512) s = p.k / 512;
-        if (s > 16) s = 16;
-        if (full > 0 && rest * 100 < slots * 85 && s >= 2 && blocks <= 0x3fffffff) {
-            long long chunk = (p.k + s - 1) / s;
+        const int parts = tail_parts(blocks, slots, p.k);
+        if (parts >= 2) {
+            long long chunk = (p.k + parts - 1) / parts;
             chunk = (chunk + 63) / 64 * 64;
-            s = (p.k + chunk - 1) / chunk;
             const int tm = lp.tall_tile ? 256 : (lp.small_tile ? 64 : 128), tn = lp.small_tile || lp.narrow_tile ? 64 : (lp.wide_tile ? 256 : (lp.mid_tile ? 192 : 128));
-            const unsigned long long bytes = (unsigned long long) rest * s * tm * tn * 4ull;
-            if (s >= 2 && bytes <= (256ull << 20)) {
+            const unsigned long long bytes = (unsigned long long) rest * parts * tm * tn * 4ull;
+            if (bytes <= (256ull << 20)) {
                 lp.head_tiles = (int) full;
-                lp.tail_split = (int) s;
+                lp.tail_split = parts;
                 lp.tail_k_chunk = (int) chunk;
                 lp.workspace_bytes = (size_t) bytes;
                 lp.counter_bytes = (size_t) rest * 4;
                 return lp;
             }
         }
+    }
+    if (f16 && lp.direct) {
+        if (model_split > 1) {
+            long long chunk = (p.k + model_split - 1) / model_split;
+            chunk = (chunk + lp.bk - 1) / lp.bk * lp.bk;
+            const long long parts = (p.k + chunk - 1) / chunk;
+            if (parts > 1) {
+                lp.split_k = (int) parts;
+                lp.k_chunk = (int) chunk;
+                lp.workspace_bytes = (size_t) ((unsigned long long) parts * p.batch * p.m * p.n * 4ull);
+            }
+        }
+        return lp;
     }
 
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;

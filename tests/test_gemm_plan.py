@@ -218,3 +218,29 @@ def test_constant_attention_masks_are_classified_by_block():
     ex = HipExecutor(0, g, batch, plan_only=True)
     steps = [ex.step_str(i) for i in range(ex.step_count())]
     assert any("attention f16 +mask" in s for s in steps) and not any("classified" in s for s in steps), steps
+
+
+def test_f16_tiles_come_from_the_cost_model():
+    """the tile and the split of K of the f16 kernel that loads global -> LDS directly: what the cost model of
+    gemm_plan.cpp picks on shapes that were timed with every tile and split forced (us of the pick / of the
+    thresholds it replaced, where they differ)"""
+    expected = {
+        (512, 11008, 4096): "direct 256x128 bk64]",
+        (512, 4096, 4096): "direct 128x64 bk64]",
+        (512, 4096, 11008): "direct 256x128 bk64 split_k=4x2752]",
+        (512, 22016, 4096): "direct 256x192 bk64]",
+        (4096, 4096, 4096): "direct 256x256 bk64]",
+        (512, 32000, 4096): "direct 256x256 bk64]",            # 166 / 187
+        (2048, 2048, 2048): "direct 128x128 bk128]",           # 29 / 34
+        (256, 4096, 4096): "direct 64x64 bk64]",               # 22 / 30
+        (512, 512, 4096): "direct 64x64 bk64 split_k=4x1024]",  # 13 / 20
+        (768, 768, 3072): "direct 128x64 bk64 split_k=3x1024]",  # 16 / 20
+        (8192, 320, 1280): "direct 128x128 bk128]",            # 20 / 25
+    }
+    for (m, n, k), want in expected.items():
+        g = Graph()
+        x = g.input([m, k], DType.F16)
+        g.output(g.linear(x, g.input([n, k], DType.F16)))
+        ex = HipExecutor(0, g, 0, plan_only=True)
+        text = [ex.step_str(i) for i in range(ex.step_count()) if "MatMul" in ex.step_str(i)][0]
+        assert want in text, (m, n, k, text)

@@ -1,8 +1,9 @@
 """The in-launch K split of the direct matmul kernel (the tiles of a sparse last round of workgroups are shared by
 2..16 workgroups that exchange f32 partial tiles and count themselves in on a per-tile counter) in every
-instantiation the launch plan can pick: f32 on 64 x 64 and 128 x 128 tiles, f16 on 64 x 64, 128 x 64, 128 x 128,
-256 x 128, 256 x 192 and 256 x 256 tiles, splits of 2, 3, 4 and 8, epilogues (bias, residual, relu) and grouped
-launches. The GPU multiplies the whole product, twice (the second run finds the counters as the first left them); the
+instantiation the launch plan picks: f32 on 64 x 64 and 128 x 128 tiles, f16 on 64 x 64, 128 x 64, 256 x 192 and
+256 x 256 tiles (with the f16 cost model a sparse last round of 128 x 128 or 256 x 128 tiles never comes out cheapest:
+a larger tile that fits one round does), splits of 2, 3, 4 and 8, epilogues (bias, residual, relu), ragged tile rows
+and grouped launches. The GPU multiplies the whole product, twice (the second run finds the counters as the first left them); the
 oracle evaluates the same graph on a sample of the rows of the left operand that reaches every tile row of every
 workgroup tile, and those rows of the GPU result are compared with it."""
 import numpy as np
@@ -21,12 +22,12 @@ CASES = [
     (DType.F16, 33, 33280, 4096, (False, False, False), 1, "direct 64x64 bk64 head=512 tail_split=8x512"),
     (DType.F16, 256, 8320, 2048, (True, False, True), 1, "direct 128x64 bk64 head=256 tail_split=4x512"),
     (DType.F16, 256, 10368, 2048, (False, True, False), 1, "direct 128x64 bk64 head=256 tail_split=3x704"),
-    (DType.F16, 130, 33280, 1024, (True, True, False), 1, "direct 128x128 bk128 head=512 tail_split=2x512"),
-    (DType.F16, 768, 16384, 1024, (False, True, True), 1, "direct 256x128 bk64 head=256 tail_split=2x512"),
-    (DType.F16, 1280, 9856, 2048, (True, False, False), 1, "direct 256x192 bk64 head=256 tail_split=4x512"),
-    (DType.F16, 1280, 14720, 1024, (False, False, True), 1, "direct 256x256 bk64 head=256 tail_split=2x512"),
-    (DType.F16, 130, 3712, 1024, (False, False, False), 3, "x3 grouped [direct 128x64 bk64 head=256 tail_split=2x512"),
-    (DType.F16, 768, 5632, 1024, (False, False, False), 3, "x3 grouped [direct 256x192 bk64 head=256 tail_split=2x512"),
+    (DType.F16, 300, 33088, 1024, (True, True, False), 1, "direct 256x192 bk64 head=256 tail_split=2x512"),
+    (DType.F16, 768, 24768, 2048, (False, True, True), 1, "direct 256x256 bk64 head=256 tail_split=4x512"),
+    (DType.F16, 768, 24768, 1536, (True, False, False), 1, "direct 256x256 bk64 head=256 tail_split=3x512"),
+    (DType.F16, 300, 2688, 1536, (False, False, False), 3, "x3 grouped [direct 64x64 bk64 head=512 tail_split=3x512"),
+    (DType.F16, 300, 11008, 1024, (False, False, False), 3, "x3 grouped [direct 256x192 bk64 head=256 tail_split=2x512"),
+    (DType.F16, 1024, 6528, 2048, (False, False, False), 3, "x3 grouped [direct 256x256 bk64 head=256 tail_split=4x512"),
 ]
 
 
