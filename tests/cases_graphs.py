@@ -1617,6 +1617,19 @@ def attention_f16_rising_scores():
 
 
 @case
+def attention_f16_causal_long():
+    """1100 queries and keys under a causal mask: 9 blocks of keys per wave, classes for 35 x 35 blocks, partial last
+    tiles of both"""
+    return _attention_f16_case(136, 2, 1100, 1100, 64, 64, True, "causal")
+
+
+@case
+def attention_f16_one_query():
+    """a single query (a decoding step) against 300 keys with a mask tensor: a workgroup with one live lane pair"""
+    return _attention_f16_case(137, 3, 1, 300, 128, 128, True, "full")
+
+
+@case
 def attention_f16_ragged_full_mask():
     """70 queries against 150 keys (partial blocks), width 64, V 40 wide, a mask tensor per batch entry"""
     return _attention_f16_case(131, 3, 70, 150, 64, 40, True, "full")
