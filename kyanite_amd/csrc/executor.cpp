@@ -110,16 +110,13 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     plan_.uploads.clear();
     plan_.uploads.shrink_to_fit();
 
-    for (auto &t : plan_.inputs) {
-        void *p = nullptr;
-        hip_check(hipHostMalloc(&p, std::max<size_t>(t.shape.size() * dtype_bytes(t.dtype), 1), hipHostMallocCoherent), "hipHostMalloc");
-        pinned_inputs_.push_back(p);
-    }
-    for (auto &t : plan_.outputs) {
-        void *p = nullptr;
-        hip_check(hipHostMalloc(&p, std::max<size_t>(t.shape.size() * dtype_bytes(t.dtype), 1), hipHostMallocCoherent), "hipHostMalloc");
-        pinned_outputs_.push_back(p);
-    }
+    // Page-locked staging for `evaluate`. Up to a few hundred MB it is set up here, so that the first evaluation is
+    // as fast as the rest; beyond that it waits for the first `evaluate`, and a caller that keeps its own device
+    // buffers and only ever calls `run_async` never pays for it.
+    size_t staging_bytes = 0;
+    for (auto &t : plan_.inputs) staging_bytes += t.shape.size() * dtype_bytes(t.dtype);
+    for (auto &t : plan_.outputs) staging_bytes += t.shape.size() * dtype_bytes(t.dtype);
+    if (staging_bytes <= ((size_t) 256 << 20)) allocate_staging();
 
     // load every distinct code object once and resolve the launch arguments
     std::map<uint64_t, hipModule_t> loaded;
@@ -155,6 +152,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     for (auto &t : plan_.inputs) own_buffer(t);
     for (auto &t : plan_.outputs) own_buffer(t);
     if (separate && io_bytes <= mapped_limit && !plan_.steps.empty()) {
+        allocate_staging();
         mapped_launches_.resize(plan_.steps.size());
         for (size_t si = 0; si < plan_.steps.size(); si++) {
             mapped_launches_[si].function = launches_[si].function;
@@ -172,6 +170,18 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
         for (auto &l : mapped_launches_) fused_mapped_ptrs_.insert(fused_mapped_ptrs_.end(), l.ptrs.begin(), l.ptrs.end());
         KN_ASSERT(fused_ptrs_.size() == fused_spec_->n_ptrs && (!mapped_io_ || fused_mapped_ptrs_.size() == fused_spec_->n_ptrs));
     }
+}
+
+void HipExecutor::allocate_staging() {
+    if (staging_ready_) return;
+    auto pinned = [](const PlanTensor &t) {
+        void *p = nullptr;
+        hip_check(hipHostMalloc(&p, std::max<size_t>(t.shape.size() * dtype_bytes(t.dtype), 1), hipHostMallocCoherent), "hipHostMalloc");
+        return p;
+    };
+    for (auto &t : plan_.inputs) pinned_inputs_.push_back(pinned(t));
+    for (auto &t : plan_.outputs) pinned_outputs_.push_back(pinned(t));
+    staging_ready_ = true;
 }
 
 const std::string &HipExecutor::fused_source() const {
@@ -411,6 +421,7 @@ const std::vector<HostTensor> &HipExecutor::evaluate(const std::vector<HostTenso
             fail("Wrong dtype for input ", i, ": expected ", dtype_name(plan_.inputs[i].dtype), ", got ", dtype_name(inputs[i].dtype));
     }
     hip_check(hipSetDevice(device_), "hipSetDevice");
+    allocate_staging();
     // The staging buffers are free: every evaluate ends with a synchronisation, and run_async never touches them.
     // Device work a caller queued through run_async is ordered before the copies below by the stream itself.
     const bool mapped = mapped_io_ && !profile_ && !graph_mode_;

@@ -102,6 +102,8 @@ private:
     uint32_t fused_seq_ = 0;
     void launch_fused(bool mapped);
     std::vector<void *> pinned_inputs_, pinned_outputs_;
+    bool staging_ready_ = false;
+    void allocate_staging();
     std::vector<HostTensor> tensor_outputs_;
     bool profile_ = false;
     std::optional<Profile> last_profile_;

@@ -1837,3 +1837,23 @@ def row_statistics_in_the_elementwise_kernel():
     g.output(g.sub(x, g.broadcast(g.view(g.reduce(x, [0], ReduceOp.MEAN), [1, 200]), [37, 200])))
     return g, 0, [rng.standard_normal((37, 200)).astype(np.float32), rng.standard_normal((3, 70000)).astype(np.float32),
                   rng.standard_normal((20, 136)).astype(np.float16)], None
+
+
+@case
+def restride_every_other_element():
+    """the data and the expected values of kn-cuda-sys/tests/restride.rs:9-26: three elements two apart read into a
+    dense tensor; here as a slice with step 2 of an input, which the copy step does"""
+    g = Graph()
+    x = g.input([6])
+    g.output(g.slice(x, 0, 0, 6, 2))
+    return g, 0, [f32((6,), [-1.0, 0.0, 2.0, 0.0, -3.0, 0.0])], [f32((3,), [-1.0, 2.0, -3.0])]
+
+
+@case
+def negative_stride_read():
+    """the layout of kn-cuda-sys/tests/negative_stride.rs:14-45: eight floats read through a stride of -1 from the
+    last element (that test prints its result; reversing 0..8 is what the layout means)"""
+    g = Graph()
+    x = g.input([1, 1, 1, 8])
+    g.output(g.flip(x, 3))
+    return g, 0, [f32((1, 1, 1, 8), np.arange(8))], [f32((1, 1, 1, 8), np.arange(8)[::-1])]

@@ -55,6 +55,26 @@ def test_upload_run_async_event_download(hip_device):
     mine.synchronize()
 
 
+@pytest.mark.gpu
+def test_device_memory_slices(hip_device):
+    """Copies into and between byte ranges of one allocation, with the data and the expected bytes of
+    kn-cuda-sys/tests/mem.rs:4-32 (`DevicePtr::offset_bytes`, `copy_linear_from_host`, `copy_linear_from_device`)."""
+    from ctypes import c_void_p
+    from kyanite_amd._lib import check, lib
+    whole = DeviceBuffer(hip_device, 512)
+    a, b, c = whole.ptr, whole.ptr + 128, whole.ptr + 256
+
+    def upload(dst, values):
+        check(lib.knhip_memcpy_h2d(whole.device, c_void_p(dst), values.ctypes.data, values.nbytes))
+
+    upload(a, np.zeros(512, np.uint8))
+    upload(a, np.full(128, 1, np.uint8))
+    upload(b, np.full(128, 2, np.uint8))
+    check(lib.knhip_memcpy_d2d(whole.device, c_void_p(c), c_void_p(a), 128))
+    expected = np.concatenate([np.full(128, v, np.uint8) for v in (1, 2, 1, 0)])
+    assert np.array_equal(whole.to_array(np.uint8, (512,)), expected)
+
+
 def _matmul_case(rng, dtype, batch, m, n, k, a_layout, b_layout, broadcast_b=False):
     """Host arrays laid out as asked plus the strides that address them as A[b, i, k], B[b, k, j]."""
     np_dtype = np.float16 if dtype == DType.F16 else np.float32
