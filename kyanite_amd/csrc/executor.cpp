@@ -72,6 +72,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     if (const char *e = getenv("KNHIP_PACK_CONSTANTS")) options.pack_matmul_constants = atoi(e) != 0;
     if (const char *e = getenv("KNHIP_POINTWISE_CONV")) options.pointwise_conv_as_matmul = atoi(e) != 0;
     if (const char *e = getenv("KNHIP_JOIN_ELEMENTWISE")) options.join_elementwise = atoi(e) != 0;
+    if (const char *e = getenv("KNHIP_SPLIT_REDUCE")) options.split_reduce = atoi(e) != 0;
     plan_ = plan_graph(graph, batch_size, options);
     for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
     if (fuse_small && plan_.steps.size() > 1) {

@@ -721,8 +721,16 @@ KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, 
 
 // ------------------------------------------------------------------------------------------------ reduce kernel
 
+// How many slices of the reduced index to fold side by side: none while there is a workgroup per compute unit or
+// little to read per workgroup; else enough for about four workgroups per compute unit, each with 64 KB or more.
+size_t reduce_parts(size_t blocks, size_t block_bytes, size_t most) {
+    if (blocks >= 256 || block_bytes < ((size_t) 512 << 10)) return 1;
+    const size_t wanted = (1024 + blocks - 1) / blocks, by_work = block_bytes / ((size_t) 64 << 10);
+    return std::max<size_t>(1, std::min({wanted, by_work, most, (size_t) 1024}));
+}
+
 KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
-                              ReduceOp rop, const ScalarExpr *pre) {
+                              ReduceOp rop, const ScalarExpr *pre, ReduceSplit *split) {
     const auto &ishape = input.shape.shape();
     // the folded values have the type of the output; with a prologue the loaded operand may be of another type
     const DType dtype = output.dtype, in_dtype = input.dtype;
@@ -790,6 +798,9 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
     ss << "KN_DEV T kn_post(T v) { return "
        << (rop == ReduceOp::Mean ? "v / (float) " + std::to_string(red_size) + ".0f" : std::string("v")) << "; }\n";
 
+    const std::string preamble = ss.str();
+    const bool may_split = split != nullptr && dtype != DType::Bool;
+    size_t parts = 1;
     std::ostringstream note;
     if (row) {
         // ---- a group of G lanes folds one output element, lanes stride over the (contiguous) reduced index
@@ -805,7 +816,12 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         size_t red_vecs = red_size / vec;
         size_t G = red_vecs >= 2048 ? 256 : red_vecs >= 128 ? 64 : red_vecs >= 16 ? 16 : 1;
         size_t block = 256, rows_per_block = block / G;
-        size_t iters = (red_vecs + G - 1) / G;
+        const size_t blocks = (kept_size + rows_per_block - 1) / rows_per_block;
+        if (may_split) parts = reduce_parts(blocks, red_size * rows_per_block * es, red_vecs / (4 * G));
+        // every slice is `chunk` vectors of the reduced index long (the last one may be shorter, none is empty)
+        const size_t chunk = (red_vecs + parts - 1) / parts;
+        parts = (red_vecs + chunk - 1) / chunk;
+        size_t iters = (chunk + G - 1) / G;
         std::vector<size_t> rdims = rc.shape;
         std::vector<std::vector<int64_t>> rstrides = rc.strides;
         if (rc.rank() > 0) {
@@ -816,7 +832,14 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_reduce(KnPtrs ptrs) {\n";
         ss << "    const SI *in = (const SI *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
         if (G == 256) ss << "    __shared__ T lds[4];\n";
-        ss << "    const idx_t row = (idx_t) blockIdx.x * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / " << G << ");\n";
+        if (parts > 1) {
+            ss << "    const idx_t part = (idx_t) blockIdx.x / (idx_t) " << blocks << ", blk = (idx_t) blockIdx.x % (idx_t) " << blocks << ";\n";
+            ss << "    const idx_t r0 = part * (idx_t) " << chunk << ";\n";
+            ss << "    const idx_t r1 = r0 + (idx_t) " << chunk << " < (idx_t) " << red_vecs << " ? r0 + (idx_t) " << chunk << " : (idx_t) " << red_vecs << ";\n";
+        } else {
+            ss << "    const idx_t blk = (idx_t) blockIdx.x, r0 = 0, r1 = (idx_t) " << red_vecs << ";\n";
+        }
+        ss << "    const idx_t row = blk * (idx_t) " << rows_per_block << " + (idx_t) (threadIdx.x / " << G << ");\n";
         ss << "    const idx_t lane = (idx_t) (threadIdx.x % " << G << ");\n";
         if (G != 256) ss << "    if (row >= (idx_t) " << kept_size << ") return;\n";
         ss << "    idx_t o_out = 0, o_in = 0;\n";
@@ -824,8 +847,8 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         ss << "    T acc[4] = {kn_identity(), kn_identity(), kn_identity(), kn_identity()};\n";
         ss << (iters <= 32 ? "#pragma unroll\n" : "#pragma unroll 8\n");
         ss << "    for (idx_t i = 0; i < (idx_t) " << iters << "; i++) {\n";
-        ss << "        const idx_t r = lane + i * (idx_t) " << G << ";\n";
-        ss << "        if (r < (idx_t) " << red_vecs << ") {\n            idx_t o = o_in;\n";
+        ss << "        const idx_t r = r0 + lane + i * (idx_t) " << G << ";\n";
+        ss << "        if (r < r1) {\n            idx_t o = o_in;\n";
         emit_decompose(ss, "            ", "r", rdims, rstrides, {"o"});
         if (vec > 1) {
             ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
@@ -837,9 +860,10 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         ss << "    T total = kn_f(kn_f(acc[0], acc[1]), kn_f(acc[2], acc[3]));\n";
         if (G == 256) ss << "    total = kn_block_reduce<4>(total, kn_f, lds);\n";
         else if (G > 1) ss << "    total = kn_group_reduce<" << G << ">(total, kn_f);\n";
-        ss << "    if (lane == 0) out[o_out] = " << to_storage(dtype, "kn_post(total)") << ";\n}\n";
+        if (parts > 1) ss << "    if (lane == 0) ((T *) ptrs.p[1])[part * (idx_t) " << kept_size << " + row] = total;\n}\n";
+        else ss << "    if (lane == 0) out[o_out] = " << to_storage(dtype, "kn_post(total)") << ";\n}\n";
         spec.block = (uint32_t) block;
-        spec.grid = ceil_div_u32(kept_size, rows_per_block);
+        spec.grid = ceil_div_u32(blocks * parts, 1);
         note << "row G=" << G << " vec=" << vec << " iters=" << iters;
     } else {
         // ---- every thread owns VEC neighbouring kept elements and walks the reduced index; TY slices of the
@@ -863,6 +887,10 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         // with plenty of independent outputs there is no need to split the reduction
         if (kept_vecs >= 256 * 1024) { TX = 256; TY = 1; }
         size_t block = TX * TY;
+        const size_t blocks = (kept_vecs + TX - 1) / TX;
+        if (may_split) parts = reduce_parts(blocks, red_size * TX * vec * es, red_size / (4 * TY));
+        const size_t chunk = (red_size + parts - 1) / parts;
+        parts = (red_size + chunk - 1) / chunk;
         std::vector<size_t> kdims = kc.shape;
         std::vector<std::vector<int64_t>> kstrides = kc.strides;
         kdims.back() /= vec;
@@ -873,13 +901,20 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         ss << "    const SI *in = (const SI *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
         if (TY > 1) ss << "    __shared__ T lds[" << TY << "][" << vec << "][" << TX << "];\n";
         ss << "    const idx_t tx = (idx_t) (threadIdx.x % " << TX << "), ty = (idx_t) (threadIdx.x / " << TX << ");\n";
-        ss << "    const idx_t kv = (idx_t) blockIdx.x * (idx_t) " << TX << " + tx;\n";
+        if (parts > 1) {
+            ss << "    const idx_t part = (idx_t) blockIdx.x / (idx_t) " << blocks << ", blk = (idx_t) blockIdx.x % (idx_t) " << blocks << ";\n";
+            ss << "    const idx_t r0 = part * (idx_t) " << chunk << ";\n";
+            ss << "    const idx_t r1 = r0 + (idx_t) " << chunk << " < (idx_t) " << red_size << " ? r0 + (idx_t) " << chunk << " : (idx_t) " << red_size << ";\n";
+        } else {
+            ss << "    const idx_t blk = (idx_t) blockIdx.x, r0 = 0, r1 = (idx_t) " << red_size << ";\n";
+        }
+        ss << "    const idx_t kv = blk * (idx_t) " << TX << " + tx;\n";
         ss << "    const bool valid = kv < (idx_t) " << kept_vecs << ";\n";
         ss << "    idx_t o_out = 0, o_in = 0;\n";
         ss << "    T acc[" << vec << "];\n    for (int j = 0; j < " << vec << "; j++) acc[j] = kn_identity();\n";
         ss << "    if (valid) {\n";
         emit_decompose(ss, "        ", "kv", kdims, kstrides, {"o_out", "o_in"});
-        ss << "#pragma unroll 4\n        for (idx_t r = ty; r < (idx_t) " << red_size << "; r += (idx_t) " << TY << ") {\n            idx_t o = o_in;\n";
+        ss << "#pragma unroll 4\n        for (idx_t r = r0 + ty; r < r1; r += (idx_t) " << TY << ") {\n            idx_t o = o_in;\n";
         emit_decompose(ss, "            ", "r", rc.shape, rc.strides, {"o"});
         if (vec > 1) {
             ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
@@ -895,7 +930,10 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         } else {
             ss << "    if (valid) {\n";
         }
-        if (vec > 1) {
+        if (parts > 1) {
+            ss << "        T *slot = (T *) ptrs.p[1] + (part * (idx_t) " << kept_vecs << " + kv) * (idx_t) " << vec << ";\n";
+            ss << "        for (int j = 0; j < " << vec << "; j++) slot[j] = acc[j];\n";
+        } else if (vec > 1) {
             ss << "        VO o;\n        for (int j = 0; j < " << vec << "; j++) o[j] = " << to_storage(dtype, "kn_post(acc[j])") << ";\n";
             ss << "        *(VO *) (out + o_out) = o;\n";
         } else {
@@ -903,8 +941,36 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         }
         ss << "    }\n}\n";
         spec.block = (uint32_t) block;
-        spec.grid = ceil_div_u32(kept_vecs, TX);
+        spec.grid = ceil_div_u32(blocks * parts, 1);
         note << "col TX=" << TX << " TY=" << TY << " vec=" << vec;
+    }
+    if (parts > 1) {
+        // the second kernel folds the slices of every result and applies the mean's division: one thread per result
+        // (neighbouring threads read neighbouring partial results), or a wave per result when there are few results
+        // and many slices, each lane folding every 64th slice before the lanes are combined
+        note << " parts=" << parts;
+        const size_t FG = kept_size <= 4096 && parts >= 64 ? 64 : 1;
+        std::ostringstream fs;
+        fs << preamble;
+        fs << "extern \"C\" __global__ __launch_bounds__(256) void kn_reduce_final(KnPtrs ptrs) {\n";
+        fs << "    const T *part = (const T *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
+        fs << "    const idx_t i = ((idx_t) blockIdx.x * (idx_t) 256 + (idx_t) threadIdx.x) / (idx_t) " << FG << ";\n";
+        fs << "    const idx_t lane = (idx_t) (threadIdx.x % " << FG << ");\n";
+        fs << "    if (i >= (idx_t) " << kept_size << ") return;\n    idx_t o_out = 0;\n";
+        emit_decompose(fs, "    ", "i", kc.shape, {kc.strides[0]}, {"o_out"});
+        fs << "    T acc = part[lane * (idx_t) " << kept_size << " + i];\n#pragma unroll 8\n";
+        fs << "    for (idx_t s = lane + (idx_t) " << FG << "; s < (idx_t) " << parts << "; s += (idx_t) " << FG << ") acc = kn_f(acc, part[s * (idx_t) " << kept_size << " + i]);\n";
+        if (FG > 1) fs << "    acc = kn_group_reduce<" << FG << ">(acc, kn_f);\n";
+        fs << "    if (lane == 0) out[o_out] = " << to_storage(dtype, "kn_post(acc)") << ";\n}\n";
+        split->parts = parts;
+        split->kept_size = kept_size;
+        split->partial_dtype = dtype == DType::F16 ? DType::F32 : dtype;
+        split->final.name = "kn_reduce_final";
+        split->final.n_ptrs = 2;
+        split->final.block = 256;
+        split->final.grid = ceil_div_u32(kept_size * FG, 256);
+        split->final.source = fs.str();
+        split->final.strategy = "fold of " + std::to_string(parts) + " partial results" + (FG > 1 ? ", a wave per result" : "");
     }
     spec.source = ss.str();
     spec.strategy = note.str();

@@ -53,8 +53,19 @@ KernelSpec make_scalar_kernel_multi(const std::vector<KernelOperand> &operands, 
 
 // output[kept] = post(fold(op, pre(input[kept, reduced...]))) (reduce.rs:35-153). `pre`: an optional elementwise
 // expression of the loaded element (its only operand is number 1), e.g. the square in a mean of squares.
+// A reduction with few results and a long reduced index has too few workgroups to pull the input at the rate of the
+// memory. With `split` given, such a reduction comes back as two kernels: the returned one folds `parts` slices of
+// the reduced index side by side into partial[parts][kept] (elements of `partial_dtype`, the type the fold computes
+// in; its second pointer is that array instead of the output), and `final` (pointers: partial, output) folds the
+// slices in order and applies the mean's division. `parts` stays 1 when there is nothing to gain.
+struct ReduceSplit {
+    size_t parts = 1;
+    size_t kept_size = 0;
+    DType partial_dtype = DType::F32;
+    KernelSpec final;
+};
 KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
-                              ReduceOp op, const ScalarExpr *pre = nullptr);
+                              ReduceOp op, const ScalarExpr *pre = nullptr, ReduceSplit *split = nullptr);
 
 // Row kernels. The value that gets normalised is `pre(load operands...)`, the value stored is
 // `post(normalised, load operands...)`: this is how a preceding scale / residual add and a following affine

@@ -205,6 +205,28 @@ private:
         return t;
     }
 
+    // One launch, or two with partial results in between when the reduction has few results and much to read.
+    void push_reduce(Value value, const PlanTensor &input, const PlanTensor &output, const std::vector<size_t> &axes,
+                     ReduceOp rop, const ScalarExpr *pre) {
+        ReduceSplit split;
+        Step step;
+        step.kind = StepKind::ReduceOp;
+        step.kernel = make_reduce_kernel(kop(input), kop(output), axes, rop, pre, options.split_reduce ? &split : nullptr);
+        if (split.parts <= 1) {
+            step.operands = {{input, OperandKind::In}, {output, OperandKind::Out}};
+            push(std::move(step), value);
+            return;
+        }
+        PlanTensor partial = alloc_tensor_shared({split.parts * split.kept_size}, split.partial_dtype);
+        step.operands = {{input, OperandKind::In}, {partial, OperandKind::Out}};
+        push(std::move(step), value);
+        Step fold;
+        fold.kind = StepKind::ReduceOp;
+        fold.kernel = std::move(split.final);
+        fold.operands = {{partial, OperandKind::In}, {output, OperandKind::Out}};
+        push(std::move(fold), value);
+    }
+
     void push(Step step, Value debug_value) {
         step.debug_value = debug_value;
         step.debug_id = graph[debug_value].debug_id;
@@ -454,21 +476,13 @@ private:
                     if (!block.row_value && block.operands.size() == 2) {
                         const PlanTensor &input = block.operands[1];
                         PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
-                        Step step;
-                        step.kind = StepKind::ReduceOp;
-                        step.kernel = make_reduce_kernel(kop(input), kop(output), op.axes, op.reduce, &block.expr);
-                        step.operands = {{input, OperandKind::In}, {output, OperandKind::Out}};
-                        push(std::move(step), value);
+                        push_reduce(value, input, output, op.axes, op.reduce, &block.expr);
                         return VT::done(output);
                     }
                 }
                 KN_TRY(input, visit(in_v));
                 PlanTensor output = alloc_tensor_shared(result_shape, result_dtype);
-                Step step;
-                step.kind = StepKind::ReduceOp;
-                step.kernel = make_reduce_kernel(kop(input), kop(output), op.axes, op.reduce);
-                step.operands = {{input, OperandKind::In}, {output, OperandKind::Out}};
-                push(std::move(step), value);
+                push_reduce(value, input, output, op.axes, op.reduce, nullptr);
                 return VT::done(output);
             }
         }

@@ -96,6 +96,7 @@ struct PlannerOptions {
     bool group_matmuls = true;   // matmuls that share their left operand and have constant right operands share a launch
     bool pointwise_conv_as_matmul = true;  // 1 x 1 convolutions with stride 1 run as one matrix product per image
     bool join_elementwise = true;  // small elementwise steps of one shape that do not depend on each other share a launch
+    bool split_reduce = true;  // a reduction with few results and a long reduced index runs as two launches
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
 };

@@ -1857,3 +1857,28 @@ def negative_stride_read():
     x = g.input([1, 1, 1, 8])
     g.output(g.flip(x, 3))
     return g, 0, [f32((1, 1, 1, 8), np.arange(8))], [f32((1, 1, 1, 8), np.arange(8)[::-1])]
+
+
+@case
+def reduce_in_two_launches():
+    """few results, much to read: slices of the reduced index are folded side by side and a second launch folds the
+    partial results. Along columns (vectors of 4, a last slice that is shorter), over everything (one result), along
+    long rows with the square folded into the load (f16, partial results in f32), with a permuted input whose kept
+    axis is not the last, and integer sums, which must stay exact"""
+    g = Graph()
+    rng = np.random.default_rng(170)
+    tall = g.input([70001, 96])
+    g.output(g.reduce(tall, [0], ReduceOp.MEAN))
+    g.output(g.reduce(tall, [0], ReduceOp.MIN))
+    whole = g.input([1500, 3001])
+    g.output(g.reduce(whole, [0, 1], ReduceOp.SUM))
+    g.output(g.reduce(whole, [0, 1], ReduceOp.MAX))
+    long_rows = g.input([3, 600000], DType.F16)
+    g.output(g.reduce(g.mul(long_rows, long_rows), [1], ReduceOp.MEAN))
+    planes = g.input([5, 300, 700])
+    g.output(g.reduce(g.permute(planes, [1, 0, 2]), [0, 2], ReduceOp.SUM))
+    counts = g.input([200000, 8], DType.I32)
+    g.output(g.reduce(counts, [0], ReduceOp.SUM))
+    return g, 0, [rng.standard_normal((70001, 96)).astype(np.float32), rng.standard_normal((1500, 3001)).astype(np.float32),
+                  rng.standard_normal((3, 600000)).astype(np.float16), rng.standard_normal((5, 300, 700)).astype(np.float32),
+                  rng.integers(-2**20, 2**20, (200000, 8)).astype(np.int32)], None
