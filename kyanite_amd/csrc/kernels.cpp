@@ -2,6 +2,7 @@
 
 #include <cinttypes>
 #include <cstdlib>
+#include <functional>
 
 namespace kn {
 
@@ -979,6 +980,11 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
 
 // ------------------------------------------------------------------------------------------------ row kernels
 
+// the row statistic of kind Reduce out of the folded value `m` (the mean divides, like the reduce kernel's last step)
+std::string stat_expr_of(bool rowred, ReduceOp rop, size_t size) {
+    return rowred && rop == ReduceOp::Mean ? "m / (float) " + std::to_string(size) + ".0f" : std::string("m");
+}
+
 KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     const auto &ops = desc.operands;
     KN_ASSERT(ops.size() >= 2);
@@ -1095,6 +1101,148 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     emit_fn("kn_pre", desc.pre, in_pre, false, row_dtype);
     emit_fn("kn_post", desc.post, in_post, true, ops[0].dtype);
 
+    // The normalised axis is not the contiguous one, a kept axis is (a softmax over the channels of [n, c, h, w]):
+    // lanes that walk along the axis would each touch a line of their own. Here TX neighbouring lanes take TX
+    // neighbouring columns instead, so that every load of a wave is a run of whole lines, TY threads share a column
+    // (every TY-th position of the axis each, in registers when those are few, else read again per pass) and
+    // combine their statistics through LDS.
+    if (sc.rank() >= 1 && axis_strides[0] != 1 && sc.strides[0].back() == 1 && sc.shape.back() >= 16 && size > 1) {
+        const size_t inner = sc.shape.back();
+        size_t n_pre = 0;
+        for (size_t k = 1; k < ops.size(); k++) n_pre += in_pre[k] ? 1 : 0;
+        size_t TX = 64, TY = 4, items = (size + 3) / 4;
+        bool held = false;
+        for (size_t tx : {64, 32, 16}) {  // fewer columns per workgroup: more threads, so more registers, per column
+            const size_t ty = 256 / tx, per_thread = (size + ty - 1) / ty;
+            if (per_thread * std::max<size_t>(n_pre, 1) <= 32) {
+                TX = tx, TY = ty, items = per_thread, held = true;
+                break;
+            }
+        }
+        std::vector<size_t> outer_shape(sc.shape.begin(), sc.shape.end() - 1);
+        if (!held) {
+            // read again per pass: what counts is how many loads are in flight, so as many workgroups as the columns
+            // give, up to four per compute unit, before whole lines per wave
+            for (size_t tx : {64, 32, 16}) {
+                TX = tx, TY = 256 / tx, items = (size + TY - 1) / TY;
+                if (concrete_size(outer_shape) * ((inner + tx - 1) / tx) >= 1024) break;
+            }
+        }
+        const size_t column_blocks = (inner + TX - 1) / TX;
+        std::vector<std::vector<int64_t>> outer_strides(ops.size());
+        for (size_t k = 0; k < ops.size(); k++) outer_strides[k].assign(sc.strides[k].begin(), sc.strides[k].end() - 1);
+        const size_t outer_size = concrete_size(outer_shape);
+        const std::string L = "(idx_t) " + std::to_string(size);
+        ss << "KN_DEV float kn_max(float a, float b) { return fmaxf(a, b); }\nKN_DEV float kn_add(float a, float b) { return a + b; }\n";
+        ss << "KN_DEV float kn_min(float a, float b) { return fminf(a, b); }\n";
+        ss << "#define TX " << TX << "\n#define TY " << TY << "\n#define ITEMS " << items << "\n";
+        // every thread of a column ends up with the fold of the TY partial values, taken in the same order
+        ss << "template<typename F> KN_DEV float kn_column_fold(float v, F f, float (*lds)[TX], int tx, int ty) {\n";
+        ss << "    lds[ty][tx] = v;\n    __syncthreads();\n    v = lds[0][tx];\n";
+        ss << "#pragma unroll\n    for (int s = 1; s < TY; s++) v = f(v, lds[s][tx]);\n    return v;\n}\n";
+        ss << "extern \"C\" __global__ __launch_bounds__(256) void " << spec.name << "(KnPtrs ptrs) {\n";
+        for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
+        ss << "    __shared__ float lds_m[TY][TX], lds_s[TY][TX];\n";
+        ss << "    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;\n";
+        ss << "    const idx_t col_raw = ((idx_t) blockIdx.x % (idx_t) " << column_blocks << ") * (idx_t) TX + (idx_t) tx;\n";
+        ss << "    const bool col_ok = col_raw < (idx_t) " << inner << ";\n";
+        ss << "    const idx_t col = col_ok ? col_raw : (idx_t) " << (inner - 1) << ";\n";
+        ss << "    const idx_t outer = (idx_t) blockIdx.x / (idx_t) " << column_blocks << ";\n";
+        ss << "    idx_t base[" << ops.size() << "];\n";
+        for (size_t k = 0; k < ops.size(); k++) ss << "    base[" << k << "] = col * (idx_t) " << i64_str(sc.strides[k].back()) << ";\n";
+        {
+            std::vector<std::string> offs;
+            for (size_t k = 0; k < ops.size(); k++) offs.push_back("base[" + std::to_string(k) + "]");
+            emit_decompose(ss, "    ", "outer", outer_shape, outer_strides, offs);
+        }
+        auto at = [&](size_t k, const std::string &i) {
+            return "p" + std::to_string(k) + "[base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k]) + "]";
+        };
+        auto pre_of = [&](const std::function<std::string(size_t)> &operand) {
+            std::string c = "kn_pre(";
+            bool first = true;
+            for (size_t k = 1; k < ops.size(); k++) {
+                if (!in_pre[k]) continue;
+                c += (first ? "" : ", ") + from_storage(ops[k].dtype, operand(k));
+                first = false;
+            }
+            return c + ")";
+        };
+        auto store = [&](const std::string &indent, const std::string &i, const std::string &value) {
+            std::string c = row_dtype == DType::F16 ? "kn_post(kn_r16(" + value + ")" : "kn_post(" + value;
+            for (size_t k = 1; k < ops.size(); k++)
+                if (in_post[k]) c += ", " + from_storage(ops[k].dtype, at(k, i));
+            ss << indent << at(0, i) << " = " << to_storage(ops[0].dtype, c + ")") << ";\n";
+        };
+        const std::string fold_stmt = fold_max ? "m = fmaxf(m, v);" : fold_min ? "m = fminf(m, v);" : "m += v;";
+        const std::string eps = DScalar::f32(desc.eps).to_c_str();
+        ss << "    float m = " << identity << ", s = 0.0f;\n";
+        if (held) {
+            for (size_t k = 1; k < ops.size(); k++)
+                if (in_pre[k]) ss << "    S" << k << " a" << k << "[ITEMS];\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n";
+            ss << "        const idx_t i = (idx_t) ty + (idx_t) it * (idx_t) TY, ic = i < " << L << " ? i : " << L << " - 1;\n";
+            for (size_t k = 1; k < ops.size(); k++)
+                if (in_pre[k]) ss << "        a" << k << "[it] = " << at(k, "ic") << ";\n";
+            ss << "    }\n    float x[ITEMS];\n";
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = (idx_t) ty + (idx_t) it * (idx_t) TY;\n";
+            ss << "        const float v = i < " << L << " ? " << pre_of([&](size_t k) { return "a" + std::to_string(k) + "[it]"; }) << " : " << identity << ";\n";
+            ss << "        x[it] = v;\n        " << fold_stmt << "\n    }\n";
+            ss << "    m = kn_column_fold(m, " << fold_fn << ", lds_m, tx, ty);\n";
+            if (rowred) {
+                ss << "    const float stat = " << stat_expr_of(rowred, rop, size) << ";\n";
+                ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) x[it] = stat;\n";
+            } else if (softmax) {
+                ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = (idx_t) ty + (idx_t) it * (idx_t) TY;\n";
+                ss << "        const float e = i < " << L << " ? expf(x[it] - m) : 0.0f;\n        x[it] = e;\n        s += e;\n    }\n";
+                ss << "    s = kn_column_fold(s, kn_add, lds_s, tx, ty);\n";
+                ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) x[it] = x[it] / s;\n";
+            } else {
+                ss << "    const float mean = m / (float) " << size << ".0f;\n";
+                ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = (idx_t) ty + (idx_t) it * (idx_t) TY;\n";
+                ss << "        const float d = i < " << L << " ? x[it] - mean : 0.0f;\n        x[it] = d;\n        s += d * d;\n    }\n";
+                ss << "    s = kn_column_fold(s, kn_add, lds_s, tx, ty);\n";
+                ss << "    const float rdenom = 1.0f / sqrtf(s / (float) " << size << ".0f + " << eps << ");\n";
+                ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) x[it] = x[it] * rdenom;\n";
+            }
+            ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = (idx_t) ty + (idx_t) it * (idx_t) TY;\n";
+            ss << "        if (col_ok && i < " << L << ") {\n";
+            store("            ", "i", "x[it]");
+            ss << "        }\n    }\n}\n";
+        } else {
+            ss << "    const idx_t len = col_ok ? " << L << " : (idx_t) 0;\n";
+            const std::string loop = "    for (idx_t i = (idx_t) ty; i < len; i += (idx_t) TY) {\n";
+            const std::string loaded = pre_of([&](size_t k) { return at(k, "i"); });
+            ss << "#pragma unroll 8\n" << loop << "        const float v = " << loaded << ";\n        " << fold_stmt << "\n    }\n";
+            ss << "    m = kn_column_fold(m, " << fold_fn << ", lds_m, tx, ty);\n";
+            if (rowred) {
+                ss << "    const float stat = " << stat_expr_of(rowred, rop, size) << ";\n";
+                ss << "#pragma unroll 8\n" << loop;
+                store("        ", "i", "stat");
+                ss << "    }\n}\n";
+            } else {
+                if (!softmax) ss << "    const float mean = m / (float) " << size << ".0f;\n";
+                ss << "#pragma unroll 8\n" << loop << "        const float v = " << loaded << ";\n";
+                if (softmax) ss << "        s += expf(v - m);\n    }\n";
+                else ss << "        const float d = v - mean;\n        s += d * d;\n    }\n";
+                ss << "    s = kn_column_fold(s, kn_add, lds_s, tx, ty);\n";
+                if (!softmax) ss << "    const float denom = sqrtf(s / (float) " << size << ".0f + " << eps << ");\n";
+                ss << "#pragma unroll 8\n" << loop << "        const float v = " << loaded << ";\n";
+                ss << "        const float r = " << (softmax ? "expf(v - m) / s" : "(v - mean) / denom") << ";\n";
+                store("        ", "i", "r");
+                ss << "    }\n}\n";
+            }
+        }
+        spec.source = ss.str();
+        spec.block = 256;
+        spec.grid = ceil_div_u32(outer_size * column_blocks, 1);
+        std::ostringstream note;
+        note << (softmax ? "softmax" : (rowred ? "row statistic + elementwise" : "layernorm")) << " columns TX=" << TX << " TY=" << TY
+             << " items=" << items << (held ? " cached" : " streamed");
+        spec.strategy = note.str();
+        return spec;
+    }
+
     // Epilogue operands (gamma, beta, ...) are requested together with the row itself when they fit in registers,
     // so that their latency overlaps with the reductions instead of following them.
     size_t n_post = 0;
@@ -1158,7 +1306,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         else ss << indent << "for (int j = 0; j < VEC; j++) m += " << src << "[j];\n";
     };
     // the row statistic of kind Reduce from the folded value `m` (like the post step of the reduce kernel)
-    const std::string stat_expr = rowred && rop == ReduceOp::Mean ? "m / (float) " + std::to_string(size) + ".0f" : std::string("m");
+    const std::string stat_expr = stat_expr_of(rowred, rop, size);
     ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << spec.name << "(KnPtrs ptrs) {\n";
     for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
     // (statistics of consecutive rows of a workgroup alternate between two sets of slots: one barrier per exchange)

@@ -1882,3 +1882,29 @@ def reduce_in_two_launches():
     return g, 0, [rng.standard_normal((70001, 96)).astype(np.float32), rng.standard_normal((1500, 3001)).astype(np.float32),
                   rng.standard_normal((3, 600000)).astype(np.float16), rng.standard_normal((5, 300, 700)).astype(np.float32),
                   rng.integers(-2**20, 2**20, (200000, 8)).astype(np.int32)], None
+
+
+@case
+def normalised_axis_is_not_the_contiguous_one():
+    """softmax, layernorm and row statistics along an axis that a contiguous axis follows (a softmax over the channels of
+    [n, c, h, w]): neighbouring lanes take neighbouring columns. Few positions per thread (in registers) with a last
+    block of columns that is partial; 300 positions (16 threads per column); 1000 positions (read again per pass); f16;
+    a sum of two tensors in front and an affine behind; a statistic with its elementwise consumer"""
+    g = Graph()
+    rng = np.random.default_rng(171)
+    maps = g.input([3, 40, 7, 9])
+    g.output(g.softmax(maps, 1))
+    g.output(g.layernorm(maps, 1, 1e-5))
+    mid = g.input([2, 300, 130], DType.F16)
+    g.output(g.softmax(mid, 1))
+    tall = g.input([1000, 50])
+    g.output(g.layernorm(tall, 0, 1e-5))
+    g.output(g.softmax(tall, 0))
+    other = g.input([1000, 50])
+    gamma, beta = g.input([1000, 1]), g.input([1000, 1])
+    normed = g.layernorm(g.add(tall, other), 0, 1e-3)
+    g.output(g.add(g.mul(normed, g.broadcast(gamma, [1000, 50])), g.broadcast(beta, [1000, 50])))
+    g.output(g.sub(tall, g.broadcast(g.view(g.reduce(tall, [0], ReduceOp.MAX), [1, 50]), [1000, 50])))
+    f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    return g, 0, [f(3, 40, 7, 9), rng.standard_normal((2, 300, 130)).astype(np.float16), f(1000, 50), f(1000, 50),
+                  f(1000, 1), f(1000, 1)], None
