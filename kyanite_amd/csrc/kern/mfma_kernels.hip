@@ -356,10 +356,17 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * T, n0 = tn * T;
-    StridedLoader<A_MODE, T, BK> la(StridedOperand{p.filter, K, 1, p.out_c, K}, m0);
+    // a launch that splits the input channels: slice blockIdx.y multiplies its own range of k and stores an f32 partial
+    // result; bias, residual and activation are applied by the pass that sums the slices
+    const int k_begin = p.splits > 1 ? blockIdx.y * p.split_channels * kh * kw : 0;
+    const int k_end = p.splits > 1 ? min(K, k_begin + p.split_channels * kh * kw) : K;
+    StridedLoader<A_MODE, T, BK> la(StridedOperand{p.filter, K, 1, p.out_c, k_end}, m0);
     PatchLoader<KH, KW, T, BK> lb(p, n0);
-    ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
-    mfma_tile_loop<TI, TI>(la, lb, s, 0, K, m0, n0);
+    lb.K = k_end;
+    ConvStore s = p.splits > 1
+        ? ConvStore{p.workspace + (long long) blockIdx.y * p.out_c * N, nullptr, nullptr, 0, p.out_c, ohw, N, 0, {0, 0}, {false, false}}
+        : ConvStore{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
+    mfma_tile_loop<TI, TI>(la, lb, s, k_begin, k_end, m0, n0);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -503,14 +510,17 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+    // a launch that splits the input channels: slice blockIdx.y takes its own range of them
+    const int c_begin = p.splits > 1 ? blockIdx.y * p.split_channels : 0;
+    const int c_end = p.splits > 1 ? min(C, c_begin + p.split_channels) : C;
     // the padding is never written again
     for (int i = t; i < PLANE_LDS; i += THREADS) Bs[i] = 0.0f;
-    fetch(0);
-    for (int c0 = 0; c0 < C; c0 += CB) {
+    fetch(c_begin);
+    for (int c0 = c_begin; c0 < c_end; c0 += CB) {
         __syncthreads();
         stage();
         __syncthreads();
-        if (c0 + CB < C) fetch(c0 + CB);
+        if (c0 + CB < c_end) fetch(c0 + CB);
         // The operands of step kk + 2 are requested from LDS before the MFMAs of step kk are issued, and the wave
         // raises its priority while it issues MFMAs. Measured on this loop alone (no global loads, two waves per
         // SIMD): operands read right before their MFMAs and masked with selects 126 TFLOP/s, without the selects 140,
@@ -549,7 +559,10 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 
     // Epilogue. Bias and residual are requested for a whole MFMA tile row at once (addresses clamped into the tensor
     // instead of branches around the loads), so their latencies overlap; only the stores are predicated.
-    ConvStore s{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
+    // (the partial results of a split launch get bias, residual and activation from the pass that sums them)
+    ConvStore s = p.splits > 1
+        ? ConvStore{p.workspace + (long long) blockIdx.y * p.out_c * N, nullptr, nullptr, 0, p.out_c, ohw, N, 0, {0, 0}, {false, false}}
+        : ConvStore{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
     const int col0 = n0 + wn * 32 * NJ + c32;
     s.prepare(col0, col0 + 32);
 #pragma unroll
@@ -801,9 +814,90 @@ int launch_gemm_f32(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     return e;
 }
 
-int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
+// Sums the partial results [split][image][channel][position] of a convolution that split its input channels and applies
+// residual, bias and activation in the order the unsplit store does. VEC = 4: every thread owns four neighbouring
+// positions (out_h * out_w a multiple of 4).
+template <int VEC>
+__global__ __launch_bounds__(256) void conv_reduce_partials_kernel(ConvParams p) {
+    const long long ohw = (long long) p.out_h * p.out_w, total = (long long) p.batch * p.out_c * ohw;
+    const long long e = ((long long) blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (e >= total) return;
+    typedef float Vec __attribute__((ext_vector_type(VEC)));
+    Vec parts[4], sum;
+    for (int j = 0; j < VEC; j++) sum[j] = 0.0f;
+    for (int s0 = 0; s0 < p.splits; s0 += 4) {  // four requests in flight, added in the order of the slices
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (s0 + i < p.splits) parts[i] = *(const Vec *) (p.workspace + (long long) (s0 + i) * total + e);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (s0 + i < p.splits) sum += parts[i];
+    }
+    const int channel = (int) ((e / ohw) % p.out_c);
+    if (p.res) sum += *(const Vec *) (p.res + e);
+    if (p.bias) {
+        const float b = p.bias[channel * p.bias_stride];
+        for (int j = 0; j < VEC; j++) sum[j] += b;
+    }
+    if (p.relu)
+        for (int j = 0; j < VEC; j++) sum[j] = fmaxf(sum[j], 0.0f);
+    *(Vec *) (p.output + e) = sum;
+}
+
+int conv_channel_split(const ConvParams &p) {
+    static const bool enabled = [] {
+        const char *env = getenv("KNHIP_SPLIT_CONV");
+        return !env || atoi(env) != 0;
+    }();
+    const long long positions = (long long) p.batch * p.out_h * p.out_w;
+    if (!enabled || positions <= 0 || p.out_c <= 0) return 1;
+    // 64 x 64 tiles of four waves each, on 1024 SIMDs. The plane kernel keeps a SIMD busy with one wave, so it splits
+    // while half of the SIMDs would be idle; the patch kernel waits for its gathers and gains up to three waves per
+    // SIMD. Measured (us, unsplit -> split), 128 -> 128 channels on 8 x 8 boards: batch 16 28.9 -> 13.6, 32 -> 16.3,
+    // 64 29.4 -> 22.6; 192 -> 192 on 19 x 19: batch 1 -> 18.5, batch 8 120 -> 54..61. Only K loops of 512 steps or
+    // more are split, into slices of 16 channels or more, up to 16 of them.
+    const long long tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64);
+    const long long k = (long long) p.in_c * p.kernel_h * p.kernel_w;
+    ConvParams shape_only = p;
+    shape_only.input = shape_only.filter = nullptr;
+    PlaneGeom geom;
+    const long long target = plane_geometry(shape_only, 64, &geom) ? 1024 : 3072;
+    if (tiles * 4 * 2 > target || k < 512) return 1;
+    const long long most = std::min<long long>({16, target / (tiles * 4), p.in_c / 16});
+    if (most < 2) return 1;
+    // whole slices of CB channels per split, and no split without channels
+    const int slices = (p.in_c + CB - 1) / CB;
+    const int per_split = (int) ((slices + most - 1) / most);
+    return (slices + per_split - 1) / per_split;
+}
+
+size_t conv_workspace_bytes(const ConvParams &p) {
+    const int splits = conv_channel_split(p);
+    if (splits <= 1) return 0;
+    return (size_t) splits * p.batch * p.out_c * p.out_h * p.out_w * sizeof(float);
+}
+
+int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
+    ConvParams p = params;
     const long long positions = (long long) p.batch * p.out_h * p.out_w;
     if (positions <= 0 || p.out_c <= 0) return 0;
+    p.splits = conv_channel_split(p);
+    if (p.splits > 1) {
+        if (!p.workspace) return (int) hipErrorInvalidValue;
+        const int slices = (p.in_c + CB - 1) / CB;
+        p.split_channels = (slices + p.splits - 1) / p.splits * CB;
+    }
+    const bool split = p.splits > 1;
+    auto sum_slices = [&]() {
+        if (!split) return (int) hipGetLastError();
+        const long long total = (long long) p.batch * p.out_c * p.out_h * p.out_w;
+        const bool vec = (p.out_h * p.out_w) % 4 == 0 && (uintptr_t) p.output % 16 == 0 && (!p.res || (uintptr_t) p.res % 16 == 0);
+        const long long threads = vec ? total / 4 : total;
+        const dim3 grid((unsigned) ((threads + 255) / 256)), block(256);
+        if (vec) hipLaunchKernelGGL((conv_reduce_partials_kernel<4>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((conv_reduce_partials_kernel<1>), grid, block, 0, stream, p);
+        return (int) hipGetLastError();
+    };
     const long long big_tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
     if (positions > 0x7fffffffll || big_tiles > 0x7fffffffll / 4) return (int) hipErrorInvalidValue;
     if ((long long) p.out_c * p.out_h * p.out_w > 0x7fffffffll) return (int) hipErrorInvalidValue;
@@ -820,6 +914,7 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     const Variant *best = nullptr;
     double best_cost = 0.0;
     for (const Variant &v : variants) {
+        if (split && v.id != 11) continue;  // (few tiles: the small one)
         if (!plane_geometry(p, v.tn, &geom)) continue;
         const long long tiles = ((positions + v.tn - 1) / v.tn) * ((p.out_c + v.bm - 1) / v.bm);
         const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost;
@@ -828,23 +923,27 @@ int launch_conv_f32(const ConvParams &p, ihipStream_t *stream) {
     if (best) {
         plane_geometry(p, best->tn, &geom);
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
-        const dim3 grid((unsigned) tiles), block(THREADS);
+        const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
         const bool ragged = p.in_c % CB != 0;
         if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true>), grid, block, 0, stream, p, geom);
         else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false>), grid, block, 0, stream, p, geom);
         else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true>), grid, block, 0, stream, p, geom);
         else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false>), grid, block, 0, stream, p, geom);
-        return (int) hipGetLastError();
+        return sum_slices();
     }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
     const int a_mode = ((uintptr_t) p.filter % 16 == 0 && K % 4 == 0) ? VecK : Scalar;
-    if (big_tiles < small_tile_threshold()) {
-        const long long tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64);
-        launch_conv_t<1>(a_mode, dim3((unsigned) tiles), stream, p);
+    // the same estimate for the patch kernel: rounds of waves on 1024 SIMDs x MFMA tiles per wave (64 output channels on
+    // 128 x 128 tiles would leave half of every tile empty)
+    const long long small_tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64);
+    const double big_cost = (double) ((big_tiles * 4 + 1023) / 1024) * 4.0, small_cost = (double) ((small_tiles * 4 + 1023) / 1024) * 1.1;
+    if (split || big_tiles < small_tile_threshold() || small_cost < big_cost) {
+        const long long tiles = small_tiles;
+        launch_conv_t<1>(a_mode, dim3((unsigned) tiles, (unsigned) p.splits), stream, p);
     } else {
         launch_conv_t<2>(a_mode, dim3((unsigned) big_tiles), stream, p);
     }
-    return (int) hipGetLastError();
+    return sum_slices();
 }
 
 }  // namespace kn

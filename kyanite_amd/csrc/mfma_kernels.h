@@ -88,7 +88,19 @@ struct ConvParams {
     int kernel_h, kernel_w, stride_y, stride_x, pad_y, pad_x;
     long long bias_stride;
     int relu;
+    // f32 scratch of `conv_workspace_bytes` bytes (256 byte aligned) when the launch splits the input channels; may
+    // be null otherwise
+    float *workspace = nullptr;
+    // filled in by the launch: slices of the input channels that are folded side by side, and channels per slice
+    int splits = 1, split_channels = 0;
 };
+
+// A convolution with few output tiles and many input channels (small batches of small boards) leaves most of the chip
+// idle while every wave works through its K loop alone. The launch then folds `conv_channel_split` slices of the input
+// channels side by side into f32 partial results and a second kernel sums them and applies bias, residual and
+// activation. A function of the shapes alone, so that the planner can reserve the scratch ahead of time.
+int conv_channel_split(const ConvParams &p);
+size_t conv_workspace_bytes(const ConvParams &p);
 
 // O[b] = softmax(scale * Q[b] K[b]^T + mask[b]) V[b] with the softmax along the keys; Q is [batch, lq, dk],
 // K [batch, lk, dk], V [batch, lk, dv], O [batch, lq, dv], mask [batch, lq, lk], with arbitrary element strides (batch,

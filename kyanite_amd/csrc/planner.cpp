@@ -26,7 +26,7 @@ std::string Step::str() const {
     else if (kind == StepKind::Conv)
         ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="
            << conv.kernel_h << "x" << conv.kernel_w << (conv_has_bias ? " +bias" : "") << (conv_has_res ? " +res" : "")
-           << (conv.relu ? " relu" : "");
+           << (conv.relu ? " relu" : "") << (conv_channel_split(conv) > 1 ? " [input channels in " + std::to_string(conv_channel_split(conv)) + " slices]" : std::string());
     else ss << " [" << kernel.strategy << "] grid=" << kernel.grid << "x" << kernel.block;
     ss << " operands:";
     for (auto &op : operands) ss << " " << dtype_name(op.tensor.dtype) << vec_str(op.tensor.shape.shape());
@@ -1328,6 +1328,9 @@ private:
             if (bias_t) step.operands.push_back({*bias_t, OperandKind::In});
             if (res_t) step.operands.push_back({*res_t, OperandKind::In});
             step.operands.push_back({output, OperandKind::Out});
+            // partial results of a launch that splits the input channels
+            if (const size_t bytes = conv_workspace_bytes(p))
+                step.operands.push_back({alloc_tensor_shared({bytes / 4}, DType::F32), OperandKind::Out});
             push(std::move(step), value);
         }
         return R::done(output);

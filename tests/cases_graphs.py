@@ -1908,3 +1908,24 @@ def normalised_axis_is_not_the_contiguous_one():
     f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
     return g, 0, [f(3, 40, 7, 9), rng.standard_normal((2, 300, 130)).astype(np.float16), f(1000, 50), f(1000, 50),
                   f(1000, 1), f(1000, 1)], None
+
+
+@case
+def conv_with_input_channels_in_slices():
+    """few output tiles, many input channels: slices of the channels are folded side by side and a second kernel sums the
+    partial results and applies bias, residual and activation. A tower block of a small batch of boards (the kernel
+    that keeps raw planes in LDS), 200 channels on 5 x 5 boards (the patch kernel; 25 slices of 8 channels in 13
+    parts, the last one shorter; 25 positions per image, so no vectors in the summing pass), a 5 x 5 filter, and a
+    stride of 2"""
+    g = Graph()
+    rng = np.random.default_rng(172)
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    boards = g.input([2, 128, 8, 8])
+    bias = g.constant([1, 128, 1, 1], rng.standard_normal(128).astype(np.float32))
+    g.output(g.relu(g.add(g.add(g.conv(boards, w(128, 128, 3, 3), 1, 1, 1, 1), bias), boards)))
+    odd = g.input([1, 200, 5, 5])
+    g.output(g.add(g.conv(odd, w(72, 200, 3, 3), 1, 1, 1, 1), g.constant([1, 72, 1, 1], rng.standard_normal(72).astype(np.float32))))
+    g.output(g.conv(g.input([3, 64, 6, 6]), w(40, 64, 5, 5), 1, 1, 2, 2))
+    g.output(g.relu(g.conv(g.input([2, 96, 9, 9]), w(64, 96, 3, 3), 2, 2, 1, 1)))
+    f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    return g, 0, [f(2, 128, 8, 8), f(1, 200, 5, 5), f(3, 64, 6, 6), f(2, 96, 9, 9)], None
