@@ -630,8 +630,8 @@ int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool 
     bool aligned = (uintptr_t) p.a % 16 == 0;
     for (int g = 0; g < groups; g++) aligned = aligned && (uintptr_t) (groups > 1 ? p.b_group[g] : p.b) % 16 == 0;
     if (!aligned) return 0;
-    const int t = lp.small_tile ? 64 : 128;
-    const long long tiles = (long long) ((p.m + t - 1) / t) * ((p.n + t - 1) / t) * groups;
+    const int t_m = lp.skinny_tile ? 32 : (lp.small_tile ? 64 : 128), t_n = lp.skinny_tile ? 128 : t_m;
+    const long long tiles = (long long) ((p.m + t_m - 1) / t_m) * ((p.n + t_n - 1) / t_n) * groups;
     if (tiles > 0x7fffffffll) return (int) hipErrorInvalidConfiguration;
     dim3 grid((unsigned) tiles, (unsigned) p.batch, (unsigned) lp.split_k);
     DirectSchedule sched{lp.k_chunk, 64, (int) tiles, 1, p.k};
@@ -644,7 +644,8 @@ int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool 
     }
     // (64 x 64 tiles on three stages: 48 KB of LDS, so three workgroups share a compute unit; on four stages and two
     // workgroups the 8192 x 320 x 320 projections of a transformer block took 26.7 us instead of 24.9 us)
-    const int e = lp.small_tile ? launch_direct<float, 1, 1, 2, 2, 3>(grid, stream, p, sched) : launch_direct<float, 2, 2, 2, 2, 2>(grid, stream, p, sched);
+    const int e = lp.skinny_tile ? launch_direct<float, 1, 1, 1, 4, 3>(grid, stream, p, sched)
+                  : lp.small_tile ? launch_direct<float, 1, 1, 2, 2, 3>(grid, stream, p, sched) : launch_direct<float, 2, 2, 2, 2, 2>(grid, stream, p, sched);
     if (e != 0) return e;
     *launched = true;
     return (int) hipGetLastError();

@@ -57,6 +57,7 @@ struct GemmLaunchPlan {
     bool narrow_tile;        // f16 direct kernel only: 128 x 64 workgroup tiles
     bool wide_tile;          // f16 direct kernel only, together with tall_tile: 256 x 256 workgroup tiles
     bool mid_tile;           // f16 direct kernel only, together with tall_tile: 256 x 192 workgroup tiles
+    bool skinny_tile;        // f32 direct kernel only: 32 x 128 workgroup tiles, for left operands of up to 32 rows
     bool direct;             // shapes and strides allow the kernel that loads global -> LDS directly
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)

@@ -1074,19 +1074,22 @@ private:
         return R::done(results[0]);
     }
 
-    // A constant right operand of an f16 matmul whose n axis is the contiguous one ([k, n] weights, as `x @ w`
-    // exports them) is laid out again, once, on the host, as [n, k]: with K contiguous in both operands the matmul
-    // takes the direct global -> LDS path (512 x 11008 x 4096 twice in one launch: 157 us -> 116 us). The original
-    // constant stays out of the arena when nothing else reads it.
+    // A constant right operand of a matmul whose n axis is the contiguous one ([k, n] weights, as `x @ w` exports
+    // them) is laid out again, once, on the host, as [n, k]: with K contiguous in both operands the matmul takes the
+    // direct global -> LDS path (f16, 512 x 11008 x 4096 twice in one launch: 157 us -> 116 us; f32,
+    // 1024 x 4672 x 2048: 281 -> 175 us). That holds for a left operand of any height: under a few rows the product
+    // is a pass over the weights, which that path streams at twice the rate (f16, 8 x 32000 x 4096: 96 -> 40 us).
+    // The original constant stays out of the arena when nothing else reads it.
     std::map<std::tuple<size_t, int64_t, std::vector<size_t>, std::vector<int64_t>>, PlanTensor> packed_rights;
 
     PlanTensor pack_right_operand(const PlanTensor &left, const PlanTensor &right, DType dt) {
-        if (!options.pack_matmul_constants || dt != DType::F16 || right.ptr.kind != BufferKind::Constant) return right;
+        if (!options.pack_matmul_constants || right.ptr.kind != BufferKind::Constant) return right;
+        if (dt != DType::F16 && dt != DType::F32) return right;
         const auto &shape = right.shape.shape();
         const auto &strides = right.shape.strides();
         const size_t b = shape[0], k = shape[1], n = shape[2];
         if (b == 0 || n < 2 || k < 64 || k % 64 != 0 || strides[2] != 1 || strides[1] == 1) return right;
-        if (left.shape.strides()[2] != 1 || left.shape.shape()[1] < 16) return right;
+        if (left.shape.strides()[2] != 1) return right;
         if (strides[0] < 0 || strides[1] < 0) return right;
         auto key = std::make_tuple(right.ptr.index, right.ptr.offset_bytes, shape, strides);
         auto it = packed_rights.find(key);
@@ -1102,19 +1105,21 @@ private:
             KN_ASSERT(right.ptr.offset_bytes >= 0 && right.ptr.offset_bytes % (int64_t) elem == 0 && last < (int64_t) src.len());
         }
         HostTensor packed(dt, {copies, n, k});
-        const uint16_t *from = (const uint16_t *) (src.bytes() + right.ptr.offset_bytes);
-        uint16_t *to = (uint16_t *) packed.bytes_mut();
         constexpr size_t TILE = 64;  // both the reads and the writes of a tile stay in cache
-        for (size_t c = 0; c < copies; c++)
-            for (size_t k0 = 0; k0 < k; k0 += TILE)
-                for (size_t n0 = 0; n0 < n; n0 += TILE) {
-                    const size_t k1 = std::min(k, k0 + TILE), n1 = std::min(n, n0 + TILE);
-                    for (size_t ni = n0; ni < n1; ni++) {
-                        uint16_t *row = to + (c * n + ni) * k;
-                        const uint16_t *col = from + c * (size_t) strides[0] + ni;
-                        for (size_t ki = k0; ki < k1; ki++) row[ki] = col[ki * (size_t) strides[1]];
+        auto turn = [&](auto *to, const auto *from) {
+            for (size_t c = 0; c < copies; c++)
+                for (size_t k0 = 0; k0 < k; k0 += TILE)
+                    for (size_t n0 = 0; n0 < n; n0 += TILE) {
+                        const size_t k1 = std::min(k, k0 + TILE), n1 = std::min(n, n0 + TILE);
+                        for (size_t ni = n0; ni < n1; ni++) {
+                            auto *row = to + (c * n + ni) * k;
+                            const auto *col = from + c * (size_t) strides[0] + ni;
+                            for (size_t ki = k0; ki < k1; ki++) row[ki] = col[ki * (size_t) strides[1]];
+                        }
                     }
-                }
+        };
+        if (elem == 2) turn((uint16_t *) packed.bytes_mut(), (const uint16_t *) (src.bytes() + right.ptr.offset_bytes));
+        else turn((uint32_t *) packed.bytes_mut(), (const uint32_t *) (src.bytes() + right.ptr.offset_bytes));
         constants.push_back(std::move(packed));
         PlanTensor t;
         t.ptr = PlanPtr{BufferKind::Constant, constants.size() - 1, 0};

@@ -92,7 +92,7 @@ struct PlannerOptions {
     bool fuse_row_epilogue = true;  // fold elementwise consumers of a layernorm / softmax into the row kernel
     bool fuse_matmul_epilogue = true;  // fold `+ d` and `max(., 0)` after a matmul into the matmul's store
     bool fuse_attention = true;  // matmul, softmax, matmul chains in f32 run as one launch
-    bool pack_matmul_constants = true;  // constant [k, n] right operands of f16 matmuls are laid out again as [n, k]
+    bool pack_matmul_constants = true;  // constant [k, n] right operands of matmuls are laid out again as [n, k]
     bool group_matmuls = true;   // matmuls that share their left operand and have constant right operands share a launch
     bool pointwise_conv_as_matmul = true;  // 1 x 1 convolutions with stride 1 run as one matrix product per image
     bool join_elementwise = true;  // small elementwise steps of one shape that do not depend on each other share a launch

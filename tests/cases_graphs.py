@@ -1929,3 +1929,30 @@ def conv_with_input_channels_in_slices():
     g.output(g.relu(g.conv(g.input([2, 96, 9, 9]), w(64, 96, 3, 3), 2, 2, 1, 1)))
     f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
     return g, 0, [f(2, 128, 8, 8), f(1, 200, 5, 5), f(3, 64, 6, 6), f(2, 96, 9, 9)], None
+
+
+@case
+def products_with_few_rows():
+    """a left operand of 1, 8 and 32 rows against constant [k, n] weights, f32 and f16: the weights are laid out again
+    as [n, k] and the product runs on the kernel that loads global -> LDS directly (f32: on 32 x 128 tiles), with a
+    last tile of columns that is partial, a bias and an activation in the store, K split where it is long, and a
+    batch of left operands against one set of weights"""
+    g = Graph()
+    rng = np.random.default_rng(173)
+    inputs = []
+
+    def inp(shape, dtype):
+        inputs.append(rng.standard_normal(shape).astype(dtype.numpy))
+        return g.input(list(shape), dtype)
+
+    def weights(k, n, dtype):
+        return g.constant([k, n], (rng.standard_normal((k, n)) * 0.1).astype(dtype.numpy), dtype)
+
+    for dtype in (DType.F32, DType.F16):
+        g.output(g.mat_mul(inp((1, 256), dtype), weights(256, 300, dtype)))
+        bias = g.constant([1, 520], rng.standard_normal((1, 520)).astype(dtype.numpy), dtype)
+        g.output(g.relu(g.add(g.mat_mul(inp((8, 192), dtype), weights(192, 520, dtype)), g.broadcast(bias, [8, 520]))))
+        g.output(g.mat_mul(inp((32, 4096), dtype), weights(4096, 136, dtype)))
+        w = g.view(weights(128, 260, dtype), [1, 128, 260])
+        g.output(g.batched_mat_mul(inp((3, 5, 128), dtype), g.broadcast(w, [3, 128, 260])))
+    return g, 0, inputs, None

@@ -15,7 +15,7 @@ def test_workspace_query_needs_no_device():
     # short K, many tiles: nothing to split; long K on few tiles: partial products; a sparse last round: counters too
     assert batched_mat_mul_workspace_bytes(matmul_args(DType.F32, 1, 1024, 1024, 64, 1, (0, 64, 1), 1, (0, 1024, 1), 1, (0, 1024, 1))) == 0
     split = batched_mat_mul_workspace_bytes(matmul_args(DType.F32, 1, 8, 4096, 4096, 1, (0, 4096, 1), 1, (0, 1, 4096), 1, (0, 4096, 1)))
-    assert split == 8 * 8 * 4096 * 4
+    assert split == 16 * 8 * 4096 * 4  # 32 tiles of 32 x 128: K in 16 parts
     tail = batched_mat_mul_workspace_bytes(matmul_args(DType.F16, 1, 33, 33280, 1024, 1, (0, 1024, 1), 1, (0, 1, 1024), 1, (0, 33280, 1)))
     assert tail == 256 + 8 * 2 * 64 * 64 * 4  # 8 counters rounded up to 256 bytes, then 8 tiles x 2 parts of 64 x 64 floats
     with pytest.raises(KnError):
