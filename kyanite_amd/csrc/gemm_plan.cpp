@@ -197,7 +197,8 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     if (lp.mid_tile) blocks = mid_blocks;
     if (f16) lp.bk = lp.small_tile || lp.tall_tile || lp.narrow_tile ? 64 : 128;
     else if (lp.direct) lp.bk = 32;
-    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= 256 && small_blocks < 512)) ? 64 : 16;
+    // (a handful of tiles is a chain of memory round trips, one per slice: deep slices from 64 on)
+    else lp.bk = lp.small_tile && (p.k >= 2048 || (p.k >= 256 && small_blocks < 512) || (p.k >= 64 && few_tiles)) ? 64 : 16;
 
     // A tile count that leaves the last round of workgroups mostly idle: the direct kernel splits the tiles of just
     // that round along K and sums the parts inside the launch, so that the round is short instead of sparse.
@@ -240,7 +241,9 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     }
 
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
-    if (can_split && blocks < split_below && groups == 1 && !lp.narrow_tile) {
+    // (a product of a few thousand multiplications is one short workgroup: a second launch to sum parts costs more)
+    const bool tiny = (long long) p.batch * p.m * p.n * p.k < (1ll << 18);
+    if (can_split && blocks < split_below && groups == 1 && !lp.narrow_tile && !tiny) {
         const int min_chunk = few_tiles ? 128 : (f16 ? 512 : 256);  // K elements a split should at least cover
         long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;
