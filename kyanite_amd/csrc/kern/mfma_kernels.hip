@@ -392,13 +392,20 @@ struct PlaneGeom {
     int w4_shift, g_shift, rw_shift;  // log2 of W / 4, G, R * W
     int n_vec;           // CB * G * plane_rows * W / 4
     int row_stride;      // W + PLANE_PAD
+    // Any image size (template flag ANYW): a tile is TN consecutive positions of the (image, y, x) order, wherever
+    // they start. Every image counts H + 2 padded rows (an empty row above and below), so that the row above / below
+    // an output row is the padded row before / after its own, across image boundaries too; the tile stages the
+    // padded rows from the one above its first output row to the one below its last, `plane_rows` at most, float by
+    // float (`n_scalar` = CB * plane_rows * W of them per slice).
+    int n_scalar;
 };
+constexpr int PLANE_MAX_SCALAR = 8;  // 32 bit loads per thread and slice for the B planes of the ANYW variant
 
 // NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64); MI: the same along
 // the output channels (2 -> 128 channels per tile, 1 -> 64); RAGGED: the channel count is not a multiple of CB (the
 // 21 planes of a board game's input): the last slice takes zeros for the channels past the end, and the filter rows,
 // whose length is no multiple of 4 floats then, are read float by float.
-template <int KH, int KW, int NJ, int MI, bool RAGGED>
+template <int KH, int KW, int NJ, int MI, bool RAGGED, bool ANYW = false>
 __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, PlaneGeom g) {
     constexpr int TN = 64 * NJ;  // positions per tile
     constexpr int BM = 64 * MI;  // output channels per tile
@@ -418,26 +425,45 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     int tm, tn;
     tile_of_block(tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * TN;
-    int img0, oy0;
-    if (g.tiles_per_image) {
+    int img0 = 0, oy0 = 0;
+    if (ANYW) {
+    } else if (g.tiles_per_image) {
         img0 = tn / g.tiles_per_image;
         oy0 = (tn - img0 * g.tiles_per_image) * g.rows;
     } else {
         img0 = tn * g.groups;
-        oy0 = 0;
     }
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, c32 = lane & 31;
     const int RS = g.row_stride;
-    const int plane = g.plane_rows * RS, gplane = plane << g.g_shift;  // LDS floats per (c, g) and per c
+    const int plane = g.plane_rows * RS, gplane = ANYW ? plane : plane << g.g_shift;  // LDS floats per (c, g) and per c
+    // ANYW: the padded row above the tile's first output row (output row rho of the (image, y) order is padded row
+    // rho + 2 * (rho / H) + 1)
+    const int rho0 = n0 / W, pi_base = rho0 + 2 * (rho0 / H);
 
     // ---- B planes: what this thread moves per slice (the same places every slice, only the channel base moves)
+    constexpr int B_SLOTS = ANYW ? PLANE_MAX_SCALAR : PLANE_MAX_VEC;
     const float *b_src[PLANE_MAX_VEC];
-    int b_dst[PLANE_MAX_VEC];  // -1: nothing to move
-    int b_channel[PLANE_MAX_VEC];  // inside the slice
+    int b_dst[B_SLOTS];  // -1: nothing to move
+    int b_channel[B_SLOTS];  // inside the slice
+    int s_off[PLANE_MAX_SCALAR];  // ANYW: offset of the float inside the input, from channel 0 of the slice; -1: a zero
+    if (ANYW) {
 #pragma unroll
-    for (int i = 0; i < PLANE_MAX_VEC; i++) {
+        for (int i = 0; i < PLANE_MAX_SCALAR; i++) {
+            const int e = t + THREADS * i;
+            const int x = e % W, t1 = e / W;
+            const int c = t1 / g.plane_rows, prow = t1 - c * g.plane_rows;
+            const int pi = pi_base + prow, img = pi / (H + 2), iy = pi - img * (H + 2) - 1;
+            const bool inside = e < g.n_scalar && iy >= 0 && iy < H && img < p.batch;
+            // (the empty rows above and below an image are never written: they keep the zeros of the first fill)
+            b_dst[i] = inside ? PLANE_SLACK + t1 * RS + PLANE_PAD + x : -1;
+            s_off[i] = inside ? ((img * C + c) * H + iy) * W + x : -1;  // below 2^31: checked on the host
+            b_channel[i] = c;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < (ANYW ? 0 : PLANE_MAX_VEC); i++) {
         const int e = t + THREADS * i;
         const int w4 = e & ((1 << g.w4_shift) - 1), t1 = e >> g.w4_shift;
         const int t2 = t1 / g.plane_rows, prow = t1 - t2 * g.plane_rows;
@@ -464,13 +490,41 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
         const int n = wn * 32 * NJ + 32 * j + c32;
+        if (ANYW) {
+            // (positions past the end take the place of the last one; their results are never stored)
+            const int pos = (int) min((long long) n0 + n, N - 1), rho = pos / W, col = pos - rho * W;
+            lane_base[j] = PLANE_SLACK + (rho + 2 * (rho / H) - pi_base) * RS + PLANE_PAD + col - p.pad_x;
+            continue;
+        }
         const int gl = n >> g.rw_shift, rem = n & ((1 << g.rw_shift) - 1), col = rem & (W - 1), r = rem >> (g.w4_shift + 2);
         lane_base[j] = PLANE_SLACK + gl * plane + r * RS + PLANE_PAD + col - p.pad_x;
     }
 
     floatx4 ra[A_ITERS], rb[PLANE_MAX_VEC];
+    float rs[PLANE_MAX_SCALAR];
+    auto fetch_planes_any = [&](int c0) {
+        const float *from = p.input + (long long) c0 * ohw;
+#pragma unroll
+        for (int i = 0; i < PLANE_MAX_SCALAR; i++)
+            rs[i] = s_off[i] >= 0 && (!RAGGED || c0 + b_channel[i] < C) ? from[s_off[i]] : 0.0f;
+    };
     auto fetch = [&](int c0) {
         const long long a_off = (long long) c0 * KH * KW, b_off = (long long) c0 * ohw;
+        if (ANYW) {
+            fetch_planes_any(c0);
+            if (RAGGED) {
+#pragma unroll
+                for (int i = 0; i < A_ITERS; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        ra[i][j] = a_src[i] && a_off + a_k[i] + j < K ? (a_src[i] + a_off)[j] : 0.0f;
+            } else {
+#pragma unroll
+                for (int i = 0; i < A_ITERS; i++)
+                    ra[i] = a_src[i] ? *(const floatx4 *) (a_src[i] + a_off) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+            return;
+        }
         if (RAGGED) {
 #pragma unroll
             for (int i = 0; i < A_ITERS; i++)
@@ -497,6 +551,12 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
 #pragma unroll
                 for (int j = 0; j < 4; j++) a_flat[a_dst[i] + j * A_STRIDE] = ra[i][j];
             }
+        if (ANYW) {
+#pragma unroll
+            for (int i = 0; i < PLANE_MAX_SCALAR; i++)
+                if (b_dst[i] >= 0) Bs[b_dst[i]] = rs[i];
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < PLANE_MAX_VEC; i++)
             if (b_dst[i] >= 0) *(floatx4 *) &Bs[b_dst[i]] = rb[i];
@@ -631,6 +691,27 @@ bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     g->row_stride = W + PLANE_PAD;
     if (g->g_shift < 0 || g->rw_shift < 0 || g->n_vec > PLANE_MAX_VEC * THREADS) return false;
     if (CB * g->groups * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
+    return true;
+}
+
+// The same for the variant that takes any image size (3 x 3, stride 1, same-size output): tiles of `tn` consecutive
+// positions.
+bool plane_geometry_any(const ConvParams &p, int tn, PlaneGeom *g) {
+    if (p.kernel_h != 3 || p.kernel_w != 3 || p.stride_y != 1 || p.stride_x != 1) return false;
+    if (p.pad_y != 1 || p.pad_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
+    if (p.in_c <= 0 || (p.in_c % CB == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
+    const int W = p.in_w, H = p.in_h;
+    if (W < 2 || H < 1 || (long long) p.batch * p.in_c * H * W >= (1ll << 31)) return false;
+    // output rows that `tn` consecutive positions can touch, image boundaries between them, and the padded rows
+    // from the one above the first to the one below the last
+    const int touched = (tn - 2) / W + 2, crossings = (touched - 2) / H + 1;
+    *g = PlaneGeom{};
+    g->groups = 1;
+    g->plane_rows = touched + 2 * crossings + 2;
+    g->row_stride = W + PLANE_PAD;
+    g->n_scalar = CB * g->plane_rows * W;
+    if (g->n_scalar > PLANE_MAX_SCALAR * THREADS) return false;
+    if (CB * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
     return true;
 }
 
@@ -861,7 +942,7 @@ int conv_channel_split(const ConvParams &p) {
     ConvParams shape_only = p;
     shape_only.input = shape_only.filter = nullptr;
     PlaneGeom geom;
-    const long long target = plane_geometry(shape_only, 64, &geom) ? 1024 : 3072;
+    const long long target = plane_geometry(shape_only, 64, &geom) || plane_geometry_any(shape_only, 64, &geom) ? 1024 : 3072;
     if (tiles * 4 * 2 > target || k < 512) return 1;
     const long long most = std::min<long long>({16, target / (tiles * 4), p.in_c / 16});
     if (most < 2) return 1;
@@ -913,12 +994,26 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
     static const Variant variants[2] = {{128, 128, 22, 4 * 1.00}, {64, 64, 11, 1 * 1.10}};
     const Variant *best = nullptr;
     double best_cost = 0.0;
+    static const bool any_enabled = !(getenv("KNHIP_PLANE_ANY") && atoi(getenv("KNHIP_PLANE_ANY")) == 0);
+    bool any_w = false;
     for (const Variant &v : variants) {
         if (split && v.id != 11) continue;  // (few tiles: the small one)
-        if (!plane_geometry(p, v.tn, &geom)) continue;
+        const bool classic = plane_geometry(p, v.tn, &geom);
+        if (!classic && !(any_enabled && plane_geometry_any(p, v.tn, &geom))) continue;
         const long long tiles = ((positions + v.tn - 1) / v.tn) * ((p.out_c + v.bm - 1) / v.bm);
         const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost;
-        if (!best || cost < best_cost) { best = &v; best_cost = cost; }
+        if (!best || cost < best_cost) { best = &v; best_cost = cost; any_w = !classic; }
+    }
+    if (best && any_w) {
+        plane_geometry_any(p, best->tn, &geom);
+        const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
+        const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
+        const bool ragged = p.in_c % CB != 0;
+        if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true, true>), grid, block, 0, stream, p, geom);
+        else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false, true>), grid, block, 0, stream, p, geom);
+        else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true, true>), grid, block, 0, stream, p, geom);
+        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false, true>), grid, block, 0, stream, p, geom);
+        return sum_slices();
     }
     if (best) {
         plane_geometry(p, best->tn, &geom);

@@ -1956,3 +1956,31 @@ def products_with_few_rows():
         w = g.view(weights(128, 260, dtype), [1, 128, 260])
         g.output(g.batched_mat_mul(inp((3, 5, 128), dtype), g.broadcast(w, [3, 128, 260])))
     return g, 0, inputs, None
+
+
+@case
+def conv_on_boards_of_any_size():
+    """3 x 3 same-size convolutions on images whose width is no power of two run on the kernel that keeps raw planes in
+    LDS too: a tile is 128 (or 64) consecutive positions wherever they start, and stages the padded rows around them,
+    across image boundaries. 9 x 9 boards with bias, residual and activation and a last tile that is partial; 7 x 7;
+    19 x 19 (a tile holds a third of an image); 5 rows of 3; 3 x 3 boards (forty images per tile); 21 input planes
+    (a channel count that is no multiple of 8); and a batch small enough that the input channels are split"""
+    g = Graph()
+    rng = np.random.default_rng(174)
+    inputs = []
+
+    def inp(*shape):
+        inputs.append(rng.standard_normal(shape).astype(np.float32))
+        return g.input(list(shape))
+
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    boards = inp(37, 72, 9, 9)
+    bias = g.constant([1, 72, 1, 1], rng.standard_normal(72).astype(np.float32))
+    g.output(g.relu(g.add(g.add(g.conv(boards, w(72, 72, 3, 3), 1, 1, 1, 1), bias), boards)))
+    g.output(g.conv(inp(20, 64, 7, 7), w(130, 64, 3, 3), 1, 1, 1, 1))
+    g.output(g.conv(inp(3, 32, 19, 19), w(64, 32, 3, 3), 1, 1, 1, 1))
+    g.output(g.conv(inp(11, 16, 5, 3), w(8, 16, 3, 3), 1, 1, 1, 1))
+    g.output(g.conv(inp(50, 16, 3, 3), w(24, 16, 3, 3), 1, 1, 1, 1))
+    g.output(g.relu(g.conv(inp(9, 21, 9, 9), w(40, 21, 3, 3), 1, 1, 1, 1)))
+    g.output(g.conv(inp(2, 128, 9, 9), w(64, 128, 3, 3), 1, 1, 1, 1))
+    return g, 0, inputs, None
