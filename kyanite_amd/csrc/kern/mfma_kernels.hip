@@ -398,15 +398,20 @@ struct PlaneGeom {
     // padded rows from the one above its first output row to the one below its last, `plane_rows` at most, float by
     // float (`n_scalar` = CB * plane_rows * W of them per slice).
     int n_scalar;
+    int by4;  // the image width is a multiple of 4 and the input 16 byte aligned: staged four floats at a time
 };
 constexpr int PLANE_MAX_SCALAR = 8;  // 32 bit loads per thread and slice for the B planes of the ANYW variant
+constexpr int PLANE_MAX_VEC4 = 4;    // 128 bit loads per thread and slice for the same when the width is a multiple of 4
 
 // NJ: MFMA tiles per wave along the positions (2 -> 128 positions per workgroup tile, 1 -> 64); MI: the same along
 // the output channels (2 -> 128 channels per tile, 1 -> 64); RAGGED: the channel count is not a multiple of CB (the
 // 21 planes of a board game's input): the last slice takes zeros for the channels past the end, and the filter rows,
 // whose length is no multiple of 4 floats then, are read float by float.
-template <int KH, int KW, int NJ, int MI, bool RAGGED, bool ANYW = false>
+template <int KH, int KW, int NJ, int MI, bool RAGGED, int ANYW = 0>
 __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, PlaneGeom g) {
+    // ANYW: 0 the power-of-two variant; 1 any image size, planes staged float by float; 2 the same with an image width
+    // that is a multiple of 4, staged four floats at a time
+    constexpr int EW = ANYW == 2 ? 4 : 1, ANY_SLOTS = ANYW == 2 ? PLANE_MAX_VEC4 : PLANE_MAX_SCALAR;
     constexpr int TN = 64 * NJ;  // positions per tile
     constexpr int BM = 64 * MI;  // output channels per tile
     constexpr int KS = CB * KH * KW;      // K slice
@@ -443,19 +448,20 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     const int rho0 = n0 / W, pi_base = rho0 + 2 * (rho0 / H);
 
     // ---- B planes: what this thread moves per slice (the same places every slice, only the channel base moves)
-    constexpr int B_SLOTS = ANYW ? PLANE_MAX_SCALAR : PLANE_MAX_VEC;
+    constexpr int B_SLOTS = ANYW ? ANY_SLOTS : PLANE_MAX_VEC;
     const float *b_src[PLANE_MAX_VEC];
     int b_dst[B_SLOTS];  // -1: nothing to move
     int b_channel[B_SLOTS];  // inside the slice
-    int s_off[PLANE_MAX_SCALAR];  // ANYW: offset of the float inside the input, from channel 0 of the slice; -1: a zero
+    int s_off[ANY_SLOTS];  // ANYW: offset of the float(s) inside the input, from channel 0 of the slice; -1: zeros
     if (ANYW) {
+        const int wq = W / EW;  // loads per image row
 #pragma unroll
-        for (int i = 0; i < PLANE_MAX_SCALAR; i++) {
+        for (int i = 0; i < ANY_SLOTS; i++) {
             const int e = t + THREADS * i;
-            const int x = e % W, t1 = e / W;
+            const int x = (e % wq) * EW, t1 = e / wq;
             const int c = t1 / g.plane_rows, prow = t1 - c * g.plane_rows;
             const int pi = pi_base + prow, img = pi / (H + 2), iy = pi - img * (H + 2) - 1;
-            const bool inside = e < g.n_scalar && iy >= 0 && iy < H && img < p.batch;
+            const bool inside = e * EW < g.n_scalar && iy >= 0 && iy < H && img < p.batch;
             // (the empty rows above and below an image are never written: they keep the zeros of the first fill)
             b_dst[i] = inside ? PLANE_SLACK + t1 * RS + PLANE_PAD + x : -1;
             s_off[i] = inside ? ((img * C + c) * H + iy) * W + x : -1;  // below 2^31: checked on the host
@@ -501,12 +507,16 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     }
 
     floatx4 ra[A_ITERS], rb[PLANE_MAX_VEC];
-    float rs[PLANE_MAX_SCALAR];
+    float rs[ANYW == 1 ? ANY_SLOTS : 1];
+    floatx4 rv[ANYW == 2 ? ANY_SLOTS : 1];
     auto fetch_planes_any = [&](int c0) {
         const float *from = p.input + (long long) c0 * ohw;
 #pragma unroll
-        for (int i = 0; i < PLANE_MAX_SCALAR; i++)
-            rs[i] = s_off[i] >= 0 && (!RAGGED || c0 + b_channel[i] < C) ? from[s_off[i]] : 0.0f;
+        for (int i = 0; i < ANY_SLOTS; i++) {
+            const bool wanted = s_off[i] >= 0 && (!RAGGED || c0 + b_channel[i] < C);
+            if constexpr (ANYW == 2) rv[i] = wanted ? *(const floatx4 *) (from + s_off[i]) : floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            else rs[i] = wanted ? from[s_off[i]] : 0.0f;
+        }
     };
     auto fetch = [&](int c0) {
         const long long a_off = (long long) c0 * KH * KW, b_off = (long long) c0 * ohw;
@@ -553,8 +563,11 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             }
         if (ANYW) {
 #pragma unroll
-            for (int i = 0; i < PLANE_MAX_SCALAR; i++)
-                if (b_dst[i] >= 0) Bs[b_dst[i]] = rs[i];
+            for (int i = 0; i < ANY_SLOTS; i++)
+                if (b_dst[i] >= 0) {
+                    if constexpr (ANYW == 2) *(floatx4 *) &Bs[b_dst[i]] = rv[i];
+                    else Bs[b_dst[i]] = rs[i];
+                }
             return;
         }
 #pragma unroll
@@ -710,7 +723,8 @@ bool plane_geometry_any(const ConvParams &p, int tn, PlaneGeom *g) {
     g->plane_rows = touched + 2 * crossings + 2;
     g->row_stride = W + PLANE_PAD;
     g->n_scalar = CB * g->plane_rows * W;
-    if (g->n_scalar > PLANE_MAX_SCALAR * THREADS) return false;
+    g->by4 = W % 4 == 0 && (uintptr_t) p.input % 16 == 0;
+    if (g->n_scalar > (g->by4 ? 4 * PLANE_MAX_VEC4 : PLANE_MAX_SCALAR) * THREADS) return false;
     if (CB * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
     return true;
 }
@@ -1009,10 +1023,15 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
         const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
         const bool ragged = p.in_c % CB != 0;
-        if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true, true>), grid, block, 0, stream, p, geom);
-        else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false, true>), grid, block, 0, stream, p, geom);
-        else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true, true>), grid, block, 0, stream, p, geom);
-        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false, true>), grid, block, 0, stream, p, geom);
+        const bool by4 = geom.by4 != 0;
+        if (best->id == 22 && ragged && by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true, 2>), grid, block, 0, stream, p, geom);
+        else if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true, 1>), grid, block, 0, stream, p, geom);
+        else if (best->id == 22 && by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false, 2>), grid, block, 0, stream, p, geom);
+        else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false, 1>), grid, block, 0, stream, p, geom);
+        else if (ragged && by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true, 2>), grid, block, 0, stream, p, geom);
+        else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true, 1>), grid, block, 0, stream, p, geom);
+        else if (by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false, 2>), grid, block, 0, stream, p, geom);
+        else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false, 1>), grid, block, 0, stream, p, geom);
         return sum_slices();
     }
     if (best) {

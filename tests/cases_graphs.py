@@ -1984,3 +1984,26 @@ def conv_on_boards_of_any_size():
     g.output(g.relu(g.conv(inp(9, 21, 9, 9), w(40, 21, 3, 3), 1, 1, 1, 1)))
     g.output(g.conv(inp(2, 128, 9, 9), w(64, 128, 3, 3), 1, 1, 1, 1))
     return g, 0, inputs, None
+
+
+@case
+def conv_on_images_with_rows_of_whole_vectors():
+    """the same kernel on image widths that are a multiple of 4 but no power of two (56, 28, 12, 20): the padded rows are
+    staged four floats at a time. A tile of 128 positions is a little over two rows of a 56 x 56 image; 21 input planes;
+    an input that is a slice of a larger tensor, so that its rows lose their alignment (float by float then)"""
+    g = Graph()
+    rng = np.random.default_rng(175)
+    inputs = []
+
+    def inp(*shape):
+        inputs.append(rng.standard_normal(shape).astype(np.float32))
+        return g.input(list(shape))
+
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    g.output(g.relu(g.conv(inp(2, 16, 56, 56), w(24, 16, 3, 3), 1, 1, 1, 1)))
+    g.output(g.conv(inp(3, 24, 28, 28), w(70, 24, 3, 3), 1, 1, 1, 1))
+    g.output(g.conv(inp(5, 8, 12, 12), w(16, 8, 3, 3), 1, 1, 1, 1))
+    g.output(g.conv(inp(2, 21, 12, 20), w(32, 21, 3, 3), 1, 1, 1, 1))
+    wide = inp(2, 8, 12, 13)
+    g.output(g.conv(g.slice(wide, 3, 1, 13), w(16, 8, 3, 3), 1, 1, 1, 1))
+    return g, 0, inputs, None
