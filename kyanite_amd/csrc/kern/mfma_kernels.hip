@@ -135,7 +135,10 @@ struct PatchLoader {
     static constexpr int EPT = BK * WIDTH / THREADS;
     static constexpr int LDS_STRIDE = WIDTH + 4;
     const float *base;  // input of this thread's image, or null when n is out of range
-    int K, in_h, in_w, kh, kw, iy0, ix0;
+    int K, in_h, in_w, kh, kw;
+    int pos_off;               // iy0 * in_w + ix0: where tap (0, 0) of channel 0 lies for this thread's position
+    unsigned long long taps;   // bit fy * kw + fx: the tap lies inside the image for this thread's position
+    int iy0, ix0;              // (filters of more than 64 taps test the bounds per element instead)
     float r[EPT];
 
     __device__ __forceinline__ PatchLoader(const ConvParams &p, int n0) {
@@ -147,28 +150,42 @@ struct PatchLoader {
         const int n = n0 + (threadIdx.x % WIDTH);
         const int ohw = p.out_h * p.out_w;
         const long long total = (long long) p.batch * ohw;
+        taps = 0;
         if (n < total) {
             const int img = n / ohw, pos = n - img * ohw;
             const int oy = pos / p.out_w, ox = pos - oy * p.out_w;
             iy0 = oy * p.stride_y - p.pad_y;
             ix0 = ox * p.stride_x - p.pad_x;
             base = p.input + (long long) img * p.in_c * in_h * in_w;
+            if (kh * kw <= 64)
+                for (int fy = 0; fy < kh; fy++)
+                    for (int fx = 0; fx < kw; fx++)
+                        if (iy0 + fy >= 0 && iy0 + fy < in_h && ix0 + fx >= 0 && ix0 + fx < in_w) taps |= 1ull << (fy * kw + fx);
         } else {
             base = nullptr;
             iy0 = ix0 = 0;
         }
+        pos_off = iy0 * in_w + ix0;
     }
 
+    // Every thread of a wave loads the same k (a wave covers 64 of the WIDTH positions of one k), so the split of k
+    // into (channel, tap) and the tap's offset run on the scalar unit; a lane adds its position and tests one bit.
     __device__ __forceinline__ void fetch(int k0) {
         const int khw = kh * kw;
+        const int k_row = __builtin_amdgcn_readfirstlane((int) threadIdx.x / WIDTH);
 #pragma unroll
         for (int i = 0; i < EPT; i++) {
-            const int k = k0 + threadIdx.x / WIDTH + (THREADS / WIDTH) * i;
+            const int k = k0 + k_row + (THREADS / WIDTH) * i;
             const int c = k / khw, rem = k - c * khw;
             const int fy = rem / kw, fx = rem - fy * kw;
-            const int iy = iy0 + fy, ix = ix0 + fx;
-            const bool ok = base != nullptr && k < K && iy >= 0 && iy < in_h && ix >= 0 && ix < in_w;
-            r[i] = ok ? base[((long long) c * in_h + iy) * in_w + ix] : 0.0f;
+            if (khw <= 64) {
+                const bool ok = k < K && ((taps >> rem) & 1ull) != 0;  // (no image: no taps)
+                r[i] = ok ? base[(c * in_h + fy) * in_w + fx + pos_off] : 0.0f;  // inside one image: below 2^31, checked on the host
+            } else {
+                const int iy = iy0 + fy, ix = ix0 + fx;
+                const bool ok = base != nullptr && k < K && iy >= 0 && iy < in_h && ix >= 0 && ix < in_w;
+                r[i] = ok ? base[((long long) c * in_h + iy) * in_w + ix] : 0.0f;
+            }
         }
     }
 
@@ -841,6 +858,8 @@ template <int TI>
 void launch_conv_t(int a_mode, dim3 grid, hipStream_t stream, const ConvParams &p) {
     if (p.kernel_h == 3 && p.kernel_w == 3) launch_conv_k<3, 3, TI>(a_mode, grid, stream, p);
     else if (p.kernel_h == 1 && p.kernel_w == 1) launch_conv_k<1, 1, TI>(a_mode, grid, stream, p);
+    else if (p.kernel_h == 5 && p.kernel_w == 5) launch_conv_k<5, 5, TI>(a_mode, grid, stream, p);
+    else if (p.kernel_h == 7 && p.kernel_w == 7) launch_conv_k<7, 7, TI>(a_mode, grid, stream, p);
     else launch_conv_k<0, 0, TI>(a_mode, grid, stream, p);
 }
 
@@ -995,7 +1014,7 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
     };
     const long long big_tiles = ((positions + BN - 1) / BN) * ((p.out_c + BM - 1) / BM);
     if (positions > 0x7fffffffll || big_tiles > 0x7fffffffll / 4) return (int) hipErrorInvalidValue;
-    if ((long long) p.out_c * p.out_h * p.out_w > 0x7fffffffll) return (int) hipErrorInvalidValue;
+    if ((long long) p.out_c * p.out_h * p.out_w > 0x7fffffffll || (long long) p.in_c * p.in_h * p.in_w > 0x7fffffffll) return (int) hipErrorInvalidValue;
     // Plane kernel tiles (output channels x positions): 128 x 128 or 64 x 64, each wave owning 4 or 1 MFMA tiles of
     // the result. The waves of all workgroups spread over 1024 SIMDs and the launch takes about as long as the
     // busiest SIMD: rounds of waves x MFMA tiles per wave. The small tile costs a tenth more per MFMA tile (more LDS
