@@ -138,6 +138,34 @@ def test_softmax_rows_past_2_31_elements(hip_device, block):
     check_outputs(small, 0, [sample], cpu_eval_graph(small, 0, [sample]), [got], "softmax rows of a 4 GiB tensor", PARITY_RECORDS)
 
 
+def test_softmax_over_a_middle_axis_past_2_31_elements(hip_device, block):
+    """the normalised axis is not the contiguous one: lanes across columns, every column read again per pass"""
+    batch, length, width = 3, 700, (1 << 20) + 8
+    g = Graph()
+    x = g.input([batch, length, width], DType.F16)
+    g.output(g.softmax(x, 1))
+    plan = HipExecutor(0, g, 0, plan_only=True)
+    assert "columns" in plan.step_str(0) and "typedef long long idx_t" in plan.step_source(0)
+    ex = HipExecutor(hip_device, g, 0)
+    _fill_input(ex, 0, block, batch * length * width)
+    _run(ex)
+    # 16 neighbouring columns at a time: the first and the last of every batch entry, and either side of the place
+    # where a 32 bit element index would wrap (flat element 2^31 lies in batch entry 2)
+    wrap_row, wrap_col = divmod(PAST_I32 - 2 * length * width, width)
+    picked = [(0, 0), (0, width - 16), (1, 524288), (2, min(wrap_col, width - 16)), (2, width - 16)]
+    small = Graph()
+    small.output(small.softmax(small.input([len(picked), length, 16], DType.F16), 1))
+    sample = np.empty((len(picked), length, 16), np.float16)
+    got = np.empty_like(sample)
+    for i, (b, col) in enumerate(picked):
+        for row in range(length):
+            first = (b * length + row) * width + col
+            sample[i, row] = _stretch(block, first, 16)
+            got[i, row] = _fetch(ex, 0, first, 16, np.float16)
+    check_outputs(small, 0, [sample], cpu_eval_graph(small, 0, [sample]), [got], "softmax over the middle axis of a 4.4 GB tensor",
+                  PARITY_RECORDS)
+
+
 def test_reduce_past_2_31_elements(hip_device, block):
     rows, width = (1 << 19) + 1, BLOCK_WIDTH
     g = Graph()
