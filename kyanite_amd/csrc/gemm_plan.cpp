@@ -110,6 +110,16 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     lp.tail_split = 1;
     lp.tail_k_chunk = p.k;
     if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return lp;
+    // A product this small is a chain of memory round trips whichever way it is tiled, and a 64 x 64 tile spends its
+    // MFMAs on rows and columns that do not exist (the value head's 1 x 1 x 256 took 15.7 us, the 32 x 64 x 128 of a
+    // 1 x 1 convolution on one board 12.1 us): one wave per result instead, lanes along K.
+    static const int dot_enabled = env_int("KNHIP_DOT_PRODUCTS", 1);
+    if (dot_enabled && p.groups <= 1 && p.k > 0 && (long long) p.batch * p.m * p.n * p.k <= (1ll << 20) && (long long) p.batch * p.m * p.n <= 16384) {
+        lp.dot = true;
+        lp.small_tile = true;
+        lp.bk = 64;
+        return lp;
+    }
 
     // 128 x 128 tiles unless there are too few of them to fill the chip. Measured thresholds: f32 344 tiles run
     // 534 us on 64 x 64 tiles against 597 us, 512 tiles 734 us against 662 us; f16 344 tiles 112 us against 85 us,
@@ -264,6 +274,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
 
 std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16) {
     std::ostringstream ss;
+    if (lp.dot) return "a wave per result";
     int tm = lp.small_tile ? 64 : 128, tn = tm;
     if (lp.tall_tile) tm = 256;
     if (lp.narrow_tile) tn = 64;

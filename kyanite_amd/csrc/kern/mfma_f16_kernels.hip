@@ -654,6 +654,7 @@ int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool 
 int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     const GemmParams &p = lp.p;
     if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
+    if (lp.dot) return launch_gemm_dot(lp, true, stream);
     const int groups = p.groups > 1 ? p.groups : 1;
     if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || lp.swapped))) return (int) hipErrorInvalidValue;
     if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;

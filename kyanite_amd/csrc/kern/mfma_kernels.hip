@@ -899,9 +899,42 @@ int launch_gemm_reduce_partials(const GemmParams &p, int split, bool f16, ihipSt
     return (int) hipGetLastError();
 }
 
+// Tiny products: one wave per result element, lanes along K, a butterfly over the lanes, and the epilogue of the tiled
+// kernels (f16: the product, and each sum with an addend, rounded to f16 like separate operations would round them).
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_dot_kernel(GemmParams p) {
+    const long long result = ((long long) blockIdx.x * 256 + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (result >= (long long) p.batch * p.m * p.n) return;  // (a whole wave at a time)
+    const int col = (int) (result % p.n), row = (int) (result / p.n % p.m), bz = (int) (result / p.n / p.m);
+    const T *a = (const T *) p.a + bz * p.a_sb + (long long) row * p.a_sm;
+    const T *b = (const T *) p.b + bz * p.b_sb + (long long) col * p.b_sn;
+    float acc = 0.0f;
+    for (int k = lane; k < p.k; k += 64) acc += (float) a[(long long) k * p.a_sk] * (float) b[(long long) k * p.b_sk];
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) acc += __shfl_xor(acc, m, 64);
+    if (lane != 0) return;
+    T r = (T) acc;
+    if (p.addend) r = (T) ((float) r + (float) ((const T *) p.addend)[bz * p.d_sb + (long long) row * p.d_sm + (long long) col * p.d_sn]);
+    if (p.addend2) r = (T) ((float) r + (float) ((const T *) p.addend2)[bz * p.d2_sb + (long long) row * p.d2_sm + (long long) col * p.d2_sn]);
+    if (p.relu) r = r > (T) 0 ? r : (T) 0;
+    ((T *) p.c)[bz * p.c_sb + (long long) row * p.c_sm + (long long) col * p.c_sn] = r;
+}
+
+int launch_gemm_dot(const GemmLaunchPlan &lp, bool f16, ihipStream_t *stream) {
+    const GemmParams &p = lp.p;
+    if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;
+    const long long results = (long long) p.batch * p.m * p.n;
+    const dim3 grid((unsigned) ((results * 64 + 255) / 256)), block(256);
+    if (f16) hipLaunchKernelGGL((gemm_dot_kernel<_Float16>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_dot_kernel<float>), grid, block, 0, stream, p);
+    return (int) hipGetLastError();
+}
+
 int launch_gemm_f32(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     const GemmParams &p = lp.p;
     if (p.batch <= 0 || p.m <= 0 || p.n <= 0) return 0;
+    if (lp.dot) return launch_gemm_dot(lp, false, stream);
     const int t = lp.small_tile ? 64 : 128;
     const int groups = p.groups > 1 ? p.groups : 1;
     if (groups > GEMM_MAX_GROUPS || (groups > 1 && (lp.split_k > 1 || p.addend || lp.swapped))) return (int) hipErrorInvalidValue;

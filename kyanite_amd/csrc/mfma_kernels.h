@@ -58,6 +58,7 @@ struct GemmLaunchPlan {
     bool wide_tile;          // f16 direct kernel only, together with tall_tile: 256 x 256 workgroup tiles
     bool mid_tile;           // f16 direct kernel only, together with tall_tile: 256 x 192 workgroup tiles
     bool skinny_tile;        // f32 direct kernel only: 32 x 128 workgroup tiles, for left operands of up to 32 rows
+    bool dot;                // a product of up to 2^20 multiplications: one wave per result, no tiles, no MFMA
     bool direct;             // shapes and strides allow the kernel that loads global -> LDS directly
     int bk;                  // depth of a K slice
     int split_k;             // workgroups along K per output tile (1 = no split)
@@ -69,6 +70,8 @@ struct GemmLaunchPlan {
     size_t counter_bytes;    // one int per shared tile
 };
 GemmLaunchPlan plan_gemm_launch(const GemmParams &p, bool f16);
+// the launch of a plan with `dot` set (both element types; `mfma_kernels.hip`)
+int launch_gemm_dot(const GemmLaunchPlan &lp, bool f16, ihipStream_t *stream);
 // "direct 256x128 bk64 head=256 tail_split=2x2048": kernel family, workgroup tile, slice depth and the splits
 std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16);
 // whether `p.groups` products may share one launch: no operand swap, no K split, no epilogue

@@ -2007,3 +2007,33 @@ def conv_on_images_with_rows_of_whole_vectors():
     wide = inp(2, 8, 12, 13)
     g.output(g.conv(g.slice(wide, 3, 1, 13), w(16, 8, 3, 3), 1, 1, 1, 1))
     return g, 0, inputs, None
+
+
+@case
+def tiny_products_one_wave_per_result():
+    """products of a few thousand multiplications run with one wave per result and lanes along K: K shorter than a wave
+    (5) and no multiple of it (200), a transposed right operand, a batch, bias and skip connection and activation in
+    the store, f16 with its roundings, and a single dot product"""
+    g = Graph()
+    rng = np.random.default_rng(176)
+    inputs = []
+
+    def inp(shape, dtype=DType.F32):
+        inputs.append(rng.standard_normal(shape).astype(dtype.numpy))
+        return g.input(list(shape), dtype)
+
+    g.output(g.mat_mul(inp((7, 5)), inp((5, 3))))
+    g.output(g.mat_mul(inp((1, 200)), g.permute(inp((9, 200)), [1, 0])))
+    x, skip = inp((3, 6, 40)), inp((3, 6, 10))
+    w = g.constant([1, 40, 10], rng.standard_normal((1, 40, 10)).astype(np.float32))
+    bias = g.constant([1, 1, 10], rng.standard_normal((1, 1, 10)).astype(np.float32))
+    g.output(g.relu(g.add(skip, g.add(g.batched_mat_mul(x, g.broadcast(w, [3, 40, 10])), g.broadcast(bias, [3, 6, 10])))))
+    h = inp((4, 100), DType.F16)
+    hw = g.constant([100, 12], (rng.standard_normal((100, 12)) * 0.2).astype(np.float16), DType.F16)
+    hb = g.constant([1, 12], rng.standard_normal((1, 12)).astype(np.float16), DType.F16)
+    g.output(g.relu(g.add(g.mat_mul(h, hw), g.broadcast(hb, [4, 12]))))
+    g.output(g.mat_mul(inp((1, 256)), inp((256, 1))))
+    from kyanite_amd import HipExecutor
+    ex = HipExecutor(0, g, 0, plan_only=True)
+    assert all("a wave per result" in ex.step_str(i) for i in range(ex.step_count()) if ex.step_kinds()[i] == "mat_mul")
+    return g, 0, inputs, None
