@@ -5,9 +5,10 @@
 Families (default: all): `elementwise`, `reduce`, `rows` (softmax / layernorm), `conv`, `matmul`. `-p` plans and
 compiles every case without a device and prints its steps instead of running it.
 
-Every case is built like a user's graph (inputs, constants for weights), runs `-n` times back to back between two
-events on the executor's stream after two untimed runs, and is reported with the bytes its inputs and outputs hold
-(TB/s) and, for convolutions and products, its arithmetic (TFLOP/s), next to the kernels the planner chose.
+Every case is built like a user's graph (inputs, constants for weights), gets normally distributed inputs (matrix
+cores run slower on real data than on zeros), runs `-n` times back to back between two events on the executor's stream
+after two untimed runs, and is reported with the bytes its inputs and outputs hold (TB/s) and, for convolutions and
+products, its arithmetic (TFLOP/s), next to the kernels the planner chose.
 The cases are the shapes that decide how the kernels were laid out: few results from much input, normalised axes that
 are not the contiguous one, small batches of small boards, left operands of a few rows.
 """
@@ -117,6 +118,28 @@ def _cases():
     return out
 
 
+def _fill_inputs(ex, rng):
+    """every input := a block of a million random values, repeated (one upload, then copies on the device that double
+    what is filled)"""
+    from ctypes import c_void_p
+
+    from ._lib import check, lib
+
+    for i, (dtype, dims) in enumerate(ex.input_info):
+        count = int(np.prod(dims)) if dims else 1
+        if count == 0:
+            continue
+        kind = np.dtype(dtype.numpy).kind
+        block = rng.standard_normal(min(count, 1 << 20)) if kind == "f" else rng.integers(0, 100, min(count, 1 << 20))
+        block = np.ascontiguousarray(block.astype(dtype.numpy))
+        base, item, filled = ex.input_ptr(i), block.itemsize, block.size
+        check(lib.knhip_memcpy_h2d(ex.device, c_void_p(base), block.ctypes.data, filled * item))
+        while filled < count:
+            step = min(filled, count - filled)
+            check(lib.knhip_memcpy_d2d(ex.device, c_void_p(base + filled * item), c_void_p(base), step * item))
+            filled += step
+
+
 def main(argv=None):
     parser = argparse.ArgumentParser(prog="op_bench", description="time single operations on the HIP executor")
     parser.add_argument("-d", "--device", type=int, default=0)
@@ -146,6 +169,7 @@ def main(argv=None):
         if args.plan_only:
             print(f"{name}\n    " + "\n    ".join(kernels))
             continue
+        _fill_inputs(ex, np.random.default_rng(1))
         for _ in range(2):
             ex.run_async()
         ex.synchronize()
