@@ -2037,3 +2037,22 @@ def tiny_products_one_wave_per_result():
     ex = HipExecutor(0, g, 0, plan_only=True)
     assert all("a wave per result" in ex.step_str(i) for i in range(ex.step_count()) if ex.step_kinds()[i] == "mat_mul")
     return g, 0, inputs, None
+
+
+@case
+def few_long_rows():
+    """a softmax or layernorm over a few rows of 64 Ki elements or more runs as separate steps that use the whole chip
+    (statistic, shifted values, statistic, division) instead of one workgroup per row: along the last axis, and along a
+    middle axis with three columns behind it"""
+    g = Graph()
+    rng = np.random.default_rng(177)
+    a, b, c = g.input([3, 70000]), g.input([2, 100000]), g.input([2, 66000, 3])
+    g.output(g.softmax(a, 1))
+    g.output(g.layernorm(b, 1, 1e-5))
+    g.output(g.softmax(c, 1))
+    g.output(g.layernorm(c, 1, 1e-3))
+    from kyanite_amd import HipExecutor
+    kinds = HipExecutor(0, g, 0, plan_only=True).step_kinds()
+    assert "softmax_op" not in kinds and "layernorm_op" not in kinds, kinds
+    f = lambda *shape: (rng.standard_normal(shape) * 3).astype(np.float32)
+    return g, 0, [f(3, 70000), f(2, 100000), f(2, 66000, 3)], None
