@@ -138,6 +138,9 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     const bool few_tiles = small_blocks < 64;
     const bool can_split = split_enabled && (p.k >= 1024 || (few_tiles && p.k >= 256));
     lp.small_tile = narrow || (big_blocks < threshold && !(can_split && p.k >= 2048 && big_blocks < 256));
+    // f32 with enough tiles either way: the tile that multiplies less padding wins, the small one counted 15 % dearer
+    // per flop (320 columns are 2.5 tiles of 128: q, k and v of the UNet block in one launch 70.8 -> 50 us)
+    if (!f16 && !lp.small_tile && (double) small_blocks * (64 * 64) * 1.15 < (double) big_blocks * (128 * 128)) lp.small_tile = true;
     // f16 with so few tiles that the K axis gets split anyway: 256 x 128 tiles (8 waves), which fetch a quarter
     // fewer bytes from L2 per flop and halve the partial products per split. Measured (us, 128 x 128 against
     // 256 x 128): 512 x 4096 x 4096 43 / 38, 512 x 4096 x 11008 89 / 75; without a split they do not pay:

@@ -16,7 +16,7 @@ from runner import PARITY_RECORDS, check_outputs
 # dtype, m, n, k, (bias, residual, relu), number of products that share the left operand, expected in the plan
 CASES = [
     (DType.F32, 33, 33280, 1536, (True, False, False), 1, "direct 64x64 bk32 head=512 tail_split=3x512"),
-    (DType.F32, 130, 33280, 1024, (True, True, True), 1, "direct 128x128 bk32 head=512 tail_split=2x512"),
+    (DType.F32, 250, 33280, 1024, (True, True, True), 1, "direct 128x128 bk32 head=512 tail_split=2x512"),
     (DType.F32, 256, 2816, 1024, (False, False, False), 3, "x3 grouped [direct 64x64 bk32 head=512 tail_split=2x512"),
     (DType.F32, 512, 5632, 2048, (False, False, False), 3, "x3 grouped [direct 128x128 bk32 head=512 tail_split=4x512"),
     (DType.F16, 33, 33280, 4096, (False, False, False), 1, "direct 64x64 bk64 head=512 tail_split=8x512"),
