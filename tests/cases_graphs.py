@@ -2056,3 +2056,31 @@ def few_long_rows():
     assert "softmax_op" not in kinds and "layernorm_op" not in kinds, kinds
     f = lambda *shape: (rng.standard_normal(shape) * 3).astype(np.float32)
     return g, 0, [f(3, 70000), f(2, 100000), f(2, 66000, 3)], None
+
+
+@case
+def special_values_on_the_split_paths():
+    """infinities and NaN through the kernels that split their work: a softmax along axis 0 (lanes across columns) with a
+    column that is all -inf, one that holds +inf and one with a NaN; reductions in two launches whose input holds NaN
+    (ignored by min and max, kept by sum) and infinities; a softmax over long rows (separate steps) with -inf entries
+    and a row that is all -inf"""
+    g = Graph()
+    rng = np.random.default_rng(179)
+    cols = rng.standard_normal((37, 40)).astype(np.float32)
+    cols[:, 3] = -np.inf
+    cols[5, 7] = np.inf
+    cols[9, 11] = np.nan
+    cols[2:30, 20] = -np.inf
+    g.output(g.softmax(g.input([37, 40]), 0))
+    tall = rng.standard_normal((70001, 96)).astype(np.float32)
+    tall[123, 4] = np.nan
+    tall[60000, 9] = np.inf
+    tall[69999, 50] = -np.inf
+    t = g.input([70001, 96])
+    for op in (ReduceOp.MIN, ReduceOp.MAX, ReduceOp.SUM):
+        g.output(g.reduce(t, [0], op))
+    rows = rng.standard_normal((3, 70000)).astype(np.float32)
+    rows[0, 100:50000] = -np.inf
+    rows[1, :] = -np.inf
+    g.output(g.softmax(g.input([3, 70000]), 1))
+    return g, 0, [cols, tall, rows], None
