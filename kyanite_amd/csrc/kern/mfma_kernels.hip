@@ -387,7 +387,7 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// "Plane" convolution: stride 1, same-size output, image width a power of two. Instead of gathering the im2col
+// "Plane" convolution: 3 x 3 or 5 x 5 filter, stride 1, same-size output, image width a power of two. Instead of gathering the im2col
 // matrix, every K slice (CB input channels x KH x KW taps) stages the raw input rows that the tile's TN = 128 or
 // 64 output positions touch into LDS once, as [channel][group][row][W], and the MFMA B operand is read straight from those
 // planes: position n of the tile sits at a fixed per-lane offset, tap (c, fy, fx) adds a wave-uniform offset. Every
@@ -395,7 +395,9 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
 // tap right of it the next row's (rows above / below the image are stored as zero rows): no masking in the K loop.
 // Global -> LDS traffic for B drops by KH * KW and no per-element index arithmetic is left in the K loop.
 // A tile is either R = TN / W whole output rows of one image (H * W >= TN) or G = TN / (H * W) whole images.
-constexpr int CB = 8;             // input channels per K slice
+constexpr int CB = 8;             // input channels per K slice of a 3 x 3 filter
+// (a 5 x 5 filter takes 4: 100 filter rows per slice in LDS instead of 200)
+constexpr int plane_slice_channels(int kh, int kw) { return kh * kw > 9 ? CB / 2 : CB; }
 constexpr int PLANE_MAX_VEC = 3;  // 128 bit loads per thread and slice for the B planes
 constexpr int PLANE_PAD = 4;      // zero floats in front of every plane row: what a tap left or right of the image reads
 constexpr int PLANE_SLACK = 4;    // zero floats in front of / behind all planes
@@ -431,7 +433,8 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     constexpr int EW = ANYW == 2 ? 4 : 1, ANY_SLOTS = ANYW == 2 ? PLANE_MAX_VEC4 : PLANE_MAX_SCALAR;
     constexpr int TN = 64 * NJ;  // positions per tile
     constexpr int BM = 64 * MI;  // output channels per tile
-    constexpr int KS = CB * KH * KW;      // K slice
+    constexpr int CBK = plane_slice_channels(KH, KW);
+    constexpr int KS = CBK * KH * KW;     // K slice
     constexpr int A_VEC = KS / 4;         // 128 bit loads per filter row and slice
     constexpr int A_ITERS = (BM * A_VEC + THREADS - 1) / THREADS;
     // rows k and k + 1, which the two halves of a wave read together, lie 32 of the 64 LDS banks apart
@@ -606,11 +609,11 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     // the padding is never written again
     for (int i = t; i < PLANE_LDS; i += THREADS) Bs[i] = 0.0f;
     fetch(c_begin);
-    for (int c0 = c_begin; c0 < c_end; c0 += CB) {
+    for (int c0 = c_begin; c0 < c_end; c0 += CBK) {
         __syncthreads();
         stage();
         __syncthreads();
-        if (c0 + CB < c_end) fetch(c0 + CB);
+        if (c0 + CBK < c_end) fetch(c0 + CBK);
         // The operands of step kk + 2 are requested from LDS before the MFMAs of step kk are issued, and the wave
         // raises its priority while it issues MFMAs. Measured on this loop alone (no global loads, two waves per
         // SIMD): operands read right before their MFMAs and masked with selects 126 TFLOP/s, without the selects 140,
@@ -695,10 +698,12 @@ int log2_exact(int x) {
 
 // Fills `g` and returns true when the plane kernel covers this convolution.
 bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
-    if (p.kernel_h != 3 || p.kernel_w != 3 || p.stride_y != 1 || p.stride_x != 1) return false;
-    if (p.pad_y != 1 || p.pad_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
-    // (a channel count that is no multiple of CB runs on the variant that reads the filter float by float)
-    if (p.in_c <= 0 || (uintptr_t) p.input % 16 != 0 || (p.in_c % CB == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
+    const bool three = p.kernel_h == 3 && p.kernel_w == 3 && p.pad_y == 1 && p.pad_x == 1;
+    const bool five = p.kernel_h == 5 && p.kernel_w == 5 && p.pad_y == 2 && p.pad_x == 2;
+    if (!(three || five) || p.stride_y != 1 || p.stride_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
+    const int cb = plane_slice_channels(p.kernel_h, p.kernel_w);
+    // (a channel count that is no multiple of the slice runs on the variant that reads the filter float by float)
+    if (p.in_c <= 0 || (uintptr_t) p.input % 16 != 0 || (p.in_c % cb == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
     const int W = p.in_w, H = p.in_h;
     if (W < 4 || W > tn || log2_exact(W) < 0) return false;
     const long long hw = (long long) H * W;
@@ -717,10 +722,10 @@ bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     g->w4_shift = log2_exact(W / 4);
     g->g_shift = log2_exact(g->groups);
     g->rw_shift = log2_exact(g->rows * W);
-    g->n_vec = CB * g->groups * g->plane_rows * W / 4;
+    g->n_vec = cb * g->groups * g->plane_rows * W / 4;
     g->row_stride = W + PLANE_PAD;
     if (g->g_shift < 0 || g->rw_shift < 0 || g->n_vec > PLANE_MAX_VEC * THREADS) return false;
-    if (CB * g->groups * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
+    if (cb * g->groups * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
     return true;
 }
 
@@ -1090,7 +1095,14 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         plane_geometry(p, best->tn, &geom);
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
         const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
-        const bool ragged = p.in_c % CB != 0;
+        const bool ragged = p.in_c % plane_slice_channels(p.kernel_h, p.kernel_w) != 0;
+        if (p.kernel_h == 5) {
+            if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 2, 2, true>), grid, block, 0, stream, p, geom);
+            else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 2, 2, false>), grid, block, 0, stream, p, geom);
+            else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, true>), grid, block, 0, stream, p, geom);
+            else hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, false>), grid, block, 0, stream, p, geom);
+            return sum_slices();
+        }
         if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true>), grid, block, 0, stream, p, geom);
         else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false>), grid, block, 0, stream, p, geom);
         else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true>), grid, block, 0, stream, p, geom);

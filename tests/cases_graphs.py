@@ -2010,6 +2010,34 @@ def conv_on_images_with_rows_of_whole_vectors():
 
 
 @case
+def conv_five_by_five_on_planes():
+    """5 x 5 filters with padding 2 on power-of-two image widths read their taps from staged planes like 3 x 3 ones, in
+    slices of four input channels: a tile that is part of an image (32 x 32), whole images per tile (8 x 8, 4 x 4), a
+    tile of 128 x 128 (128 output channels on many positions), 6 input channels (the last slice half empty, the filter
+    read float by float), bias + skip connection + relu in the store, and a batch small enough for the input
+    channels to go in slices"""
+    g = Graph()
+    rng = np.random.default_rng(181)
+    inputs = []
+
+    def inp(*shape):
+        inputs.append(rng.standard_normal(shape).astype(np.float32))
+        return g.input(list(shape))
+
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    g.output(g.conv(inp(3, 8, 32, 32), w(24, 8, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(37, 12, 8, 8), w(70, 12, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(9, 4, 4, 4), w(8, 4, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(256, 8, 16, 16), w(128, 8, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(2, 6, 16, 8), w(16, 6, 5, 5), 1, 1, 2, 2))
+    x, skip = inp(4, 8, 16, 16), inp(4, 16, 16, 16)
+    y = g.add(g.conv(x, w(16, 8, 5, 5), 1, 1, 2, 2), g.broadcast(w(1, 16, 1, 1), [4, 16, 16, 16]))
+    g.output(g.relu(g.add(y, skip)))
+    g.output(g.conv(inp(2, 64, 8, 8), w(32, 64, 5, 5), 1, 1, 2, 2))
+    return g, 0, inputs, None
+
+
+@case
 def tiny_products_one_wave_per_result():
     """products of a few thousand multiplications run with one wave per result and lanes along K: K shorter than a wave
     (5) and no multiple of it (200), a transposed right operand, a batch, bias and skip connection and activation in
