@@ -1581,27 +1581,56 @@ KernelSpec make_gather_kernel(const KernelOperand &input, const KernelOperand &i
     std::vector<KernelOperand> all{input, indices, output};
     bool idx64 = !fits_i32(all, total + 4096);
 
+    // Rows that are gathered whole (an embedding lookup, a selection of channels): when the fastest axis of the
+    // result is not the gathered one and contiguous on both sides, a thread moves 16 bytes of it at a time.
+    const size_t last = c.rank() - 1, es = dtype_bytes(input.dtype);
+    const int64_t gathered_stride = input.shape.strides()[axis];
+    size_t vec = 1;
+    if (c.strides[0][last] == 1 && c.strides[1][last] == 1 && c.strides[2][last] == 0) {
+        for (vec = 16 / es; vec > 1; vec /= 2) {
+            bool ok = c.shape[last] % vec == 0 && gathered_stride % (int64_t) vec == 0;
+            ok &= input.offset_bytes % (int64_t) (vec * es) == 0 && output.offset_bytes % (int64_t) (vec * es) == 0;
+            for (size_t a = 0; a < last; a++) ok &= c.strides[0][a] % (int64_t) vec == 0 && c.strides[1][a] % (int64_t) vec == 0;
+            if (ok) break;
+        }
+    }
+    if (vec > 1) {
+        c.shape[last] /= vec;
+        c.strides[0][last] = c.strides[1][last] = (int64_t) vec;
+    }
+    const size_t items = total / vec;
+    // four independent loads per thread once there are workgroups to spare
+    const size_t unroll = items >= ((size_t) 1 << 20) ? 4 : 1;
+    const bool nt = is_streaming(output);
+
     std::ostringstream ss;
     emit_header(ss, idx64, 3);
     ss << "typedef " << storage_type(input.dtype) << " S;\ntypedef " << dtype_c_name(indices.dtype) << " I;\n";
+    if (vec > 1) ss << vec_type_decl("V", input.dtype, vec);
+    else ss << "typedef S V;\n";
     ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_gather(KnPtrs ptrs) {\n";
     ss << "    const S *in = (const S *) ptrs.p[0];\n    const I *indices = (const I *) ptrs.p[1];\n    S *out = (S *) ptrs.p[2];\n";
-    ss << "    const idx_t flat = (idx_t) blockIdx.x * 256 + (idx_t) threadIdx.x;\n";
-    ss << "    if (flat >= (idx_t) " << total << ") return;\n";
-    ss << "    idx_t o_out = 0, o_in = 0, o_idx = 0;\n";
-    emit_decompose(ss, "    ", "flat", c.shape, c.strides, {"o_out", "o_in", "o_idx"});
-    ss << "    const I index = indices[o_idx];\n";
-    ss << "    S value = 0;\n";
+    ss << "    const idx_t first = (idx_t) blockIdx.x * " << 256 * unroll << " + (idx_t) threadIdx.x;\n";
+    ss << "    V value[" << unroll << "];\n    idx_t where[" << unroll << "];\n";
+    ss << "#pragma unroll\n    for (int u = 0; u < " << unroll << "; u++) {\n";
+    ss << "        const idx_t flat = first + u * 256;\n";
+    ss << "        __builtin_memset(&value[u], 0, sizeof(V));\n        where[u] = -1;\n";
+    ss << "        if (flat < (idx_t) " << items << ") {\n";
+    ss << "            idx_t o_out = 0, o_in = 0, o_idx = 0;\n";
+    emit_decompose(ss, "            ", "flat", c.shape, c.strides, {"o_out", "o_in", "o_idx"});
+    ss << "            const I index = indices[o_idx];\n            where[u] = o_out;\n";
     if (dtype_is_signed(indices.dtype))
-        ss << "    if (index >= 0 && (unsigned long long) index < " << ishape[axis] << "ull)";
+        ss << "            if (index >= 0 && (unsigned long long) index < " << ishape[axis] << "ull)";
     else
-        ss << "    if ((unsigned long long) index < " << ishape[axis] << "ull)";
-    ss << " value = in[o_in + (idx_t) index * (idx_t) " << input.shape.strides()[axis] << "];\n";
-    ss << "    out[o_out] = value;\n}\n";
+        ss << "            if ((unsigned long long) index < " << ishape[axis] << "ull)";
+    ss << " value[u] = *(const V *) (in + o_in + (idx_t) index * (idx_t) " << gathered_stride << ");\n";
+    ss << "        }\n    }\n";
+    ss << "#pragma unroll\n    for (int u = 0; u < " << unroll << "; u++)\n";
+    ss << "        if (first + u * 256 < (idx_t) " << items << ") " << store_stmt("V", "out + where[u]", "value[u]", nt) << "\n}\n";
 
     spec.source = ss.str();
-    spec.grid = ceil_div_u32(total, 256);
-    spec.strategy = "rank=" + std::to_string(c.rank());
+    spec.grid = ceil_div_u32(items, 256 * unroll);
+    spec.strategy = "rank=" + std::to_string(c.rank()) + " vec=" + std::to_string(vec) + " unroll=" + std::to_string(unroll);
     return spec;
 }
 

@@ -2,7 +2,7 @@
 
     python -m kyanite_amd.op_bench [-d DEVICE] [-n ITERATIONS] [-p] [FAMILY ...]
 
-Families (default: all): `elementwise`, `reduce`, `rows` (softmax / layernorm), `conv`, `matmul`. `-p` plans and
+Families (default: all): `elementwise`, `gather`, `reduce`, `rows` (softmax / layernorm), `conv`, `matmul`. `-p` plans and
 compiles every case without a device and prints its steps instead of running it.
 
 Every case is built like a user's graph (inputs, constants for weights), gets normally distributed inputs (matrix
@@ -42,6 +42,25 @@ def _cases():
          lambda g: g.output(g.add(g.permute(g.input([64, 256, 64, 64]), [0, 2, 3, 1]), one(g))), 512 * M)
     case("elementwise", "x + column, f32 8192 x 8192",
          lambda g: g.output(g.add(g.input([8192, 8192]), g.broadcast(g.input([8192, 1]), [8192, 8192]))), 512 * M)
+
+    def gather_case(name, shape, axis, count, dtype=f32):
+        elem = np.dtype(dtype.numpy).itemsize
+        result = list(shape)
+        result[axis] = count
+
+        def build(g):
+            where = g.constant([count], rng.integers(0, shape[axis], count).astype(np.int64), DType.I64)
+            g.output(g.gather(g.input(list(shape), dtype), axis, where))
+
+        # (what the result holds, read and written once; repeated indices are read again from the caches)
+        case("gather", f"{name}: {count} along axis {axis} of {dtype.name.lower()} {list(shape)}", build, 2 * elem * int(np.prod(result)))
+
+    gather_case("embedding rows", (32000, 4096), 0, 8192, f16)
+    gather_case("embedding rows", (50000, 768), 0, 16384)
+    gather_case("tokens of a sequence", (64, 4096, 1024), 1, 2048)
+    gather_case("channels of bytes", (256, 64, 64, 64), 1, 64, u8)
+    gather_case("policy moves", (1024, 4672), 1, 1858)
+    gather_case("columns", (4096, 4096), 1, 4096)
 
     def reduce_case(shape, axes, op=ReduceOp.SUM, dtype=f32):
         elem = 2 if dtype == f16 else 4
@@ -150,7 +169,7 @@ def main(argv=None):
 
     from . import Graph, HipExecutor
 
-    known = ["elementwise", "reduce", "rows", "conv", "matmul"]
+    known = ["elementwise", "gather", "reduce", "rows", "conv", "matmul"]
     for family in args.families:
         if family not in known:
             parser.error(f"unknown family {family!r}; choose from {', '.join(known)}")

@@ -189,6 +189,37 @@ def gather_real():
 
 
 @case
+def gather_whole_rows_as_vectors():
+    """a gather whose fastest result axis is not the gathered one moves 16 bytes per thread: an embedding lookup in
+    f16 (enough of it for four loads per thread), channels selected out of [n, c, hw] in f32, rows of 10 floats (8 byte
+    vectors), bytes (16 per vector), rows cut out of a wider tensor (no alignment: element by element) and an index
+    tensor that is an input"""
+    g = Graph()
+    rng = np.random.default_rng(182)
+    inputs = []
+
+    def inp(shape, dtype=DType.F32):
+        if np.dtype(dtype.numpy).kind == "f":
+            inputs.append(rng.standard_normal(shape).astype(dtype.numpy))
+        else:
+            inputs.append(rng.integers(0, 200, shape).astype(dtype.numpy))
+        return g.input(list(shape), dtype)
+
+    def idx(count, below):
+        return g.constant([count], rng.integers(0, below, count).astype(np.int64), DType.I64)
+
+    g.output(g.gather(inp((5000, 2048), DType.F16), 0, idx(5000, 5000)))
+    g.output(g.gather(inp((37, 50, 24)), 1, idx(70, 50)))
+    g.output(g.gather(inp((64, 10)), 0, idx(33, 64)))
+    g.output(g.gather(inp((300, 48), DType.U8), 0, idx(500, 300)))
+    g.output(g.gather(g.slice(inp((40, 25)), 1, 1, 25), 0, idx(90, 40)))
+    where = g.input([11], DType.I32)
+    g.output(g.gather(inp((9, 6, 32)), 0, where))
+    inputs.insert(len(inputs) - 1, rng.integers(0, 9, 11).astype(np.int32))
+    return g, 0, inputs, None
+
+
+@case
 def linear():
     """graphs.rs:262-283, expected values from the reference"""
     g = Graph()
