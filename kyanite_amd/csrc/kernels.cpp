@@ -1598,6 +1598,49 @@ KernelSpec make_gather_kernel(const KernelOperand &input, const KernelOperand &i
         c.shape[last] /= vec;
         c.strides[0][last] = c.strides[1][last] = (int64_t) vec;
     }
+    // A gather along the contiguous axis of the input (the moves of a policy picked out of its planes): lanes that
+    // read `in[row, index[j]]` touch a cache line each. With enough rows, and at least a quarter of a row wanted,
+    // a workgroup stages the row in LDS with whole vectors and gathers from there.
+    const size_t row_len = ishape[axis], rows = total / n_idx;
+    if (c.strides[2][last] != 0 && c.shape[last] == n_idx && gathered_stride == 1 && row_len * es <= 65536 && rows >= 128 &&
+        n_idx * 4 >= row_len && n_idx >= 64) {
+        size_t rvec = 16 / es;
+        for (; rvec > 1; rvec /= 2) {
+            bool ok = row_len % rvec == 0 && input.offset_bytes % (int64_t) (rvec * es) == 0;
+            for (size_t a = 0; a < last; a++) ok &= c.strides[1][a] % (int64_t) rvec == 0;
+            if (ok) break;
+        }
+        std::vector<size_t> outer(c.shape.begin(), c.shape.begin() + (ptrdiff_t) last);
+        std::vector<std::vector<int64_t>> outer_strides{
+            std::vector<int64_t>(c.strides[0].begin(), c.strides[0].begin() + (ptrdiff_t) last),
+            std::vector<int64_t>(c.strides[1].begin(), c.strides[1].begin() + (ptrdiff_t) last)};
+        std::ostringstream ss;
+        emit_header(ss, idx64, 3);
+        ss << "typedef " << storage_type(input.dtype) << " S;\ntypedef " << dtype_c_name(indices.dtype) << " I;\n";
+        if (rvec > 1) ss << vec_type_decl("V", input.dtype, rvec);
+        else ss << "typedef S V;\n";
+        ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_gather(KnPtrs ptrs) {\n";
+        ss << "    const S *in = (const S *) ptrs.p[0];\n    const I *indices = (const I *) ptrs.p[1];\n    S *out = (S *) ptrs.p[2];\n";
+        ss << "    __shared__ __attribute__((aligned(16))) S row[" << row_len << "];\n";
+        ss << "    const idx_t r = (idx_t) blockIdx.x;\n    idx_t o_out = 0, o_in = 0;\n";
+        emit_decompose(ss, "    ", "r", outer, outer_strides, {"o_out", "o_in"});
+        ss << "    for (int i = threadIdx.x * " << rvec << "; i < " << row_len << "; i += " << 256 * rvec << ")\n";
+        ss << "        *(V *) (row + i) = *(const V *) (in + o_in + i);\n";
+        ss << "    __syncthreads();\n";
+        ss << "    for (int j = threadIdx.x; j < " << n_idx << "; j += 256) {\n";
+        ss << "        const I index = indices[(idx_t) j * (idx_t) " << c.strides[2][last] << "];\n";
+        ss << "        S value = 0;\n";
+        if (dtype_is_signed(indices.dtype))
+            ss << "        if (index >= 0 && (unsigned long long) index < " << row_len << "ull)";
+        else
+            ss << "        if ((unsigned long long) index < " << row_len << "ull)";
+        ss << " value = row[index];\n";
+        ss << "        out[o_out + (idx_t) j * (idx_t) " << c.strides[0][last] << "] = value;\n    }\n}\n";
+        spec.source = ss.str();
+        spec.grid = ceil_div_u32(rows, 1);
+        spec.strategy = "rank=" + std::to_string(c.rank()) + " rows staged in LDS vec=" + std::to_string(rvec);
+        return spec;
+    }
     const size_t items = total / vec;
     // four independent loads per thread once there are workgroups to spare
     const size_t unroll = items >= ((size_t) 1 << 20) ? 4 : 1;

@@ -220,6 +220,37 @@ def gather_whole_rows_as_vectors():
 
 
 @case
+def gather_along_the_contiguous_axis_through_lds():
+    """a gather along the axis the input is contiguous in, with many rows and a good share of every row wanted: a
+    workgroup stages its row in LDS and picks from there. Rows of whole 16 byte vectors, rows of halves that only
+    allow 4 byte vectors, bytes, a row cut out of a wider tensor (element by element), indices that are an input,
+    and a result that a concatenation takes on"""
+    g = Graph()
+    rng = np.random.default_rng(183)
+    inputs = []
+
+    def inp(shape, dtype=DType.F32):
+        if np.dtype(dtype.numpy).kind == "f":
+            inputs.append(rng.standard_normal(shape).astype(dtype.numpy))
+        else:
+            inputs.append(rng.integers(0, 200, shape).astype(dtype.numpy))
+        return g.input(list(shape), dtype)
+
+    def idx(count, below):
+        return g.constant([count], rng.integers(0, below, count).astype(np.int64), DType.I64)
+
+    g.output(g.gather(inp((200, 300)), 1, idx(150, 300)))
+    g.output(g.gather(inp((130, 7, 90), DType.F16), 2, idx(64, 90)))
+    g.output(g.gather(inp((256, 100), DType.U8), 1, idx(100, 100)))
+    g.output(g.gather(g.slice(inp((140, 131)), 1, 1, 129), 1, idx(200, 128)))
+    where = g.input([77], DType.I32)
+    inputs.append(rng.integers(0, 96, 77).astype(np.int32))
+    g.output(g.gather(inp((128, 96)), 1, where))
+    g.output(g.concat([g.gather(inp((300, 64)), 1, idx(64, 64)), inp((300, 8))], 1))
+    return g, 0, inputs, None
+
+
+@case
 def linear():
     """graphs.rs:262-283, expected values from the reference"""
     g = Graph()
