@@ -1110,13 +1110,27 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         const size_t inner = sc.shape.back();
         size_t n_pre = 0;
         for (size_t k = 1; k < ops.size(); k++) n_pre += in_pre[k] ? 1 : 0;
-        size_t TX = 64, TY = 4, items = (size + 3) / 4;
+        size_t TX = 64, TY = 4, items = (size + 3) / 4, threads = 256;
         bool held = false;
         for (size_t tx : {64, 32, 16}) {  // fewer columns per workgroup: more threads, so more registers, per column
             const size_t ty = 256 / tx, per_thread = (size + ty - 1) / ty;
             if (per_thread * std::max<size_t>(n_pre, 1) <= 32) {
                 TX = tx, TY = ty, items = per_thread, held = true;
                 break;
+            }
+        }
+        // A run of less than a cache line per row of lanes (16 or 32 halves, 16 floats), or a column too long for 256
+        // threads: a workgroup of 1024 threads holds four times as much, a whole line per row of lanes. (f16
+        // [64, 512, 32, 32] along axis 1: 61.0 -> 27.1 us; f32 [8, 1000, 4096] along axis 1, read three times before:
+        // 94.3 -> 60.7 us; runs of two lines per row of lanes on 1024 threads where 256 threads manage one: 113 -> 123 us.)
+        const size_t elem_bytes = dtype_bytes(ops[1].dtype);
+        if ((!held || TX * elem_bytes < 128) && sc.shape.back() >= 64) {
+            for (size_t tx : {64, 32}) {
+                const size_t ty = 1024 / tx, per_thread = (size + ty - 1) / ty;
+                if (tx * elem_bytes >= 128 && per_thread * std::max<size_t>(n_pre, 1) <= 32) {
+                    TX = tx, TY = ty, items = per_thread, held = true, threads = 1024;
+                    break;
+                }
             }
         }
         std::vector<size_t> outer_shape(sc.shape.begin(), sc.shape.end() - 1);
@@ -1140,7 +1154,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         ss << "template<typename F> KN_DEV float kn_column_fold(float v, F f, float (*lds)[TX], int tx, int ty) {\n";
         ss << "    lds[ty][tx] = v;\n    __syncthreads();\n    v = lds[0][tx];\n";
         ss << "#pragma unroll\n    for (int s = 1; s < TY; s++) v = f(v, lds[s][tx]);\n    return v;\n}\n";
-        ss << "extern \"C\" __global__ __launch_bounds__(256) void " << spec.name << "(KnPtrs ptrs) {\n";
+        ss << "extern \"C\" __global__ __launch_bounds__(" << threads << ") void " << spec.name << "(KnPtrs ptrs) {\n";
         for (size_t k = 0; k < ops.size(); k++) ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
         ss << "    __shared__ float lds_m[TY][TX], lds_s[TY][TX];\n";
         ss << "    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;\n";
@@ -1234,11 +1248,12 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             }
         }
         spec.source = ss.str();
-        spec.block = 256;
+        spec.block = (uint32_t) threads;
         spec.grid = ceil_div_u32(outer_size * column_blocks, 1);
         std::ostringstream note;
         note << (softmax ? "softmax" : (rowred ? "row statistic + elementwise" : "layernorm")) << " columns TX=" << TX << " TY=" << TY
              << " items=" << items << (held ? " cached" : " streamed");
+        if (threads != 256) note << " threads=" << threads;
         spec.strategy = note.str();
         return spec;
     }
