@@ -1973,6 +1973,27 @@ def normalised_axis_is_not_the_contiguous_one():
 
 
 @case
+def columns_on_workgroups_of_1024_threads():
+    """the same kernels where 256 threads would see less than a cache line per row of lanes, or could not hold the
+    column in registers: 1000 positions over 96 columns (32 threads per column), layernorm over 512 channels of f16
+    with an affine behind, 70 columns (the second block of 64 mostly empty), a sum in front (two tensors to hold, so
+    read again per pass on 256 threads), and a column mean with its elementwise consumer"""
+    g = Graph()
+    rng = np.random.default_rng(184)
+    tall = g.input([1000, 96])
+    g.output(g.softmax(tall, 0))
+    g.output(g.layernorm(g.add(tall, g.input([1000, 96])), 0, 1e-5))
+    g.output(g.sub(tall, g.broadcast(g.view(g.reduce(tall, [0], ReduceOp.MEAN), [1, 96]), [1000, 96])))
+    maps = g.input([3, 512, 70], DType.F16)
+    gamma, beta = g.input([1, 512, 1], DType.F16), g.input([1, 512, 1], DType.F16)
+    normed = g.layernorm(maps, 1, 1e-5)
+    g.output(g.add(g.mul(normed, g.broadcast(gamma, [3, 512, 70])), g.broadcast(beta, [3, 512, 70])))
+    f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    h = lambda *shape: rng.standard_normal(shape).astype(np.float16)
+    return g, 0, [f(1000, 96), f(1000, 96), h(3, 512, 70), h(1, 512, 1), h(1, 512, 1)], None
+
+
+@case
 def conv_with_input_channels_in_slices():
     """few output tiles, many input channels: slices of the channels are folded side by side and a second kernel sums the
     partial results and applies bias, residual and activation. A tower block of a small batch of boards (the kernel
