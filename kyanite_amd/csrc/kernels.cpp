@@ -530,10 +530,28 @@ std::optional<KernelSpec> make_transposed_tile_kernel(const std::vector<KernelOp
         ss << "    S" << k << " *p" << k << " = (S" << k << " *) ptrs.p[" << k << "];\n";
         if (transposed[k]) ss << "    __shared__ S" << k << " tile" << k << "[" << TILE << "][" << pitch_of(operands[k].dtype) << "];\n";
     }
-    // which tile: the output axis fastest, then the operands' axis, then everything else
+    // Which tile: the output axis fastest, then the operands' axis, then everything else. Consecutive workgroups then
+    // write neighbouring pieces of the same 64 rows, and read tiles that lie 64 rows of the transposed operand
+    // apart: when that distance is (nearly) a multiple of 1 MB, as with rows of 16 KB or more whose length is a
+    // power of two, all workgroups in flight read through the same few memory channels. Those shapes walk the tiles
+    // along diagonals instead, which moves both sides on by a tile's width per workgroup (f32 8192 x 8192: 135 ->
+    // 103 us, f16 16384 x 16384: 298 -> 227 us); other shapes lose the order of their writes that way (f32
+    // 32768 x 2048: 119 -> 153 us) and keep the straight order.
+    bool diagonal = false;
+    for (size_t k = n_out; k < n_ops && !diagonal; k++) {
+        if (!transposed[k]) continue;
+        const uint64_t apart = (uint64_t) std::llabs(c.strides[k][last]) * dtype_bytes(operands[k].dtype) * TILE;
+        const uint64_t off = apart % (1u << 20);
+        diagonal = tiles_a > 1 && tiles_l > 1 && (off <= (1u << 15) || off >= (1u << 20) - (1u << 15));
+        break;
+    }
     ss << "    idx_t blk = (idx_t) blockIdx.x;\n";
-    ss << "    const idx_t l0 = (blk % (idx_t) " << tiles_l << ") * " << TILE << "; blk /= (idx_t) " << tiles_l << ";\n";
-    ss << "    const idx_t a0 = (blk % (idx_t) " << tiles_a << ") * " << TILE << "; blk /= (idx_t) " << tiles_a << ";\n";
+    ss << "    const idx_t tl = blk % (idx_t) " << tiles_l << "; blk /= (idx_t) " << tiles_l << ";\n";
+    if (!diagonal)
+        ss << "    const idx_t ta = blk % (idx_t) " << tiles_a << "; blk /= (idx_t) " << tiles_a << ";\n";
+    else
+        ss << "    const idx_t ta = (blk % (idx_t) " << tiles_a << " + tl) % (idx_t) " << tiles_a << "; blk /= (idx_t) " << tiles_a << ";\n";
+    ss << "    const idx_t l0 = tl * " << TILE << ", a0 = ta * " << TILE << ";\n";
     for (size_t k = 0; k < n_ops; k++) ss << "    idx_t off" << k << " = 0;\n";
     {
         std::vector<std::string> offs;
@@ -586,7 +604,7 @@ std::optional<KernelSpec> make_transposed_tile_kernel(const std::vector<KernelOp
     spec.source = ss.str();
     spec.grid = (uint32_t) blocks;
     std::ostringstream note;
-    note << "rank=" << rank << " transposed tiles " << TILE << "x" << TILE << " idx=" << (idx64 ? 64 : 32);
+    note << "rank=" << rank << " transposed tiles " << TILE << "x" << TILE << (diagonal ? " along diagonals" : "") << " idx=" << (idx64 ? 64 : 32);
     if (n_out > 1) note << " outputs=" << n_out;
     spec.strategy = note.str();
     return spec;
