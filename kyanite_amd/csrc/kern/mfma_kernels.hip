@@ -387,7 +387,7 @@ __global__ __launch_bounds__(THREADS) void conv_f32_kernel(ConvParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// "Plane" convolution: 3 x 3 or 5 x 5 filter, stride 1, same-size output, image width a power of two. Instead of gathering the im2col
+// "Plane" convolution: 3 x 3 or 5 x 5 filter, stride 1, same-size output (image width a power of two in the variant described first). Instead of gathering the im2col
 // matrix, every K slice (CB input channels x KH x KW taps) stages the raw input rows that the tile's TN = 128 or
 // 64 output positions touch into LDS once, as [channel][group][row][W], and the MFMA B operand is read straight from those
 // planes: position n of the tile sits at a fixed per-lane offset, tap (c, fy, fx) adds a wave-uniform offset. Every
@@ -412,10 +412,10 @@ struct PlaneGeom {
     int n_vec;           // CB * G * plane_rows * W / 4
     int row_stride;      // W + PLANE_PAD
     // Any image size (template flag ANYW): a tile is TN consecutive positions of the (image, y, x) order, wherever
-    // they start. Every image counts H + 2 padded rows (an empty row above and below), so that the row above / below
-    // an output row is the padded row before / after its own, across image boundaries too; the tile stages the
-    // padded rows from the one above its first output row to the one below its last, `plane_rows` at most, float by
-    // float (`n_scalar` = CB * plane_rows * W of them per slice).
+    // they start. Every image counts H + 2 (5 x 5: H + 4) padded rows (empty rows above and below), so that the rows
+    // above / below an output row are the padded rows before / after its own, across image boundaries too; the tile
+    // stages the padded rows from the first one its first output row reads to the last one its last reads,
+    // `plane_rows` at most, float by float (`n_scalar` = slice channels * plane_rows * W of them per slice).
     int n_scalar;
     int by4;  // the image width is a multiple of 4 and the input 16 byte aligned: staged four floats at a time
 };
@@ -463,9 +463,10 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, c32 = lane & 31;
     const int RS = g.row_stride;
     const int plane = g.plane_rows * RS, gplane = ANYW ? plane : plane << g.g_shift;  // LDS floats per (c, g) and per c
-    // ANYW: the padded row above the tile's first output row (output row rho of the (image, y) order is padded row
-    // rho + 2 * (rho / H) + 1)
-    const int rho0 = n0 / W, pi_base = rho0 + 2 * (rho0 / H);
+    // ANYW: the first padded row the tile's first output row reads (with PY = KH / 2 empty rows above and below every
+    // image, output row rho of the (image, y) order is padded row rho + 2 * PY * (rho / H) + PY)
+    constexpr int PY = KH / 2;
+    const int rho0 = n0 / W, pi_base = rho0 + 2 * PY * (rho0 / H);
 
     // ---- B planes: what this thread moves per slice (the same places every slice, only the channel base moves)
     constexpr int B_SLOTS = ANYW ? ANY_SLOTS : PLANE_MAX_VEC;
@@ -480,7 +481,7 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             const int e = t + THREADS * i;
             const int x = (e % wq) * EW, t1 = e / wq;
             const int c = t1 / g.plane_rows, prow = t1 - c * g.plane_rows;
-            const int pi = pi_base + prow, img = pi / (H + 2), iy = pi - img * (H + 2) - 1;
+            const int pi = pi_base + prow, img = pi / (H + 2 * PY), iy = pi - img * (H + 2 * PY) - PY;
             const bool inside = e * EW < g.n_scalar && iy >= 0 && iy < H && img < p.batch;
             // (the empty rows above and below an image are never written: they keep the zeros of the first fill)
             b_dst[i] = inside ? PLANE_SLACK + t1 * RS + PLANE_PAD + x : -1;
@@ -519,7 +520,7 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         if (ANYW) {
             // (positions past the end take the place of the last one; their results are never stored)
             const int pos = (int) min((long long) n0 + n, N - 1), rho = pos / W, col = pos - rho * W;
-            lane_base[j] = PLANE_SLACK + (rho + 2 * (rho / H) - pi_base) * RS + PLANE_PAD + col - p.pad_x;
+            lane_base[j] = PLANE_SLACK + (rho + 2 * PY * (rho / H) - pi_base) * RS + PLANE_PAD + col - p.pad_x;
             continue;
         }
         const int gl = n >> g.rw_shift, rem = n & ((1 << g.rw_shift) - 1), col = rem & (W - 1), r = rem >> (g.w4_shift + 2);
@@ -702,6 +703,9 @@ bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     const bool five = p.kernel_h == 5 && p.kernel_w == 5 && p.pad_y == 2 && p.pad_x == 2;
     if (!(three || five) || p.stride_y != 1 || p.stride_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
     const int cb = plane_slice_channels(p.kernel_h, p.kernel_w);
+    // (5 x 5 with channels that do not fill their slices of four gathers faster: the 22 planes of a Go network's stem on
+    // 19 x 19 -> 192 channels at batch 256 383 us here, 319 us on the patch kernel)
+    if (five && p.in_c % cb != 0) return false;
     // (a channel count that is no multiple of the slice runs on the variant that reads the filter float by float)
     if (p.in_c <= 0 || (uintptr_t) p.input % 16 != 0 || (p.in_c % cb == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
     const int W = p.in_w, H = p.in_h;
@@ -729,12 +733,15 @@ bool plane_geometry(const ConvParams &p, int tn, PlaneGeom *g) {
     return true;
 }
 
-// The same for the variant that takes any image size (3 x 3, stride 1, same-size output): tiles of `tn` consecutive
-// positions.
+// The same for the variant that takes any image size (3 x 3 or 5 x 5, stride 1, same-size output): tiles of `tn`
+// consecutive positions.
 bool plane_geometry_any(const ConvParams &p, int tn, PlaneGeom *g) {
-    if (p.kernel_h != 3 || p.kernel_w != 3 || p.stride_y != 1 || p.stride_x != 1) return false;
-    if (p.pad_y != 1 || p.pad_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
-    if (p.in_c <= 0 || (p.in_c % CB == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
+    const bool three = p.kernel_h == 3 && p.kernel_w == 3 && p.pad_y == 1 && p.pad_x == 1;
+    const bool five = p.kernel_h == 5 && p.kernel_w == 5 && p.pad_y == 2 && p.pad_x == 2;
+    if (!(three || five) || p.stride_y != 1 || p.stride_x != 1 || p.out_h != p.in_h || p.out_w != p.in_w) return false;
+    const int cb = plane_slice_channels(p.kernel_h, p.kernel_w);
+    if (five && p.in_c % cb != 0) return false;
+    if (p.in_c <= 0 || (p.in_c % cb == 0 && (uintptr_t) p.filter % 16 != 0)) return false;
     const int W = p.in_w, H = p.in_h;
     if (W < 2 || H < 1 || (long long) p.batch * p.in_c * H * W >= (1ll << 31)) return false;
     // output rows that `tn` consecutive positions can touch, image boundaries between them, and the padded rows
@@ -742,12 +749,12 @@ bool plane_geometry_any(const ConvParams &p, int tn, PlaneGeom *g) {
     const int touched = (tn - 2) / W + 2, crossings = (touched - 2) / H + 1;
     *g = PlaneGeom{};
     g->groups = 1;
-    g->plane_rows = touched + 2 * crossings + 2;
+    g->plane_rows = touched + 2 * p.pad_y * crossings + 2 * p.pad_y;
     g->row_stride = W + PLANE_PAD;
-    g->n_scalar = CB * g->plane_rows * W;
+    g->n_scalar = cb * g->plane_rows * W;
     g->by4 = W % 4 == 0 && (uintptr_t) p.input % 16 == 0;
     if (g->n_scalar > (g->by4 ? 4 * PLANE_MAX_VEC4 : PLANE_MAX_SCALAR) * THREADS) return false;
-    if (CB * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
+    if (cb * g->plane_rows * g->row_stride + 2 * PLANE_SLACK > PLANE_LDS) return false;
     return true;
 }
 
@@ -1069,6 +1076,9 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
     bool any_w = false;
     for (const Variant &v : variants) {
         if (split && v.id != 11) continue;  // (few tiles: the small one)
+        // (5 x 5: 100 filter rows per slice for 128 channels leave LDS for one workgroup per compute unit; 64 x 64 tiles
+        // run 101 TFLOP/s where 128 x 128 run 94, on 128 -> 128 channels at 32 x 32, 16 x 16 and 8 x 8 alike)
+        if (p.kernel_h == 5 && v.id != 11) continue;
         const bool classic = plane_geometry(p, v.tn, &geom);
         if (!classic && !(any_enabled && plane_geometry_any(p, v.tn, &geom))) continue;
         const long long tiles = ((positions + v.tn - 1) / v.tn) * ((p.out_c + v.bm - 1) / v.bm);
@@ -1079,8 +1089,13 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         plane_geometry_any(p, best->tn, &geom);
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
         const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
-        const bool ragged = p.in_c % CB != 0;
+        const bool ragged = p.in_c % plane_slice_channels(p.kernel_h, p.kernel_w) != 0;
         const bool by4 = geom.by4 != 0;
+        if (p.kernel_h == 5) {
+            if (by4) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, false, 2>), grid, block, 0, stream, p, geom);
+            else hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, false, 1>), grid, block, 0, stream, p, geom);
+            return sum_slices();
+        }
         if (best->id == 22 && ragged && by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true, 2>), grid, block, 0, stream, p, geom);
         else if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true, 1>), grid, block, 0, stream, p, geom);
         else if (best->id == 22 && by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false, 2>), grid, block, 0, stream, p, geom);
@@ -1097,10 +1112,7 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
         const bool ragged = p.in_c % plane_slice_channels(p.kernel_h, p.kernel_w) != 0;
         if (p.kernel_h == 5) {
-            if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 2, 2, true>), grid, block, 0, stream, p, geom);
-            else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 2, 2, false>), grid, block, 0, stream, p, geom);
-            else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, true>), grid, block, 0, stream, p, geom);
-            else hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, false>), grid, block, 0, stream, p, geom);
+            hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, false>), grid, block, 0, stream, p, geom);
             return sum_slices();
         }
         if (best->id == 22 && ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, true>), grid, block, 0, stream, p, geom);

@@ -2095,10 +2095,10 @@ def conv_on_images_with_rows_of_whole_vectors():
 @case
 def conv_five_by_five_on_planes():
     """5 x 5 filters with padding 2 on power-of-two image widths read their taps from staged planes like 3 x 3 ones, in
-    slices of four input channels: a tile that is part of an image (32 x 32), whole images per tile (8 x 8, 4 x 4), a
-    tile of 128 x 128 (128 output channels on many positions), 6 input channels (the last slice half empty, the filter
-    read float by float), bias + skip connection + relu in the store, and a batch small enough for the input
-    channels to go in slices"""
+    slices of four input channels: a tile that is part of an image (32 x 32), whole images per tile (8 x 8, 4 x 4),
+    128 output channels on many positions (two tiles of 64), 6 input channels (no whole slices: the kernel that
+    gathers patches), bias + skip connection + relu in the store, and a batch small enough for the input channels
+    to go in slices"""
     g = Graph()
     rng = np.random.default_rng(181)
     inputs = []
@@ -2117,6 +2117,31 @@ def conv_five_by_five_on_planes():
     y = g.add(g.conv(x, w(16, 8, 5, 5), 1, 1, 2, 2), g.broadcast(w(1, 16, 1, 1), [4, 16, 16, 16]))
     g.output(g.relu(g.add(y, skip)))
     g.output(g.conv(inp(2, 64, 8, 8), w(32, 64, 5, 5), 1, 1, 2, 2))
+    return g, 0, inputs, None
+
+
+@case
+def conv_five_by_five_on_boards_of_any_size():
+    """the same on image sizes that are no power of two: the 22 input planes of a Go network on 19 x 19 (no whole
+    slices of four channels: the kernel that gathers patches), 20 planes on the same boards, 9 x 9 boards, 28 x 28 images (rows of whole vectors), a 5 x 3 and a 2 x 2
+    image (smaller than the filter), bias and relu in the store, and few boards with many channels (in slices)"""
+    g = Graph()
+    rng = np.random.default_rng(185)
+    inputs = []
+
+    def inp(*shape):
+        inputs.append(rng.standard_normal(shape).astype(np.float32))
+        return g.input(list(shape))
+
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    stem = g.add(g.conv(inp(3, 22, 19, 19), w(96, 22, 5, 5), 1, 1, 2, 2), g.broadcast(w(1, 96, 1, 1), [3, 96, 19, 19]))
+    g.output(g.relu(stem))
+    g.output(g.conv(inp(2, 20, 19, 19), w(40, 20, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(11, 8, 9, 9), w(24, 8, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(2, 12, 28, 28), w(70, 12, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(7, 4, 5, 3), w(8, 4, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(40, 5, 2, 2), w(8, 5, 5, 5), 1, 1, 2, 2))
+    g.output(g.conv(inp(1, 64, 9, 9), w(32, 64, 5, 5), 1, 1, 2, 2))
     return g, 0, inputs, None
 
 
