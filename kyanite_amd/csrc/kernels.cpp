@@ -1636,7 +1636,7 @@ KernelSpec make_gather_kernel(const KernelOperand &input, const KernelOperand &i
     // a workgroup stages the row in LDS with whole vectors and gathers from there.
     const size_t row_len = ishape[axis], rows = total / n_idx;
     if (c.strides[2][last] != 0 && c.shape[last] == n_idx && gathered_stride == 1 && row_len * es <= 65536 && rows >= 128 &&
-        n_idx * 4 >= row_len && n_idx >= 64) {
+        n_idx * 4 >= row_len && n_idx >= 64 && n_idx < ((size_t) 1 << 30)) {
         size_t rvec = 16 / es;
         for (; rvec > 1; rvec /= 2) {
             bool ok = row_len % rvec == 0 && input.offset_bytes % (int64_t) (rvec * es) == 0;
