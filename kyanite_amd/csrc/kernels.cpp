@@ -1060,8 +1060,11 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         if (ok) break;
     }
     size_t nv = size / vec;
-    // G lanes share a row; the row stays in registers when every lane holds at most MAX_ITEMS vectors
-    const size_t MAX_ITEMS = 16;
+    // G lanes share a row; the row stays in registers when every lane holds at most MAX_ITEMS vectors: 64 elements,
+    // which the kernel keeps as floats. (With 16 vectors of 8 halves a lane of 1024 would hold 128 and spill: f16
+    // [1046, 128256] 396 us held against 240 us read again per pass; single elements held up to 64 instead of 16: f32
+    // rows of 50257 486 us read again per pass.)
+    const size_t MAX_ITEMS = std::max<size_t>(1, 64 / vec);
     size_t G = 1024;
     for (size_t g : {1, 4, 16, 64, 256, 1024}) {
         size_t per_lane = (nv + g - 1) / g;
