@@ -2195,6 +2195,31 @@ def few_long_rows():
 
 
 @case
+def rows_too_long_for_registers():
+    """rows of more than 64 elements per lane of 1024 are read again per pass, by a softmax twice (maximum and sum of
+    exponentials in one pass): an odd length (element by element), whole vectors, f16; rows that start with -inf (the
+    running maximum is still -inf there), hold +inf, a NaN, or nothing but -inf; and a layernorm, which takes three
+    passes"""
+    g = Graph()
+    rng = np.random.default_rng(186)
+    odd = rng.standard_normal((70, 70001)).astype(np.float32) * 3
+    odd[0, :5000] = -np.inf
+    odd[1, 1::2] = -np.inf
+    odd[2, 40000] = np.inf
+    odd[3, 69000] = np.nan
+    odd[4, :] = -np.inf
+    odd[5, :60000] = -np.inf
+    odd[5, 60000] = np.nan
+    g.output(g.softmax(g.input([70, 70001]), 1))
+    whole = rng.standard_normal((66, 132000)).astype(np.float32)
+    g.output(g.softmax(g.input([66, 132000]), 1))
+    halves = (rng.standard_normal((65, 90000)) * 2).astype(np.float16)
+    g.output(g.softmax(g.input([65, 90000], DType.F16), 1))
+    g.output(g.layernorm(g.input([66, 132000]), 1, 1e-5))
+    return g, 0, [odd, whole, halves, whole.copy()], None
+
+
+@case
 def special_values_on_the_split_paths():
     """infinities and NaN through the kernels that split their work: a softmax along axis 0 (lanes across columns) with a
     column that is all -inf, one that holds +inf and one with a NaN; reductions in two launches whose input holds NaN
