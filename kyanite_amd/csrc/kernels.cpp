@@ -34,7 +34,8 @@ KN_DEV float kn_r16(float x) { return (float) (_Float16) x; }
 // Abramowitz-Stegun erf, evaluated in f64 exactly like the host reference does
 KN_DEV double kn_erf(double x) {
     double s = (x != x) ? x : (__builtin_signbit(x) ? -1.0 : 1.0);
-    double a = __builtin_fabs(x);
+    // (from 10 on the result is 1 to the last bit of an f64; the sixteenth power stays finite for the reciprocal below)
+    double a = __builtin_fmin(__builtin_fabs(x), 10.0);
     double d = 1.0, p = a;
     d += 0.0705230784 * p; p *= a;
     d += 0.0422820123 * p; p *= a;
@@ -43,7 +44,12 @@ KN_DEV double kn_erf(double x) {
     d += 0.0002765672 * p; p *= a;
     d += 0.0000430638 * p;
     double d2 = d * d, d4 = d2 * d2, d8 = d4 * d4, d16 = d8 * d8;
-    return s * (1.0 - 1.0 / d16);
+    // 1 / d16 from the hardware's approximation and two Newton steps (d16 is finite and at least 1) instead of a
+    // division with its scaling and fix-up, which was most of the function: 64M halves 99 -> 89 us, GELU over 64M floats 100 -> 89 us
+    double r = __builtin_amdgcn_rcp(d16);
+    r = __builtin_fma(__builtin_fma(-d16, r, 1.0), r, r);
+    r = __builtin_fma(__builtin_fma(-d16, r, 1.0), r, r);
+    return s * (1.0 - r);
 }
 
 // x * tanh(log(1 + e^x)) with tanh(log(u)) = (u^2 - 1) / (u^2 + 1) written out: n = e^x (e^x + 2), n / (n + 2). One
