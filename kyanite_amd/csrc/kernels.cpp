@@ -240,6 +240,9 @@ std::string unary_expr(const ScalarNode &n, DType in, const std::string &x) {
         case UnaryOp::Log: return fn(d, "log") + "(" + x + ")";
         case UnaryOp::Sqrt: return fn(d, "sqrt") + "(" + x + ")";
         case UnaryOp::Sigmoid:
+            // (halves: the hardware's 2^x and reciprocal, a few 1e-6 off before the result is rounded to 11 bits;
+            // 64M halves 54.9 -> 43.8 us)
+            if (in == DType::F16) return "__frcp_rn(1.0f + __expf(-(" + x + ")))";
             return d ? "(1.0 / (1.0 + exp(-(" + x + "))))" : "(1.0f / (1.0f + expf(-(" + x + "))))";
         case UnaryOp::Tanh: return fn(d, "tanh") + "(" + x + ")";
         case UnaryOp::Erf: return d ? "kn_erf(" + x + ")" : "((float) kn_erf((double) (" + x + ")))";
