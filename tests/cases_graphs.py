@@ -251,6 +251,26 @@ def gather_along_the_contiguous_axis_through_lds():
 
 
 @case
+def square_written_as_a_power():
+    """`x ** 2` and `x ** 3` with a constant exponent are emitted as products and `x ** 0.5` as a square root:
+    negative values, zeros of both signs, infinities, NaN, values whose square overflows or underflows, f16; other
+    constant exponents stay with the library"""
+    g = Graph()
+    rng = np.random.default_rng(187)
+    special = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 3e19, -3e19, 1e-23, -1e-30, 2.5, -7.25], np.float32)
+    values = np.concatenate([special, rng.standard_normal(3000).astype(np.float32) * 100])
+    x = g.input([len(values)])
+    g.output(g.pow(x, g.scalar(2.0, DType.F32)))
+    g.output(g.pow(x, g.scalar(0.5, DType.F32)))
+    g.output(g.pow(x, g.scalar(3.0, DType.F32)))
+    g.output(g.pow(x, g.scalar(1.5, DType.F32)))
+    h = g.input([len(values)], DType.F16)
+    g.output(g.add(g.pow(h, g.scalar(2.0, DType.F16)), g.scalar(1.0, DType.F16)))
+    g.output(g.pow(h, g.scalar(0.5, DType.F16)))
+    return g, 0, [values, values.astype(np.float16)], None
+
+
+@case
 def linear():
     """graphs.rs:262-283, expected values from the reference"""
     g = Graph()
