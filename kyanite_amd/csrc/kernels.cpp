@@ -1295,6 +1295,21 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "    const idx_t len = col_ok ? " << L << " : (idx_t) 0;\n";
             const std::string loop = "    for (idx_t i = (idx_t) ty; i < len; i += (idx_t) TY) {\n";
             const std::string loaded = pre_of([&](size_t k) { return at(k, "i"); });
+            if (softmax) {
+                // two passes, as for rows too long for registers: the sum of exponentials is kept relative to the
+                // running maximum, and the threads of a column scale theirs to the column's maximum before adding
+                ss << "#pragma unroll 8\n" << loop << "        const float v = " << loaded << ";\n";
+                ss << "        if (v > m) { s *= kn_exp(m - v); m = v; }\n";
+                ss << "        s += v == -KN_INF ? 0.0f : kn_exp(v - m);\n    }\n";
+                ss << "    const float m_mine = m;\n";
+                ss << "    m = kn_column_fold(m, " << fold_fn << ", lds_m, tx, ty);\n";
+                ss << "    s = m_mine == -KN_INF ? s : s * kn_exp(m_mine - m);\n";
+                ss << "    s = kn_column_fold(s, kn_add, lds_s, tx, ty);\n";
+                ss << "#pragma unroll 8\n" << loop << "        const float v = " << loaded << ";\n";
+                ss << "        const float r = kn_exp(v - m) / s;\n";
+                store("        ", "i", "r");
+                ss << "    }\n}\n";
+            } else {
             ss << "#pragma unroll 8\n" << loop << "        const float v = " << loaded << ";\n        " << fold_stmt << "\n    }\n";
             ss << "    m = kn_column_fold(m, " << fold_fn << ", lds_m, tx, ty);\n";
             if (rowred) {
@@ -1314,13 +1329,14 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
                 store("        ", "i", "r");
                 ss << "    }\n}\n";
             }
+            }
         }
         spec.source = ss.str();
         spec.block = (uint32_t) threads;
         spec.grid = ceil_div_u32(outer_size * column_blocks, 1);
         std::ostringstream note;
         note << (softmax ? "softmax" : (rowred ? "row statistic + elementwise" : "layernorm")) << " columns TX=" << TX << " TY=" << TY
-             << " items=" << items << (held ? " cached" : " streamed");
+             << " items=" << items << (held ? " cached" : (softmax ? " streamed twice" : " streamed"));
         if (threads != 256) note << " threads=" << threads;
         spec.strategy = note.str();
         return spec;

@@ -2244,7 +2244,7 @@ def special_values_on_the_split_paths():
     """infinities and NaN through the kernels that split their work: a softmax along axis 0 (lanes across columns) with a
     column that is all -inf, one that holds +inf and one with a NaN; reductions in two launches whose input holds NaN
     (ignored by min and max, kept by sum) and infinities; a softmax over long rows (separate steps) with -inf entries
-    and a row that is all -inf"""
+    and a row that is all -inf; the same down columns of 1000 that are read twice"""
     g = Graph()
     rng = np.random.default_rng(179)
     cols = rng.standard_normal((37, 40)).astype(np.float32)
@@ -2264,4 +2264,12 @@ def special_values_on_the_split_paths():
     rows[0, 100:50000] = -np.inf
     rows[1, :] = -np.inf
     g.output(g.softmax(g.input([3, 70000]), 1))
-    return g, 0, [cols, tall, rows], None
+    # columns too long to hold (read twice): one that starts with -inf, one that is all -inf, a NaN, a +inf
+    long_cols = (rng.standard_normal((1000, 50)) * 3).astype(np.float32)
+    long_cols[:700, 2] = -np.inf
+    long_cols[:, 5] = -np.inf
+    long_cols[321, 8] = np.nan
+    long_cols[999, 13] = np.inf
+    long_cols[::2, 21] = -np.inf
+    g.output(g.softmax(g.input([1000, 50]), 0))
+    return g, 0, [cols, tall, rows, long_cols], None
