@@ -2,7 +2,8 @@
 
     python -m kyanite_amd.op_bench [-d DEVICE] [-n ITERATIONS] [-p] [FAMILY ...]
 
-Families (default: all): `elementwise`, `gather`, `reduce`, `rows` (softmax / layernorm), `conv`, `matmul`. `-p` plans and
+Families (default: all): `elementwise`, `activations`, `gather`, `reduce`, `rows` (softmax / layernorm), `conv`,
+`matmul`. `-p` plans and
 compiles every case without a device and prints its steps instead of running it.
 
 Every case is built like a user's graph (inputs, constants for weights), gets normally distributed inputs (matrix
@@ -19,7 +20,7 @@ import numpy as np
 
 
 def _cases():
-    from . import DType, Graph, ReduceOp
+    from . import DType, Graph, ReduceOp, UnaryOp
 
     f32, f16, u8 = DType.F32, DType.F16, DType.U8
     rng = np.random.default_rng(0)
@@ -42,6 +43,23 @@ def _cases():
          lambda g: g.output(g.add(g.permute(g.input([64, 256, 64, 64]), [0, 2, 3, 1]), one(g))), 512 * M)
     case("elementwise", "x + column, f32 8192 x 8192",
          lambda g: g.output(g.add(g.input([8192, 8192]), g.broadcast(g.input([8192, 1]), [8192, 8192]))), 512 * M)
+
+    def activation_case(name, build, dtype=f32):
+        elem = 2 if dtype == f16 else 4
+        case("activations", f"{name}, {dtype.name.lower()} [64M]", lambda g: g.output(build(g, g.input([64 * M], dtype), dtype)), 2 * elem * 64 * M)
+
+    def gelu_erf(g, x, dtype):
+        inner = g.unary(UnaryOp.ERF, g.mul(x, g.scalar(0.7071067811865476, dtype)))
+        return g.mul(g.mul(x, g.scalar(0.5, dtype)), g.add(g.scalar(1, dtype), inner))
+
+    for dtype in (f32, f16):
+        activation_case("sigmoid", lambda g, x, dt: g.unary(UnaryOp.SIGMOID, x), dtype)
+        activation_case("tanh", lambda g, x, dt: g.unary(UnaryOp.TANH, x), dtype)
+        activation_case("mish", lambda g, x, dt: g.unary(UnaryOp.MISH, x), dtype)
+        activation_case("softplus", lambda g, x, dt: g.unary(UnaryOp.SOFTPLUS, x), dtype)
+        activation_case("gelu through erf", gelu_erf, dtype)
+        activation_case("x ** 2", lambda g, x, dt: g.pow(x, g.scalar(2.0, dt)), dtype)
+        activation_case("x ** 1.5", lambda g, x, dt: g.pow(x, g.scalar(1.5, dt)), dtype)
 
     def gather_case(name, shape, axis, count, dtype=f32):
         elem = np.dtype(dtype.numpy).itemsize
@@ -169,7 +187,7 @@ def main(argv=None):
 
     from . import Graph, HipExecutor
 
-    known = ["elementwise", "gather", "reduce", "rows", "conv", "matmul"]
+    known = ["elementwise", "activations", "gather", "reduce", "rows", "conv", "matmul"]
     for family in args.families:
         if family not in known:
             parser.error(f"unknown family {family!r}; choose from {', '.join(known)}")

@@ -6,7 +6,7 @@ from kyanite_amd import op_bench
 
 
 def test_plans_without_a_device(capsys):
-    assert op_bench.main(["-p", "reduce", "rows", "elementwise", "gather"]) == 0
+    assert op_bench.main(["-p", "reduce", "rows", "elementwise", "gather", "activations"]) == 0
     text = capsys.readouterr().out
     assert "fold of 1024 partial results" in text and "columns TX=32 TY=8" in text and "transposed tiles 64x64" in text
     assert "rank=2 vec=8 unroll=4" in text  # embedding rows of halves: 16 bytes per thread
