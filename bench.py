@@ -51,12 +51,46 @@ MFMA_PEAK_TFLOPS = {"f32": 157.3, "f16": 2500.0}
 TRAFFIC_PROFILE = "profiles/bandwidth_graphs_counters.md"
 
 
+def traffic_from_profile(kernel_name):
+    """HBM bytes per launch of one of the bandwidth kernels as the committed counter summary states it: the row of its
+    table `| kernel | reads (B) | writes (B) | HBM traffic per launch (B) | algorithmic bytes | ratio |` whose first
+    cell ends in the graph's number ("2b"); None when the file or the row is missing."""
+    tag = kernel_name.split("_")[0]
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) == 6 and cells[0].endswith(" " + tag) and re.fullmatch(r"[\d,]+", cells[3]):
+                    return int(cells[3].replace(",", ""))
+    except OSError:
+        pass
+    return None
+
+
 def log(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
+def elements_over_bar(expected, actual):
+    """(elements whose relative error under the 1e-3 rms floor exceeds the bar of the dtype, elements compared)"""
+    import numpy as np
+    from oracle.parity import F16_MAX_REL, F32_MAX_REL, SMALL_FLOOR
+    e = np.asarray(expected)
+    bar = F16_MAX_REL if e.dtype == np.float16 else F32_MAX_REL
+    e64 = e.astype(np.float64).reshape(-1)
+    a64 = np.asarray(actual).astype(np.float64).reshape(-1)
+    keep = np.isfinite(e64)
+    e64, a64 = e64[keep], a64[keep]
+    if e64.size == 0:
+        return 0, 0
+    floor = SMALL_FLOOR * float(np.sqrt(np.mean(e64 * e64)))
+    rel = np.abs(a64 - e64) / np.maximum(np.abs(e64), max(floor, 1e-300))
+    return int(np.count_nonzero(rel > bar)), int(e64.size)
+
+
 def check_parity(graph, batch, inputs, expected, actual, what):
     """The rules of oracle/parity.py; returns a summary for the JSON line, ends the run when a rule fails."""
+    import numpy as np
     from oracle.parity import check_outputs
     records = []
     try:
@@ -64,10 +98,22 @@ def check_parity(graph, batch, inputs, expected, actual, what):
     except AssertionError as failure:
         log(f"PARITY FAILURE: {failure}")
         sys.exit(1)
-    summary = {"rules": sorted({r["rule"] for r in records})}
+    summary = {"rules": sorted({r["rule"] for r in records}), "elements_compared": int(sum(r["elements"] for r in records))}
     errs = [r["err"] for r in records if "err" in r]
     if errs:
         summary["max_rel_err_floor_1e-3_rms"] = float(f"{max(errs):.3e}")
+        # the floor (fraction of the tensor's rms) at which every element would lie within the bar
+        summary["floor_needed_rms_fraction"] = float(f"{max(r.get('floor_needed', 0.0) for r in records):.3e}")
+        # how many elements, not only the worst one, lie outside the stated bar under the small floor
+        over, floats = 0, 0
+        for e, a in zip(expected, actual):
+            if np.asarray(e).dtype.kind != "f":
+                continue
+            n_over, n = elements_over_bar(e, a)
+            over += n_over
+            floats += n
+        summary["elements_over_bar_floor_1e-3_rms"] = over
+        summary["fraction_over_bar"] = float(f"{over / max(floats, 1):.3e}")
     acc = [r for r in records if r["rule"] == "accumulated"]
     if acc:
         worst = max(acc, key=lambda r: r["gpu_max"])
@@ -75,7 +121,8 @@ def check_parity(graph, batch, inputs, expected, actual, what):
             "terms_per_sum": worst["k"], "floor_rms_fraction": float(f"{worst['floor_k']:.3g}"),
             "max_rel_err_with_that_floor": float(f"{max(r['err_k'] for r in acc):.3e}"),
             "gpu_vs_f64_max": float(f"{worst['gpu_max']:.3e}"), "oracle_vs_f64_max": float(f"{worst['oracle_max']:.3e}"),
-            "gpu_vs_f64_rms": float(f"{worst['gpu_rms']:.3e}"), "oracle_vs_f64_rms": float(f"{worst['oracle_rms']:.3e}")}
+            "gpu_vs_f64_rms": float(f"{worst['gpu_rms']:.3e}"), "oracle_vs_f64_rms": float(f"{worst['oracle_rms']:.3e}"),
+            "agreement_rule_waived": bool(any(r.get("rule2_waived") for r in acc))}
     return summary
 
 
@@ -88,6 +135,19 @@ def timed_steps(ex, steps, warmup):
         ex.run_async()
     ex.synchronize()
     return time.perf_counter() - t0
+
+
+def evaluate_with_copies(ex, inputs, n):
+    """Wall clock of `evaluate` (host buffers in, host buffers out: staging copies, H2D, launches, D2H), timed like
+    kn-cuda-eval/src/bin/profile_net.rs:146-180 times it: max(1, n / 10) untimed evaluations, then n."""
+    for _ in range(max(1, n // 10)):
+        ex.evaluate(inputs)
+    t0 = time.perf_counter()
+    for _ in range(n):
+        ex.evaluate(inputs)
+    dt = (time.perf_counter() - t0) / n
+    return {"ms_per_eval": float(f"{dt * 1e3:.5g}"), "evals_per_s": float(f"{1.0 / dt:.5g}"), "evaluations": n,
+            "input_bytes": int(sum(x.nbytes for x in inputs))}
 
 
 def per_step_seconds(ex, iters):
@@ -188,7 +248,14 @@ def run_bandwidth(args, device, steps, warmup):
                         "sample": "oracle (C++ restatement of cpu_eval_graph, single thread) on the whole workload, one "
                                   "evaluation of each graph at full shape: " + ", ".join(sample_desc)}
 
+    # the same step with the copies: `evaluate` of the combined graph from host buffers (1.3 GB in, 0.9 GB out)
+    all_inputs = [x for name, *_ in parts for x in host_inputs[name]]
+    with_copies = evaluate_with_copies(ex, all_inputs, 3)
+    with_copies["graph_evals_per_s"] = float(f"{len(parts) * with_copies['evals_per_s']:.5g}")
+    log(f"evaluate with copies: {with_copies}")
+
     dom = kernels[dominant]
+    traffic = traffic_from_profile(dominant)
     return {
         "metric": "graph evals/sec at 1 GPU (bandwidth-bound op graphs 2a-2d, device only)",
         "value": round(evals_per_s, 2),
@@ -207,9 +274,13 @@ def run_bandwidth(args, device, steps, warmup):
                                "once, back to back on one stream",
                    "inputs_resident_in_hbm": True},
         "roofline": {"bound": "hbm", "kernel": f"{dominant} ({dom['step']})", "achieved": dom["achieved_gbs"],
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"], "traffic": None,
-                     "traffic_note": f"not measured in this run; counter runs of the same kernels: {TRAFFIC_PROFILE}"},
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac"], "traffic": traffic,
+                     "traffic_note": (f"HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy kernel) from the "
+                                      f"committed counter runs of this kernel, {TRAFFIC_PROFILE}; not measured in this run"
+                                      if traffic is not None else
+                                      f"not measured in this run; counter runs of the same kernels: {TRAFFIC_PROFILE}")},
         "kernels": kernels,
+        "evaluate_with_copies": with_copies,
         "cpu_baseline": cpu_baseline,
         "device": device.name(),
     }
@@ -330,44 +401,53 @@ def run_model(args, device, workload, steps, warmup):
             cpu_seconds = (time.perf_counter() - t) / n
             sample_graph, sample_batch, sample_inputs, sample_outputs = graph, batch, inputs, gpu_outputs
             cpu_evals = 1.0 / cpu_seconds
+            sample_kind = "all"
             sample = f"{n} evaluations of the whole graph at batch 8 ({cpu_seconds * 1e6:.1f} us each)"
         elif workload == "resnet":
-            rows = args.resnet_rows  # positions are independent of each other: the first rows of the batch must match
+            # positions are independent of each other: any leading part of the batch must match; default all of it
+            rows = args.resnet_rows or batch
             sample_graph, sample_batch, sample_inputs = graph, rows, [x[:rows] for x in inputs]
             t = time.perf_counter()
             expected = cpu_eval_graph(sample_graph, sample_batch, sample_inputs)
             cpu_seconds = time.perf_counter() - t
             sample_outputs = [g[:rows] for g in gpu_outputs]
             cpu_evals = rows / cpu_seconds / batch
-            sample = (f"the first {rows} of the 1024 positions ({cpu_seconds:.2f} s), scaled to evaluations of 1024 "
-                      f"positions; the GPU's first {rows} rows at batch 1024 are checked against them")
+            sample_kind = "all" if rows == batch else f"first {rows} of {batch} positions"
+            sample = (f"all {batch} positions ({cpu_seconds:.2f} s for one evaluation)" if rows == batch else
+                      f"the first {rows} of the {batch} positions ({cpu_seconds:.2f} s), scaled to evaluations of {batch} "
+                      f"positions; the GPU's first {rows} rows at batch {batch} are checked against them")
         elif workload == "llama":
-            # causal attention: the first tokens do not depend on the later ones; 128 tokens span two key blocks of
-            # the fused attention kernel and rows of every wave of a matmul tile
-            rows = args.llama_rows
-            sample_graph, _, _ = configs.build_llama(seed=0, seq=rows)
+            # default: the whole prefill. With fewer rows: by causality the first tokens do not depend on the later ones
+            rows = args.llama_rows or 512
+            sample_graph = graph if rows == 512 else configs.build_llama(seed=0, seq=rows)[0]
             sample_batch, sample_inputs = 0, [inputs[0][:, :rows]]
             t = time.perf_counter()
             expected = cpu_eval_graph(sample_graph, 0, sample_inputs)
             cpu_seconds = time.perf_counter() - t
             sample_outputs = [gpu_outputs[0][:, :rows]]
             cpu_evals = rows / cpu_seconds / 512
-            sample = (f"the same decoder on the first {rows} of the 512 tokens ({cpu_seconds:.2f} s), scaled to "
+            sample_kind = "all" if rows == 512 else f"first {rows} of 512 tokens"
+            sample = (f"all 512 tokens ({cpu_seconds:.2f} s for one evaluation)" if rows == 512 else
+                      f"the same decoder on the first {rows} of the 512 tokens ({cpu_seconds:.2f} s), scaled to "
                       f"evaluations of 512 tokens; by causality the GPU's first {rows} output rows at sequence 512 are "
                       "checked against them")
         else:
-            # samples of the batch are independent: the first one at full resolution
-            sample_graph, _, _ = configs.build_unet_block(seed=0, batch=1)
-            sample_batch, sample_inputs = 0, [x[:1] for x in inputs]
+            # samples of the batch are independent; default both
+            n = args.unet_samples or 2
+            sample_graph = graph if n == 2 else configs.build_unet_block(seed=0, batch=n)[0]
+            sample_batch, sample_inputs = 0, [x[:n] for x in inputs]
             t = time.perf_counter()
             expected = cpu_eval_graph(sample_graph, 0, sample_inputs)
             cpu_seconds = time.perf_counter() - t
-            sample_outputs = [gpu_outputs[0][:1]]
-            cpu_evals = 1.0 / cpu_seconds / 2
-            sample = (f"the first of the 2 samples at full resolution ({cpu_seconds:.2f} s), scaled to evaluations of "
+            sample_outputs = [gpu_outputs[0][:n]]
+            cpu_evals = n / cpu_seconds / 2
+            sample_kind = "all" if n == 2 else f"first {n} of 2 samples"
+            sample = (f"both samples at full resolution ({cpu_seconds:.2f} s for one evaluation)" if n == 2 else
+                      f"the first of the 2 samples at full resolution ({cpu_seconds:.2f} s), scaled to evaluations of "
                       "batch 2; the GPU's first sample at batch 2 is checked against it")
         log(f"oracle sample took {cpu_seconds:.2f} s")
         extra["parity"] = check_parity(sample_graph, sample_batch, sample_inputs, expected, sample_outputs, workload)
+        extra["parity"]["sample"] = sample_kind
         log(f"parity {extra['parity']}")
         cpu_baseline = {"value": float(f"{cpu_evals:.4g}"), "unit": "graph evals/s", "cores": 1, "kind": "port",
                         "sample": "oracle (C++ restatement of cpu_eval_graph, single thread) on " + sample}
@@ -378,16 +458,11 @@ def run_model(args, device, workload, steps, warmup):
         dt = timed_steps(ex, steps, warmup) / steps
         extra["hip_graph_replay"] = {"ms_per_step": round(dt * 1e3, 5), "evals_per_s": round(1.0 / dt, 1)}
         ex.set_graph_mode(False)
-        # the reference's executor contract includes the copies: time `evaluate` (H2D, launches, D2H) as well
-        n = 2000
-        for _ in range(20):
-            ex.evaluate(inputs)
-        t = time.perf_counter()
-        for _ in range(n):
-            ex.evaluate(inputs)
-        dt = (time.perf_counter() - t) / n
-        extra["evaluate_with_copies_us"] = round(dt * 1e6, 2)
-        extra["evaluate_with_copies_evals_per_s"] = round(1.0 / dt, 1)
+
+    # the reference's executor contract includes the copies: `evaluate` (staging, H2D, launches, D2H) next to the
+    # device-only figure, for every configuration
+    extra["evaluate_with_copies"] = evaluate_with_copies(ex, inputs, 2000 if workload == "mlp" else 20)
+    log(f"evaluate with copies: {extra['evaluate_with_copies']}")
 
     mfma_s = sum(float(per_step[i]) for i in range(ex.step_count()) if ex.step_work(i)[0] > 0)
     mfma_flops = sum(ex.step_work(i)[0] for i in range(ex.step_count()))
@@ -425,7 +500,7 @@ WORKLOADS = {"mlp": "configs[0]", "bandwidth": "configs[1]", "resnet": "configs[
 def summary_of(result):
     """What the `configs` table of the combined line keeps of one workload's result."""
     keep = ("metric", "value", "unit", "steps", "warmup", "ms_per_step", "dtype", "roofline", "matmul_conv_total", "parity",
-            "cpu_baseline", "hip_graph_replay", "evaluate_with_copies_us", "evaluate_with_copies_evals_per_s")
+            "cpu_baseline", "hip_graph_replay", "evaluate_with_copies")
     out = {k: result[k] for k in keep if k in result}
     out["workload"] = result["config"]["workload"]
     if "whole_graph_tflops" in result["config"]:
@@ -436,6 +511,39 @@ def summary_of(result):
     elif kernels:
         out["kernels"] = [{k: e[k] for k in ("kernel", "launches", "avg_ms", "share", "achieved_tflops", "mfma_frac", "achieved_gbs",
                                               "hbm_frac") if k in e} for e in kernels[:6]]
+    return out
+
+
+def compact_summary(entry):
+    """One short flat record per configuration for the top level of the combined line: step time, throughput with and
+    without copies, roofline fraction of the dominant kernel, matmul / conv total against the MFMA peak, parity."""
+    out = {"ms_per_step": entry["ms_per_step"], "evals_per_s": entry["value"], "frac": entry["roofline"]["frac"],
+           "bound": entry["roofline"]["bound"]}
+    if "matmul_conv_total" in entry:
+        out["mfma_frac_all_matmul_conv"] = entry["matmul_conv_total"]["mfma_frac"]
+    if "evaluate_with_copies" in entry:
+        out["ms_per_eval_with_copies"] = entry["evaluate_with_copies"]["ms_per_eval"]
+    parity = entry.get("parity")
+    kernels = entry.get("kernels")
+    if parity is None and isinstance(kernels, dict):
+        parts = [k["parity"] for k in kernels.values() if "parity" in k]
+        if parts:
+            parity = {"rules": sorted({r for p in parts for r in p["rules"]}), "sample": "all",
+                      "elements_compared": sum(p["elements_compared"] for p in parts),
+                      "max_rel_err_floor_1e-3_rms": max(p.get("max_rel_err_floor_1e-3_rms", 0.0) for p in parts)}
+        out["hbm_frac_per_kernel"] = {name: k["frac"] for name, k in kernels.items()}
+    if parity is not None:
+        out["parity_rules"] = parity["rules"]
+        out["parity_sample"] = parity.get("sample", "all")
+        out["parity_elements"] = parity.get("elements_compared")
+        if "max_rel_err_floor_1e-3_rms" in parity:
+            out["parity_max_rel_err"] = parity["max_rel_err_floor_1e-3_rms"]
+        if "fraction_over_bar" in parity:
+            out["parity_fraction_over_bar"] = parity["fraction_over_bar"]
+        if "floor_needed_rms_fraction" in parity:
+            out["parity_floor_needed"] = parity["floor_needed_rms_fraction"]
+    if entry.get("cpu_baseline"):
+        out["cpu_evals_per_s"] = entry["cpu_baseline"]["value"]
     return out
 
 
@@ -453,8 +561,12 @@ def main():
                              "to calibrate hardware counters against)")
     parser.add_argument("--order", default="abcd", help="order of the four graphs inside one step (letters a-d)")
     parser.add_argument("--kernel-iters", type=int, default=20, help="profiled runs for the per-kernel timing")
-    parser.add_argument("--resnet-rows", type=int, default=64, help="positions of the ResNet batch the oracle evaluates")
-    parser.add_argument("--llama-rows", type=int, default=128, help="leading tokens of the LLaMA prefill the oracle evaluates")
+    parser.add_argument("--resnet-rows", type=int, default=0,
+                        help="leading positions of the ResNet batch the oracle evaluates (default 0: all 1024)")
+    parser.add_argument("--llama-rows", type=int, default=0,
+                        help="leading tokens of the LLaMA prefill the oracle evaluates (default 0: all 512)")
+    parser.add_argument("--unet-samples", type=int, default=0,
+                        help="leading samples of the UNet batch the oracle evaluates (default 0: both)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on exactly one GPU (one executor, one arena, no collectives); "
@@ -478,6 +590,7 @@ def main():
             log(f"---- {name} ({time.time() - t0:.0f} s so far)")
             table[f"{WORKLOADS[name]} {name}"] = summary_of(run_model(args, device, name, None, None))
         result["configs"] = dict(sorted(table.items()))
+        result["configs_summary"] = {name: compact_summary(entry) for name, entry in result["configs"].items()}
         result["config"]["also_run"] = "every other BASELINE configuration, see `configs`"
         log(f"all workloads took {time.time() - t0:.0f} s")
     print(json.dumps(result))

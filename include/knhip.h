@@ -70,16 +70,6 @@ int knhip_memcpy_d2d(int device, void *dst, const void *src, size_t bytes);
 int knhip_host_alloc(size_t bytes, void **ptr);
 int knhip_host_free(void *ptr);
 int knhip_device_synchronize(int device);
-/* No counterpart in the reference. What the matrix cores of the device sustain when nothing else limits them: a
- * register-only loop of independent MFMAs on one wave per SIMD and the shader clock it ran at. `mode` is a sum of
- * KNHIP_PROBE_NORMAL (operands N(0, 1) instead of small integers), KNHIP_PROBE_F32 (v_mfma_f32_32x32x2_f32 instead
- * of v_mfma_f32_32x32x16_f16) and KNHIP_PROBE_RECTIFIED (the B operands max(x, 0), like activations after a relu).
- * The rate on N(0, 1) data is the ceiling that matmul / convolution rates on real data should be read against (the
- * clock drops under the power they draw). */
-#define KNHIP_PROBE_NORMAL 1
-#define KNHIP_PROBE_F32 2
-#define KNHIP_PROBE_RECTIFIED 4
-int knhip_device_mfma_probe(int device, int mode, int iterations, double *tflops, double *shader_mhz);
 
 /* streams and events (replaces CudaStream, kn-cuda-sys/src/wrapper/handle.rs:105-174, and CudaEvent, event.rs:7-45).
  * Handles are the HIP objects themselves (hipStream_t / hipEvent_t behind void *); a NULL stream is the device's
@@ -109,7 +99,8 @@ int knhip_memcpy_d2d_async(int device, void *dst, const void *src, size_t bytes,
  * (kn-cuda-eval/src/planner.rs:606-648). Elements are f32, or f16 with f32 accumulation and one rounding at the store.
  * Launches that split the K axis between workgroups keep f32 partial products and tile counters in `workspace`
  * (device memory, 256 byte aligned, knhip_batched_mat_mul_workspace_bytes(args) bytes; may be NULL when that is 0);
- * the call returns once the work is queued on `stream`, and the workspace must stay untouched until it has run. */
+ * the call returns once the work is queued on `stream`, and the workspace must stay untouched until it has run.
+ * A batch of more than 65535 entries runs as several launches, one after the other on `stream`. */
 typedef struct {
     int dtype; /* KNHIP_F32 or KNHIP_F16 */
     int batch, m, n, k;
@@ -130,6 +121,66 @@ int knhip_batched_mat_mul(int device, void *stream, const knhip_matmul_args *arg
  * work overlaps on one GPU (two streams, two threads) race, the caller orders them. */
 #define KNHIP_STATIC_SCRATCH_BYTES (32u << 20)
 int knhip_batched_mat_mul_static(int device, void *stream, const knhip_matmul_args *args);
+/* The first use of the static array on a device looks its address up, which is no stream operation and may be refused
+ * while a stream capture is open: call this once per device beforehand (any earlier knhip_batched_mat_mul_static on the
+ * device does the same). Allocates nothing. */
+int knhip_static_scratch_prepare(int device);
+
+/* ---- device tensors and stand-alone kernels, outside any executor ------------------------------------------------
+ * A tensor in device memory that the caller owns: DeviceTensor = PtrTensor<DevicePtr> (kn-cuda-eval/src/
+ * offset_tensor.rs:14-20, device_tensor.rs:12). `ptr` is the address of the element with index 0 along every axis,
+ * strides are in elements and may be zero (broadcast) or negative (flipped); the views of offset_tensor.rs:52-114
+ * (permute, view, broadcast, slice, index, flip, repeat_unary) are edits of shape, strides and address that the
+ * binding does on its side (knhip_strided_view / knhip_strided_slice below give the layout algebra). */
+typedef struct {
+    void *ptr;
+    int dtype; /* KNHIP_F32 ... KNHIP_F16 */
+    size_t rank;
+    const size_t *shape;
+    const int64_t *strides;
+} knhip_tensor;
+
+/* DeviceTensor::copy_from (device_tensor.rs:101-126): dst[i] = src[i] for every index i of the common shape, same
+ * dtype. One linear device-to-device copy when both sides have the same dense strides, else the elementwise kernel
+ * with the operation `y = x` on the two layouts (the reference's "restride trick", copy_from_as_scalar_op
+ * :73-99). Returns once the work is queued on `stream` (the reference synchronises a stream of its own; a binding that
+ * wants that calls knhip_stream_synchronize). The destination may not have a broadcast axis. */
+int knhip_strided_copy(int device, void *stream, const knhip_tensor *dst, const knhip_tensor *src);
+
+/* The five run-time compiled kernel types of kn-cuda-eval/src/autokernel/, on caller-owned tensors. A constructor
+ * specialises the kernel for shapes, strides and element types (tensor descriptors whose `ptr` may be NULL: the tensor
+ * is then assumed to start on a 16 byte boundary; run refuses addresses of another alignment than the constructor
+ * saw) and compiles it (cached). `device` -1 compiles without a GPU; such a kernel cannot run. knhip_kernel_run takes
+ * the addresses in the order of the constructor's tensors and returns once the launch is queued on `stream`. */
+typedef struct knhip_kernel knhip_kernel;
+/* ScalarKernel::new_for_shapes (autokernel/scalar.rs:33-121): `operation` in the reference's form, "*x0 = *x1 + *x2;"
+ * (it must end in ';'). x0 points at the element of operand 0, which is written; xk (k >= 1) at the element of
+ * operand k, which is read. Inside the operation a value has its register type: float for f16, bool for bool, else the
+ * C type of its dtype. All operands have one shape; run: one address per operand. */
+int knhip_scalar_kernel_new(int device, const char *operation, const knhip_tensor *operands, size_t operand_count,
+                            knhip_kernel **out);
+/* ReduceKernel::new (autokernel/reduce.rs:35-123) with the operation as a code (KNHIP_REDUCE_*, identities and mean
+ * as in kn-graph/src/graph.rs:1746-1786) where the reference takes C text; `output` has the kept axes of `input` in
+ * order. run: (input, output). */
+int knhip_reduce_kernel_new(int device, int reduce_op, const knhip_tensor *input, const knhip_tensor *output, const size_t *axes,
+                            size_t axis_count, knhip_kernel **out);
+/* SoftmaxKernel::new (autokernel/softmax.rs:28-91): output = softmax(input_scale * input) along `axis`, f32.
+ * run: (input, output). */
+int knhip_softmax_kernel_new(int device, const knhip_tensor *input, const knhip_tensor *output, size_t axis, float input_scale,
+                             knhip_kernel **out);
+/* LayernormKernel::new (autokernel/layernorm.rs:33-93): x = alpha0 * input0 + alpha1 * input1, output =
+ * beta * (x - mean) / sqrt(var + eps) along `axis`, f32; input1 has input0's layout and is only read when alpha1 is
+ * not 0. run: (input0, input1 or NULL, output), like layernorm.rs:95-111. */
+int knhip_layernorm_kernel_new(int device, const knhip_tensor *input, const knhip_tensor *output, size_t axis, float eps,
+                               float alpha0, float alpha1, float beta, knhip_kernel **out);
+/* GatherKernel::new (autokernel/gather.rs:30-98): output[.., i, ..] = input[.., indices[i], ..] along `axis`, zero where
+ * the index is out of range; indices of any integer type, rank 1. run: (input, indices, output). */
+int knhip_gather_kernel_new(int device, const knhip_tensor *input, const knhip_tensor *indices, const knhip_tensor *output,
+                            size_t axis, knhip_kernel **out);
+int knhip_kernel_run(const knhip_kernel *kernel, void *stream, void *const *ptrs, size_t count);
+/* the specialisation that was picked (a short text), and the launch size */
+int knhip_kernel_info(const knhip_kernel *kernel, char *strategy, size_t cap, size_t *needed, unsigned *grid, unsigned *block);
+void knhip_kernel_free(knhip_kernel *kernel);
 
 /* ---- graph (kn-graph/src/graph.rs) ------------------------------------------------------------------------- */
 typedef struct knhip_graph knhip_graph;
@@ -232,18 +283,49 @@ int knhip_graph_optimize(const knhip_graph *g, const knhip_optimizer_settings *s
 /* ---- executor (kn-cuda-eval/src/executor.rs:60-258, kn-runtime/src/lib.rs:85-126) ------------------------------ */
 typedef struct knhip_executor knhip_executor;
 
-/* CudaExecutor::new(device, &graph, batch_size) (executor.rs:61); `flags` is 0 for the reference's behaviour.
- * KNHIP_PLAN_ONLY: nothing touches a device, the graph is planned and its kernels are compiled (works on a machine
- * without a GPU). KNHIP_PRESERVE_INPUTS: input buffers are never reused for later values, for callers that write
- * the inputs on the device once and then call run_async many times (the reference re-uploads them per evaluate).
- * KNHIP_STEP_BY_STEP: every run launches the planned steps one by one, also where the whole plan is small enough to
- * run as one kernel (knhip_executor_fused_source). */
-#define KNHIP_PLAN_ONLY 1
-#define KNHIP_PRESERVE_INPUTS 2
-#define KNHIP_STEP_BY_STEP 4
-int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int flags, knhip_executor **out);
-int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int flags,
-                                 knhip_executor **out);
+/* What an executor is built with beyond (device, graph, batch size). Fill the struct with
+ * knhip_executor_options_default() and change what is needed; a NULL pointer means the defaults: the reference's
+ * behaviour with every planned path of this library switched on. The options belong to the one executor (nothing is
+ * read from the environment), so two executors of one process can be planned differently. The reference's own knob
+ * surface is the optimizer's (kn-graph/src/optimizer/mod.rs:11-22, knhip_optimizer_settings above); its executor has
+ * none (executor.rs:61).
+ * plan_only: nothing touches a device, the graph is planned and its kernels are compiled (works on a machine without
+ *   a GPU). preserve_inputs: input buffers are never reused for later values, for callers that write the inputs on the
+ *   device once and then call run_async many times (the reference re-uploads them per evaluate). step_by_step: every
+ *   run launches the planned steps one by one, also where the whole plan is small enough to run as one kernel
+ *   (knhip_executor_fused_source).
+ * The remaining int fields are 1 by default; 0 switches that path off:
+ *   fuse_attention            matmul, softmax, matmul chains as one launch (off: three launches)
+ *   group_matmuls             matmuls that share their left operand in one launch (off: one launch each)
+ *   pack_matmul_constants     constant [k, n] right operands laid out again as [n, k] when the plan is made
+ *   pointwise_conv_as_matmul  1 x 1 convolutions with stride 1 as one matrix product per image (off: the conv kernel)
+ *   join_elementwise          neighbouring independent elementwise steps of one shape share a launch
+ *   split_reduce              reductions with few results and a long reduced index run as two launches
+ *   tiled_transpose           elementwise kernels with a transposed operand turn tiles through LDS
+ *   split_conv_channels       convolutions with few tiles fold slices of their input channels side by side
+ *   plane_conv_any_width      3 x 3 convolutions on images without a power-of-two width use the plane kernel
+ *   direct_gemm               matmul kernels that load global -> LDS directly (off: staged through registers)
+ *   split_k, tail_split       workgroups that share a tile along K (either kind) / only the last round's tiles
+ *   dot_products              one wave per result for products of up to 2^20 multiplications
+ * streaming_bytes: operands of at least this size that are touched once per element are read and written with
+ *   non-temporal accesses (default 64 MiB; 0: never). mapped_io_bytes: evaluate() of a graph whose inputs and outputs
+ *   are at most this many bytes in all reads and writes them in page-locked host memory instead of copying them
+ *   to and from the arena (default 64 KiB; 0: never). */
+typedef struct {
+    size_t struct_bytes; /* sizeof(knhip_executor_options), set by knhip_executor_options_default */
+    int plan_only, preserve_inputs, step_by_step;
+    int fuse_attention, group_matmuls, pack_matmul_constants, pointwise_conv_as_matmul, join_elementwise, split_reduce;
+    int tiled_transpose, split_conv_channels, plane_conv_any_width;
+    int direct_gemm, split_k, tail_split, dot_products;
+    uint64_t streaming_bytes, mapped_io_bytes;
+} knhip_executor_options;
+int knhip_executor_options_default(knhip_executor_options *options);
+
+/* CudaExecutor::new(device, &graph, batch_size) (executor.rs:61) */
+int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, const knhip_executor_options *options,
+                       knhip_executor **out);
+int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size,
+                                 const knhip_executor_options *options, knhip_executor **out);
 void knhip_executor_free(knhip_executor *ex);
 
 int knhip_executor_io_count(const knhip_executor *ex, size_t *inputs, size_t *outputs);
@@ -266,7 +348,11 @@ int knhip_executor_synchronize(knhip_executor *ex);
  * `iterations` back-to-back run_async calls bracketed by two HIP events recorded on the executor's stream;
  * returns the elapsed device time in milliseconds for all iterations together. */
 int knhip_executor_time_runs(knhip_executor *ex, size_t iterations, float *elapsed_ms);
-/* device addresses of the dense input / output tensors inside the arena (pub device_inputs / device_outputs) */
+/* Device addresses of the dense input / output tensors inside the arena (pub device_inputs / device_outputs). Their
+ * contents are what run_async reads and writes. evaluate() leaves its inputs and outputs there too, EXCEPT for
+ * graphs under the mapped_io_bytes option (64 KiB of inputs + outputs by default), whose evaluate() works on page-locked
+ * host memory and never touches these buffers: a caller that mixes evaluate() with device-side reads of these
+ * addresses sets mapped_io_bytes to 0. */
 int knhip_executor_input_ptr(const knhip_executor *ex, size_t index, void **ptr);
 int knhip_executor_output_ptr(const knhip_executor *ex, size_t index, void **ptr);
 /* the HIP stream (hipStream_t) every step is launched on (CudaExecutor::stream, executor.rs:112-114) */

@@ -7,6 +7,8 @@ from ._lib import KnError, LIB_PATH
 from .executor import Device, HipDevice, HipExecutor, PreparedGraph, Profile, compile_stats
 from .runtime import (STATIC_SCRATCH_BYTES, DeviceBuffer, HipEvent, HipStream, PinnedMem, batched_mat_mul,
                       batched_mat_mul_static, batched_mat_mul_workspace_bytes, matmul_args)
+from .device_tensor import DeviceTensor, StridedShape
+from .autokernel import GatherKernel, LayernormKernel, ReduceKernel, ScalarKernel, SoftmaxKernel
 from .graph import (BATCH, BINARY_ALL, REDUCE_ALL, UNARY_ALL, BinaryOp, DType, Graph, OpKind, OptimizerSettings,
                     ReduceOp, Size, UnaryOp, Value, optimize_graph, shape)
 
@@ -16,4 +18,5 @@ __all__ = [
     "ReduceOp", "Size", "UnaryOp", "Value", "optimize_graph", "shape",
     "DeviceBuffer", "HipEvent", "HipStream", "PinnedMem", "batched_mat_mul", "batched_mat_mul_workspace_bytes", "matmul_args",
     "STATIC_SCRATCH_BYTES", "batched_mat_mul_static",
+    "DeviceTensor", "StridedShape", "ScalarKernel", "ReduceKernel", "SoftmaxKernel", "LayernormKernel", "GatherKernel",
 ]

@@ -43,6 +43,19 @@ class MatmulArgsT(Structure):
                 ("c", c_void_p), ("c_batch_stride", c_int64), ("c_row_stride", c_int64), ("c_col_stride", c_int64)]
 
 
+class ExecutorOptionsT(Structure):
+    _fields_ = ([("struct_bytes", c_size_t)] +
+                [(name, c_int) for name in (
+                    "plan_only", "preserve_inputs", "step_by_step", "fuse_attention", "group_matmuls", "pack_matmul_constants",
+                    "pointwise_conv_as_matmul", "join_elementwise", "split_reduce", "tiled_transpose", "split_conv_channels",
+                    "plane_conv_any_width", "direct_gemm", "split_k", "tail_split", "dot_products")] +
+                [("streaming_bytes", c_uint64), ("mapped_io_bytes", c_uint64)])
+
+
+class TensorT(Structure):
+    _fields_ = [("ptr", c_void_p), ("dtype", c_int), ("rank", c_size_t), ("shape", POINTER(c_size_t)), ("strides", POINTER(c_int64))]
+
+
 class MemUsageT(Structure):
     _fields_ = [("dedicated_bytes", c_size_t), ("shared_bytes", c_size_t), ("zero_bytes", c_size_t),
                 ("hypo_shared_bytes_peak", c_size_t), ("hypo_shared_bytes_total", c_size_t), ("arena_bytes", c_size_t)]
@@ -67,7 +80,6 @@ SIGNATURES = {
     "knhip_host_alloc": [c_size_t, POINTER(c_void_p)],
     "knhip_host_free": [c_void_p],
     "knhip_device_synchronize": [c_int],
-    "knhip_device_mfma_probe": [c_int, c_int, c_int, POINTER(c_double), POINTER(c_double)],
     "knhip_stream_create": [c_int, POINTER(c_void_p)],
     "knhip_stream_destroy": [c_int, c_void_p],
     "knhip_stream_synchronize": [c_int, c_void_p],
@@ -83,6 +95,16 @@ SIGNATURES = {
     "knhip_batched_mat_mul_workspace_bytes": [POINTER(MatmulArgsT), PZ],
     "knhip_batched_mat_mul": [c_int, c_void_p, POINTER(MatmulArgsT), c_void_p, c_size_t],
     "knhip_batched_mat_mul_static": [c_int, c_void_p, POINTER(MatmulArgsT)],
+    "knhip_static_scratch_prepare": [c_int],
+    "knhip_strided_copy": [c_int, c_void_p, POINTER(TensorT), POINTER(TensorT)],
+    "knhip_scalar_kernel_new": [c_int, c_char_p, POINTER(TensorT), c_size_t, POINTER(c_void_p)],
+    "knhip_reduce_kernel_new": [c_int, c_int, POINTER(TensorT), POINTER(TensorT), PZ, c_size_t, POINTER(c_void_p)],
+    "knhip_softmax_kernel_new": [c_int, POINTER(TensorT), POINTER(TensorT), c_size_t, c_float, POINTER(c_void_p)],
+    "knhip_layernorm_kernel_new": [c_int, POINTER(TensorT), POINTER(TensorT), c_size_t, c_float, c_float, c_float, c_float,
+                                   POINTER(c_void_p)],
+    "knhip_gather_kernel_new": [c_int, POINTER(TensorT), POINTER(TensorT), POINTER(TensorT), c_size_t, POINTER(c_void_p)],
+    "knhip_kernel_run": [c_void_p, c_void_p, POINTER(c_void_p), c_size_t],
+    "knhip_kernel_info": [c_void_p, c_char_p, c_size_t, PZ, POINTER(ctypes.c_uint), POINTER(ctypes.c_uint)],
     "knhip_graph_new": [POINTER(G)],
     "knhip_graph_clone": [G, POINTER(G)],
     "knhip_graph_deserialize": [POINTER(c_uint8), c_size_t, POINTER(G)],
@@ -129,8 +151,9 @@ SIGNATURES = {
     "knhip_graph_infer_batch_size": [G, PZ, PZ, c_size_t, POINTER(c_int), POINTER(c_int), POINTER(c_uint64)],
     "knhip_optimizer_settings_default": [POINTER(OptimizerSettingsT)],
     "knhip_graph_optimize": [G, POINTER(OptimizerSettingsT), POINTER(G)],
-    "knhip_executor_new": [c_int, G, c_size_t, c_int, POINTER(E)],
-    "knhip_executor_new_from_blob": [c_int, POINTER(c_uint8), c_size_t, c_size_t, c_int, POINTER(E)],
+    "knhip_executor_options_default": [POINTER(ExecutorOptionsT)],
+    "knhip_executor_new": [c_int, G, c_size_t, POINTER(ExecutorOptionsT), POINTER(E)],
+    "knhip_executor_new_from_blob": [c_int, POINTER(c_uint8), c_size_t, c_size_t, POINTER(ExecutorOptionsT), POINTER(E)],
     "knhip_executor_io_count": [E, PZ, PZ],
     "knhip_executor_io_info": [E, c_int, c_size_t, POINTER(c_int), PZ, PZ, c_size_t],
     "knhip_executor_evaluate": [E, POINTER(c_void_p), PZ, c_size_t, POINTER(c_void_p), PZ, c_size_t],
@@ -163,6 +186,7 @@ SPECIAL = {
     "knhip_last_error": ([], c_char_p),
     "knhip_graph_free": ([G], None),
     "knhip_executor_free": ([E], None),
+    "knhip_kernel_free": ([c_void_p], None),
 }
 
 

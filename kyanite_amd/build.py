@@ -16,10 +16,10 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HOST_SOURCES = [
     "dtype.cpp", "graph.cpp", "serialize.cpp", "const_eval.cpp", "optimizer.cpp", "strided_shape.cpp",
-    "kernels.cpp", "fused_graph.cpp", "rtc.cpp", "gemm_plan.cpp", "planner.cpp", "executor.cpp", "capi.cpp",
+    "kernels.cpp", "fused_graph.cpp", "rtc.cpp", "gemm_plan.cpp", "planner.cpp", "executor.cpp", "capi.cpp", "standalone.cpp",
 ]
 DEVICE_SOURCES = ["kern/mfma_kernels.hip", "kern/mfma_f16_kernels.hip", "kern/attention_kernels.hip", "kern/attention_f16_kernels.hip",
-                  "kern/static_scratch.hip", "kern/probe_kernels.hip"]
+                  "kern/static_scratch.hip"]
 
 COMMON_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-D__HIP_PLATFORM_AMD__",
                 f"-I{ROCM}/include"]

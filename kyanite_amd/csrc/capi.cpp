@@ -16,8 +16,7 @@ struct knhip_graph {
 };
 struct knhip_executor {
     HipExecutor ex;
-    knhip_executor(int device, const Graph &g, size_t batch, int flags)
-        : ex(device, g, batch, (flags & KNHIP_PLAN_ONLY) != 0, (flags & KNHIP_PRESERVE_INPUTS) != 0, (flags & KNHIP_STEP_BY_STEP) == 0) {}
+    knhip_executor(int device, const Graph &g, size_t batch, const ExecutorOptions &options) : ex(device, g, batch, options) {}
 };
 
 namespace {
@@ -94,17 +93,18 @@ namespace kn {
 
 void set_last_error(const std::string &message) { g_last_error = message; }
 
-GemmLaunchPlan matmul_api_plan(const knhip_matmul_args &a, MatmulWorkspace *ws) {
-    if (a.dtype != KNHIP_F32 && a.dtype != KNHIP_F16) fail("batched_mat_mul: dtype must be f32 or f16, got code ", a.dtype);
-    if (a.batch < 0 || a.m < 0 || a.n < 0 || a.k < 0) fail("batched_mat_mul: negative size");
-    const bool empty = a.batch == 0 || a.m == 0 || a.n == 0;
-    if (!empty && (a.c == nullptr || (a.k > 0 && (a.a == nullptr || a.b == nullptr)))) fail("batched_mat_mul: null operand");
-    if (a.batch > 65535) fail("batched_mat_mul: at most 65535 batch entries per call, got ", a.batch);
+namespace {
+
+// grid.y carries the batch index: at most this many batch entries per launch, longer batches run as several launches
+constexpr int MATMUL_BATCH_SLAB = 65535;
+
+GemmLaunchPlan matmul_plan_slab(const knhip_matmul_args &a, int first, int count, MatmulWorkspace *ws) {
+    const size_t elem = a.dtype == KNHIP_F16 ? 2 : 4;
     GemmParams p{};
-    p.a = a.a;
-    p.b = a.b;
-    p.c = a.c;
-    p.batch = a.batch;
+    p.a = a.a ? (const char *) a.a + (int64_t) first * a.a_batch_stride * (int64_t) elem : nullptr;
+    p.b = a.b ? (const char *) a.b + (int64_t) first * a.b_batch_stride * (int64_t) elem : nullptr;
+    p.c = a.c ? (char *) a.c + (int64_t) first * a.c_batch_stride * (int64_t) elem : nullptr;
+    p.batch = count;
     p.m = a.m;
     p.n = a.n;
     p.k = a.k;
@@ -117,23 +117,48 @@ GemmLaunchPlan matmul_api_plan(const knhip_matmul_args &a, MatmulWorkspace *ws) 
     return lp;
 }
 
-void matmul_api_launch(const knhip_matmul_args &args, void *workspace, size_t workspace_bytes, ihipStream_t *stream) {
-    MatmulWorkspace ws;
-    GemmLaunchPlan lp = matmul_api_plan(args, &ws);
-    if (args.batch == 0 || args.m == 0 || args.n == 0) return;
-    if (ws.total() > 0) {
-        if (workspace == nullptr || workspace_bytes < ws.total())
-            fail("batched_mat_mul: this product needs ", ws.total(), " bytes of workspace, got ", workspace_bytes);
+}  // namespace
+
+MatmulPlan matmul_api_plan(const knhip_matmul_args &a) {
+    if (a.dtype != KNHIP_F32 && a.dtype != KNHIP_F16) fail("batched_mat_mul: dtype must be f32 or f16, got code ", a.dtype);
+    if (a.batch < 0 || a.m < 0 || a.n < 0 || a.k < 0) fail("batched_mat_mul: negative size");
+    const bool empty = a.batch == 0 || a.m == 0 || a.n == 0;
+    if (!empty && (a.c == nullptr || (a.k > 0 && (a.a == nullptr || a.b == nullptr)))) fail("batched_mat_mul: null operand");
+    MatmulPlan plan;
+    plan.f16 = a.dtype == KNHIP_F16;
+    plan.empty = empty;
+    // the slabs run one after the other on the stream and share the workspace, which has room for the largest
+    for (int first = 0; first < a.batch || plan.slabs.empty(); first += MATMUL_BATCH_SLAB) {
+        MatmulWorkspace ws;
+        plan.slabs.push_back(matmul_plan_slab(a, first, std::min(MATMUL_BATCH_SLAB, a.batch - first), &ws));
+        plan.slab_workspaces.push_back(ws);
+        plan.workspace.counter_bytes = std::max(plan.workspace.counter_bytes, ws.counter_bytes);
+        plan.workspace.partial_bytes = std::max(plan.workspace.partial_bytes, ws.partial_bytes);
+        if (a.batch == 0) break;
+    }
+    return plan;
+}
+
+void matmul_api_launch(MatmulPlan &plan, void *workspace, size_t workspace_bytes, ihipStream_t *stream) {
+    if (plan.empty) return;
+    const size_t total = plan.workspace.total();
+    if (total > 0) {
+        if (workspace == nullptr || workspace_bytes < total)
+            fail("batched_mat_mul: this product needs ", total, " bytes of workspace, got ", workspace_bytes);
         if ((uintptr_t) workspace % 256 != 0) fail("batched_mat_mul: the workspace must be 256 byte aligned");
+    }
+    for (size_t i = 0; i < plan.slabs.size(); i++) {
+        GemmLaunchPlan &lp = plan.slabs[i];
+        const MatmulWorkspace &ws = plan.slab_workspaces[i];
         if (ws.counter_bytes > 0) {
             // the tile counters start at zero (a fill kernel, not a memset: the call may be under stream capture)
             hip_check((hipError_t) launch_fill_zero(workspace, ws.counter_bytes, stream), "counter fill launch");
             lp.p.counters = workspace;
         }
-        if (ws.partial_bytes > 0) lp.p.workspace = (char *) workspace + ws.partial_offset();
+        // (the partial products sit behind the room of the largest slab's counters)
+        if (ws.partial_bytes > 0) lp.p.workspace = (char *) workspace + plan.workspace.partial_offset();
+        hip_check((hipError_t) (plan.f16 ? launch_gemm_f16(lp, stream) : launch_gemm_f32(lp, stream)), "matmul launch");
     }
-    const bool f16 = args.dtype == KNHIP_F16;
-    hip_check((hipError_t) (f16 ? launch_gemm_f16(lp, stream) : launch_gemm_f32(lp, stream)), "matmul launch");
 }
 
 }  // namespace kn
@@ -268,9 +293,7 @@ int knhip_event_elapsed_seconds(int device, void *start, void *end, float *secon
 int knhip_batched_mat_mul_workspace_bytes(const knhip_matmul_args *args, size_t *bytes) {
     return guarded([&] {
         KN_REQUIRE(args != nullptr && bytes != nullptr);
-        MatmulWorkspace ws;
-        (void) matmul_api_plan(*args, &ws);
-        *bytes = ws.total();
+        *bytes = matmul_api_plan(*args).workspace.total();
         return KNHIP_OK;
     });
 }
@@ -278,7 +301,8 @@ int knhip_batched_mat_mul_workspace_bytes(const knhip_matmul_args *args, size_t 
 int knhip_batched_mat_mul(int device, void *stream, const knhip_matmul_args *args, void *workspace, size_t workspace_bytes) {
     return on_device(device, [&] {
         KN_REQUIRE(args != nullptr);
-        matmul_api_launch(*args, workspace, workspace_bytes, (ihipStream_t *) stream);
+        MatmulPlan plan = matmul_api_plan(*args);
+        matmul_api_launch(plan, workspace, workspace_bytes, (ihipStream_t *) stream);
     });
 }
 
@@ -657,20 +681,81 @@ int knhip_graph_optimize(const knhip_graph *g, const knhip_optimizer_settings *s
 
 // ---------------------------------------------------------------------------------------------- executor
 
-int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, int flags, knhip_executor **out) {
+int knhip_executor_options_default(knhip_executor_options *o) {
     return guarded([&] {
-        KN_REQUIRE(graph != nullptr && out != nullptr);
-        *out = new knhip_executor(device, graph->graph, batch_size, flags);
+        KN_REQUIRE(o != nullptr);
+        const ExecutorOptions d;
+        std::memset(o, 0, sizeof *o);
+        o->struct_bytes = sizeof *o;
+        o->plan_only = d.plan_only;
+        o->preserve_inputs = d.planner.preserve_inputs;
+        o->step_by_step = !d.fuse_small;
+        o->fuse_attention = d.planner.fuse_attention;
+        o->group_matmuls = d.planner.group_matmuls;
+        o->pack_matmul_constants = d.planner.pack_matmul_constants;
+        o->pointwise_conv_as_matmul = d.planner.pointwise_conv_as_matmul;
+        o->join_elementwise = d.planner.join_elementwise;
+        o->split_reduce = d.planner.split_reduce;
+        o->tiled_transpose = d.planner.generator.tiled_transpose;
+        o->split_conv_channels = d.planner.split_conv_channels;
+        o->plane_conv_any_width = d.planner.plane_conv_any_width;
+        o->direct_gemm = d.planner.gemm.direct;
+        o->split_k = d.planner.gemm.split_k;
+        o->tail_split = d.planner.gemm.tail_split;
+        o->dot_products = d.planner.gemm.dot_products;
+        o->streaming_bytes = d.planner.generator.streaming_bytes;
+        o->mapped_io_bytes = d.mapped_io_bytes;
         return KNHIP_OK;
     });
 }
 
-int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size, int flags,
-                                 knhip_executor **out) {
+namespace {
+
+ExecutorOptions executor_options_from(const knhip_executor_options *o) {
+    ExecutorOptions e;
+    if (o == nullptr) return e;
+    if (o->struct_bytes != sizeof *o)
+        fail("knhip_executor_options.struct_bytes is ", o->struct_bytes, ", this library expects ", sizeof *o,
+             " (fill the struct with knhip_executor_options_default first)");
+    e.plan_only = o->plan_only != 0;
+    e.fuse_small = o->step_by_step == 0;
+    e.mapped_io_bytes = (size_t) o->mapped_io_bytes;
+    PlannerOptions &p = e.planner;
+    p.preserve_inputs = o->preserve_inputs != 0;
+    p.fuse_attention = o->fuse_attention != 0;
+    p.group_matmuls = o->group_matmuls != 0;
+    p.pack_matmul_constants = o->pack_matmul_constants != 0;
+    p.pointwise_conv_as_matmul = o->pointwise_conv_as_matmul != 0;
+    p.join_elementwise = o->join_elementwise != 0;
+    p.split_reduce = o->split_reduce != 0;
+    p.generator.tiled_transpose = o->tiled_transpose != 0;
+    p.generator.streaming_bytes = (size_t) o->streaming_bytes;
+    p.split_conv_channels = o->split_conv_channels != 0;
+    p.plane_conv_any_width = o->plane_conv_any_width != 0;
+    p.gemm.direct = o->direct_gemm != 0;
+    p.gemm.split_k = o->split_k != 0;
+    p.gemm.tail_split = o->tail_split != 0;
+    p.gemm.dot_products = o->dot_products != 0;
+    return e;
+}
+
+}  // namespace
+
+int knhip_executor_new(int device, const knhip_graph *graph, size_t batch_size, const knhip_executor_options *options,
+                       knhip_executor **out) {
+    return guarded([&] {
+        KN_REQUIRE(graph != nullptr && out != nullptr);
+        *out = new knhip_executor(device, graph->graph, batch_size, executor_options_from(options));
+        return KNHIP_OK;
+    });
+}
+
+int knhip_executor_new_from_blob(int device, const uint8_t *blob, size_t len, size_t batch_size,
+                                 const knhip_executor_options *options, knhip_executor **out) {
     return guarded([&] {
         KN_REQUIRE(blob != nullptr && out != nullptr);
         Graph g = Graph::deserialize(blob, len);
-        *out = new knhip_executor(device, g, batch_size, flags);
+        *out = new knhip_executor(device, g, batch_size, executor_options_from(options));
         return KNHIP_OK;
     });
 }

@@ -62,17 +62,11 @@ hipModule_t load_code_object(std::shared_ptr<const CodeObject> &code, const std:
 
 }  // namespace
 
-HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only, bool preserve_inputs, bool fuse_small)
-    : device_(device), batch_size_(batch_size), plan_only_(plan_only) {
+HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, const ExecutorOptions &executor_options)
+    : device_(device), batch_size_(batch_size), plan_only_(executor_options.plan_only) {
+    const bool plan_only = executor_options.plan_only, fuse_small = executor_options.fuse_small;
     if (!plan_only) HipDevice::check(device);
-    PlannerOptions options;
-    options.preserve_inputs = preserve_inputs;
-    if (const char *e = getenv("KNHIP_FUSE_ATTENTION")) options.fuse_attention = atoi(e) != 0;
-    if (const char *e = getenv("KNHIP_GROUP_MATMULS")) options.group_matmuls = atoi(e) != 0;
-    if (const char *e = getenv("KNHIP_PACK_CONSTANTS")) options.pack_matmul_constants = atoi(e) != 0;
-    if (const char *e = getenv("KNHIP_POINTWISE_CONV")) options.pointwise_conv_as_matmul = atoi(e) != 0;
-    if (const char *e = getenv("KNHIP_JOIN_ELEMENTWISE")) options.join_elementwise = atoi(e) != 0;
-    if (const char *e = getenv("KNHIP_SPLIT_REDUCE")) options.split_reduce = atoi(e) != 0;
+    const PlannerOptions &options = executor_options.planner;
     plan_ = plan_graph(graph, batch_size, options);
     for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
     if (fuse_small && plan_.steps.size() > 1) {
@@ -140,7 +134,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     }
 
     // Mapped inputs / outputs for small graphs: every input and output in a shared buffer of its own, a few KB in all
-    static const size_t mapped_limit = getenv("KNHIP_MAPPED_IO_BYTES") ? (size_t) atoll(getenv("KNHIP_MAPPED_IO_BYTES")) : 64 * 1024;
+    const size_t mapped_limit = executor_options.mapped_io_bytes;
     size_t io_bytes = 0;
     bool separate = true;
     std::vector<size_t> seen;
@@ -152,7 +146,7 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, bool
     };
     for (auto &t : plan_.inputs) own_buffer(t);
     for (auto &t : plan_.outputs) own_buffer(t);
-    if (separate && io_bytes <= mapped_limit && !plan_.steps.empty()) {
+    if (separate && mapped_limit > 0 && io_bytes <= mapped_limit && !plan_.steps.empty()) {
         allocate_staging();
         mapped_launches_.resize(plan_.steps.size());
         for (size_t si = 0; si < plan_.steps.size(); si++) {
@@ -451,8 +445,8 @@ const std::vector<HostTensor> &HipExecutor::evaluate(const std::vector<HostTenso
     // That is a bus write away from the end of the kernel, where the runtime's own completion path adds about 6 us.
     bool done = false;
     if (mapped && fused_function_) {
-        volatile uint32_t *flag = fused_done_;
-        for (int spin = 0; spin < 400000 && !done; spin++) done = *flag == fused_seq_;
+        // (an acquire load: the outputs are read from page-locked memory right behind it)
+        for (int spin = 0; spin < 400000 && !done; spin++) done = __atomic_load_n(fused_done_, __ATOMIC_ACQUIRE) == fused_seq_;
     }
     if (!done) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
     for (size_t i = 0; i < plan_.outputs.size(); i++) {

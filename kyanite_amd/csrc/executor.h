@@ -25,14 +25,22 @@ public:
     static std::string name(int device);
 };
 
+// What an executor is built with beyond (device, graph, batch size); the defaults are the reference's behaviour plus
+// every planned path of this library switched on. One executor's options do not touch another's.
+struct ExecutorOptions {
+    bool plan_only = false;   // build and compile the plan without touching a device (no allocation, no launches)
+    bool fuse_small = true;   // a plan of a few tiny steps is launched as one kernel (fused_graph.h)
+    // `evaluate` of a graph whose inputs and outputs are at most this many bytes in all reads and writes them in
+    // page-locked host memory instead of copying them to and from the arena (0: never)
+    size_t mapped_io_bytes = 64 * 1024;
+    // (`planner.preserve_inputs` keeps the input buffers from being reused for later values, for callers that write
+    // the inputs on the device once and then call run_async many times)
+    PlannerOptions planner;
+};
+
 class HipExecutor {
 public:
-    // `plan_only` builds and compiles the plan without touching a device (no allocation, no launches)
-    // `preserve_inputs` keeps the input buffers from being reused for later values, for callers that write the
-    // inputs on the device once and then call run_async many times
-    // `fuse_small`: a plan of a few tiny steps is launched as one kernel (fused_graph.h)
-    HipExecutor(int device, const Graph &graph, size_t batch_size, bool plan_only = false, bool preserve_inputs = false,
-                bool fuse_small = true);
+    HipExecutor(int device, const Graph &graph, size_t batch_size, const ExecutorOptions &options = ExecutorOptions());
     ~HipExecutor();
     HipExecutor(const HipExecutor &) = delete;
     HipExecutor &operator=(const HipExecutor &) = delete;

@@ -103,7 +103,13 @@ std::optional<KernelSpec> make_fused_graph_kernel(const std::vector<FusedPart> &
         if (grid > 0) {
             ss << "    {\n        kn_s" << i << "::KnPtrs q;\n";
             for (size_t k = 0; k < n; k++) ss << "        q.p[" << k << "] = all.p[" << offset + k << "];\n";
-            ss << "        for (unsigned b = 0; b < " << grid << "u; b++) kn_s" << i << "::kn_step(q, b);\n    }\n";
+            // A step body is written for a fresh workgroup: its LDS arrays are used once, behind one barrier. When one
+            // workgroup plays several, a fast wave must not write the arrays for workgroup b + 1 while a slow one
+            // still reads what workgroup b left there: a barrier between the turns.
+            if (grid > 1)
+                ss << "        for (unsigned b = 0; b < " << grid << "u; b++) {\n            kn_s" << i << "::kn_step(q, b);\n            __syncthreads();\n        }\n    }\n";
+            else
+                ss << "        kn_s" << i << "::kn_step(q, 0u);\n    }\n";
             if (i + 1 < parts.size()) ss << "    __syncthreads();\n";
         }
         offset += n;

@@ -11,11 +11,6 @@ namespace kn {
 
 namespace {
 
-int env_int(const char *name, int fallback) {
-    const char *env = getenv(name);
-    return env && *env ? atoi(env) : fallback;
-}
-
 // ---- Cost model of the f16 kernel that loads global -> LDS directly.
 //
 // What a compute unit can do per slice of 64 along K is bounded by the 128 byte lines it can request - it keeps
@@ -113,7 +108,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // A product this small is a chain of memory round trips whichever way it is tiled, and a 64 x 64 tile spends its
     // MFMAs on rows and columns that do not exist (the value head's 1 x 1 x 256 took 15.7 us, the 32 x 64 x 128 of a
     // 1 x 1 convolution on one board 12.1 us): one wave per result instead, lanes along K.
-    static const int dot_enabled = env_int("KNHIP_DOT_PRODUCTS", 1);
+    const bool dot_enabled = p.tuning.dot_products;
     if (dot_enabled && p.groups <= 1 && p.k > 0 && (long long) p.batch * p.m * p.n * p.k <= (1ll << 20) && (long long) p.batch * p.m * p.n <= 16384) {
         lp.dot = true;
         lp.small_tile = true;
@@ -126,7 +121,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // 128 tiles 47 us against 56 us. An output no wider than 64 would leave most of a 128 wide tile unused
     // (16 x [4096 x 4096] x [4096 x 40] in f32: 450 us on 64 x 64 tiles against 682 us).
     const long long threshold = f16 ? 256 : 512;
-    static const int split_enabled = env_int("KNHIP_SPLIT_K", 1);
+    const bool split_enabled = p.tuning.split_k;
     const int groups = p.groups > 1 ? p.groups : 1;
     const long long big_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch * groups;
     const bool narrow = p.m <= 64 || p.n <= 64;
@@ -155,7 +150,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     const int vec = f16 ? 8 : 4;
     // (row strides: positive and small enough for the 32 bit byte offsets that the kernel keeps per lane within a tile)
     constexpr long long max_row_stride = 1ll << 21;
-    lp.direct = p.k > 0 && p.k % (8 * vec) == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % vec == 0 && p.b_sn % vec == 0 &&
+    lp.direct = p.tuning.direct && p.k > 0 && p.k % (8 * vec) == 0 && p.a_sk == 1 && p.b_sk == 1 && p.a_sm % vec == 0 && p.b_sn % vec == 0 &&
                 p.a_sm > 0 && p.b_sn > 0 && p.a_sm < max_row_stride && p.b_sn < max_row_stride &&
                 (p.batch <= 1 || (p.a_sb % vec == 0 && p.b_sb % vec == 0));
     const long long narrow_blocks = (long long) ((p.m + 127) / 128) * ((p.n + 63) / 64) * p.batch * groups;
@@ -167,7 +162,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // 256 x 128 with K in four parts for down, 128 x 64 for o - what sweeps over those shapes had arrived at before -
     // and on shapes nobody swept it is what the thresholds it replaces were not: 256 x 4096 x 4096 22 us instead of
     // 30 us, 512 x 512 x 4096 13 / 20, 768 x 768 x 3072 16 / 20, 8192 x 320 x 1280 20 / 25, 512 x 32000 x 4096 166 / 187.
-    static const int tail_enabled = env_int("KNHIP_TAIL_SPLIT", 1);
+    const bool tail_enabled = p.tuning.tail_split;
     int model_split = 0;
     if (f16 && lp.direct) {
         int best_tile = TILE_SMALL, best_split = 1;

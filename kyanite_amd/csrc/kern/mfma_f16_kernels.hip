@@ -624,8 +624,7 @@ void launch_a(int a_mode, int b_mode, dim3 grid, hipStream_t stream, const GemmP
 int launch_gemm_f32_direct(const GemmLaunchPlan &lp, ihipStream_t *stream, bool *launched) {
     *launched = false;
     const GemmParams &p = lp.p;
-    static const int direct_env = getenv("KNHIP_F32_DIRECT") ? atoi(getenv("KNHIP_F32_DIRECT")) : 1;
-    if (!direct_env || !lp.direct || lp.k_chunk % 32 != 0) return 0;
+    if (!lp.direct || lp.k_chunk % 32 != 0) return 0;
     const int groups = p.groups > 1 ? p.groups : 1;
     bool aligned = (uintptr_t) p.a % 16 == 0;
     for (int g = 0; g < groups; g++) aligned = aligned && (uintptr_t) (groups > 1 ? p.b_group[g] : p.b) % 16 == 0;
@@ -667,8 +666,7 @@ int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
         if (mode != b_mode) b_mode = Scalar;
     }
     // both operands K contiguous and K (and every split of it) whole slices: the direct-to-LDS kernel
-    static const int direct_env = getenv("KNHIP_F16_DIRECT") ? atoi(getenv("KNHIP_F16_DIRECT")) : 1;
-    const bool direct = direct_env && lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % 64 == 0;
+    const bool direct = lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % 64 == 0;
     // (128 x 64 tiles exist in the direct kernel only; without it they run as 64 x 64)
     // (so do 256 x 256 and 256 x 192 tiles, which otherwise run as 256 x 128)
     const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct);

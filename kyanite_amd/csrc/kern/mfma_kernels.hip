@@ -876,13 +876,7 @@ void launch_conv_t(int a_mode, dim3 grid, hipStream_t stream, const ConvParams &
 }
 
 // convolutions: 128 x 128 tiles unless there are too few of them to give every compute unit two workgroups
-int small_tile_threshold() {
-    static const int value = [] {
-        const char *env = getenv("KNHIP_SMALL_TILE_BELOW");
-        return env ? atoi(env) : 512;
-    }();
-    return value;
-}
+int small_tile_threshold() { return 512; }
 
 }  // namespace
 
@@ -1004,10 +998,7 @@ __global__ __launch_bounds__(256) void conv_reduce_partials_kernel(ConvParams p)
 }
 
 int conv_channel_split(const ConvParams &p) {
-    static const bool enabled = [] {
-        const char *env = getenv("KNHIP_SPLIT_CONV");
-        return !env || atoi(env) != 0;
-    }();
+    const bool enabled = p.channel_split;
     const long long positions = (long long) p.batch * p.out_h * p.out_w;
     if (!enabled || positions <= 0 || p.out_c <= 0) return 1;
     // 64 x 64 tiles of four waves each, on 1024 SIMDs. The plane kernel keeps a SIMD busy with one wave, so it splits
@@ -1072,7 +1063,7 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
     static const Variant variants[2] = {{128, 128, 22, 4 * 1.00}, {64, 64, 11, 1 * 1.10}};
     const Variant *best = nullptr;
     double best_cost = 0.0;
-    static const bool any_enabled = !(getenv("KNHIP_PLANE_ANY") && atoi(getenv("KNHIP_PLANE_ANY")) == 0);
+    const bool any_enabled = p.plane_any_width;
     bool any_w = false;
     for (const Variant &v : variants) {
         if (split && v.id != 11) continue;  // (few tiles: the small one)

@@ -37,18 +37,35 @@ void *scratch_of_current_device(int device) {
 
 }  // namespace
 
+// The address lookup is no stream operation and may be refused while a stream capture is open: a caller that will
+// capture resolves it ahead of time with this call (any earlier knhip_batched_mat_mul_static on the device does too).
+extern "C" int knhip_static_scratch_prepare(int device) {
+    try {
+        kn::HipDevice::check(device);
+        kn::hip_check(hipSetDevice(device), "hipSetDevice");
+        (void) scratch_of_current_device(device);
+        return KNHIP_OK;
+    } catch (const std::exception &e) {
+        kn::set_last_error(e.what());
+        return KNHIP_ERROR;
+    } catch (...) {
+        kn::set_last_error("unknown failure");
+        return KNHIP_ERROR;
+    }
+}
+
 extern "C" int knhip_batched_mat_mul_static(int device, void *stream, const knhip_matmul_args *args) {
     try {
         if (args == nullptr) kn::fail("invalid argument: args is null");
         kn::HipDevice::check(device);
         kn::hip_check(hipSetDevice(device), "hipSetDevice");
-        kn::MatmulWorkspace ws;
-        (void) kn::matmul_api_plan(*args, &ws);
-        if (ws.total() > (size_t) KNHIP_STATIC_SCRATCH_BYTES)
-            kn::fail("batched_mat_mul_static: this product needs ", ws.total(), " bytes of scratch, the static scratch holds ",
+        kn::MatmulPlan plan = kn::matmul_api_plan(*args);
+        const size_t total = plan.workspace.total();
+        if (total > (size_t) KNHIP_STATIC_SCRATCH_BYTES)
+            kn::fail("batched_mat_mul_static: this product needs ", total, " bytes of scratch, the static scratch holds ",
                      (size_t) KNHIP_STATIC_SCRATCH_BYTES, "; use knhip_batched_mat_mul with a workspace of the caller's");
         void *ptr = scratch_of_current_device(device);
-        kn::matmul_api_launch(*args, ws.total() > 0 ? ptr : nullptr, ws.total() > 0 ? (size_t) KNHIP_STATIC_SCRATCH_BYTES : 0,
+        kn::matmul_api_launch(plan, total > 0 ? ptr : nullptr, total > 0 ? (size_t) KNHIP_STATIC_SCRATCH_BYTES : 0,
                               (ihipStream_t *) stream);
         return KNHIP_OK;
     } catch (const std::exception &e) {

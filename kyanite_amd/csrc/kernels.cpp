@@ -6,6 +6,18 @@
 
 namespace kn {
 
+namespace {
+thread_local const GeneratorOptions *g_generator_options = nullptr;
+const GeneratorOptions g_default_generator_options{};
+}  // namespace
+
+GeneratorScope::GeneratorScope(const GeneratorOptions &options) : previous_(g_generator_options), mine_(options) {
+    g_generator_options = &mine_;
+}
+GeneratorScope::~GeneratorScope() { g_generator_options = previous_; }
+const GeneratorOptions &generator_options() { return g_generator_options ? *g_generator_options : g_default_generator_options; }
+
+
 // ------------------------------------------------------------------------------------------------ prelude
 
 const char *kernel_prelude() {
@@ -341,9 +353,24 @@ std::string emit_expr(std::ostringstream &ss, const ScalarExpr &expr, const std:
                     rhs = binary_expr(n.binary, expr.nodes[n.a].dtype, prefix + std::to_string(n.a), prefix + std::to_string(n.b));
                 break;
             }
+            case ScalarNode::Raw: {
+                // the caller's statements in a block of their own, with x0 pointing at the result and xk at loaded operand k
+                KN_ASSERT(i + 1 == expr.nodes.size(), "a raw operation is the last node of its expression");
+                ss << indent << compute_type(n.dtype) << " " << name << "_v = " << compute_type(n.dtype) << "();\n" << indent << "{\n";
+                ss << indent << "    " << compute_type(n.dtype) << " *const x0 = &" << name << "_v;\n";
+                for (size_t j = 0; j < i; j++) {
+                    const ScalarNode &in = expr.nodes[j];
+                    if (in.kind != ScalarNode::Load) continue;
+                    ss << indent << "    const " << compute_type(in.dtype) << " *const x" << in.operand << " = &" << prefix << j << ";\n";
+                    ss << indent << "    (void) x" << in.operand << ";\n";
+                }
+                ss << indent << "    " << n.raw << "\n" << indent << "}\n";
+                rhs = name + "_v";
+                break;
+            }
         }
         // values of type f16 are kept as floats that are exactly representable in f16
-        if (n.dtype == DType::F16 && (n.kind == ScalarNode::Unary || n.kind == ScalarNode::Binary)) rhs = "kn_r16(" + rhs + ")";
+        if (n.dtype == DType::F16 && (n.kind == ScalarNode::Unary || n.kind == ScalarNode::Binary || n.kind == ScalarNode::Raw)) rhs = "kn_r16(" + rhs + ")";
         ss << indent << "const " << compute_type(n.dtype) << " " << name << " = " << rhs << ";\n";
     }
     return prefix + std::to_string(expr.result());
@@ -419,17 +446,10 @@ void emit_decompose(std::ostringstream &ss, const std::string &indent, const std
 
 // Streaming heuristics: a big tensor that is touched exactly once per element gains nothing from the caches, and
 // its dirty lines would only delay whatever runs next. Such operands are read and written with non-temporal
-// accesses. The threshold can be overridden with KNHIP_NT_BYTES (0 switches the hint off).
+// accesses (GeneratorOptions::streaming_bytes).
 size_t nt_threshold_bytes() {
-    static const size_t value = [] {
-        const char *env = getenv("KNHIP_NT_BYTES");
-        if (env && *env) {
-            unsigned long long v = strtoull(env, nullptr, 10);
-            return v == 0 ? SIZE_MAX : (size_t) v;
-        }
-        return (size_t) 64 << 20;
-    }();
-    return value;
+    const size_t v = generator_options().streaming_bytes;
+    return v == 0 ? SIZE_MAX : v;
 }
 
 bool is_streaming(const KernelOperand &op) {
@@ -508,10 +528,7 @@ namespace {
 // directions are free of bank conflicts.
 std::optional<KernelSpec> make_transposed_tile_kernel(const std::vector<KernelOperand> &operands, const std::vector<ScalarExpr> &exprs,
                                                       const Collapsed &c, size_t total) {
-    static const bool enabled = [] {
-        const char *env = getenv("KNHIP_TILED_TRANSPOSE");
-        return !(env && *env == '0');
-    }();
+    const bool enabled = generator_options().tiled_transpose;
     const size_t n_out = exprs.size(), n_ops = operands.size(), rank = c.rank();
     if (!enabled || rank < 2 || total < (1u << 16)) return std::nullopt;
     const size_t last = rank - 1;

@@ -9,6 +9,29 @@
 
 namespace kn {
 
+// Choices of the generators that a caller may move; the generators of a thread read the options of the innermost
+// GeneratorScope alive on it (the defaults when there is none).
+struct GeneratorOptions {
+    // operands of at least this many bytes that are touched once per element are read and written with non-temporal
+    // accesses (0: never)
+    size_t streaming_bytes = (size_t) 64 << 20;
+    // elementwise kernels with an operand that is contiguous along another axis than the outputs turn 64 x 64 tiles
+    // through LDS (off: the plain kernel with strided accesses)
+    bool tiled_transpose = true;
+};
+class GeneratorScope {
+public:
+    explicit GeneratorScope(const GeneratorOptions &options);
+    ~GeneratorScope();
+    GeneratorScope(const GeneratorScope &) = delete;
+    GeneratorScope &operator=(const GeneratorScope &) = delete;
+
+private:
+    const GeneratorOptions *previous_;
+    GeneratorOptions mine_;
+};
+const GeneratorOptions &generator_options();
+
 // A kernel ready to be compiled: every shape, stride and expression is baked into `source`; the only launch
 // arguments are the operand base addresses, in `operands` order.
 struct KernelSpec {
@@ -22,8 +45,11 @@ struct KernelSpec {
 
 // One node of a fused elementwise expression: operands are loaded (`Load`), single-valued constants are inlined
 // (`Const`), everything else refers to earlier nodes.
+// `Raw`: statements in the form the reference writes its operations in, "*x0 = *x1 + *x2;" (autokernel/scalar.rs:36):
+// x0 points at the result, xk at the loaded operand k, each in its register type (f16 as float, bool as bool).
+// A Raw node is the last node of its expression and follows one Load node per operand it may read.
 struct ScalarNode {
-    enum Kind { Load, Const, Unary, Binary } kind = Load;
+    enum Kind { Load, Const, Unary, Binary, Raw } kind = Load;
     DType dtype = DType::F32;  // type of the produced value
     size_t operand = 0;        // Load: index into the operand list
     DScalar constant;          // Const
@@ -31,6 +57,7 @@ struct ScalarNode {
     DType cast_to = DType::F32;
     BinaryOp binary = BinaryOp::Add;
     size_t a = 0, b = 0;  // argument node indices
+    std::string raw;      // Raw: the statements
 };
 
 // An expression DAG in evaluation order, the last node being the result.

@@ -15,6 +15,15 @@ namespace kn {
 // The element type (float or _Float16, the same for all three matrices) is fixed by the launch function.
 constexpr int GEMM_MAX_GROUPS = 4;
 
+// Launch paths a caller may switch off (all on by default); part of the parameters, so that the plan made ahead of
+// time and the launch see the same choice.
+struct GemmTuning {
+    bool direct = true;        // the kernels that load global -> LDS directly (off: every product stages through registers)
+    bool split_k = true;       // workgroups that share a tile along K, of either kind
+    bool tail_split = true;    // the split of just the last, sparse round of tiles inside one launch
+    bool dot_products = true;  // one wave per result for products of up to 2^20 multiplications
+};
+
 struct GemmParams {
     const void *a;
     const void *b;
@@ -45,6 +54,7 @@ struct GemmParams {
     // zero-filled ints that the launch hands back zero-filled (`GemmLaunchPlan::counter_bytes` bytes) when tiles
     // are shared between workgroups; may be null otherwise
     void *counters = nullptr;
+    GemmTuning tuning;
 };
 
 // How a matrix multiply is launched; a pure function of the shapes, strides and alignments, so the planner can ask
@@ -97,6 +107,9 @@ struct ConvParams {
     float *workspace = nullptr;
     // filled in by the launch: slices of the input channels that are folded side by side, and channels per slice
     int splits = 1, split_channels = 0;
+    // launch paths a caller may switch off
+    bool channel_split = true;    // slices of the input channels folded side by side when the tiles are few
+    bool plane_any_width = true;  // the plane kernel for 3 x 3 convolutions on images without a power-of-two width
 };
 
 // A convolution with few output tiles and many input channels (small batches of small boards) leaves most of the chip

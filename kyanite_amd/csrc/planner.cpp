@@ -1128,6 +1128,7 @@ private:
         step.kind = StepKind::MatMul;
         step.gemm_f16 = dt == DType::F16;
         GemmParams &g = step.gemm;
+            g.tuning = options.gemm;
         g.batch = (int) b; g.m = (int) m; g.n = (int) n; g.k = (int) k;
         g.a_sb = l.shape.strides()[0]; g.a_sm = l.shape.strides()[1]; g.a_sk = l.shape.strides()[2];
         g.b_sb = r0.shape.strides()[0]; g.b_sk = r0.shape.strides()[1]; g.b_sn = r0.shape.strides()[2];
@@ -1260,6 +1261,7 @@ private:
             step.kind = StepKind::MatMul;
             step.gemm_f16 = dt == DType::F16;
             GemmParams &g = step.gemm;
+            g.tuning = options.gemm;
             g.batch = (int) b; g.m = (int) m; g.n = (int) n; g.k = (int) k;
             g.a_sb = left.shape.strides()[0]; g.a_sm = left.shape.strides()[1]; g.a_sk = left.shape.strides()[2];
             g.b_sb = right.shape.strides()[0]; g.b_sk = right.shape.strides()[1]; g.b_sn = right.shape.strides()[2];
@@ -1365,6 +1367,7 @@ private:
             Step step;
             step.kind = StepKind::MatMul;
             GemmParams &g = step.gemm;
+            g.tuning = options.gemm;
             g.batch = (int) out_shape[0]; g.m = (int) cout; g.n = (int) hw; g.k = (int) cin;
             g.a_sb = 0; g.a_sm = cin; g.a_sk = 1;
             g.b_sb = cin * hw; g.b_sk = hw; g.b_sn = 1;
@@ -1392,6 +1395,8 @@ private:
             Step step;
             step.kind = StepKind::Conv;
             ConvParams &p = step.conv;
+            p.channel_split = options.split_conv_channels;
+            p.plane_any_width = options.plane_conv_any_width;
             KN_ASSERT(out_shape[0] <= INT32_MAX);
             p.batch = (int) out_shape[0];
             p.in_c = (int) d.input_channels; p.in_h = (int) d.input_h; p.in_w = (int) d.input_w;
@@ -1656,6 +1661,7 @@ size_t align_up(size_t v) { return (v + ARENA_ALIGN - 1) / ARENA_ALIGN * ARENA_A
 }  // namespace
 
 Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &options) {
+    GeneratorScope generator_scope(options.generator);
     Planner planner(graph, batch_size, options);
     Plan plan;
 

@@ -99,6 +99,10 @@ struct PlannerOptions {
     bool split_reduce = true;  // a reduction with few results and a long reduced index runs as two launches
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
+    GemmTuning gemm;                   // launch paths of the matmul kernels
+    bool split_conv_channels = true;   // convolutions with few tiles fold slices of their input channels side by side
+    bool plane_conv_any_width = true;  // 3 x 3 convolutions on images without a power-of-two width on the plane kernel
+    GeneratorOptions generator;        // what the generated kernels may use (streaming accesses, transposing tiles)
 };
 
 Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &options);

@@ -5,7 +5,7 @@ from ctypes import byref, c_double, c_float, c_int, c_size_t, c_void_p
 
 import numpy as np
 
-from ._lib import KnError, MemUsageT, ProfileT, check, get_string, lib
+from ._lib import ExecutorOptionsT, KnError, MemUsageT, ProfileT, check, get_string, lib
 from .graph import DType, Graph
 
 STEP_KINDS = ["conv", "mat_mul", "scalar_op", "reduce_op", "softmax_op", "layernorm_op", "gather_op"]
@@ -51,14 +51,28 @@ class Profile:
         return self.text
 
 
+def executor_options(**fields):
+    """A `knhip_executor_options` struct with the library's defaults and the given fields changed."""
+    opts = ExecutorOptionsT()
+    check(lib.knhip_executor_options_default(byref(opts)))
+    known = {name for name, _ in ExecutorOptionsT._fields_} - {"struct_bytes"}
+    for name, value in fields.items():
+        if name not in known:
+            raise KnError(f"unknown executor option {name!r}; known: {sorted(known)}")
+        setattr(opts, name, int(value))
+    return opts
+
+
 class HipExecutor:
     """`HipExecutor(device, graph, batch_size)` / `evaluate(inputs) -> outputs`."""
 
-    def __init__(self, device, graph, batch_size, plan_only=False, preserve_inputs=False, step_by_step=False):
+    def __init__(self, device, graph, batch_size, plan_only=False, preserve_inputs=False, step_by_step=False, **options):
+        """`options`: any further field of `knhip_executor_options` (include/knhip.h), e.g. `fuse_attention=False`,
+        `mapped_io_bytes=0`; what is not named keeps its default. The options belong to this executor alone."""
         index = device.index if isinstance(device, HipDevice) else int(device)
         h = c_void_p()
-        flags = (1 if plan_only else 0) | (2 if preserve_inputs else 0) | (4 if step_by_step else 0)
-        check(lib.knhip_executor_new(index, graph._h, batch_size, flags, byref(h)))
+        opts = executor_options(plan_only=plan_only, preserve_inputs=preserve_inputs, step_by_step=step_by_step, **options)
+        check(lib.knhip_executor_new(index, graph._h, batch_size, byref(opts), byref(h)))
         self._h = h
         self.device = index
         self.batch_size = batch_size

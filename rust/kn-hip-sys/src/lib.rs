@@ -58,17 +58,56 @@ pub struct knhip_matmul_args {
     pub c_col_stride: i64,
 }
 
+/// What an executor is built with beyond (device, graph, batch size); fill it with `knhip_executor_options_default`.
+#[repr(C)]
+#[derive(Debug, Copy, Clone)]
+pub struct knhip_executor_options {
+    pub struct_bytes: usize,
+    pub plan_only: c_int,
+    pub preserve_inputs: c_int,
+    pub step_by_step: c_int,
+    pub fuse_attention: c_int,
+    pub group_matmuls: c_int,
+    pub pack_matmul_constants: c_int,
+    pub pointwise_conv_as_matmul: c_int,
+    pub join_elementwise: c_int,
+    pub split_reduce: c_int,
+    pub tiled_transpose: c_int,
+    pub split_conv_channels: c_int,
+    pub plane_conv_any_width: c_int,
+    pub direct_gemm: c_int,
+    pub split_k: c_int,
+    pub tail_split: c_int,
+    pub dot_products: c_int,
+    pub streaming_bytes: u64,
+    pub mapped_io_bytes: u64,
+}
+
+/// A strided tensor in device memory that the caller owns (`DeviceTensor`); strides in elements.
+#[repr(C)]
+#[derive(Debug, Copy, Clone)]
+pub struct knhip_tensor {
+    pub ptr: *mut c_void,
+    pub dtype: c_int,
+    pub rank: usize,
+    pub shape: *const usize,
+    pub strides: *const i64,
+}
+
+#[repr(C)]
+pub struct knhip_kernel {
+    _private: [u8; 0],
+}
+
 pub const KNHIP_OK: c_int = 0;
 pub const KNHIP_ERROR: c_int = 1;
 pub const KNHIP_BUFFER_TOO_SMALL: c_int = 2;
 
-pub const KNHIP_PLAN_ONLY: c_int = 1;
-pub const KNHIP_PRESERVE_INPUTS: c_int = 2;
-pub const KNHIP_STEP_BY_STEP: c_int = 4;
-
-pub const KNHIP_PROBE_NORMAL: c_int = 1;
-pub const KNHIP_PROBE_F32: c_int = 2;
-pub const KNHIP_PROBE_RECTIFIED: c_int = 4;
+pub const KNHIP_REDUCE_SUM: c_int = 0;
+pub const KNHIP_REDUCE_MEAN: c_int = 1;
+pub const KNHIP_REDUCE_PROD: c_int = 2;
+pub const KNHIP_REDUCE_MAX: c_int = 3;
+pub const KNHIP_REDUCE_MIN: c_int = 4;
 
 pub const KNHIP_F32: c_int = 0;
 pub const KNHIP_F64: c_int = 1;
@@ -99,7 +138,6 @@ extern "C" {
     pub fn knhip_host_alloc(bytes: usize, ptr: *mut *mut c_void) -> c_int;
     pub fn knhip_host_free(ptr: *mut c_void) -> c_int;
     pub fn knhip_device_synchronize(device: c_int) -> c_int;
-    pub fn knhip_device_mfma_probe(device: c_int, mode: c_int, iterations: c_int, tflops: *mut f64, shader_mhz: *mut f64) -> c_int;
 
     // streams, events, asynchronous copies
     pub fn knhip_stream_create(device: c_int, stream: *mut *mut c_void) -> c_int;
@@ -120,10 +158,36 @@ extern "C" {
     pub fn knhip_batched_mat_mul(device: c_int, stream: *mut c_void, args: *const knhip_matmul_args, workspace: *mut c_void,
                                  workspace_bytes: usize) -> c_int;
     pub fn knhip_batched_mat_mul_static(device: c_int, stream: *mut c_void, args: *const knhip_matmul_args) -> c_int;
+    pub fn knhip_static_scratch_prepare(device: c_int) -> c_int;
+
+    // device tensors and stand-alone kernels
+    pub fn knhip_strided_copy(device: c_int, stream: *mut c_void, dst: *const knhip_tensor, src: *const knhip_tensor) -> c_int;
+    pub fn knhip_scalar_kernel_new(device: c_int, operation: *const c_char, operands: *const knhip_tensor, operand_count: usize,
+                                   out: *mut *mut knhip_kernel) -> c_int;
+    pub fn knhip_reduce_kernel_new(device: c_int, reduce_op: c_int, input: *const knhip_tensor, output: *const knhip_tensor,
+                                   axes: *const usize, axis_count: usize, out: *mut *mut knhip_kernel) -> c_int;
+    pub fn knhip_softmax_kernel_new(device: c_int, input: *const knhip_tensor, output: *const knhip_tensor, axis: usize,
+                                    input_scale: f32, out: *mut *mut knhip_kernel) -> c_int;
+    pub fn knhip_layernorm_kernel_new(device: c_int, input: *const knhip_tensor, output: *const knhip_tensor, axis: usize, eps: f32,
+                                      alpha0: f32, alpha1: f32, beta: f32, out: *mut *mut knhip_kernel) -> c_int;
+    pub fn knhip_gather_kernel_new(device: c_int, input: *const knhip_tensor, indices: *const knhip_tensor,
+                                   output: *const knhip_tensor, axis: usize, out: *mut *mut knhip_kernel) -> c_int;
+    pub fn knhip_kernel_run(kernel: *const knhip_kernel, stream: *mut c_void, ptrs: *const *mut c_void, count: usize) -> c_int;
+    pub fn knhip_kernel_info(kernel: *const knhip_kernel, strategy: *mut c_char, cap: usize, needed: *mut usize, grid: *mut u32,
+                             block: *mut u32) -> c_int;
+    pub fn knhip_kernel_free(kernel: *mut knhip_kernel);
+
+    // layout algebra (kn-cuda-eval/src/shape.rs:25-285), computed by the library
+    pub fn knhip_strided_flags(shape: *const usize, strides: *const i64, rank: usize, simple: *mut c_int, dense: *mut c_int) -> c_int;
+    pub fn knhip_strided_view(shape: *const usize, strides: *const i64, rank: usize, new_shape: *const usize, new_rank: usize,
+                              ok: *mut c_int, new_strides: *mut i64) -> c_int;
+    pub fn knhip_strided_slice(shape: *const usize, strides: *const i64, rank: usize, axis: usize, start: usize, end: usize,
+                               step: usize, out_shape: *mut usize, out_strides: *mut i64) -> c_int;
 
     // executor
-    pub fn knhip_executor_new_from_blob(device: c_int, blob: *const u8, len: usize, batch_size: usize, flags: c_int,
-                                        out: *mut *mut knhip_executor) -> c_int;
+    pub fn knhip_executor_options_default(options: *mut knhip_executor_options) -> c_int;
+    pub fn knhip_executor_new_from_blob(device: c_int, blob: *const u8, len: usize, batch_size: usize,
+                                        options: *const knhip_executor_options, out: *mut *mut knhip_executor) -> c_int;
     pub fn knhip_executor_free(ex: *mut knhip_executor);
     pub fn knhip_executor_io_count(ex: *const knhip_executor, inputs: *mut usize, outputs: *mut usize) -> c_int;
     pub fn knhip_executor_io_info(ex: *const knhip_executor, is_output: c_int, index: usize, dtype: *mut c_int, rank: *mut usize,

@@ -224,12 +224,14 @@ impl Drop for PinnedMem {
     }
 }
 
-/// mem/device.rs:18-46: one allocation, freed when the last pointer into it is dropped.
+/// mem/device.rs:18-46: one allocation, freed when the last pointer into it is dropped. A buffer that somebody else
+/// owns (the arena of an executor) is only described, never freed.
 #[derive(Debug)]
 struct DeviceBuffer {
     device: HipDevice,
     base: *mut c_void,
     len_bytes: usize,
+    owned: bool,
 }
 
 unsafe impl Send for DeviceBuffer {}
@@ -237,7 +239,9 @@ unsafe impl Sync for DeviceBuffer {}
 
 impl Drop for DeviceBuffer {
     fn drop(&mut self) {
-        unsafe { knhip_free(self.device.inner(), self.base) }.unwrap_in_drop()
+        if self.owned {
+            unsafe { knhip_free(self.device.inner(), self.base) }.unwrap_in_drop()
+        }
     }
 }
 
@@ -252,7 +256,13 @@ impl DevicePtr {
     pub fn alloc(device: HipDevice, len_bytes: usize) -> Self {
         let mut base = null_mut();
         unsafe { knhip_malloc(device.inner(), len_bytes.max(1), &mut base) }.unwrap();
-        DevicePtr { buffer: Arc::new(DeviceBuffer { device, base, len_bytes }), offset_bytes: 0 }
+        DevicePtr { buffer: Arc::new(DeviceBuffer { device, base, len_bytes, owned: true }), offset_bytes: 0 }
+    }
+
+    /// `len_bytes` of device memory at `base` that is owned elsewhere (an executor's input or output tensor).
+    /// Safety: the memory outlives every pointer made from the result.
+    pub unsafe fn borrowed(device: HipDevice, base: *mut c_void, len_bytes: usize) -> Self {
+        DevicePtr { buffer: Arc::new(DeviceBuffer { device, base, len_bytes, owned: false }), offset_bytes: 0 }
     }
 
     pub fn device(&self) -> HipDevice {
@@ -300,6 +310,35 @@ impl DevicePtr {
         assert!(len_bytes <= self.room() && len_bytes <= buffer.len_bytes());
         knhip_memcpy_d2h_async(self.device().inner(), buffer.ptr(), self.ptr(), len_bytes, stream.inner()).unwrap()
     }
+}
+
+/// `knhip_executor_options` with the library's defaults; change fields before building an executor. The options
+/// belong to that executor alone: nothing is read from the environment.
+#[derive(Debug, Copy, Clone)]
+pub struct ExecutorOptions(pub knhip_executor_options);
+
+impl Default for ExecutorOptions {
+    fn default() -> Self {
+        let mut raw = std::mem::MaybeUninit::<knhip_executor_options>::zeroed();
+        unsafe {
+            knhip_executor_options_default(raw.as_mut_ptr()).unwrap();
+            ExecutorOptions(raw.assume_init())
+        }
+    }
+}
+
+impl ExecutorOptions {
+    /// for callers that write the device inputs once and call `run_async` many times
+    pub fn preserve_inputs(mut self) -> Self {
+        self.0.preserve_inputs = 1;
+        self
+    }
+}
+
+/// Resolves the address of the static scratch of `knhip_batched_mat_mul_static` on `device`; call it once before a
+/// stream capture that will contain `run_static`.
+pub fn static_scratch_prepare(device: HipDevice) {
+    unsafe { knhip_static_scratch_prepare(device.inner()) }.unwrap()
 }
 
 /// One matrix of a batched product: group.rs:87-105 (`MatMulOperand`), with element strides spelled out

@@ -2273,3 +2273,19 @@ def special_values_on_the_split_paths():
     long_cols[::2, 21] = -np.inf
     g.output(g.softmax(g.input([1000, 50]), 0))
     return g, 0, [cols, tall, rows, long_cols], None
+
+
+@case
+def one_workgroup_plays_several():
+    """graphs small enough to run as one kernel whose steps were written for 2 to 4 workgroups with LDS of their own:
+    rows folded by all 256 lanes (one LDS exchange per row), columns folded through LDS, a softmax of 4 long rows; the
+    one workgroup takes the turns of all of them, with a barrier between the turns"""
+    g = Graph()
+    rng = np.random.default_rng(211)
+    rows = rng.standard_normal((3, 16384)).astype(np.float32)
+    g.output(g.unary(UnaryOp.SIGMOID, g.reduce(g.input([3, 16384]), [1], ReduceOp.SUM)))
+    cols = rng.standard_normal((512, 96)).astype(np.float32)
+    g.output(g.unary(UnaryOp.EXP, g.reduce(g.input([512, 96]), [0], ReduceOp.MAX)))
+    soft = rng.standard_normal((4, 3000)).astype(np.float32)
+    g.output(g.softmax(g.input([4, 3000]), 1))
+    return g, 0, [rows, cols, soft], None

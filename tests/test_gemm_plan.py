@@ -181,10 +181,8 @@ def test_constant_weights_are_laid_out_again_for_f16_matmuls(monkeypatch):
     weight_bytes = 128 * 256 * 2
     assert HipExecutor(0, graph(False), 0, plan_only=True).mem_usage["dedicated_bytes"] == weight_bytes
     assert HipExecutor(0, graph(True), 0, plan_only=True).mem_usage["dedicated_bytes"] == 2 * weight_bytes
-    monkeypatch.setenv("KNHIP_PACK_CONSTANTS", "0")
-    assert HipExecutor(0, graph(True), 0, plan_only=True).mem_usage["dedicated_bytes"] == weight_bytes
+    assert HipExecutor(0, graph(True), 0, plan_only=True, pack_matmul_constants=False).mem_usage["dedicated_bytes"] == weight_bytes
     # f32 matmuls and K axes that are no multiple of 64 keep the operand as it is
-    monkeypatch.delenv("KNHIP_PACK_CONSTANTS")
     g = Graph()
     x = g.input([64, 96], DType.F16)
     w = g.constant([96, 256], np.ones((96, 256), np.float16), DType.F16)
