@@ -88,7 +88,15 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, cons
             parts.push_back(part);
         }
         if (ok) fused_spec_ = make_fused_graph_kernel(parts);
-        if (fused_spec_) fused_code_ = compile_kernel(fused_spec_->source);
+        if (fused_spec_) {
+            fused_code_ = compile_kernel(fused_spec_->source);
+            // What launch_fused passes: the pointer table by value (at least one slot), the address of the completion
+            // word and the number of the launch. The compiled kernel must expect exactly that many bytes of arguments.
+            const size_t host_bytes = 8 * std::max<size_t>(fused_spec_->n_ptrs, 1) + 8 + 4;
+            const size_t kernel_bytes = kernarg_segment_bytes(*fused_code_);
+            if (kernel_bytes != host_bytes)
+                fail("the one-kernel plan expects ", kernel_bytes, " bytes of launch arguments, the launch passes ", host_bytes);
+        }
     }
     if (plan_only) return;
 
@@ -164,6 +172,9 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, cons
         for (auto &l : launches_) fused_ptrs_.insert(fused_ptrs_.end(), l.ptrs.begin(), l.ptrs.end());
         for (auto &l : mapped_launches_) fused_mapped_ptrs_.insert(fused_mapped_ptrs_.end(), l.ptrs.begin(), l.ptrs.end());
         KN_ASSERT(fused_ptrs_.size() == fused_spec_->n_ptrs && (!mapped_io_ || fused_mapped_ptrs_.size() == fused_spec_->n_ptrs));
+        // (the kernel's table has at least one slot: the launch must never read it through a null data pointer)
+        if (fused_ptrs_.empty()) fused_ptrs_.push_back(nullptr);
+        if (mapped_io_ && fused_mapped_ptrs_.empty()) fused_mapped_ptrs_.push_back(nullptr);
     }
 }
 

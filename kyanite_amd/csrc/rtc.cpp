@@ -172,6 +172,28 @@ std::string library_dir() {
     return ".";
 }
 
+size_t kernarg_segment_bytes(const CodeObject &code) {
+    // the metadata is a MessagePack map; the key is a string, the value behind it an unsigned integer
+    static const char key[] = ".kernarg_segment_size";
+    const size_t key_len = sizeof key - 1;
+    const std::vector<char> &b = code.binary;
+    size_t found = 0, value = 0;
+    for (size_t i = 0; i + key_len < b.size(); i++) {
+        if (memcmp(b.data() + i, key, key_len) != 0) continue;
+        const unsigned char *p = (const unsigned char *) b.data() + i + key_len;
+        const size_t left = b.size() - i - key_len;
+        size_t v = 0;
+        if (p[0] <= 0x7f) v = p[0];
+        else if (p[0] == 0xcc && left >= 2) v = p[1];
+        else if (p[0] == 0xcd && left >= 3) v = ((size_t) p[1] << 8) | p[2];
+        else if (p[0] == 0xce && left >= 5) v = ((size_t) p[1] << 24) | ((size_t) p[2] << 16) | ((size_t) p[3] << 8) | p[4];
+        else continue;
+        found++;
+        value = v;
+    }
+    return found == 1 ? value : 0;
+}
+
 CompileStats compile_stats() {
     std::lock_guard<std::mutex> lock(g_mutex);
     return g_stats;

@@ -27,6 +27,10 @@ std::shared_ptr<const CodeObject> compile_kernel(const std::string &source);
 // cache that passed the checks above and still does not load.
 std::shared_ptr<const CodeObject> recompile_kernel(const std::string &source);
 
+// Bytes of launch arguments the (single) kernel of a code object expects, read from the code object's metadata note
+// (the value behind the key ".kernarg_segment_size"); 0 when the note does not hold exactly one such key.
+size_t kernarg_segment_bytes(const CodeObject &code);
+
 struct CompileStats {
     size_t compiled = 0, memory_hits = 0, disk_hits = 0, discarded = 0;
 };

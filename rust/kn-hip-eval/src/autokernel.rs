@@ -24,7 +24,7 @@ struct Descriptor {
 fn describe(shape: &StridedShape, dtype: DType) -> Descriptor {
     let dims = shape.shape().to_vec();
     let strides = shape.strides_i64();
-    let raw = knhip_tensor { ptr: null_mut(), dtype: dtype_code(dtype), rank: dims.len(), shape: dims.as_ptr(), strides: strides.as_ptr() };
+    let raw = knhip_tensor { ptr: null_mut(), dtype: dtype_code(dtype) as c_int, rank: dims.len(), shape: dims.as_ptr(), strides: strides.as_ptr() };
     Descriptor { raw, _shape: dims, _strides: strides }
 }
 

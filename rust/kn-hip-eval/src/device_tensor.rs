@@ -63,7 +63,7 @@ impl DeviceTensor {
         let strides = self.shape.strides_i64();
         let raw = knhip_tensor {
             ptr: self.ptr.ptr(),
-            dtype: dtype_code(self.dtype),
+            dtype: dtype_code(self.dtype) as std::os::raw::c_int,
             rank: shape.len(),
             shape: shape.as_ptr(),
             strides: strides.as_ptr(),

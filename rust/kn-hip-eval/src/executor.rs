@@ -6,10 +6,12 @@ use std::ptr::null_mut;
 use kn_graph::dispatch_dtype;
 use kn_graph::dtype::{DBool, DTensor, DType, Tensor};
 use kn_graph::graph::Graph;
-use kn_hip_sys::wrapper::{read_string, HipDevice, HipStream, Status};
+use kn_hip_sys::wrapper::{read_string, DevicePtr, ExecutorOptions, HipDevice, HipStream, Status};
 use kn_hip_sys::*;
 
+use crate::device_tensor::DeviceTensor;
 use crate::serialize::{dtype_from_code, serialize_graph};
+use crate::shape::StridedShape;
 
 /// planner.rs:67-81, plus the size of the one arena every buffer lives in.
 #[derive(Debug, Clone, Copy)]
@@ -40,26 +42,14 @@ pub struct Profile {
     pub timing_overhead: f32,
 }
 
-/// A dense row-major tensor inside the executor's arena (the role of `DeviceTensor` for inputs and outputs).
-#[derive(Debug, Clone)]
-pub struct DeviceIo {
-    pub ptr: *mut c_void,
-    pub dtype: DType,
-    pub shape: Vec<usize>,
-}
-
-impl DeviceIo {
-    pub fn len_bytes(&self) -> usize {
-        self.shape.iter().product::<usize>() * self.dtype.size().bytes()
-    }
-}
-
 pub struct HipExecutor {
     raw: *mut knhip_executor,
     stream: HipStream,
 
-    pub device_inputs: Vec<DeviceIo>,
-    pub device_outputs: Vec<DeviceIo>,
+    /// the dense input and output tensors inside the executor's arena (executor.rs:26-27); they live as long as the
+    /// executor does
+    pub device_inputs: Vec<DeviceTensor>,
+    pub device_outputs: Vec<DeviceTensor>,
 
     pub batch_size: usize,
     pub mem_usage: MemoryUsage,
@@ -72,7 +62,7 @@ pub struct HipExecutor {
 // executor.rs:41: used from one thread at a time (&mut self), may move between threads
 unsafe impl Send for HipExecutor {}
 
-fn io_infos(raw: *const knhip_executor, is_output: bool, count: usize) -> Vec<DeviceIo> {
+fn io_tensors(device: HipDevice, raw: *const knhip_executor, is_output: bool, count: usize) -> Vec<DeviceTensor> {
     (0..count)
         .map(|index| unsafe {
             let mut dtype: c_int = 0;
@@ -85,7 +75,10 @@ fn io_infos(raw: *const knhip_executor, is_output: bool, count: usize) -> Vec<De
             } else {
                 knhip_executor_input_ptr(raw, index, &mut ptr).unwrap();
             }
-            DeviceIo { ptr, dtype: dtype_from_code(dtype), shape: dims[..rank].to_vec() }
+            let dtype = dtype_from_code(dtype);
+            let shape = StridedShape::new_simple(dims[..rank].to_vec());
+            let len_bytes = shape.size() * dtype.size().bytes();
+            DeviceTensor::from_parts(DevicePtr::borrowed(device, ptr, len_bytes), shape, dtype)
         })
         .collect()
 }
@@ -117,20 +110,21 @@ impl HipExecutor {
     /// `CudaExecutor::new` (executor.rs:61-110): plans the graph for one concrete batch size, allocates the arena,
     /// uploads the constants and compiles the kernels.
     pub fn new(device: HipDevice, graph: &Graph, batch_size: usize) -> Self {
-        Self::new_with_flags(device, graph, batch_size, 0)
+        Self::new_with_options(device, graph, batch_size, &ExecutorOptions::default())
     }
 
-    /// `flags`: `KNHIP_PRESERVE_INPUTS` for callers that write `device_inputs` once and call `run_async` many times.
-    pub fn new_with_flags(device: HipDevice, graph: &Graph, batch_size: usize, flags: c_int) -> Self {
+    /// `options`: e.g. `ExecutorOptions::default().preserve_inputs()` for callers that write `device_inputs` once and
+    /// call `run_async` many times, or `mapped_io_bytes = 0` for callers that read `device_outputs` after `evaluate`.
+    pub fn new_with_options(device: HipDevice, graph: &Graph, batch_size: usize, options: &ExecutorOptions) -> Self {
         let blob = serialize_graph(graph);
         let mut raw = null_mut();
-        unsafe { knhip_executor_new_from_blob(device.inner(), blob.as_ptr(), blob.len(), batch_size, flags, &mut raw) }.unwrap();
+        unsafe { knhip_executor_new_from_blob(device.inner(), blob.as_ptr(), blob.len(), batch_size, &options.0, &mut raw) }.unwrap();
 
         let (mut input_count, mut output_count) = (0usize, 0usize);
         unsafe { knhip_executor_io_count(raw, &mut input_count, &mut output_count) }.unwrap();
-        let device_inputs = io_infos(raw, false, input_count);
-        let device_outputs = io_infos(raw, true, output_count);
-        let tensor_outputs = device_outputs.iter().map(|io| zeros_dtensor(io.dtype, &io.shape)).collect();
+        let device_inputs = io_tensors(device, raw, false, input_count);
+        let device_outputs = io_tensors(device, raw, true, output_count);
+        let tensor_outputs = device_outputs.iter().map(|t| zeros_dtensor(t.dtype(), t.strided_shape().shape())).collect();
 
         let mut usage = knhip_mem_usage::default();
         unsafe { knhip_executor_mem_usage(raw, &mut usage) }.unwrap();
@@ -166,8 +160,8 @@ impl HipExecutor {
     pub fn evaluate(&mut self, inputs: &[DTensor]) -> &[DTensor] {
         assert_eq!(inputs.len(), self.device_inputs.len(), "Wrong input count");
         for (i, (input, io)) in inputs.iter().zip(&self.device_inputs).enumerate() {
-            assert_eq!(input.shape(), &io.shape[..], "Wrong shape for input {}", i);
-            assert_eq!(input.dtype(), io.dtype, "Wrong dtype for input {}", i);
+            assert_eq!(input.shape(), io.strided_shape().shape(), "Wrong shape for input {}", i);
+            assert_eq!(input.dtype(), io.dtype(), "Wrong dtype for input {}", i);
         }
 
         let dense: Vec<DTensor> = inputs.iter().map(as_standard_layout).collect();

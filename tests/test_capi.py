@@ -49,3 +49,21 @@ def test_oracle_is_not_linked_into_the_product():
             if name.endswith((".py", ".cpp", ".h", ".hip")):
                 with open(os.path.join(root, name)) as f:
                     assert "oracle" not in f.read().lower(), f"{name} mentions the oracle"
+
+
+def test_one_kernel_plans_pass_the_launch_argument_check():
+    """A plan that runs as one generated kernel is only built when the compiled kernel expects exactly the bytes of
+    launch arguments that the executor passes (pointer table by value, completion word, launch number): read from the
+    code object's metadata when the executor is made, with or without a device. Every small case of the graph tests goes
+    through the same check; here the count is spelled out for the tiny MLP: 8 operands of 3 steps."""
+    import re
+
+    from kyanite_amd import HipExecutor
+    from kyanite_amd.configs import build_tiny_mlp
+
+    graph, _ = build_tiny_mlp(seed=0, batch=8)
+    ex = HipExecutor(0, graph, 8, plan_only=True)
+    source = ex.fused_source()
+    assert source, "the tiny MLP plans as one kernel"
+    slots = int(re.search(r"struct KnFusedPtrs \{ void \*p\[(\d+)\]; \};", source).group(1))
+    assert slots == sum(len(re.findall(r"\bf32\[", ex.step_str(i).split("operands:")[1])) for i in range(ex.step_count())) == 8

@@ -39,7 +39,7 @@ def test_every_bound_function_matches_the_header():
     assert not [n for n in rust if n not in c], "bound in Rust but not declared in knhip.h"
     assert {n: c[n] for n in rust} == rust
     # the whole runtime and executor tiers are bound; only builder / query / layout-test entry points may be left out
-    unbound = [n for n in c if n not in rust and not n.startswith(("knhip_graph_", "knhip_strided_", "knhip_optimizer_"))]
+    unbound = [n for n in c if n not in rust and not n.startswith(("knhip_graph_", "knhip_optimizer_"))]
     assert sorted(unbound) == ["knhip_executor_new", "knhip_executor_step_source"]
 
 
@@ -62,8 +62,32 @@ def _rust_struct_fields(name):
 
 
 def test_repr_c_structs_have_the_fields_of_the_header():
-    for name in ("knhip_mem_usage", "knhip_profile", "knhip_matmul_args"):
+    for name in ("knhip_mem_usage", "knhip_profile", "knhip_matmul_args", "knhip_executor_options", "knhip_tensor"):
         assert _rust_struct_fields(name) == _c_struct_fields(name), name
+
+
+def test_the_python_struct_has_the_fields_of_the_header_too():
+    from kyanite_amd._lib import ExecutorOptionsT, MatmulArgsT, TensorT
+    for name, struct in (("knhip_executor_options", ExecutorOptionsT), ("knhip_matmul_args", MatmulArgsT), ("knhip_tensor", TensorT)):
+        assert [f for f, _ in struct._fields_] == _c_struct_fields(name), name
+
+
+def test_device_tensor_and_autokernels_of_the_rust_crate_call_what_the_header_declares():
+    """every knhip_* name used by kn-hip-eval is bound in kn-hip-sys, and the reference's public methods are there"""
+    rust = _rust_functions()
+    for module in ("device_tensor.rs", "autokernel.rs", "shape.rs", "executor.rs"):
+        text = _read("rust", "kn-hip-eval", "src", module)
+        for name in set(re.findall(r"\b(knhip_[a-z0-9_]+)\s*\(", text)):
+            assert name in rust, f"{module} calls {name}, which kn-hip-sys does not bind"
+    tensor = _read("rust", "kn-hip-eval", "src", "device_tensor.rs")
+    for method in ("alloc_simple", "deep_clone", "copy_simple_from_host", "copy_simple_to_host", "copy_from", "copy_from_host_staged",
+                   "copy_to_host_staged", "permute", "view", "broadcast", "slice", "index", "flip", "repeat_unary", "to_mat_mul_arg"):
+        assert re.search(r"pub (unsafe )?fn " + method + r"\b", tensor), method
+    kernels = _read("rust", "kn-hip-eval", "src", "autokernel.rs")
+    for kernel in ("ScalarKernel", "ReduceKernel", "SoftmaxKernel", "LayernormKernel", "GatherKernel"):
+        assert f"pub struct {kernel}" in kernels and re.search(r"impl " + kernel + r" \{.*?pub unsafe fn run", kernels, flags=re.S), kernel
+    executor = _read("rust", "kn-hip-eval", "src", "executor.rs")
+    assert "pub device_inputs: Vec<DeviceTensor>" in executor and "pub device_outputs: Vec<DeviceTensor>" in executor
 
 
 def test_codes_of_the_rust_serialiser_are_the_header_codes():
@@ -93,7 +117,7 @@ def test_codes_of_the_rust_serialiser_are_the_header_codes():
     for name, value in re.findall(r"pub const (KNHIP_[A-Z0-9_]+): c_int = (\d+);", sys_lib):
         if name in enums:
             assert enums[name] == int(value), name
-    for name in ("KNHIP_OK", "KNHIP_ERROR", "KNHIP_BUFFER_TOO_SMALL", "KNHIP_PLAN_ONLY", "KNHIP_PRESERVE_INPUTS"):
+    for name in ("KNHIP_OK", "KNHIP_ERROR", "KNHIP_BUFFER_TOO_SMALL"):
         value = re.search(r"#define " + name + r" (\d+)", header).group(1)
         assert re.search(r"pub const " + name + r": c_int = " + value + ";", sys_lib), name
 
