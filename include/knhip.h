@@ -296,6 +296,8 @@ typedef struct knhip_executor knhip_executor;
  *   (knhip_executor_fused_source).
  * The remaining int fields are 1 by default; 0 switches that path off:
  *   fuse_attention            matmul, softmax, matmul chains as one launch (off: three launches)
+ *   fuse_gated_matmul         (x w_g) sigmoid(x w_g) (x w_u) in f16 as one launch whose store computes the gated
+ *                             product (off: the two products, then an elementwise launch)
  *   group_matmuls             matmuls that share their left operand in one launch (off: one launch each)
  *   pack_matmul_constants     constant [k, n] right operands laid out again as [n, k] when the plan is made
  *   pointwise_conv_as_matmul  1 x 1 convolutions with stride 1 as one matrix product per image (off: the conv kernel)
@@ -314,7 +316,7 @@ typedef struct knhip_executor knhip_executor;
 typedef struct {
     size_t struct_bytes; /* sizeof(knhip_executor_options), set by knhip_executor_options_default */
     int plan_only, preserve_inputs, step_by_step;
-    int fuse_attention, group_matmuls, pack_matmul_constants, pointwise_conv_as_matmul, join_elementwise, split_reduce;
+    int fuse_attention, fuse_gated_matmul, group_matmuls, pack_matmul_constants, pointwise_conv_as_matmul, join_elementwise, split_reduce;
     int tiled_transpose, split_conv_channels, plane_conv_any_width;
     int direct_gemm, split_k, tail_split, dot_products;
     uint64_t streaming_bytes, mapped_io_bytes;

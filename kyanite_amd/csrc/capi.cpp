@@ -691,6 +691,7 @@ int knhip_executor_options_default(knhip_executor_options *o) {
         o->preserve_inputs = d.planner.preserve_inputs;
         o->step_by_step = !d.fuse_small;
         o->fuse_attention = d.planner.fuse_attention;
+        o->fuse_gated_matmul = d.planner.fuse_gated_matmul;
         o->group_matmuls = d.planner.group_matmuls;
         o->pack_matmul_constants = d.planner.pack_matmul_constants;
         o->pointwise_conv_as_matmul = d.planner.pointwise_conv_as_matmul;
@@ -723,6 +724,7 @@ ExecutorOptions executor_options_from(const knhip_executor_options *o) {
     PlannerOptions &p = e.planner;
     p.preserve_inputs = o->preserve_inputs != 0;
     p.fuse_attention = o->fuse_attention != 0;
+    p.fuse_gated_matmul = o->fuse_gated_matmul != 0;
     p.group_matmuls = o->group_matmuls != 0;
     p.pack_matmul_constants = o->pack_matmul_constants != 0;
     p.pointwise_conv_as_matmul = o->pointwise_conv_as_matmul != 0;

@@ -240,6 +240,20 @@ void HipExecutor::realise_launch(size_t index, Launch &l, bool mapped) {
         gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;
         gemm.counters = lp.counter_bytes > 0 ? l.ptrs[next++] : nullptr;
         l.gemm_plan = plan_gemm_launch(gemm, step.gemm_f16);
+    } else if (step.kind == StepKind::MatMul && step.gemm.pair_op) {
+        // a gated pair: left operand, the two right operands, the result
+        GemmParams gemm = step.gemm;
+        KN_ASSERT(l.ptrs.size() == 4);
+        gemm.a = l.ptrs[0];
+        gemm.b = l.ptrs[1];
+        gemm.b_pair = l.ptrs[2];
+        gemm.c = l.ptrs[3];
+        // the kernel reaches both right operands with 32 bit byte offsets from the lower of the two
+        const long long apart = std::llabs((const char *) gemm.b_pair - (const char *) gemm.b);
+        if (apart + ((long long) (gemm.n / 2) * gemm.b_sn + gemm.k) * 2 >= 0xffffffffll)
+            fail("the two weights of a gated matmul lie ", apart, " bytes apart in the arena, out of the kernel's reach; "
+                 "build the executor with fuse_gated_matmul = 0");
+        l.gemm_plan = plan_gemm_launch(gemm, step.gemm_f16);
     } else if (step.kind == StepKind::MatMul) {
         GemmParams gemm = step.gemm;
         gemm.a = l.ptrs[0];

@@ -77,7 +77,7 @@ std::optional<KernelSpec> make_fused_graph_kernel(const std::vector<FusedPart> &
             if (part.kernel->block != 256 || part.kernel->grid > FUSED_MAX_WORKGROUPS) return std::nullopt;
         } else {
             const GemmParams &p = part.gemm;
-            if (p.groups > 1 || p.batch <= 0 || p.m <= 0 || p.n <= 0 || p.k < 0) return std::nullopt;
+            if (p.groups > 1 || p.pair_op || p.batch <= 0 || p.m <= 0 || p.n <= 0 || p.k < 0) return std::nullopt;
             const long long outputs = (long long) p.batch * p.m * p.n;
             if (outputs > FUSED_MAX_MATMUL_OUTPUTS || outputs * (long long) p.k > FUSED_MAX_MATMUL_MACS) return std::nullopt;
         }

@@ -109,7 +109,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // MFMAs on rows and columns that do not exist (the value head's 1 x 1 x 256 took 15.7 us, the 32 x 64 x 128 of a
     // 1 x 1 convolution on one board 12.1 us): one wave per result instead, lanes along K.
     const bool dot_enabled = p.tuning.dot_products;
-    if (dot_enabled && p.groups <= 1 && p.k > 0 && (long long) p.batch * p.m * p.n * p.k <= (1ll << 20) && (long long) p.batch * p.m * p.n <= 16384) {
+    if (dot_enabled && p.groups <= 1 && !p.pair_op && p.k > 0 && (long long) p.batch * p.m * p.n * p.k <= (1ll << 20) && (long long) p.batch * p.m * p.n <= 16384) {
         lp.dot = true;
         lp.small_tile = true;
         lp.bk = 64;
@@ -174,9 +174,9 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
             for (int split : split_choices) {
                 if (split > 1) {
                     const unsigned long long bytes = (unsigned long long) split * p.batch * p.m * p.n * 4ull;
-                    if (!split_enabled || groups > 1 || p.k / split < 256 || bytes > (256ull << 20)) continue;
+                    if (!split_enabled || groups > 1 || p.pair_op || p.k / split < 256 || bytes > (256ull << 20)) continue;
                 }
-                const double us = estimate_f16_direct_us(p, groups, tile, split, tail_enabled && split_enabled);
+                const double us = estimate_f16_direct_us(p, groups, tile, split, tail_enabled && split_enabled && !p.pair_op);
                 if (best_us == 0.0 || us < best_us) {
                     best_us = us;
                     best_tile = tile;
@@ -215,7 +215,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // pass between workgroups with accesses that bypass the L2 caches, which costs more than the second launch
     // of a plain split; so a launch with less than one round of tiles keeps that (512 x 4096 x 11008: 69 us
     // against 82 us).
-    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled && model_split <= 1 && !lp.skinny_tile) {
+    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled && model_split <= 1 && !lp.skinny_tile && !p.pair_op) {
         const long long slots = 256 * (lp.tall_tile || lp.narrow_tile ? 1 : 2);
         const long long full = blocks / slots * slots, rest = blocks - full;
         const int parts = tail_parts(blocks, slots, p.k);
@@ -251,7 +251,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     const long long split_below = lp.tall_tile ? 128 : 256, split_target = lp.tall_tile ? 256 : 512;
     // (a product of a few thousand multiplications is one short workgroup: a second launch to sum parts costs more)
     const bool tiny = (long long) p.batch * p.m * p.n * p.k < (1ll << 18);
-    if (can_split && blocks < split_below && groups == 1 && !lp.narrow_tile && !tiny) {
+    if (can_split && blocks < split_below && groups == 1 && !lp.narrow_tile && !tiny && !p.pair_op) {
         const int min_chunk = few_tiles ? 128 : (f16 ? 512 : 256);  // K elements a split should at least cover
         long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;
@@ -284,6 +284,7 @@ std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16) {
     }
     if (lp.skinny_tile) tm = 32, tn = 128;
     ss << (lp.direct ? "direct " : "staged ") << tm << "x" << tn << " bk" << lp.bk;
+    if (lp.p.pair_op) ss << " gated pairs";
     if (lp.split_k > 1) ss << " split_k=" << lp.split_k << "x" << lp.k_chunk;
     if (lp.tail_split > 1) ss << " head=" << lp.head_tiles << " tail_split=" << lp.tail_split << "x" << lp.tail_k_chunk;
     return ss.str();

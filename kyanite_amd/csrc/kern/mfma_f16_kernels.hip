@@ -205,6 +205,35 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
         }
 }
 
+// The store of a gated pair (GemmParams::pair_op): lanes c and c + 16 of an MFMA tile hold G and U of one element of
+// C, column 16 * (virtual column / 32) + c % 16. Both lanes compute the element (the partner's factor comes by a lane
+// exchange) and each stores half of the tile's rows. Roundings as the separate operations place them: the two products,
+// the sigmoid (the hardware's 2^x and reciprocal, like the generated elementwise kernels use for halves) and both
+// multiplications are each rounded to f16.
+template <int MI, int NI>
+__device__ __forceinline__ void store_tiles_gated(const GemmParams &p, const floatx16 (&acc)[MI][NI], int bz, int row0, int col0) {
+    const int lane = threadIdx.x & 63, c = lane & 31, half = lane >> 5;
+    const bool low = c < 16;
+    const int n_out = p.n / 2;
+    half_t *out = (half_t *) p.c + bz * p.c_sb;
+    auto r16 = [](float x) { return (float) (half_t) x; };
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NI; j++) {
+            const int col = ((col0 + 32 * j) >> 5) * 16 + (c & 15);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float own = acc[i][j][v], other = __shfl_xor(own, 16);
+                const float g = r16(low ? own : other), u = r16(low ? other : own);
+                const float sig = r16(__frcp_rn(1.0f + __expf(-g)));
+                const float act = r16(r16(g * sig) * u);
+                const int row = row0 + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
+                if ((v < 8) == low && row < p.m && col < n_out) out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) act;
+            }
+        }
+}
+
 // TI: MFMA tiles per wave and axis; WM: waves along M (2 along N), so the workgroup tile is (32 TI WM) x (64 TI):
 // 128 x 128 (TI 2, WM 2), 64 x 64 (TI 1, WM 2) or 256 x 128 with 8 waves (TI 2, WM 4), which fetches a quarter less
 // from L2 per flop. BK: depth of a K slice; NBUF: LDS buffers per operand (2 = double buffered, one barrier per
@@ -435,7 +464,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
     constexpr int LD = A_LD + B_LD;
     const int lr = lane / CHUNKS, pos = lane % CHUNKS;
     const char *a_tile = (const char *) ((const T *) p.a + bz * p.a_sb + k_begin + (long long) m0 * p.a_sm);
-    const char *b_tile = (const char *) ((const T *) b_base + bz * p.b_sb + k_begin + (long long) n0 * p.b_sn);
+    // (a gated pair reads rows of two matrices: offsets from the lower of the two bases, see below)
+    const char *pair_lo = (const char *) p.b < (const char *) p.b_pair ? (const char *) p.b : (const char *) p.b_pair;
+    const char *b_tile = p.pair_op ? pair_lo + ((long long) bz * p.b_sb + k_begin) * (long long) sizeof(T)
+                                   : (const char *) ((const T *) b_base + bz * p.b_sb + k_begin + (long long) n0 * p.b_sn);
     unsigned a_off[A_LD], b_off[B_LD];
 #pragma unroll
     for (int i = 0; i < A_LD; i++) {
@@ -446,6 +478,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
     for (int i = 0; i < B_LD; i++) {
         const int row = (wave * B_LD + i) * ROWS_PER_LOAD + lr;
         b_off[i] = (unsigned) (((long long) (min(n0 + row, p.n - 1) - n0) * p.b_sn + VEC * (pos ^ swz(row))) * (long long) sizeof(T));
+        if (p.pair_op) {
+            // virtual column -> (matrix, column): the first 16 columns of a block of 32 are G's, the others U's
+            const int vcol = n0 + row, col = min((vcol >> 5) * 16 + (vcol & 15), p.n / 2 - 1);
+            const char *base = (vcol & 16) ? (const char *) p.b_pair : (const char *) p.b;
+            b_off[i] = (unsigned) ((long long) (base - pair_lo) + ((long long) col * p.b_sn + VEC * (pos ^ swz(row))) * (long long) sizeof(T));
+        }
     }
     char *const dst_a = lds + wave * A_LD * 1024, *const dst_b = lds + A_BYTES + wave * B_LD * 1024;
     // load l of a slice: the first A_LD fill rows of A, the others rows of B
@@ -567,6 +605,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
         store_tiles<T, MI, NI>(p, sum, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
         return;
     }
+    if constexpr (sizeof(T) == 2) {
+        if (p.pair_op) {
+            store_tiles_gated<MI, NI>(p, acc, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
+            return;
+        }
+    }
     store_tiles<T, MI, NI>(p, acc, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
 }
 
@@ -659,6 +703,14 @@ int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     if (p.addend2 != nullptr && p.addend == nullptr) return (int) hipErrorInvalidValue;
     if (p.batch > 65535 || (long long) p.m * p.n > 0x7fffffffll * 256) return (int) hipErrorInvalidConfiguration;
     if (lp.split_k > 1 && p.workspace == nullptr) return (int) hipErrorInvalidValue;
+    if (p.pair_op) {
+        // a gated pair: only what the plan promised (direct kernel, one product per launch, whole K per workgroup), and
+        // both matrices within reach of the 32 bit offsets from the lower of the two
+        const long long apart = (const char *) p.b_pair - (const char *) p.b, span = ((long long) (p.n / 2) * p.b_sn + p.k) * 2;
+        if (p.pair_op != GEMM_PAIR_SWIGLU || p.b_pair == nullptr || groups > 1 || p.addend || lp.split_k > 1 || lp.tail_split > 1 || lp.swapped ||
+            !lp.direct || p.n % 2 != 0 || (apart < 0 ? -apart : apart) + span >= 0xffffffffll || (uintptr_t) p.b_pair % 16 != 0)
+            return (int) hipErrorInvalidValue;
+    }
     const int a_mode = pick_mode(p.a, p.a_sm, p.a_sk, p.m, p.k, p.a_sb, p.batch);
     int b_mode = pick_mode(groups > 1 ? p.b_group[0] : p.b, p.b_sn, p.b_sk, p.n, p.k, p.b_sb, p.batch);
     for (int g = 1; g < groups; g++) {  // the loader that every operand of the group allows
@@ -667,6 +719,7 @@ int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
     }
     // both operands K contiguous and K (and every split of it) whole slices: the direct-to-LDS kernel
     const bool direct = lp.direct && a_mode == VecK && b_mode == VecK && lp.k_chunk % 64 == 0;
+    if (p.pair_op && !direct) return (int) hipErrorInvalidValue;
     // (128 x 64 tiles exist in the direct kernel only; without it they run as 64 x 64)
     // (so do 256 x 256 and 256 x 192 tiles, which otherwise run as 256 x 128)
     const bool narrow = lp.narrow_tile && direct, small = lp.small_tile || (lp.narrow_tile && !direct);

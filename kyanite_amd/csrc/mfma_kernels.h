@@ -55,7 +55,16 @@ struct GemmParams {
     // are shared between workgroups; may be null otherwise
     void *counters = nullptr;
     GemmTuning tuning;
+    // Gated pair (f16, the kernel that loads global -> LDS directly, no groups, no addend, no split of K):
+    // C = (G * sigmoid(G)) * U with G = A * B and U = A * B_pair, each product, the sigmoid and each multiplication
+    // rounded to f16 like separate operations would. `n` counts VIRTUAL columns, two per column of C: the block of 32
+    // virtual columns t holds the columns 16 t .. 16 t + 15 of G in its first half and those of U in its second, so
+    // that the two factors of an element of C sit in one MFMA tile, 16 lanes apart. c_sm / c_sn address C itself
+    // ([m, n / 2]); b_sn / b_sk address B and B_pair alike.
+    int pair_op = 0;
+    const void *b_pair = nullptr;
 };
+constexpr int GEMM_PAIR_SWIGLU = 1;
 
 // How a matrix multiply is launched; a pure function of the shapes, strides and alignments, so the planner can ask
 // for it ahead of time (to reserve the workspace) and the launch reproduces it.

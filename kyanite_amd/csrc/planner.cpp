@@ -21,6 +21,7 @@ std::string Step::str() const {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm_has_addend2 ? " +add" : "") << (gemm.relu ? " relu" : "");
         if (gemm.groups > 1) ss << " x" << gemm.groups << " grouped";
+        if (gemm.pair_op) ss << " (x w_g) sigmoid(x w_g) (x w_u), n counts both";
         ss << " [" << describe_gemm_plan(plan_gemm_launch(gemm, gemm_f16), gemm_f16) << "]";
     }
     else if (kind == StepKind::Conv)
@@ -45,7 +46,7 @@ double Step::bytes() const {
     double total = 0.0;
     for (size_t i = 0; i < operands.size(); i++) {
         // split-K scratch is not algorithmic traffic
-        if (kind == StepKind::MatMul && !attention && i >= (gemm.groups > 1 ? 1u + 2u * (unsigned) gemm.groups : 3u + (gemm_has_addend ? 1u : 0u) + (gemm_has_addend2 ? 1u : 0u))) break;
+        if (kind == StepKind::MatMul && !attention && i >= (gemm.pair_op ? 4u : gemm.groups > 1 ? 1u + 2u * (unsigned) gemm.groups : 3u + (gemm_has_addend ? 1u : 0u) + (gemm_has_addend2 ? 1u : 0u))) break;
         auto &op = operands[i];
         double elements = 1.0;
         const auto &shape = op.tensor.shape.shape();
@@ -300,6 +301,11 @@ private:
         }
         if (options.fuse_matmul_epilogue) {
             auto fused = try_visit_fused_matmul(value);
+            if (!fused.ok) return VT::missing(fused.need);
+            if (fused.value) return VT::done(*fused.value);
+        }
+        if (options.fuse_gated_matmul) {
+            auto fused = try_visit_gated_matmul(value);
             if (!fused.ok) return VT::missing(fused.need);
             if (fused.value) return VT::done(*fused.value);
         }
@@ -1081,6 +1087,91 @@ private:
         static const std::vector<Value> none;
         auto it = matmuls_by_left.find(left);
         return it == matmuls_by_left.end() ? none : it->second;
+    }
+
+    // `(g * sigmoid(g)) * u` with g = x w_g and u = x w_u, two f16 matmuls of one left operand with constant right
+    // operands of one shape, every intermediate value hidden and used only here (the gate twice): the feed-forward gate
+    // of a LLaMA style block. Planned as ONE launch of the matmul kernel that loads global -> LDS directly: its tiles
+    // interleave 16 columns of g with the same 16 columns of u, and the store computes the gated product, so neither
+    // product is written to memory and the elementwise launch behind them is gone (the reference plans two cuBLAS calls
+    // and a scalar kernel, planner.rs:606-648, :835-954). Roundings are those of the separate operations.
+    Visit<std::optional<PlanTensor>> try_visit_gated_matmul(Value value) {
+        using R = Visit<std::optional<PlanTensor>>;
+        const ValueInfo &info = graph[value];
+        const Operation &top = info.operation;
+        if (info.dtype != DType::F16 || top.kind != OpKind::Binary || top.binary != BinaryOp::Mul) return R::done(std::nullopt);
+        // through single-use hidden views down to a matmul; `from` itself has been checked by the caller
+        auto matmul_under = [&](Value from) -> std::optional<Value> {
+            Value v = from;
+            while (graph[v].operation.kind == OpKind::View) {
+                Value inner = graph[v].operation.inputs[0];
+                if (!can_fuse(inner) || graph[inner].shape.rank() == 0) return std::nullopt;
+                v = inner;
+            }
+            if (graph[v].operation.kind != OpKind::MatMul || map.count(v)) return std::nullopt;
+            return v;
+        };
+        std::optional<Value> gate_mm, up_mm;
+        for (int side = 0; side < 2 && !gate_mm; side++) {
+            const Value inner = top.inputs[side], up_side = top.inputs[1 - side];
+            const Operation &iop = graph[inner].operation;
+            if (!can_fuse(inner) || !can_fuse(up_side) || iop.kind != OpKind::Binary || iop.binary != BinaryOp::Mul) continue;
+            if (graph[inner].shape != info.shape || graph[up_side].shape != info.shape) continue;
+            for (int s = 0; s < 2; s++) {
+                const Value sig = iop.inputs[s], gate = iop.inputs[1 - s];
+                const Operation &sop = graph[sig].operation;
+                if (!can_fuse(sig) || sop.kind != OpKind::Unary || sop.unary != UnaryOp::Sigmoid || sop.inputs[0] != gate) continue;
+                if (!graph.is_hidden_with_uses(gate, 2) || graph[gate].shape != info.shape || map.count(gate) || map.count(up_side)) continue;
+                auto g = matmul_under(gate), u = matmul_under(up_side);
+                if (!g || !u || *g == *u) continue;
+                gate_mm = g;
+                up_mm = u;
+                break;
+            }
+        }
+        if (!gate_mm) return R::done(std::nullopt);
+        const Operation &gop = graph[*gate_mm].operation, &uop = graph[*up_mm].operation;
+        if (gop.inputs[0] != uop.inputs[0] || !graph.is_const(gop.inputs[1]) || !graph.is_const(uop.inputs[1]) || graph.is_const(gop.inputs[0])) return R::done(std::nullopt);
+        if (graph[*gate_mm].dtype != DType::F16 || graph[*gate_mm].shape != graph[*up_mm].shape ||
+            graph[gop.inputs[1]].shape != graph[uop.inputs[1]].shape)
+            return R::done(std::nullopt);
+
+        auto left = visit(gop.inputs[0]);
+        if (!left.ok) return R::missing(left.need);
+        auto gate_w = visit(gop.inputs[1]);
+        if (!gate_w.ok) return R::missing(gate_w.need);
+        auto up_w = visit(uop.inputs[1]);
+        if (!up_w.ok) return R::missing(up_w.need);
+        if (gate_w.value.shape.strides() != up_w.value.shape.strides()) return R::done(std::nullopt);
+        KN_ASSERT(left.value.shape.rank() == 3 && gate_w.value.shape.rank() == 3);
+        const PlanTensor wg = pack_right_operand(left.value, gate_w.value, DType::F16), wu = pack_right_operand(left.value, up_w.value, DType::F16);
+        if (wg.shape.strides() != wu.shape.strides()) return R::done(std::nullopt);
+
+        const PlanTensor &l = left.value;
+        const size_t b = l.shape.shape()[0], m = l.shape.shape()[1], k = l.shape.shape()[2], n = wg.shape.shape()[2];
+        if (b != 1 || m * n == 0 || m > INT32_MAX || 2 * n > INT32_MAX || k > INT32_MAX) return R::done(std::nullopt);
+        Step step;
+        step.kind = StepKind::MatMul;
+        step.gemm_f16 = true;
+        GemmParams &g = step.gemm;
+        g.tuning = options.gemm;
+        g.batch = 1; g.m = (int) m; g.n = (int) (2 * n); g.k = (int) k;
+        g.a_sb = l.shape.strides()[0]; g.a_sm = l.shape.strides()[1]; g.a_sk = l.shape.strides()[2];
+        g.b_sb = wg.shape.strides()[0]; g.b_sk = wg.shape.strides()[1]; g.b_sn = wg.shape.strides()[2];
+        g.c_sb = (long long) (m * n); g.c_sm = (long long) n; g.c_sn = 1;
+        g.pair_op = GEMM_PAIR_SWIGLU;
+        // only on the kernel that loads global -> LDS directly, whole K per workgroup (operands in the arena are aligned)
+        const GemmLaunchPlan lp = plan_gemm_launch(g, true);
+        if (!lp.direct || lp.swapped || lp.split_k > 1 || lp.tail_split > 1 || lp.dot) return R::done(std::nullopt);
+        // both weights lie within the reach of the kernel's 32 bit offsets wherever the arena puts them
+        if (dtype_bytes(DType::F16) * (n * (size_t) std::llabs(g.b_sn) + k) * 2 >= ((size_t) 1 << 31)) return R::done(std::nullopt);
+
+        PlanTensor result = alloc_tensor_shared({1, m, n}, DType::F16);
+        step.operands = {{l, OperandKind::In}, {wg, OperandKind::In}, {wu, OperandKind::In}, {result, OperandKind::Out}};
+        push(std::move(step), value);
+        auto viewed = result.view(info.shape.eval(batch_size));
+        KN_ASSERT(viewed.has_value(), "a dense matmul result can always be viewed");
+        return R::done(*viewed);
     }
 
     Visit<std::optional<PlanTensor>> try_visit_matmul_group(Value value) {

@@ -93,6 +93,8 @@ struct PlannerOptions {
     bool fuse_matmul_epilogue = true;  // fold `+ d` and `max(., 0)` after a matmul into the matmul's store
     bool fuse_attention = true;  // matmul, softmax, matmul chains in f32 run as one launch
     bool pack_matmul_constants = true;  // constant [k, n] right operands of matmuls are laid out again as [n, k]
+    // (x w_g) * sigmoid(x w_g) * (x w_u) in f16 with constant weights: one launch whose store computes the gated product
+    bool fuse_gated_matmul = true;
     bool group_matmuls = true;   // matmuls that share their left operand and have constant right operands share a launch
     bool pointwise_conv_as_matmul = true;  // 1 x 1 convolutions with stride 1 run as one matrix product per image
     bool join_elementwise = true;  // small elementwise steps of one shape that do not depend on each other share a launch

@@ -67,6 +67,7 @@ pub struct knhip_executor_options {
     pub preserve_inputs: c_int,
     pub step_by_step: c_int,
     pub fuse_attention: c_int,
+    pub fuse_gated_matmul: c_int,
     pub group_matmuls: c_int,
     pub pack_matmul_constants: c_int,
     pub pointwise_conv_as_matmul: c_int,

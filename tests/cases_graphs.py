@@ -2289,3 +2289,61 @@ def one_workgroup_plays_several():
     soft = rng.standard_normal((4, 3000)).astype(np.float32)
     g.output(g.softmax(g.input([4, 3000]), 1))
     return g, 0, [rows, cols, soft], None
+
+
+def _gated_feed_forward(seed, m, k, n, order=0, extra_use=False, weights_kn=False):
+    """act = (x w_g) sigmoid(x w_g) (x w_u) in f16, spelled in one of four operand orders"""
+    g = Graph()
+    rng = np.random.default_rng(seed)
+    x = g.input([m, k], DType.F16)
+
+    def weight():
+        w = (rng.standard_normal((n, k)) / np.sqrt(k)).astype(np.float16)
+        if weights_kn:
+            return g.mat_mul(x, g.constant([k, n], np.ascontiguousarray(w.T), DType.F16))
+        return g.linear(x, g.constant([n, k], w, DType.F16))
+
+    gate, up = weight(), weight()
+    sig = g.sigmoid(gate)
+    inner = g.mul(gate, sig) if order & 1 == 0 else g.mul(sig, gate)
+    act = g.mul(inner, up) if order & 2 == 0 else g.mul(up, inner)
+    g.output(act)
+    if extra_use:
+        g.output(g.unary(UnaryOp.NEG, gate))  # the gate is needed on its own as well: nothing to fuse
+    return g, 0, [(rng.standard_normal((m, k)) * 1.5).astype(np.float16)], None
+
+
+@case
+def gated_matmul_ragged():
+    """rows and columns that fill no tile (m 200 of 256, 424 = 26.5 blocks of 16 columns), K of two slices"""
+    return _gated_feed_forward(301, 200, 128, 424)
+
+
+@case
+def gated_matmul_orders():
+    """sigmoid(g) * g and u * (...): the other operand orders of the same product"""
+    g1, _, in1, _ = _gated_feed_forward(302, 64, 64, 48, order=3)
+    return g1, 0, in1, None
+
+
+@case
+def gated_matmul_order_1():
+    return _gated_feed_forward(303, 130, 192, 256, order=1)
+
+
+@case
+def gated_matmul_order_2_kn_weights():
+    """weights stored [k, n] (`x @ w`): laid out again as [n, k] when the plan is made, then paired"""
+    return _gated_feed_forward(304, 256, 256, 512, order=2, weights_kn=True)
+
+
+@case
+def gated_matmul_wide():
+    """more than one tile in both directions on the 256 x 192 tiles a tall product picks"""
+    return _gated_feed_forward(305, 512, 256, 1000)
+
+
+@case
+def gated_matmul_gate_used_elsewhere():
+    """the gate is an output too: the three launches stay"""
+    return _gated_feed_forward(306, 96, 128, 160, extra_use=True)

@@ -33,6 +33,15 @@ def shared_left_linears():
     return g, 0, [_normal(192, 256, dtype=np.float16)]
 
 
+def gated_feed_forward():
+    g = Graph()
+    x = g.input([96, 128], DType.F16)
+    gate = g.linear(x, g.constant([208, 128], (_normal(208, 128) / 11).astype(np.float16), DType.F16))
+    up = g.linear(x, g.constant([208, 128], (_normal(208, 128) / 11).astype(np.float16), DType.F16))
+    g.output(g.mul(g.mul(gate, g.sigmoid(gate)), up))
+    return g, 0, [_normal(96, 128, dtype=np.float16)]
+
+
 def constant_kn_weight():
     g = Graph()
     x = g.input([64, 128], DType.F16)
@@ -128,6 +137,8 @@ def sources(ex):
 # option -> (graph builder, the option's value, what the default plan shows, what the plan with the option shows)
 OPTIONS = {
     "fuse_attention": (attention_f32, 0, lambda ex: "attention" in plan_text(ex), lambda ex: "attention" not in plan_text(ex) and ex.step_count() >= 3),
+    "fuse_gated_matmul": (gated_feed_forward, 0, lambda ex: "gated pairs" in plan_text(ex) and ex.step_count() == 1,
+                          lambda ex: "gated" not in plan_text(ex) and ex.step_count() == 2),
     "group_matmuls": (shared_left_linears, 0, lambda ex: "grouped" in plan_text(ex), lambda ex: "grouped" not in plan_text(ex) and ex.step_count() == 3),
     "pack_matmul_constants": (constant_kn_weight, 0, lambda ex: "f16[1, 256, 128]" not in plan_text(ex) and "direct" in plan_text(ex),
                               lambda ex: "staged" in plan_text(ex)),
