@@ -80,6 +80,26 @@ KN_DEV float kn_log1p_unit(float w) {
     return u == 1.0f ? w : logf(u) * (w / (u - 1.0f));
 }
 
+// The same three functions for halves. A result that is rounded to 11 bits does not need the library's exponential and
+// logarithm (about twenty instructions each, which rows of halves then wait for instead of memory): the hardware's 2^x
+// and log2 are a few 1e-7 off. The error function keeps the reference's polynomial (kn-graph/src/graph.rs:1677-1690)
+// but in f32, written without the cancellation of 1 - 1 / d^16: with d = 1 + t, d^16 - 1 comes from squaring
+// (1 + t)^2 - 1 = t (2 + t) four times, all terms positive, and erf = (d^16 - 1) / d^16.
+KN_DEV float kn_mish_half(float x) {
+    const float w = __expf(x), n = w * (w + 2.0f);
+    return x > 20.0f ? x : x * (n * __frcp_rn(n + 2.0f));
+}
+KN_DEV float kn_erf_half(float x) {
+    if (x != x) return x;
+    const float a = fminf(__builtin_fabsf(x), 4.5f);
+    float t = a * (0.0705230784f + a * (0.0422820123f + a * (0.0092705272f + a * (0.0001520143f + a * (0.0002765672f + a * 0.0000430638f)))));
+    t = t * (2.0f + t);
+    t = t * (2.0f + t);
+    t = t * (2.0f + t);
+    t = t * (2.0f + t);
+    return __builtin_copysignf(t * __frcp_rn(1.0f + t), x);
+}
+
 // low 64 bits of the value converted to a 128 bit signed integer: truncation toward zero, saturation at the
 // 128 bit bounds, NaN gives 0. Narrower integer targets wrap from here.
 KN_DEV kn_u64 kn_f2i(double x) {
@@ -257,11 +277,17 @@ std::string unary_expr(const ScalarNode &n, DType in, const std::string &x) {
             if (in == DType::F16) return "__frcp_rn(1.0f + __expf(-(" + x + ")))";
             return d ? "(1.0 / (1.0 + exp(-(" + x + "))))" : "(1.0f / (1.0f + expf(-(" + x + "))))";
         case UnaryOp::Tanh: return fn(d, "tanh") + "(" + x + ")";
-        case UnaryOp::Erf: return d ? "kn_erf(" + x + ")" : "((float) kn_erf((double) (" + x + ")))";
+        case UnaryOp::Erf:
+            if (in == DType::F16) return "kn_erf_half(" + x + ")";
+            return d ? "kn_erf(" + x + ")" : "((float) kn_erf((double) (" + x + ")))";
         case UnaryOp::Mish:
+            if (in == DType::F16) return "kn_mish_half(" + x + ")";
             if (!d) return "kn_mish(" + x + ")";
             return "((" + x + ") * " + fn(d, "tanh") + "(" + fn(d, "log1p") + "(" + fn(d, "exp") + "(" + x + "))))";
         case UnaryOp::Softplus:
+            // (halves: 1 + e^-|x| rounded to f32 is off by at most 6e-8, half a unit of the last place of the smallest
+            // normal half; the hardware's 2^x and log2)
+            if (in == DType::F16) return "(__logf(1.0f + __expf(-__builtin_fabsf(" + x + "))) + fmaxf(" + x + ", 0.0f))";
             if (!d) return "(kn_log1p_unit(expf(-__builtin_fabsf(" + x + "))) + fmaxf(" + x + ", 0.0f))";
             return "(" + fn(d, "log1p") + "(" + fn(d, "exp") + "(-" + fn(d, "__builtin_fabs") + "(" + x + "))) + " + fn(d, "fmax") + "(" + x + ", " + (d ? "0.0" : "0.0f") + "))";
         case UnaryOp::ValueCast: {
@@ -346,6 +372,10 @@ std::string emit_expr(std::ostringstream &ss, const ScalarExpr &expr, const std:
                     rhs = "((" + base + ") * (" + base + "))";
                 else if (const_power && rn.constant.f == 3.0)
                     rhs = "((" + base + ") * (" + base + ") * (" + base + "))";
+                else if (const_power && rn.constant.f == 1.5 && rn.constant.dtype != DType::F64)
+                    // x sqrt(x): NaN below zero like the power, +0 for -0 (the product of two -0); only -inf needs a word
+                    // (64M floats: 238 -> what the memory takes)
+                    rhs = "((" + base + ") == -KN_INF ? KN_INF : ((" + base + ") * sqrtf(" + base + ")))";
                 else if (const_power && rn.constant.f == 0.5 && rn.constant.dtype != DType::F64)
                     // (pow(-0, 0.5) is +0 and pow(-inf, 0.5) is +inf, where the square root gives -0 and NaN)
                     rhs = "((" + base + ") == -KN_INF ? KN_INF : (sqrtf(" + base + ") + 0.0f))";
@@ -481,8 +511,12 @@ void emit_header(std::ostringstream &ss, bool idx64, size_t n_ptrs) {
     ss << "struct KnPtrs { void *p[" << std::max<size_t>(n_ptrs, 1) << "]; };\n";
 }
 
-std::string vec_type_decl(const std::string &name, DType t, size_t vec) {
-    return std::string("typedef ") + storage_type(t) + " " + name + " __attribute__((ext_vector_type(" + std::to_string(vec) + ")));\n";
+// `element_aligned`: the vector may start at any element (the hardware takes 128 bit accesses at any address; the type
+// says so, so that the compiler does not assume 16 byte alignment)
+std::string vec_type_decl(const std::string &name, DType t, size_t vec, bool element_aligned = false) {
+    std::string decl = std::string("typedef ") + storage_type(t) + " " + name + " __attribute__((ext_vector_type(" + std::to_string(vec) + ")";
+    if (element_aligned) decl += ", aligned(" + std::to_string(dtype_bytes(t)) + ")";
+    return decl + "));\n";
 }
 
 // Largest power-of-two vector width (in elements) such that every operand can be accessed with aligned vectors
@@ -891,6 +925,40 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
                 if (ok) break;
             }
         }
+        // Many short rows whose length is no multiple of the vector (sums over 33 floats of [2097152, 33]): lanes that
+        // walk a row each would fetch single elements, a line per few lanes. The rows of a dense input follow each other
+        // in memory, so a workgroup takes 256 of them as ONE contiguous run with 128 bit loads into LDS and every
+        // thread folds a row from there.
+        const size_t row_bytes = red_size * es;
+        if (vec == 1 && 16 / es > 1 && kc.rank() == 1 && rc.rank() == 1 && rc.strides[0][0] == 1 && kc.strides[0][0] == 1 &&
+            kc.strides[1][0] == (int64_t) red_size && red_size >= 3 && row_bytes <= 240 && kept_size >= 16384 &&
+            input.offset_bytes % 16 == 0 && kept_size * red_size < (1ull << 31)) {
+            const size_t ve = 16 / es;
+            ss << vec_type_decl("V", in_dtype, ve);
+            ss << "extern \"C\" __global__ __launch_bounds__(256) void kn_reduce(KnPtrs ptrs) {\n";
+            ss << "    const SI *in = (const SI *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
+            ss << "    __shared__ __attribute__((aligned(16))) SI tile[" << 256 * red_size << "];\n";
+            ss << "    const idx_t row0 = (idx_t) blockIdx.x * (idx_t) 256;\n";
+            ss << "    const idx_t rows = (idx_t) " << kept_size << " - row0 < (idx_t) 256 ? (idx_t) " << kept_size << " - row0 : (idx_t) 256;\n";
+            ss << "    const SI *src = in + row0 * (idx_t) " << red_size << ";\n";
+            ss << "    const idx_t elems = rows * (idx_t) " << red_size << ", vecs = elems / (idx_t) " << ve << ";\n";
+            // (256 rows are a whole number of vectors: every run starts on a 16 byte boundary)
+            ss << "#pragma unroll 4\n    for (idx_t v = (idx_t) threadIdx.x; v < vecs; v += (idx_t) 256) ((V *) tile)[v] = "
+               << load_expr("V", "(const V *) src + v", is_streaming(input)) << ";\n";
+            ss << "    for (idx_t e = vecs * (idx_t) " << ve << " + (idx_t) threadIdx.x; e < elems; e += (idx_t) 256) tile[e] = src[e];\n";
+            ss << "    __syncthreads();\n";
+            ss << "    if ((idx_t) threadIdx.x < rows) {\n        T acc = kn_identity();\n";
+            ss << "        const SI *mine = tile + (idx_t) threadIdx.x * (idx_t) " << red_size << ";\n";
+            ss << "#pragma unroll 11\n        for (int j = 0; j < " << red_size << "; j++) acc = kn_f(acc, kn_pre(" << from_storage(in_dtype, "mine[j]") << "));\n";
+            ss << "        out[row0 + (idx_t) threadIdx.x] = " << to_storage(dtype, "kn_post(acc)") << ";\n    }\n}\n";
+            spec.block = 256;
+            spec.grid = ceil_div_u32(kept_size, 256);
+            spec.source = ss.str();
+            note << "short rows, 256 at a time through LDS";
+            spec.strategy = note.str();
+            if (split) split->parts = 1;
+            return spec;
+        }
         size_t red_vecs = red_size / vec;
         size_t G = red_vecs >= 2048 ? 256 : red_vecs >= 128 ? 64 : red_vecs >= 16 ? 16 : 1;
         size_t block = 256, rows_per_block = block / G;
@@ -1118,7 +1186,21 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         }
         if (ok) break;
     }
-    size_t nv = size / vec;
+    // Rows whose length is no multiple of the vector, or that start at any element (rows of 50257 floats follow each
+    // other at every alignment): still whole vectors. Vectors may start at any element, and the last vector of a row
+    // ends with the row, overlapping the one before it: the elements it repeats are left out of the sums and written
+    // twice with the same value. Only for rows that are held in registers, from a few vectors per lane on.
+    bool ragged = false;
+    if (vec == 1 && 16 / max_bytes > 1 && size >= 4096 && size <= (size_t) 64 * 1024) {
+        bool ok = true;
+        for (size_t k = 0; k < ops.size() && ok; k++) ok = k == 0 ? axis_strides[k] == 1 : (axis_strides[k] == 0 || axis_strides[k] == 1);
+        if (ok) {
+            vec = 16 / max_bytes;
+            ragged = true;
+        }
+    }
+    const size_t rem = size % vec;  // elements of the last vector that are its own (0: all of them)
+    size_t nv = (size + vec - 1) / vec;
     // G lanes share a row; the row stays in registers when every lane holds at most MAX_ITEMS vectors: 64 elements,
     // which the kernel keeps as floats. (With 16 vectors of 8 halves a lane of 1024 would hold 128 and spill: f16
     // [1046, 128256] 396 us held against 240 us read again per pass; single elements held up to 64 instead of 16: f32
@@ -1147,7 +1229,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     emit_header(ss, idx64, ops.size());
     for (size_t k = 0; k < ops.size(); k++) {
         ss << "typedef " << storage_type(ops[k].dtype) << " S" << k << ";\n";
-        if (vec > 1) ss << vec_type_decl("V" + std::to_string(k), ops[k].dtype, vec);
+        if (vec > 1) ss << vec_type_decl("V" + std::to_string(k), ops[k].dtype, vec, ragged);
     }
     // which operands feed the prologue / epilogue
     std::vector<bool> in_pre(ops.size(), false), in_post(ops.size(), false);
@@ -1389,7 +1471,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     // `seq` rows, as long as enough workgroups remain to fill the chip.
     std::vector<bool> staged(ops.size(), false);
     size_t seq = 1, staged_bytes = 0;
-    if (cached && vec > 1) {
+    if (cached && vec > 1 && !ragged) {
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_post[k] || in_pre[k] || axis_strides[k] != 1) continue;
             bool invariant = true;
@@ -1414,6 +1496,8 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     const bool check_i = cached && items * G != nv;
 
     ss << "#define VEC " << vec << "\n#define ITEMS " << items << "\n#define G " << G << "\n";
+    // whether element j of vector position i is that vector's own (not a repeat of the vector before the row's last)
+    if (ragged && rem != 0) ss << "#define KN_OWN(i, j) ((i) != (idx_t) " << (nv - 1) << " || (j) >= " << (vec - rem) << ")\n";
     ss << "KN_DEV float kn_max(float a, float b) { return fmaxf(a, b); }\nKN_DEV float kn_add(float a, float b) { return a + b; }\n";
     ss << "KN_DEV float kn_min(float a, float b) { return fminf(a, b); }\n";
     auto emit_fold = [&](const std::string &indent, const std::string &src) {
@@ -1448,13 +1532,21 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         if (nw > 1) ss << "    " << var << " = kn_block_reduce<" << nw << ">(" << var << ", " << f << ", lds_" << var << ");\n";
         else ss << "    " << var << " = kn_group_reduce<G>(" << var << ", " << f << ");\n";
     };
+    // element offset along the axis of vector position `i` of operand k: the last vector of a ragged row ends with the row
+    const bool overlap = ragged && rem != 0;
+    auto axis_offset = [&](size_t k, const std::string &i) {
+        if (axis_strides[k] == 0) return std::string("(idx_t) 0");
+        if (!overlap) return i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec);
+        KN_ASSERT(axis_strides[k] == 1);
+        return "(" + i + " == (idx_t) " + std::to_string(nv - 1) + " ? (idx_t) " + std::to_string(size - vec) + " : " + i + " * (idx_t) " + std::to_string(vec) + ")";
+    };
     // the prologue operands of vector position `i` (in vector units along the axis): loaded into `a<k>`, either
     // declared on the spot or assigned to an element of a register array that was declared earlier (`slot`)
     std::string pre_base = "base";  // the row offsets that the prologue loads start from
     auto emit_pre_loads = [&](const std::string &indent, const std::string &i, const std::string &slot) {
         for (size_t k = 1; k < ops.size(); k++) {
             if (!in_pre[k]) continue;
-            std::string o = "(" + pre_base + "[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
+            std::string o = "(" + pre_base + "[" + std::to_string(k) + "] + " + axis_offset(k, i) + ")";
             bool v = vec > 1 && axis_strides[k] == 1;
             std::string lhs = slot.empty() ? std::string("const ") + (v ? "V" : "S") + std::to_string(k) + " a" + std::to_string(k)
                                            : "a" + std::to_string(k) + "[" + slot + "]";
@@ -1490,7 +1582,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
                 ss << indent << "const V" << k << " b" << k << " = lds_b" << k << "[" << i << "];\n";
                 continue;
             }
-            std::string o = "(base[" + std::to_string(k) + "] + " + i + " * (idx_t) " + i64_str(axis_strides[k] * (int64_t) vec) + ")";
+            std::string o = "(base[" + std::to_string(k) + "] + " + axis_offset(k, i) + ")";
             bool v = vec > 1 && axis_strides[k] == 1;
             std::string lhs = slot.empty() ? std::string("const ") + (v ? "V" : "S") + std::to_string(k) + " b" + std::to_string(k)
                                            : "b" + std::to_string(k) + "[" + slot + "]";
@@ -1501,7 +1593,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     auto emit_post_store = [&](const std::string &indent, const std::string &i, const std::string &src, const std::string &slot) {
         emit_post_loads(indent, i, "");  // (those not requested ahead)
         const std::string pick = slot.empty() ? std::string() : "[" + slot + "]";
-        std::string o0 = "(base[0] + " + i + " * (idx_t) " + i64_str(axis_strides[0] * (int64_t) vec) + ")";
+        std::string o0 = "(base[0] + " + axis_offset(0, i) + ")";
         auto call = [&](const std::string &j) {
             std::string c = row_dtype == DType::F16 ? "kn_post(kn_r16(" + src + "[" + j + "])" : "kn_post(" + src + "[" + j + "]";
             for (size_t k = 1; k < ops.size(); k++) {
@@ -1564,7 +1656,14 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         emit_pre_apply("        ", "x[it]", "it");
         if (check_i)
             ss << "        if (!(i < (idx_t) " << nv << ")) for (int j = 0; j < VEC; j++) x[it][j] = " << identity << ";\n";
-        emit_fold("        ", "x[it]");
+        if (overlap) {
+            // the last vector repeats VEC - rem elements of the one before it: those stay out of the fold
+            ss << "        {\n            float own[VEC];\n            for (int j = 0; j < VEC; j++) own[j] = KN_OWN(i, j) ? x[it][j] : " << identity << ";\n";
+            emit_fold("            ", "own");
+            ss << "        }\n";
+        } else {
+            emit_fold("        ", "x[it]");
+        }
         ss << "    }\n";
         if (seq > 1) {
             ss << "    if (rs + 1 < " << seq << ") {\n    const idx_t row = " << seq_row << " + (idx_t) (rs + 1) * (idx_t) " << rows_per_block << ";\n";
@@ -1577,7 +1676,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         // layernorm with the same number of elements in every lane: per-lane mean and centred sum of squares,
         // combined pairwise in a single pass over the lanes instead of one pass for the mean and one for the
         // variance (one barrier instead of two when a row spans several waves)
-        const bool one_pass = !softmax && !rowred && !check_i && G > 1;
+        const bool one_pass = !softmax && !rowred && !check_i && !overlap && G > 1;
         if (!one_pass) reduce("m", fold_fn);
         if (!rowred) ss << "    float s = 0.0f;\n";
         if (rowred) {
@@ -1586,7 +1685,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
         } else if (softmax) {
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
             ss << "        for (int j = 0; j < VEC; j++) {\n            const float e = (i < (idx_t) " << nv << ") ? kn_exp(x[it][j] - m) : 0.0f;\n";
-            ss << "            x[it][j] = e;\n            s += e;\n        }\n    }\n";
+            ss << "            x[it][j] = e;\n            s += " << (overlap ? "KN_OWN(i, j) ? e : 0.0f" : "e") << ";\n        }\n    }\n";
             reduce("s", "kn_add");
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        for (int j = 0; j < VEC; j++) x[it][j] = x[it][j] / s;\n    }\n";
         } else if (one_pass) {
@@ -1601,7 +1700,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
             ss << "    const float mean = m / (float) " << size << ".0f;\n";
             ss << "#pragma unroll\n    for (int it = 0; it < ITEMS; it++) {\n        const idx_t i = lane + (idx_t) it * (idx_t) G;\n";
             ss << "        for (int j = 0; j < VEC; j++) {\n            const float d = (i < (idx_t) " << nv << ") ? (x[it][j] - mean) : 0.0f;\n";
-            ss << "            x[it][j] = d;\n            s += d * d;\n        }\n    }\n";
+            ss << "            x[it][j] = d;\n            s += " << (overlap ? "KN_OWN(i, j) ? d * d : 0.0f" : "d * d") << ";\n        }\n    }\n";
             reduce("s", "kn_add");
         }
         if (!softmax && !rowred) {
@@ -1686,6 +1785,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     spec.grid = ceil_div_u32(static_size, rows_per_block * seq);
     std::ostringstream note;
     note << (softmax ? "softmax" : (rowred ? "row statistic + elementwise" : "layernorm")) << " G=" << G << " vec=" << vec << " items=" << items << (cached ? " cached" : " streamed");
+    if (ragged) note << " vectors at any element" << (rem != 0 ? ", last one overlapping" : "");
     if (seq > 1) note << " rows=" << seq;
     spec.strategy = note.str();
     return spec;

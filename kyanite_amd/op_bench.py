@@ -112,6 +112,10 @@ def _cases():
     rows_case("softmax", (8, 1000, 4096), 1)
     rows_case("softmax", (4096, 16384), 0)
     rows_case("layernorm", (32, M), 1)
+    # rows whose length is no multiple of the 128 bit vector: a vocabulary of 50257 entries
+    rows_case("softmax", (2048, 50257), 1)
+    rows_case("layernorm", (2048, 50257), 1)
+    rows_case("softmax", (4096, 50257), 1, f16)
 
     def conv_case(name, n, c, h, w, oc, k, stride=1, pad=None):
         pad = k // 2 if pad is None else pad

@@ -2347,3 +2347,53 @@ def gated_matmul_wide():
 def gated_matmul_gate_used_elsewhere():
     """the gate is an output too: the three launches stay"""
     return _gated_feed_forward(306, 96, 128, 160, extra_use=True)
+
+
+@case
+def rows_of_odd_length():
+    """rows held in registers whose length is no multiple of the 128 bit vector and whose start falls on any element:
+    vectors at any alignment, the last one overlapping its neighbour (its repeated elements stay out of the sums);
+    softmax with a scaled input, layernorm with gamma / beta, an RMS norm, in f32 and f16; a slice that starts one
+    element into each row (length a multiple of the vector, start not); -inf entries next to the row's end"""
+    g = Graph()
+    rng = np.random.default_rng(307)
+    a = rng.standard_normal((5, 4097)).astype(np.float32)
+    a[2, 4090:] = -np.inf
+    a[3, 4096] = 30.0
+    xa = g.input([5, 4097])
+    g.output(g.softmax(g.mul(xa, g.scalar(0.5)), 1))
+    gamma, beta = g.constant([4097], rng.standard_normal(4097).astype(np.float32)), g.constant([4097], rng.standard_normal(4097).astype(np.float32))
+    b = rng.standard_normal((7, 4097)).astype(np.float32)
+    g.output(g.add(g.mul(g.layernorm(g.input([7, 4097]), 1, 1e-5), gamma), beta))
+    c = rng.standard_normal((3, 8191)).astype(np.float16)
+    xc = g.input([3, 8191], DType.F16)
+    g.output(g.softmax(xc, 1))
+    g.output(g.layernorm(xc, 1, 1e-3))
+    d = rng.standard_normal((6, 5003)).astype(np.float32)
+    xd = g.input([6, 5003])
+    ms = g.view(g.reduce(g.mul(xd, xd), [1], ReduceOp.MEAN), [6, 1])
+    g.output(g.binary(BinaryOp.DIV, xd, g.unary(UnaryOp.SQRT, g.add(ms, g.scalar(1e-6)))))
+    e = rng.standard_normal((4, 4100)).astype(np.float32)
+    g.output(g.softmax(g.slice(g.input([4, 4100]), 1, 1, 4097), 1))
+    return g, 0, [a, b, c, d, e], None
+
+
+@case
+def reduce_many_short_rows():
+    """sums, maxima and means over short rows whose length is no multiple of the vector: 256 rows at a time through LDS
+    (the last workgroup has fewer; 16500 rows of 7 halves are no whole number of vectors)"""
+    g = Graph()
+    rng = np.random.default_rng(311)
+    a = rng.standard_normal((20001, 33)).astype(np.float32)
+    xa = g.input([20001, 33])
+    g.output(g.reduce(xa, [1], ReduceOp.SUM))
+    g.output(g.reduce(xa, [1], ReduceOp.MEAN))
+    b = rng.standard_normal((16500, 7)).astype(np.float16)
+    b[5, :] = -np.inf
+    b[9, 3] = np.nan
+    g.output(g.reduce(g.input([16500, 7], DType.F16), [1], ReduceOp.MAX))
+    c = rng.integers(-1000, 1000, size=(17000, 13), dtype=np.int32)
+    g.output(g.reduce(g.input([17000, 13], DType.I32), [1], ReduceOp.SUM))
+    d = rng.integers(0, 255, size=(40000, 5), dtype=np.uint8)
+    g.output(g.reduce(g.input([40000, 5], DType.U8), [1], ReduceOp.MIN))
+    return g, 0, [a, b, c, d], None
