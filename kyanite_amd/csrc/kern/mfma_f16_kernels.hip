@@ -206,10 +206,11 @@ __device__ __forceinline__ void store_tiles(const GemmParams &p, const floatx16 
 }
 
 // The store of a gated pair (GemmParams::pair_op): lanes c and c + 16 of an MFMA tile hold G and U of one element of
-// C, column 16 * (virtual column / 32) + c % 16. Both lanes compute the element (the partner's factor comes by a lane
-// exchange) and each stores half of the tile's rows. Roundings as the separate operations place them: the two products,
-// the sigmoid (the hardware's 2^x and reciprocal, like the generated elementwise kernels use for halves) and both
-// multiplications are each rounded to f16.
+// C, column 16 * (virtual column / 32) + c % 16. Each of the two lanes computes and stores half of the tile's rows: the
+// lower lane registers 0 .. 7, the upper one registers 8 .. 15, and one lane exchange per pair of registers hands each
+// the factor it lacks (the lower lane sends its register v + 8 and gets the partner's register v, the upper lane the
+// other way round). Roundings as the separate operations place them: the two products, the sigmoid (the hardware's 2^x
+// and reciprocal, like the generated elementwise kernels use for halves) and both multiplications are each rounded to f16.
 template <int MI, int NI>
 __device__ __forceinline__ void store_tiles_gated(const GemmParams &p, const floatx16 (&acc)[MI][NI], int bz, int row0, int col0) {
     const int lane = threadIdx.x & 63, c = lane & 31, half = lane >> 5;
@@ -223,13 +224,15 @@ __device__ __forceinline__ void store_tiles_gated(const GemmParams &p, const flo
         for (int j = 0; j < NI; j++) {
             const int col = ((col0 + 32 * j) >> 5) * 16 + (c & 15);
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float own = acc[i][j][v], other = __shfl_xor(own, 16);
-                const float g = r16(low ? own : other), u = r16(low ? other : own);
+            for (int v = 0; v < 8; v++) {
+                const float lo = acc[i][j][v], hi = acc[i][j][v + 8];
+                const float got = __shfl_xor(low ? hi : lo, 16);
+                const float g = r16(low ? lo : got), u = r16(low ? got : hi);
                 const float sig = r16(__frcp_rn(1.0f + __expf(-g)));
                 const float act = r16(r16(g * sig) * u);
-                const int row = row0 + 32 * i + 8 * (v >> 2) + 4 * half + (v & 3);
-                if ((v < 8) == low && row < p.m && col < n_out) out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) act;
+                const int w = low ? v : v + 8;
+                const int row = row0 + 32 * i + 8 * (w >> 2) + 4 * half + (w & 3);
+                if (row < p.m && col < n_out) out[(long long) row * p.c_sm + (long long) col * p.c_sn] = (half_t) act;
             }
         }
 }
