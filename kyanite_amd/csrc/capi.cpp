@@ -805,13 +805,11 @@ int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const
         if (output_count != plan.outputs.size()) fail("Wrong output count: expected ", plan.outputs.size(), ", got ", output_count);
         KN_REQUIRE(input_count == 0 || (inputs != nullptr && input_bytes != nullptr));
         KN_REQUIRE(output_count == 0 || (outputs != nullptr && output_bytes != nullptr));
-        std::vector<HostTensor> in;
         for (size_t i = 0; i < input_count; i++) {
             const PlanTensor &t = plan.inputs[i];
             size_t expected = t.shape.size() * dtype_bytes(t.dtype);
             if (input_bytes[i] != expected) fail("Wrong size for input ", i, ": expected ", expected, " bytes, got ", input_bytes[i]);
             KN_REQUIRE(inputs[i] != nullptr || expected == 0);
-            in.push_back(HostTensor(t.dtype, t.shape.shape(), inputs[i]));
         }
         for (size_t i = 0; i < output_count; i++) {
             const PlanTensor &t = plan.outputs[i];
@@ -819,9 +817,7 @@ int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const
             if (output_bytes[i] != expected) fail("Wrong size for output ", i, ": expected ", expected, " bytes, got ", output_bytes[i]);
             KN_REQUIRE(outputs[i] != nullptr || expected == 0);
         }
-        const std::vector<HostTensor> &out = ex->ex.evaluate(in);
-        for (size_t i = 0; i < output_count; i++)
-            if (out[i].nbytes()) std::memcpy(outputs[i], out[i].bytes(), out[i].nbytes());
+        ex->ex.evaluate(inputs, outputs);
         return KNHIP_OK;
     });
 }

@@ -8,9 +8,75 @@ extern "C" hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalW
                                                uint32_t flags);
 
 #include <chrono>
+#include <condition_variable>
+#include <cstring>
+#include <deque>
 #include <map>
+#include <memory>
+#include <mutex>
+#include <thread>
 
 namespace kn {
+
+// The host side of big staging copies, spread over a few threads: one thread copies 10 to 20 GB/s out of memory, less
+// than the copy engine moves across the bus, so a tensor of hundreds of MB would wait for the host otherwise.
+class HostCopyPool {
+public:
+    explicit HostCopyPool(size_t workers) {
+        for (size_t i = 0; i < workers; i++) threads_.emplace_back([this] { work(); });
+    }
+    ~HostCopyPool() {
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            stop_ = true;
+        }
+        wake_.notify_all();
+        for (auto &t : threads_) t.join();
+    }
+    // returns when all of [dst, dst + bytes) is written
+    void copy(void *dst, const void *src, size_t bytes) {
+        const size_t parts = threads_.size() + 1;
+        const size_t part = (bytes / parts + 4095) & ~(size_t) 4095;
+        size_t own = std::min(part, bytes);
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            for (size_t off = own; off < bytes; off += part) {
+                jobs_.push_back({(char *) dst + off, (const char *) src + off, std::min(part, bytes - off)});
+                pending_++;
+            }
+        }
+        wake_.notify_all();
+        std::memcpy(dst, src, own);
+        std::unique_lock<std::mutex> lock(mutex_);
+        done_.wait(lock, [this] { return pending_ == 0; });
+    }
+
+private:
+    struct Job {
+        char *dst;
+        const char *src;
+        size_t bytes;
+    };
+    void work() {
+        std::unique_lock<std::mutex> lock(mutex_);
+        while (true) {
+            wake_.wait(lock, [this] { return stop_ || !jobs_.empty(); });
+            if (stop_) return;
+            Job job = jobs_.front();
+            jobs_.pop_front();
+            lock.unlock();
+            std::memcpy(job.dst, job.src, job.bytes);
+            lock.lock();
+            if (--pending_ == 0) done_.notify_all();
+        }
+    }
+    std::vector<std::thread> threads_;
+    std::mutex mutex_;
+    std::condition_variable wake_, done_;
+    std::deque<Job> jobs_;
+    size_t pending_ = 0;
+    bool stop_ = false;
+};
 
 void hip_check(hipError_t e, const char *what) {
     if (e != hipSuccess) fail("HIP failure in ", what, ": ", hipGetErrorName(e), " (", hipGetErrorString(e), ")");
@@ -68,7 +134,6 @@ HipExecutor::HipExecutor(int device, const Graph &graph, size_t batch_size, cons
     if (!plan_only) HipDevice::check(device);
     const PlannerOptions &options = executor_options.planner;
     plan_ = plan_graph(graph, batch_size, options);
-    for (auto &t : plan_.outputs) tensor_outputs_.push_back(HostTensor(t.dtype, t.shape.shape()));
     if (fuse_small && plan_.steps.size() > 1) {
         std::vector<FusedPart> parts;
         bool ok = true;
@@ -286,6 +351,7 @@ HipExecutor::~HipExecutor() {
     if (stream_) (void) hipStreamSynchronize(stream_);
     if (graph_exec_) (void) hipGraphExecDestroy(graph_exec_);
     if (fused_done_) (void) hipHostFree(fused_done_);
+    for (hipEvent_t e : chunk_events_) (void) hipEventDestroy(e);
     for (void *p : pinned_inputs_) (void) hipHostFree(p);
     for (void *p : pinned_outputs_) (void) hipHostFree(p);
     for (hipModule_t m : modules_) (void) hipModuleUnload(m);
@@ -432,37 +498,61 @@ void HipExecutor::run_async() {
     last_profile_ = std::move(profile);
 }
 
-const std::vector<HostTensor> &HipExecutor::evaluate(const std::vector<HostTensor> &inputs) {
-    if (plan_only_) fail("this executor was created without a device and cannot run");
-    if (inputs.size() != plan_.inputs.size()) fail("Wrong input count: expected ", plan_.inputs.size(), ", got ", inputs.size());
-    for (size_t i = 0; i < inputs.size(); i++) {
-        if (inputs[i].shape != plan_.inputs[i].shape.shape())
-            fail("Wrong shape for input ", i, ": expected ", vec_str(plan_.inputs[i].shape.shape()), ", got ", vec_str(inputs[i].shape));
-        if (inputs[i].dtype != plan_.inputs[i].dtype)
-            fail("Wrong dtype for input ", i, ": expected ", dtype_name(plan_.inputs[i].dtype), ", got ", dtype_name(inputs[i].dtype));
+void HipExecutor::host_copy(void *dst, const void *src, size_t bytes) {
+    // below a few MB a second thread would still be waking up when the first one is done
+    if (bytes < ((size_t) 4 << 20)) {
+        std::memcpy(dst, src, bytes);
+        return;
     }
+    if (!copy_pool_) copy_pool_ = std::make_unique<HostCopyPool>(3);
+    copy_pool_->copy(dst, src, bytes);
+}
+
+void HipExecutor::evaluate(const void *const *inputs, void *const *outputs) {
+    if (plan_only_) fail("this executor was created without a device and cannot run");
     hip_check(hipSetDevice(device_), "hipSetDevice");
     allocate_staging();
     // The staging buffers are free: every evaluate ends with a synchronisation, and run_async never touches them.
     // Device work a caller queued through run_async is ordered before the copies below by the stream itself.
     const bool mapped = mapped_io_ && !profile_ && !graph_mode_;
-    for (size_t i = 0; i < inputs.size(); i++) {
-        size_t bytes = inputs[i].nbytes();
-        if (bytes == 0) continue;
-        std::memcpy(pinned_inputs_[i], inputs[i].bytes(), bytes);
+    for (size_t i = 0; i < plan_.inputs.size(); i++) {
+        const size_t bytes = plan_.inputs[i].shape.size() * dtype_bytes(plan_.inputs[i].dtype);
         KN_ASSERT(plan_.inputs[i].shape.has_simple_strides());
-        if (!mapped) hip_check(hipMemcpyAsync(input_ptr(i), pinned_inputs_[i], bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync(H2D)");
+        for (size_t off = 0; off < bytes; off += kCopyChunkBytes) {
+            const size_t n = std::min(kCopyChunkBytes, bytes - off);
+            host_copy((char *) pinned_inputs_[i] + off, (const char *) inputs[i] + off, n);
+            if (!mapped)
+                hip_check(hipMemcpyAsync((char *) input_ptr(i) + off, (char *) pinned_inputs_[i] + off, n, hipMemcpyHostToDevice, stream_),
+                          "hipMemcpyAsync(H2D)");
+        }
     }
+    struct Chunk {
+        size_t output, offset, bytes;
+    };
+    std::vector<Chunk> chunks;
+    for (size_t i = 0; i < plan_.outputs.size(); i++) {
+        const size_t bytes = plan_.outputs[i].shape.size() * dtype_bytes(plan_.outputs[i].dtype);
+        for (size_t off = 0; off < bytes; off += kCopyChunkBytes) chunks.push_back({i, off, std::min(kCopyChunkBytes, bytes - off)});
+    }
+    // an event behind every chunk but the last, so that the host can copy a chunk out while the next ones still move
+    const size_t n_events = chunks.empty() ? 0 : chunks.size() - 1;
     if (mapped) {
         last_profile_ = std::nullopt;
         if (fused_function_) launch_fused(true);
         else for (size_t si = 0; si < plan_.steps.size(); si++) launch_step(si, nullptr, nullptr, true);
     } else {
         run_async();
-        for (size_t i = 0; i < plan_.outputs.size(); i++) {
-            size_t bytes = tensor_outputs_[i].nbytes();
-            if (bytes == 0) continue;
-            hip_check(hipMemcpyAsync(pinned_outputs_[i], output_ptr(i), bytes, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync(D2H)");
+        while (chunk_events_.size() < n_events) {
+            hipEvent_t e = nullptr;
+            hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
+            chunk_events_.push_back(e);
+        }
+        for (size_t c = 0; c < chunks.size(); c++) {
+            const Chunk &ch = chunks[c];
+            hip_check(hipMemcpyAsync((char *) pinned_outputs_[ch.output] + ch.offset, (char *) output_ptr(ch.output) + ch.offset, ch.bytes,
+                                     hipMemcpyDeviceToHost, stream_),
+                      "hipMemcpyAsync(D2H)");
+            if (c < n_events) hip_check(hipEventRecord(chunk_events_[c], stream_), "hipEventRecord");
         }
     }
     // The fused kernel of a small graph reports its own completion: after its last store every thread fences at
@@ -473,20 +563,22 @@ const std::vector<HostTensor> &HipExecutor::evaluate(const std::vector<HostTenso
         // (an acquire load: the outputs are read from page-locked memory right behind it)
         for (int spin = 0; spin < 400000 && !done; spin++) done = __atomic_load_n(fused_done_, __ATOMIC_ACQUIRE) == fused_seq_;
     }
-    if (!done) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
-    for (size_t i = 0; i < plan_.outputs.size(); i++) {
-        HostTensor &t = tensor_outputs_[i];
-        size_t bytes = t.nbytes();
-        if (bytes == 0) continue;
-        // outputs are handed out as shared tensors: never write into storage a caller may still hold
-        if (t.data.use_count() > 1) t = HostTensor(t.dtype, t.shape);
-        std::memcpy(t.bytes_mut(), pinned_outputs_[i], bytes);
-        if (t.dtype == DType::Bool) {
-            for (size_t k = 0; k < bytes; k++)
-                if (t.bytes()[k] > 1) fail("bool output ", i, " holds a value other than 0 or 1");
+    if (mapped && !done) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    for (size_t c = 0; c < chunks.size(); c++) {
+        const Chunk &ch = chunks[c];
+        if (!mapped) {
+            if (c < n_events) hip_check(hipEventSynchronize(chunk_events_[c]), "hipEventSynchronize");
+            else hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
         }
+        host_copy((char *) outputs[ch.output] + ch.offset, (char *) pinned_outputs_[ch.output] + ch.offset, ch.bytes);
     }
-    return tensor_outputs_;
+    if (chunks.empty() && !mapped) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    for (size_t i = 0; i < plan_.outputs.size(); i++) {
+        if (plan_.outputs[i].dtype != DType::Bool) continue;
+        const uint8_t *bytes = (const uint8_t *) outputs[i];
+        for (size_t k = 0, n = plan_.outputs[i].shape.size(); k < n; k++)
+            if (bytes[k] > 1) fail("bool output ", i, " holds a value other than 0 or 1");
+    }
 }
 
 std::string HipExecutor::str() const {

@@ -38,6 +38,8 @@ struct ExecutorOptions {
     PlannerOptions planner;
 };
 
+class HostCopyPool;
+
 class HipExecutor {
 public:
     HipExecutor(int device, const Graph &graph, size_t batch_size, const ExecutorOptions &options = ExecutorOptions());
@@ -45,8 +47,12 @@ public:
     HipExecutor(const HipExecutor &) = delete;
     HipExecutor &operator=(const HipExecutor &) = delete;
 
-    // host tensors in, host tensors out; the returned tensors stay valid until the next call
-    const std::vector<HostTensor> &evaluate(const std::vector<HostTensor> &inputs);
+    // Dense host buffers in, dense host buffers out (executor.rs:117-195; the C ABI has checked counts and sizes).
+    // Every byte crosses host memory once on each side: caller -> page-locked staging -> device and back. Tensors of
+    // more than `kCopyChunkBytes` move in chunks, so that the copy engine works on one chunk while the host copies
+    // the next one (inputs) or the one before (outputs), with the host copies of big chunks spread over a few threads.
+    void evaluate(const void *const *inputs, void *const *outputs);
+    static constexpr size_t kCopyChunkBytes = (size_t) 8 << 20;
     // launch the steps on the executor's stream without any synchronisation (executor.rs:197-258)
     void run_async();
     void synchronize();
@@ -112,7 +118,9 @@ private:
     std::vector<void *> pinned_inputs_, pinned_outputs_;
     bool staging_ready_ = false;
     void allocate_staging();
-    std::vector<HostTensor> tensor_outputs_;
+    std::unique_ptr<HostCopyPool> copy_pool_;   // threads for the host side of big copies, started on first need
+    std::vector<hipEvent_t> chunk_events_;      // one per output chunk of the largest evaluation so far
+    void host_copy(void *dst, const void *src, size_t bytes);
     bool profile_ = false;
     std::optional<Profile> last_profile_;
     bool graph_mode_ = false;

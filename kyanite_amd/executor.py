@@ -95,9 +95,10 @@ class HipExecutor:
         check(lib.knhip_executor_io_info(self._h, is_output, i, byref(dtype), byref(rank), dims, rank.value))
         return DType(dtype.value), [dims[k] for k in range(rank.value)]
 
-    def evaluate(self, inputs):
-        """Dense numpy arrays in, freshly allocated numpy arrays out. Shapes and dtypes are checked like
-        executor.rs:118-127 does."""
+    def evaluate(self, inputs, out=None):
+        """Dense numpy arrays in, numpy arrays out: freshly allocated ones, or the dense arrays of `out` (as the
+        reference hands out the same tensors again on every call, executor.rs:117, 194). Shapes and dtypes are checked
+        like executor.rs:118-127 does."""
         if len(inputs) != len(self.input_info):
             raise KnError(f"Wrong input count: expected {len(self.input_info)}, got {len(inputs)}")
         arrays = []
@@ -108,7 +109,16 @@ class HipExecutor:
             if x.dtype != dtype.numpy:
                 raise KnError(f"Wrong dtype for input {i}: expected {dtype.name}, got {x.dtype}")
             arrays.append(np.ascontiguousarray(x))
-        outputs = [np.empty(dims, dtype.numpy) for dtype, dims in self.output_info]
+        if out is None:
+            outputs = [np.empty(dims, dtype.numpy) for dtype, dims in self.output_info]
+        else:
+            outputs = list(out)
+            if len(outputs) != len(self.output_info):
+                raise KnError(f"Wrong output count: expected {len(self.output_info)}, got {len(outputs)}")
+            for i, (y, (dtype, dims)) in enumerate(zip(outputs, self.output_info)):
+                if not isinstance(y, np.ndarray) or list(y.shape) != dims or y.dtype != dtype.numpy or not y.flags.c_contiguous \
+                        or not y.flags.writeable:
+                    raise KnError(f"Output {i} must be a writeable dense {dtype.name} array of shape {dims}")
         n_in, n_out = len(arrays), len(outputs)
         in_ptrs = (c_void_p * max(n_in, 1))(*[a.ctypes.data for a in arrays])
         in_bytes = (c_size_t * max(n_in, 1))(*[a.nbytes for a in arrays])
