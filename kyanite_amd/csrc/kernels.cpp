@@ -128,10 +128,11 @@ template<typename T> KN_DEV T kn_shfl_xor(T v, int mask) {
         __builtin_memcpy(&v, &w, sizeof(T));
         return v;
     } else {
-        int w[2]; __builtin_memcpy(w, &v, 8);
-        w[0] = __shfl_xor(w[0], mask, 64);
-        w[1] = __shfl_xor(w[1], mask, 64);
-        __builtin_memcpy(&v, w, 8);
+        static_assert(sizeof(T) % 4 == 0, "shuffled word by word");
+        int w[sizeof(T) / 4]; __builtin_memcpy(w, &v, sizeof(T));
+#pragma unroll
+        for (unsigned i = 0; i < sizeof(T) / 4; i++) w[i] = __shfl_xor(w[i], mask, 64);
+        __builtin_memcpy(&v, w, sizeof(T));
         return v;
     }
 }
@@ -842,11 +843,17 @@ size_t reduce_parts(size_t blocks, size_t block_bytes, size_t most) {
 }
 
 KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
-                              ReduceOp rop, const ScalarExpr *pre, ReduceSplit *split) {
+                              ReduceOp rop, const ScalarExpr *pre, ReduceSplit *split, const ReduceStat *stat) {
     const auto &ishape = input.shape.shape();
     // the folded values have the type of the output; with a prologue the loaded operand may be of another type
     const DType dtype = output.dtype, in_dtype = input.dtype;
-    KN_ASSERT(pre ? pre->nodes.back().dtype == dtype : in_dtype == dtype);
+    if (stat) {
+        // pairs of floats out of floats or halves (a prologue gives floats)
+        KN_ASSERT(dtype == DType::F32 && (pre ? pre->nodes.back().dtype == DType::F32 : (in_dtype == DType::F32 || in_dtype == DType::F16)));
+        rop = ReduceOp::Sum;
+    } else {
+        KN_ASSERT(pre ? pre->nodes.back().dtype == dtype : in_dtype == dtype);
+    }
 
     // split axes into kept and reduced
     std::vector<size_t> kept_shape, red_shape;
@@ -893,9 +900,11 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
 
     std::ostringstream ss;
     emit_header(ss, idx64, 2);
-    ss << "typedef " << storage_type(dtype) << " S;\ntypedef " << storage_type(in_dtype) << " SI;\ntypedef " << T << " T;\n";
+    ss << "typedef " << storage_type(dtype) << " S;\ntypedef " << storage_type(in_dtype) << " SI;\n";
+    if (!stat) ss << "typedef " << T << " T;\ntypedef T X;\n";
+    else ss << "typedef float X;\n#define KN_PLANE ((idx_t) " << stat->plane << ")\n";
     // the value that is folded: the loaded element, or an elementwise expression of it
-    ss << "KN_DEV T kn_pre(" << compute_type(in_dtype) << " x1) {\n";
+    ss << "KN_DEV X kn_pre(" << compute_type(in_dtype) << " x1) {\n";
     if (pre) {
         std::string res = emit_expr(ss, *pre, "y", [&](size_t operand) {
             KN_ASSERT(operand == 1);
@@ -905,10 +914,51 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
     } else {
         ss << "    return x1;\n}\n";
     }
-    ss << "KN_DEV T kn_f(T a, T b) { return " << binary_expr(bop, dtype, "a", "b") << "; }\n";
-    ss << "KN_DEV T kn_identity() { return " << identity.to_c_str() << "; }\n";
-    ss << "KN_DEV T kn_post(T v) { return "
-       << (rop == ReduceOp::Mean ? "v / (float) " + std::to_string(red_size) + ".0f" : std::string("v")) << "; }\n";
+    if (!stat) {
+        ss << "KN_DEV T kn_f(T a, T b) { return " << binary_expr(bop, dtype, "a", "b") << "; }\n";
+        ss << "KN_DEV T kn_identity() { return " << identity.to_c_str() << "; }\n";
+        ss << "KN_DEV void kn_acc(T &t, X x) { t = kn_f(t, x); }\n";
+        ss << "KN_DEV T kn_post(T v) { return "
+           << (rop == ReduceOp::Mean ? "v / (float) " + std::to_string(red_size) + ".0f" : std::string("v")) << "; }\n";
+        ss << "KN_DEV void kn_store(S *at, T v) { *at = " << to_storage(dtype, "kn_post(v)") << "; }\n";
+    } else if (stat->kind == ReduceStat::MaxSumExp) {
+        // a: the maximum so far, b: sum of exp(x - a). An element of -inf adds nothing (a row of nothing else ends as
+        // (-inf, 0) and its results as NaN, like exp(-inf - -inf)); +inf or NaN make the sum NaN, like exp(inf - inf).
+        ss << R"KN(struct T { float a, b; };
+KN_DEV T kn_identity() { return T{-KN_INF, 0.0f}; }
+KN_DEV void kn_acc(T &t, float x) {
+    const float e = __expf(-fabsf(x - t.a));  // (a term of a sum of many: the hardware's 2^x, a few 1e-7 off)
+    const float b = x > t.a ? t.b * e + 1.0f : t.b + e;
+    t.b = x == -KN_INF ? t.b : (x == KN_INF ? __builtin_nanf("") : b);
+    t.a = fmaxf(t.a, x);
+}
+KN_DEV T kn_f(T p, T q) {
+    const float m = fmaxf(p.a, q.a);
+    const float sp = p.a == m ? p.b : p.b * expf(p.a - m), sq = q.a == m ? q.b : q.b * expf(q.a - m);
+    return T{m, sp + sq};
+}
+KN_DEV void kn_store(S *at, T v) { at[0] = v.a; at[KN_PLANE] = 1.0f / v.b; }
+)KN";
+    } else {
+        // (count, mean, M2): Welford per element, the reciprocal of the count from the hardware (the mean moves by
+        // d / n, so an ulp of 1 / n is an ulp of a correction); Chan's combination between accumulators
+        ss << R"KN(struct T { float n, mean, m2; };
+KN_DEV T kn_identity() { return T{0.0f, 0.0f, 0.0f}; }
+KN_DEV void kn_acc(T &t, float x) {
+    t.n += 1.0f;
+    const float d = x - t.mean;
+    t.mean += d * __frcp_rn(t.n);
+    t.m2 += d * (x - t.mean);
+}
+KN_DEV T kn_f(T p, T q) {
+    const float n = p.n + q.n;
+    if (n == 0.0f) return p;
+    const float d = q.mean - p.mean, r = q.n / n;
+    return T{n, p.mean + d * r, (p.m2 + q.m2) + d * d * (p.n * r)};
+}
+)KN";
+        ss << "KN_DEV void kn_store(S *at, T v) { at[0] = v.mean; at[KN_PLANE] = 1.0f / sqrtf(v.m2 / v.n + " << DScalar::f32(stat->eps).to_c_str() << "); }\n";
+    }
 
     const std::string preamble = ss.str();
     const bool may_split = split != nullptr && dtype != DType::Bool;
@@ -930,7 +980,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         // in memory, so a workgroup takes 256 of them as ONE contiguous run with 128 bit loads into LDS and every
         // thread folds a row from there.
         const size_t row_bytes = red_size * es;
-        if (vec == 1 && 16 / es > 1 && kc.rank() == 1 && rc.rank() == 1 && rc.strides[0][0] == 1 && kc.strides[0][0] == 1 &&
+        if (!stat && vec == 1 && 16 / es > 1 && kc.rank() == 1 && rc.rank() == 1 && rc.strides[0][0] == 1 && kc.strides[0][0] == 1 &&
             kc.strides[1][0] == (int64_t) red_size && red_size >= 3 && row_bytes <= 240 && kept_size >= 16384 &&
             input.offset_bytes % 16 == 0 && kept_size * red_size < (1ull << 31)) {
             const size_t ve = 16 / es;
@@ -998,16 +1048,16 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         emit_decompose(ss, "            ", "r", rdims, rstrides, {"o"});
         if (vec > 1) {
             ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
-            ss << "            for (int j = 0; j < " << vec << "; j++) acc[(i + j) & 3] = kn_f(acc[(i + j) & 3], " << "kn_pre(" + from_storage(in_dtype, "v[j]") + ")" << ");\n";
+            ss << "            for (int j = 0; j < " << vec << "; j++) kn_acc(acc[(i + j) & 3], " << "kn_pre(" + from_storage(in_dtype, "v[j]") + ")" << ");\n";
         } else {
-            ss << "            acc[i & 3] = kn_f(acc[i & 3], " << "kn_pre(" + from_storage(in_dtype, "in[o]") + ")" << ");\n";
+            ss << "            kn_acc(acc[i & 3], " << "kn_pre(" + from_storage(in_dtype, "in[o]") + ")" << ");\n";
         }
         ss << "        }\n    }\n";
         ss << "    T total = kn_f(kn_f(acc[0], acc[1]), kn_f(acc[2], acc[3]));\n";
         if (G == 256) ss << "    total = kn_block_reduce<4>(total, kn_f, lds);\n";
         else if (G > 1) ss << "    total = kn_group_reduce<" << G << ">(total, kn_f);\n";
         if (parts > 1) ss << "    if (lane == 0) ((T *) ptrs.p[1])[part * (idx_t) " << kept_size << " + row] = total;\n}\n";
-        else ss << "    if (lane == 0) out[o_out] = " << to_storage(dtype, "kn_post(total)") << ";\n}\n";
+        else ss << "    if (lane == 0) kn_store(out + o_out, total);\n}\n";
         spec.block = (uint32_t) block;
         spec.grid = ceil_div_u32(blocks * parts, 1);
         note << "row G=" << G << " vec=" << vec << " iters=" << iters;
@@ -1017,10 +1067,11 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         size_t vec = 1;
         if (kc.strides[1].back() == 1 && kc.strides[0].back() == 1) {
             for (vec = 16 / es; vec > 1; vec /= 2) {
+                // (pairs are stored float by float: only the loads are vectors then)
                 bool ok = kc.shape.back() % vec == 0 && input.offset_bytes % (int64_t) (vec * es) == 0 &&
-                          output.offset_bytes % (int64_t) (vec * dtype_bytes(dtype)) == 0;
+                          (stat || output.offset_bytes % (int64_t) (vec * dtype_bytes(dtype)) == 0);
                 for (size_t a = 0; a + 1 < kc.rank(); a++)
-                    ok &= kc.strides[0][a] % (int64_t) vec == 0 && kc.strides[1][a] % (int64_t) vec == 0;
+                    ok &= (stat || kc.strides[0][a] % (int64_t) vec == 0) && kc.strides[1][a] % (int64_t) vec == 0;
                 for (size_t a = 0; a < rc.rank(); a++) ok &= rc.strides[0][a] % (int64_t) vec == 0;
                 if (ok) break;
             }
@@ -1042,7 +1093,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         kdims.back() /= vec;
         kstrides[0].back() *= (int64_t) vec;
         kstrides[1].back() *= (int64_t) vec;
-        if (vec > 1) ss << vec_type_decl("V", in_dtype, vec) << vec_type_decl("VO", dtype, vec);
+        if (vec > 1) ss << vec_type_decl("V", in_dtype, vec) << (stat ? std::string() : vec_type_decl("VO", dtype, vec));
         ss << "extern \"C\" __global__ __launch_bounds__(" << block << ") void kn_reduce(KnPtrs ptrs) {\n";
         ss << "    const SI *in = (const SI *) ptrs.p[0];\n    S *out = (S *) ptrs.p[1];\n";
         if (TY > 1) ss << "    __shared__ T lds[" << TY << "][" << vec << "][" << TX << "];\n";
@@ -1064,9 +1115,9 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         emit_decompose(ss, "            ", "r", rc.shape, rc.strides, {"o"});
         if (vec > 1) {
             ss << "            const V v = " << load_expr("V", "in + o", is_streaming(input)) << ";\n#pragma unroll\n";
-            ss << "            for (int j = 0; j < " << vec << "; j++) acc[j] = kn_f(acc[j], " << "kn_pre(" + from_storage(in_dtype, "v[j]") + ")" << ");\n";
+            ss << "            for (int j = 0; j < " << vec << "; j++) kn_acc(acc[j], " << "kn_pre(" + from_storage(in_dtype, "v[j]") + ")" << ");\n";
         } else {
-            ss << "            acc[0] = kn_f(acc[0], " << "kn_pre(" + from_storage(in_dtype, "in[o]") + ")" << ");\n";
+            ss << "            kn_acc(acc[0], " << "kn_pre(" + from_storage(in_dtype, "in[o]") + ")" << ");\n";
         }
         ss << "        }\n    }\n";
         if (TY > 1) {
@@ -1079,11 +1130,11 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         if (parts > 1) {
             ss << "        T *slot = (T *) ptrs.p[1] + (part * (idx_t) " << kept_vecs << " + kv) * (idx_t) " << vec << ";\n";
             ss << "        for (int j = 0; j < " << vec << "; j++) slot[j] = acc[j];\n";
-        } else if (vec > 1) {
+        } else if (vec > 1 && !stat) {
             ss << "        VO o;\n        for (int j = 0; j < " << vec << "; j++) o[j] = " << to_storage(dtype, "kn_post(acc[j])") << ";\n";
             ss << "        *(VO *) (out + o_out) = o;\n";
         } else {
-            ss << "        out[o_out] = " << to_storage(dtype, "kn_post(acc[0])") << ";\n";
+            ss << "        for (int j = 0; j < " << vec << "; j++) kn_store(out + o_out + j, acc[j]);\n";
         }
         ss << "    }\n}\n";
         spec.block = (uint32_t) block;
@@ -1095,7 +1146,7 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         // (neighbouring threads read neighbouring partial results), or a wave per result when there are few results
         // and many slices, each lane folding every 64th slice before the lanes are combined
         note << " parts=" << parts;
-        const size_t FG = kept_size <= 4096 && parts >= 64 ? 64 : 1;
+        const size_t FG = kept_size <= 4096 && parts >= 16 ? 64 : 1;
         std::ostringstream fs;
         fs << preamble;
         fs << "extern \"C\" __global__ __launch_bounds__(256) void kn_reduce_final(KnPtrs ptrs) {\n";
@@ -1104,13 +1155,15 @@ KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &o
         fs << "    const idx_t lane = (idx_t) (threadIdx.x % " << FG << ");\n";
         fs << "    if (i >= (idx_t) " << kept_size << ") return;\n    idx_t o_out = 0;\n";
         emit_decompose(fs, "    ", "i", kc.shape, {kc.strides[0]}, {"o_out"});
-        fs << "    T acc = part[lane * (idx_t) " << kept_size << " + i];\n#pragma unroll 8\n";
+        if (FG > parts) fs << "    T acc = lane < (idx_t) " << parts << " ? part[lane * (idx_t) " << kept_size << " + i] : kn_identity();\n#pragma unroll 8\n";
+        else fs << "    T acc = part[lane * (idx_t) " << kept_size << " + i];\n#pragma unroll 8\n";
         fs << "    for (idx_t s = lane + (idx_t) " << FG << "; s < (idx_t) " << parts << "; s += (idx_t) " << FG << ") acc = kn_f(acc, part[s * (idx_t) " << kept_size << " + i]);\n";
         if (FG > 1) fs << "    acc = kn_group_reduce<" << FG << ">(acc, kn_f);\n";
-        fs << "    if (lane == 0) out[o_out] = " << to_storage(dtype, "kn_post(acc)") << ";\n}\n";
+        fs << "    if (lane == 0) kn_store(out + o_out, acc);\n}\n";
         split->parts = parts;
         split->kept_size = kept_size;
         split->partial_dtype = dtype == DType::F16 ? DType::F32 : dtype;
+        split->partial_words = !stat ? 1 : (stat->kind == ReduceStat::MaxSumExp ? 2 : 3);
         split->final.name = "kn_reduce_final";
         split->final.n_ptrs = 2;
         split->final.block = 256;
@@ -1219,6 +1272,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
     }
     size_t items = (nv + G - 1) / G;
     bool cached = items <= MAX_ITEMS;
+    if (!cached) spec.row_access = KernelSpec::RowsStreamed;
     constexpr size_t min_block = 256;  // (rows that span several waves get a workgroup each: G is 256 or 1024 then)
     size_t block = std::max<size_t>(G, min_block);
     size_t rows_per_block = block / G;
@@ -1309,6 +1363,7 @@ KernelSpec make_row_kernel(const RowKernelDesc &desc) {
                 if (concrete_size(outer_shape) * ((inner + tx - 1) / tx) >= 1024) break;
             }
         }
+        spec.row_access = held ? KernelSpec::RowsHeld : KernelSpec::ColumnsStreamed;
         const size_t column_blocks = (inner + TX - 1) / TX;
         std::vector<std::vector<int64_t>> outer_strides(ops.size());
         for (size_t k = 0; k < ops.size(); k++) outer_strides[k].assign(sc.strides[k].begin(), sc.strides[k].end() - 1);

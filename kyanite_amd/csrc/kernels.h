@@ -41,6 +41,9 @@ struct KernelSpec {
     uint32_t block = 0;  // threads per workgroup
     size_t n_ptrs = 0;
     std::string strategy;  // human readable note on the specialisation that was picked
+    // Row kernels only: whether the rows are held in registers (read once), or read again per pass by the one workgroup
+    // that owns a row (lanes along the row) or a few columns (lanes across neighbouring columns)
+    enum RowAccess { RowsHeld, RowsStreamed, ColumnsStreamed } row_access = RowsHeld;
 };
 
 // One node of a fused elementwise expression: operands are loaded (`Load`), single-valued constants are inlined
@@ -89,10 +92,24 @@ struct ReduceSplit {
     size_t parts = 1;
     size_t kept_size = 0;
     DType partial_dtype = DType::F32;
+    size_t partial_words = 1;  // elements of `partial_dtype` per partial result (more than one for a ReduceStat)
     KernelSpec final;
 };
+// The statistics of a softmax or a layernorm as a reduction of its own, for rows (or columns) that no workgroup can
+// hold: instead of one value per kept element the kernel folds a pair and stores TWO floats, one at its place in
+// `output` and one `plane` floats behind that (two planes of the kept shape, one after the other):
+//   MaxSumExp: the maximum m of the row and 1 / sum(exp(x - m)), the sum kept relative to the running maximum;
+//   MeanRstd:  the mean and 1 / sqrt(variance + eps), from (count, mean, M2) triples (Welford per element, combined
+//              pairwise after Chan, Golub and LeVeque).
+// `op` is ignored then; -inf, +inf and NaN elements give what exp(x - max) / sum gives element by element.
+struct ReduceStat {
+    enum Kind { MaxSumExp, MeanRstd } kind = MaxSumExp;
+    float eps = 0;
+    size_t plane = 0;
+};
 KernelSpec make_reduce_kernel(const KernelOperand &input, const KernelOperand &output, const std::vector<size_t> &axes,
-                              ReduceOp op, const ScalarExpr *pre = nullptr, ReduceSplit *split = nullptr);
+                              ReduceOp op, const ScalarExpr *pre = nullptr, ReduceSplit *split = nullptr,
+                              const ReduceStat *stat = nullptr);
 
 // Row kernels. The value that gets normalised is `pre(load operands...)`, the value stored is
 // `post(normalised, load operands...)`: this is how a preceding scale / residual add and a following affine

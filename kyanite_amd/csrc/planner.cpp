@@ -458,7 +458,6 @@ private:
                 KN_ASSERT(result_dtype == DType::F32 || result_dtype == DType::F16);
                 auto row = visit_row_inputs(value);
                 if (!row.ok) return VT::missing(row.need);
-                if (auto y = plan_few_long_rows(value, row.value)) return VT::done(*y);
                 // no elementwise consumer was fused: the epilogue is the identity
                 ScalarExpr post;
                 ScalarNode n;
@@ -636,77 +635,126 @@ private:
         return R::done(row);
     }
 
-    // A softmax or layernorm over a few rows of 64 Ki elements or more. The row kernel gives a row to one workgroup,
-    // which reads it three times at what one compute unit can pull (8 rows of 4 Mi floats: 1.6 ms, 0.17 TB/s). The
-    // same arithmetic as separate steps uses the whole chip: the statistic of every row with the reduction that folds
-    // slices of the reduced index side by side, the shifted values, their statistic, and the division. Six passes
-    // over the tensor instead of two, at the rate of the memory.
-    std::optional<PlanTensor> plan_few_long_rows(Value value, const FusedRow &row) {
-        const ValueInfo &info = graph[value];
-        if (!options.split_reduce || info.dtype != DType::F32 || row.inputs.size() != 1 || row.pre.nodes.size() != 1) return std::nullopt;
+    // A softmax or layernorm whose rows no workgroup can hold. The row kernel reads such a row again per pass, with
+    // the one workgroup that owns it: a few rows of a million elements move at what a few compute units can pull
+    // (8 rows of 4 Mi floats: 1.6 ms, 0.17 TB/s), and columns of a tall matrix in runs of 64 bytes per row of lanes
+    // ([4096, 16384] along axis 0: 309 us). As two steps that each use the whole chip the tensor is read twice and
+    // written once at the rate of the memory: the statistics of every row as a reduction that folds pairs (maximum
+    // and sum of exponentials in one pass, or mean and variance; slices of the reduced index side by side when the
+    // rows are few), then an elementwise kernel over (x, statistics) that also applies the epilogue.
+    bool two_pass_rows_ok(const FusedRow &row, const KernelSpec &kernel, DType result_dtype, size_t rows,
+                          const std::vector<PlanTensor> &extra) const {
+        if (!options.split_reduce || result_dtype != DType::F32 || row.kind == RowKernelDesc::Reduce) return false;
+        if (row.inputs.size() != 1 || row.pre.nodes.size() != 1 || row.inputs[0].dtype != DType::F32) return false;
+        for (size_t k = 1; k < extra.size(); k++)
+            if (extra[k].dtype != DType::F32) return false;
+        if (kernel.row_access == KernelSpec::ColumnsStreamed) return true;
+        // lanes along the rows: a workgroup per row is enough once there are four per compute unit
+        return kernel.row_access == KernelSpec::RowsStreamed && rows < 1024;
+    }
+
+    void plan_two_pass_rows(Value value, const FusedRow &row, const PlanTensor &output, const ScalarExpr &post,
+                            const std::vector<PlanTensor> &extra) {
         const PlanTensor &x = row.inputs[0];
         const std::vector<size_t> shape = x.shape.shape();
-        const size_t axis = row.axis, length = shape[axis];
-        if (length < 65536 || concrete_size(shape) / length > 64) return std::nullopt;
-        std::vector<size_t> kept, unit = shape;
+        const size_t axis = row.axis;
+        std::vector<size_t> kept, unit = shape, planes{2};
         for (size_t a = 0; a < shape.size(); a++)
             if (a != axis) kept.push_back(shape[a]);
         unit[axis] = 1;
-        auto along = [&](const PlanTensor &stat) { return stat.view(unit)->broadcast(shape); };
-        auto node = [](ScalarNode::Kind kind) {
+        planes.insert(planes.end(), kept.begin(), kept.end());
+        const bool softmax = row.kind == RowKernelDesc::Softmax;
+
+        // step 1: (maximum, 1 / sum of exponentials) or (mean, 1 / sqrt(variance + eps)) of every row, as two planes
+        PlanTensor stats = alloc_tensor_shared(planes, DType::F32);
+        auto plane = [&](size_t which) { return *stats.slice(0, SliceRange{which, which + 1, 1}).view(kept); };
+        const PlanTensor first = plane(0), second = plane(1);
+        ReduceStat stat;
+        stat.kind = softmax ? ReduceStat::MaxSumExp : ReduceStat::MeanRstd;
+        stat.eps = row.eps;
+        stat.plane = concrete_size(kept);
+        {
+            ReduceSplit split;
+            Step step;
+            step.kind = StepKind::ReduceOp;
+            step.kernel = make_reduce_kernel(kop(x), kop(first), {axis}, ReduceOp::Sum, nullptr, &split, &stat);
+            step.kernel.strategy = std::string(softmax ? "maximum and sum of exponentials: " : "mean and variance: ") + step.kernel.strategy;
+            if (split.parts <= 1) {
+                step.operands = {{x, OperandKind::In}, {stats, OperandKind::Out}};
+                push(std::move(step), value);
+            } else {
+                PlanTensor partial = alloc_tensor_shared({split.parts * split.kept_size * split.partial_words}, split.partial_dtype);
+                step.operands = {{x, OperandKind::In}, {partial, OperandKind::Out}};
+                push(std::move(step), value);
+                Step fold;
+                fold.kind = StepKind::ReduceOp;
+                fold.kernel = std::move(split.final);
+                fold.operands = {{partial, OperandKind::In}, {stats, OperandKind::Out}};
+                push(std::move(fold), value);
+            }
+        }
+
+        // step 2: post(exp(x - maximum) * (1 / sum)) or post((x - mean) * (1 / sqrt(variance + eps)))
+        auto along = [&](const PlanTensor &s) { return s.view(unit)->broadcast(shape); };
+        ScalarExpr expr;
+        auto node = [&](ScalarNode::Kind kind) {
             ScalarNode n;
             n.kind = kind;
             n.dtype = DType::F32;
             return n;
         };
+        auto push_node = [&](ScalarNode n) {
+            expr.nodes.push_back(std::move(n));
+            return expr.nodes.size() - 1;
+        };
         auto load = [&](size_t operand) {
             ScalarNode n = node(ScalarNode::Load);
             n.operand = operand;
-            return n;
+            return push_node(n);
         };
         auto binary = [&](BinaryOp op, size_t a, size_t b) {
             ScalarNode n = node(ScalarNode::Binary);
             n.binary = op;
             n.a = a;
             n.b = b;
-            return n;
+            return push_node(n);
         };
-        auto unary = [&](UnaryOp op, size_t a) {
-            ScalarNode n = node(ScalarNode::Unary);
-            n.unary = op;
-            n.a = a;
-            return n;
-        };
-        auto constant = [&](float v) {
-            ScalarNode n = node(ScalarNode::Const);
-            n.constant = DScalar::f32(v);
-            return n;
-        };
-        const bool softmax = row.kind == RowKernelDesc::Softmax;
-        // the maximum (softmax) or the mean (layernorm) of every row, then the values shifted by it: exp(x - max) or x - mean
-        PlanTensor first = alloc_tensor_shared(kept, DType::F32);
-        push_reduce(value, x, first, {axis}, softmax ? ReduceOp::Max : ReduceOp::Mean, nullptr);
-        PlanTensor shifted = alloc_tensor_shared(shape, DType::F32);
-        ScalarExpr shift;
-        shift.nodes = {load(1), load(2), binary(BinaryOp::Sub, 0, 1)};
-        if (softmax) shift.nodes.push_back(unary(UnaryOp::Exp, 2));
-        plan_scalar_op(shift, {shifted, x, along(first)}, value);
-        // their sum (softmax) or the mean of their squares (layernorm)
-        PlanTensor second = alloc_tensor_shared(kept, DType::F32);
-        ScalarExpr square;
-        square.nodes = {load(1), binary(BinaryOp::Mul, 0, 0)};
-        push_reduce(value, shifted, second, {axis}, softmax ? ReduceOp::Sum : ReduceOp::Mean, softmax ? nullptr : &square);
-        // e / sum, or d * (1 / sqrt(var + eps)) as the row kernel computes it
-        PlanTensor output = alloc_tensor_shared(shape, DType::F32);
-        ScalarExpr last;
+        const size_t lx = load(1), la = load(2), lb = load(3);
+        size_t centred = binary(BinaryOp::Sub, lx, la);
         if (softmax) {
-            last.nodes = {load(1), load(2), binary(BinaryOp::Div, 0, 1)};
-        } else {
-            last.nodes = {load(1), load(2), constant(row.eps), binary(BinaryOp::Add, 1, 2), unary(UnaryOp::Sqrt, 3), constant(1.0f),
-                          binary(BinaryOp::Div, 5, 4), binary(BinaryOp::Mul, 0, 6)};
+            ScalarNode e = node(ScalarNode::Unary);
+            e.unary = UnaryOp::Exp;
+            e.a = centred;
+            centred = push_node(e);
         }
-        plan_scalar_op(last, {output, shifted, along(second)}, value);
-        return output;
+        const size_t normalised = binary(BinaryOp::Mul, centred, lb);
+        // the epilogue behind it: its loads of the normalised value become references to that node, its other loads
+        // move behind (output, x, the two statistics)
+        std::vector<PlanTensor> operands{output, x, along(first), along(second)};
+        for (size_t k = 1; k < extra.size(); k++) operands.push_back(extra[k]);
+        std::vector<size_t> at(post.nodes.size());
+        for (size_t i = 0; i < post.nodes.size(); i++) {
+            ScalarNode n = post.nodes[i];
+            KN_ASSERT(n.kind != ScalarNode::Raw);
+            if (n.kind == ScalarNode::Load && n.operand == SIZE_MAX) {
+                at[i] = normalised;
+                continue;
+            }
+            if (n.kind == ScalarNode::Load) n.operand = 4 + n.operand - 1;
+            if (n.kind == ScalarNode::Unary || n.kind == ScalarNode::Binary) n.a = at[n.a];
+            if (n.kind == ScalarNode::Binary) n.b = at[n.b];
+            at[i] = push_node(n);
+        }
+        // (an epilogue that is the normalised value itself leaves `normalised` as the last node only if nothing
+        // follows it: the result of the expression is its last node)
+        if (at.back() != expr.nodes.size() - 1) {
+            // the result is an earlier node: repeat it through a multiplication by one, which changes no bit of a float
+            ScalarNode one = node(ScalarNode::Const);
+            one.constant = DScalar::f32(1.0f);
+            const size_t c = push_node(one);
+            binary(BinaryOp::Mul, at.back(), c);
+        }
+        plan_scalar_op(expr, operands, value);
     }
 
     // Emit the row kernel for `row_value`, storing `post(normalised, extra...)` as the result of `result_value`.
@@ -735,6 +783,14 @@ private:
         step.kind = row.kind == RowKernelDesc::Softmax ? StepKind::SoftmaxOp
                                                       : (row.kind == RowKernelDesc::Reduce ? StepKind::ReduceOp : StepKind::LayernormOp);
         step.kernel = make_row_kernel(desc);
+        {
+            const auto &full = output.shape.shape();
+            const size_t rows = full[row.axis] == 0 ? 0 : concrete_size(full) / full[row.axis];
+            if (two_pass_rows_ok(row, step.kernel, info.dtype, rows, extra)) {
+                plan_two_pass_rows(row_value, row, output, post_in, extra);
+                return output;
+            }
+        }
         step.operands.push_back({output, OperandKind::Out});
         for (size_t k = 1; k < all.size(); k++) step.operands.push_back({all[k], OperandKind::In});
         push(std::move(step), row_value);

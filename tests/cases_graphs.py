@@ -2197,9 +2197,9 @@ def tiny_products_one_wave_per_result():
 
 @case
 def few_long_rows():
-    """a softmax or layernorm over a few rows of 64 Ki elements or more runs as separate steps that use the whole chip
-    (statistic, shifted values, statistic, division) instead of one workgroup per row: along the last axis, and along a
-    middle axis with three columns behind it"""
+    """a softmax or layernorm over a few rows of 64 Ki elements or more runs as two steps that use the whole chip (the
+    statistics of every row as a reduction over pairs, slices of a row side by side; then one elementwise kernel)
+    instead of one workgroup per row: along the last axis, and along a middle axis with three columns behind it"""
     g = Graph()
     rng = np.random.default_rng(177)
     a, b, c = g.input([3, 70000]), g.input([2, 100000]), g.input([2, 66000, 3])
@@ -2212,6 +2212,41 @@ def few_long_rows():
     assert "softmax_op" not in kinds and "layernorm_op" not in kinds, kinds
     f = lambda *shape: (rng.standard_normal(shape) * 3).astype(np.float32)
     return g, 0, [f(3, 70000), f(2, 100000), f(2, 66000, 3)], None
+
+
+@case
+def rows_in_two_passes():
+    """rows or columns that no workgroup can hold, as a reduction to (maximum, 1 / sum of exponentials) or (mean,
+    1 / sqrt(variance + eps)) and an elementwise kernel that also applies the epilogue: columns of a tall matrix (with
+    columns of -inf, with +inf, with a NaN), a layernorm along axis 0 with gamma and beta behind it, a softmax over a
+    long middle axis, a few long rows with an affine epilogue, and enough rows that no row is cut into slices"""
+    from kyanite_amd import HipExecutor
+    g = Graph()
+    rng = np.random.default_rng(977)
+    tall = (rng.standard_normal((2500, 192)) * 4).astype(np.float32)
+    tall[:, 3] = -np.inf
+    tall[:700, 5] = -np.inf
+    tall[1200, 7] = np.inf
+    tall[2499, 9] = np.nan
+    tall[0, 11] = -np.inf
+    g.output(g.softmax(g.input([2500, 192]), 0))
+    cols = (rng.standard_normal((1500, 96)) * 2 + 5).astype(np.float32)
+    gamma, beta = rng.standard_normal((1, 96)).astype(np.float32), rng.standard_normal((1500, 1)).astype(np.float32)
+    y = g.layernorm(g.input([1500, 96]), 0, 1e-5)
+    g.output(g.add(g.mul(y, g.constant([1, 96], gamma)), g.constant([1500, 1], beta)))
+    middle = rng.standard_normal((40, 3000, 48)).astype(np.float32)
+    g.output(g.softmax(g.input([40, 3000, 48]), 1))
+    long_rows = (rng.standard_normal((4, 100000)) * 3 - 2).astype(np.float32)
+    w = rng.standard_normal((1, 100000)).astype(np.float32)
+    g.output(g.add(g.mul(g.layernorm(g.input([4, 100000]), 1, 1e-3), g.constant([1, 100000], w)), g.scalar(0.5)))
+    many = rng.standard_normal((300, 70000)).astype(np.float32)
+    g.output(g.softmax(g.input([300, 70000]), 1))
+    plan = HipExecutor(0, g, 0, plan_only=True)
+    kinds = plan.step_kinds()
+    assert "softmax_op" not in kinds and "layernorm_op" not in kinds, kinds
+    text = "\n".join(plan.step_str(i) for i in range(plan.step_count()))
+    assert text.count("maximum and sum of exponentials") == 3 and text.count("mean and variance") == 2, text
+    return g, 0, [tall, cols, middle, long_rows, many], None
 
 
 @case
