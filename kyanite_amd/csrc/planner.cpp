@@ -644,10 +644,10 @@ private:
     // rows are few), then an elementwise kernel over (x, statistics) that also applies the epilogue.
     bool two_pass_rows_ok(const FusedRow &row, const KernelSpec &kernel, DType result_dtype, size_t rows,
                           const std::vector<PlanTensor> &extra) const {
-        if (!options.split_reduce || result_dtype != DType::F32 || row.kind == RowKernelDesc::Reduce) return false;
-        if (row.inputs.size() != 1 || row.pre.nodes.size() != 1 || row.inputs[0].dtype != DType::F32) return false;
+        if (!options.split_reduce || (result_dtype != DType::F32 && result_dtype != DType::F16) || row.kind == RowKernelDesc::Reduce) return false;
+        if (row.inputs.size() != 1 || row.pre.nodes.size() != 1 || row.inputs[0].dtype != result_dtype) return false;
         for (size_t k = 1; k < extra.size(); k++)
-            if (extra[k].dtype != DType::F32) return false;
+            if (extra[k].dtype != result_dtype) return false;
         if (kernel.row_access == KernelSpec::ColumnsStreamed) return true;
         // lanes along the rows: a workgroup per row is enough once there are four per compute unit
         return kernel.row_access == KernelSpec::RowsStreamed && rows < 1024;
@@ -719,7 +719,20 @@ private:
             n.b = b;
             return push_node(n);
         };
-        const size_t lx = load(1), la = load(2), lb = load(3);
+        // (halves: computed in f32 from the loaded half and rounded once, like the row kernel's result)
+        const DType dt = x.dtype;
+        auto cast = [&](size_t a, DType to) {
+            ScalarNode n = node(ScalarNode::Unary);
+            n.unary = UnaryOp::ValueCast;
+            n.cast_to = to;
+            n.dtype = to;
+            n.a = a;
+            return push_node(n);
+        };
+        size_t lx = load(1);
+        expr.nodes[lx].dtype = dt;
+        if (dt != DType::F32) lx = cast(lx, DType::F32);
+        const size_t la = load(2), lb = load(3);
         size_t centred = binary(BinaryOp::Sub, lx, la);
         if (softmax) {
             ScalarNode e = node(ScalarNode::Unary);
@@ -727,7 +740,8 @@ private:
             e.a = centred;
             centred = push_node(e);
         }
-        const size_t normalised = binary(BinaryOp::Mul, centred, lb);
+        size_t normalised = binary(BinaryOp::Mul, centred, lb);
+        if (dt != DType::F32) normalised = cast(normalised, dt);
         // the epilogue behind it: its loads of the normalised value become references to that node, its other loads
         // move behind (output, x, the two statistics)
         std::vector<PlanTensor> operands{output, x, along(first), along(second)};

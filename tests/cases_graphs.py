@@ -2219,7 +2219,8 @@ def rows_in_two_passes():
     """rows or columns that no workgroup can hold, as a reduction to (maximum, 1 / sum of exponentials) or (mean,
     1 / sqrt(variance + eps)) and an elementwise kernel that also applies the epilogue: columns of a tall matrix (with
     columns of -inf, with +inf, with a NaN), a layernorm along axis 0 with gamma and beta behind it, a softmax over a
-    long middle axis, a few long rows with an affine epilogue, and enough rows that no row is cut into slices"""
+    long middle axis, a few long rows with an affine epilogue, enough rows that no row is cut into slices, and columns
+    of halves (computed in f32, rounded once)"""
     from kyanite_amd import HipExecutor
     g = Graph()
     rng = np.random.default_rng(977)
@@ -2241,12 +2242,16 @@ def rows_in_two_passes():
     g.output(g.add(g.mul(g.layernorm(g.input([4, 100000]), 1, 1e-3), g.constant([1, 100000], w)), g.scalar(0.5)))
     many = rng.standard_normal((300, 70000)).astype(np.float32)
     g.output(g.softmax(g.input([300, 70000]), 1))
+    halves = (rng.standard_normal((3000, 128)) * 2 + 1).astype(np.float16)
+    scale = rng.standard_normal((1, 128)).astype(np.float16)
+    g.output(g.mul(g.layernorm(g.input([3000, 128], DType.F16), 0, 1e-3), g.constant([1, 128], scale, DType.F16)))
+    g.output(g.softmax(g.input([3000, 128], DType.F16), 0))
     plan = HipExecutor(0, g, 0, plan_only=True)
     kinds = plan.step_kinds()
     assert "softmax_op" not in kinds and "layernorm_op" not in kinds, kinds
     text = "\n".join(plan.step_str(i) for i in range(plan.step_count()))
-    assert text.count("maximum and sum of exponentials") == 3 and text.count("mean and variance") == 2, text
-    return g, 0, [tall, cols, middle, long_rows, many], None
+    assert text.count("maximum and sum of exponentials") == 4 and text.count("mean and variance") == 3, text
+    return g, 0, [tall, cols, middle, long_rows, many, halves, halves.copy()], None
 
 
 @case
