@@ -2215,6 +2215,38 @@ def few_long_rows():
 
 
 @case
+def byte_transposes():
+    """elementwise kernels over one-byte elements with a transposed operand: tiles of 128 x 128 with a word of four
+    elements per thread (u8 with a straight operand next to the transposed one, sizes that are no multiple of the tile,
+    i8 with batch axes, bool), and shapes that keep the tiles of 64 x 64 (a length that is no multiple of 4, a
+    broadcast operand)"""
+    from kyanite_amd import HipExecutor
+    g = Graph()
+    rng = np.random.default_rng(433)
+    u8 = lambda *shape: rng.integers(0, 256, size=shape, dtype=np.uint8)
+    a, b = u8(300, 520), u8(520, 300)
+    xa, xb = g.input([300, 520], DType.U8), g.input([520, 300], DType.U8)
+    g.output(g.add(g.permute(xa, [1, 0]), xb))
+    c = rng.integers(-128, 128, size=(3, 5, 132, 260), dtype=np.int8)
+    xc = g.input([3, 5, 132, 260], DType.I8)
+    g.output(g.mul(g.permute(xc, [0, 1, 3, 2]), g.scalar(3, DType.I8)))
+    d = rng.integers(0, 2, size=(256, 384)).astype(bool)
+    e = rng.integers(0, 2, size=(384, 256)).astype(bool)
+    xd, xe = g.input([256, 384], DType.BOOL), g.input([384, 256], DType.BOOL)
+    g.output(g.mul(g.permute(xd, [1, 0]), xe))
+    f = u8(258, 514)
+    xf = g.input([258, 514], DType.U8)
+    g.output(g.add(g.permute(xf, [1, 0]), g.scalar(1, DType.U8)))
+    h, column = u8(260, 512), u8(512, 1)
+    xh = g.input([260, 512], DType.U8)
+    g.output(g.add(g.permute(xh, [1, 0]), g.constant([512, 1], column, DType.U8)))
+    plan = HipExecutor(0, g, 0, plan_only=True)
+    text = [plan.step_str(i) for i in range(plan.step_count())]
+    assert sum("128x128 of bytes" in t for t in text) == 3 and sum("tiles 64x64" in t for t in text) == 2, text
+    return g, 0, [a, b, c, d, e, f, h], None
+
+
+@case
 def rows_in_two_passes():
     """rows or columns that no workgroup can hold, as a reduction to (maximum, 1 / sum of exponentials) or (mean,
     1 / sqrt(variance + eps)) and an elementwise kernel that also applies the epilogue: columns of a tall matrix (with
