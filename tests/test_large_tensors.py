@@ -138,15 +138,23 @@ def test_softmax_rows_past_2_31_elements(hip_device, block):
     check_outputs(small, 0, [sample], cpu_eval_graph(small, 0, [sample]), [got], "softmax rows of a 4 GiB tensor", PARITY_RECORDS)
 
 
-def test_softmax_over_a_middle_axis_past_2_31_elements(hip_device, block):
-    """the normalised axis is not the contiguous one: lanes across columns, every column read again per pass"""
+@pytest.mark.parametrize("two_steps", [True, False])
+def test_softmax_over_a_middle_axis_past_2_31_elements(hip_device, block, two_steps):
+    """the normalised axis is not the contiguous one and no workgroup can hold a column: as a reduction to (maximum,
+    1 / sum of exponentials) and an elementwise kernel, or (with that plan switched off) the row kernel with lanes
+    across columns that reads every column again per pass"""
     batch, length, width = 3, 700, (1 << 20) + 8
     g = Graph()
     x = g.input([batch, length, width], DType.F16)
     g.output(g.softmax(x, 1))
-    plan = HipExecutor(0, g, 0, plan_only=True)
-    assert "columns" in plan.step_str(0) and "typedef long long idx_t" in plan.step_source(0)
-    ex = HipExecutor(hip_device, g, 0)
+    options = {} if two_steps else {"split_reduce": False}
+    plan = HipExecutor(0, g, 0, plan_only=True, **options)
+    if two_steps:
+        assert plan.step_count() == 2 and "maximum and sum of exponentials" in plan.step_str(0)
+        assert all("typedef long long idx_t" in plan.step_source(i) for i in range(2))
+    else:
+        assert "columns" in plan.step_str(0) and "typedef long long idx_t" in plan.step_source(0)
+    ex = HipExecutor(hip_device, g, 0, **options)
     _fill_input(ex, 0, block, batch * length * width)
     _run(ex)
     # 16 neighbouring columns at a time: the first and the last of every batch entry, and either side of the place
