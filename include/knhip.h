@@ -312,14 +312,17 @@ typedef struct knhip_executor knhip_executor;
  * streaming_bytes: operands of at least this size that are touched once per element are read and written with
  *   non-temporal accesses (default 64 MiB; 0: never). mapped_io_bytes: evaluate() of a graph whose inputs and outputs
  *   are at most this many bytes in all reads and writes them in page-locked host memory instead of copying them
- *   to and from the arena (default 64 KiB; 0: never). */
+ *   to and from the arena (default 64 KiB; 0: never). stream_weights_bytes: a plan with at least this many bytes of
+ *   constants reads the constant right operands of its matmuls (under left operands of up to 1024 rows) with the
+ *   non-temporal hint, as streams that cannot stay in the last-level cache from one evaluation to the next (default
+ *   256 MiB; 0: never). */
 typedef struct {
     size_t struct_bytes; /* sizeof(knhip_executor_options), set by knhip_executor_options_default */
     int plan_only, preserve_inputs, step_by_step;
     int fuse_attention, fuse_gated_matmul, group_matmuls, pack_matmul_constants, pointwise_conv_as_matmul, join_elementwise, split_reduce;
     int tiled_transpose, split_conv_channels, plane_conv_any_width;
     int direct_gemm, split_k, tail_split, dot_products;
-    uint64_t streaming_bytes, mapped_io_bytes;
+    uint64_t streaming_bytes, mapped_io_bytes, stream_weights_bytes;
 } knhip_executor_options;
 int knhip_executor_options_default(knhip_executor_options *options);
 

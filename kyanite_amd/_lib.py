@@ -49,7 +49,7 @@ class ExecutorOptionsT(Structure):
                     "plan_only", "preserve_inputs", "step_by_step", "fuse_attention", "fuse_gated_matmul", "group_matmuls", "pack_matmul_constants",
                     "pointwise_conv_as_matmul", "join_elementwise", "split_reduce", "tiled_transpose", "split_conv_channels",
                     "plane_conv_any_width", "direct_gemm", "split_k", "tail_split", "dot_products")] +
-                [("streaming_bytes", c_uint64), ("mapped_io_bytes", c_uint64)])
+                [("streaming_bytes", c_uint64), ("mapped_io_bytes", c_uint64), ("stream_weights_bytes", c_uint64)])
 
 
 class TensorT(Structure):

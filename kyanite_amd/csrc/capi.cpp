@@ -706,6 +706,7 @@ int knhip_executor_options_default(knhip_executor_options *o) {
         o->dot_products = d.planner.gemm.dot_products;
         o->streaming_bytes = d.planner.generator.streaming_bytes;
         o->mapped_io_bytes = d.mapped_io_bytes;
+        o->stream_weights_bytes = d.planner.stream_weights_bytes;
         return KNHIP_OK;
     });
 }
@@ -738,6 +739,7 @@ ExecutorOptions executor_options_from(const knhip_executor_options *o) {
     p.gemm.split_k = o->split_k != 0;
     p.gemm.tail_split = o->tail_split != 0;
     p.gemm.dot_products = o->dot_products != 0;
+    p.stream_weights_bytes = (size_t) o->stream_weights_bytes;
     return e;
 }
 

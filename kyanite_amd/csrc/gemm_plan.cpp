@@ -98,6 +98,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         q.d2_sm = p.d2_sn; q.d2_sn = p.d2_sm;
         p = q;
         lp.swapped = true;
+        p.tuning.stream_b = false;  // (the weight is the left operand now)
     }
     lp.p = p;
     lp.split_k = 1;
@@ -285,6 +286,7 @@ std::string describe_gemm_plan(const GemmLaunchPlan &lp, bool f16) {
     if (lp.skinny_tile) tm = 32, tn = 128;
     ss << (lp.direct ? "direct " : "staged ") << tm << "x" << tn << " bk" << lp.bk;
     if (lp.p.pair_op) ss << " gated pairs";
+    if (lp.direct && lp.p.tuning.stream_b) ss << " weights streamed";
     if (lp.split_k > 1) ss << " split_k=" << lp.split_k << "x" << lp.k_chunk;
     if (lp.tail_split > 1) ss << " head=" << lp.head_tiles << " tail_split=" << lp.tail_split << "x" << lp.tail_k_chunk;
     return ss.str();

@@ -404,7 +404,8 @@ struct DirectSchedule {
     int head_tiles, tail_split, tail_k_chunk;
 };
 
-template <typename T, int MI, int NI, int WM, int WN, int NSTAGE>
+// BSTREAM: the loads of the right operand carry the non-temporal hint (GemmTuning::stream_b)
+template <typename T, int MI, int NI, int WM, int WN, int NSTAGE, bool BSTREAM>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p, DirectSchedule sched) {
     constexpr int WAVES = WM * WN, TM = 32 * MI * WM, TN = 32 * NI * WN, ROW = DIRECT_ROW, BK = ROW / (int) sizeof(T), VEC = 16 / (int) sizeof(T);
     constexpr int A_BYTES = TM * ROW, STAGE = (TM + TN) * ROW;
@@ -494,7 +495,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
         constexpr int l = decltype(lc)::value;
 #if defined(__HIP_DEVICE_COMPILE__)
         if constexpr (l < A_LD) __builtin_amdgcn_global_load_lds((const void *) (a_tile + a_off[l]), dst_a + stage + l * 1024, 16, 0, 0);
-        else __builtin_amdgcn_global_load_lds((const void *) (b_tile + b_off[l - A_LD]), dst_b + stage + (l - A_LD) * 1024, 16, 0, 0);
+        else __builtin_amdgcn_global_load_lds((const void *) (b_tile + b_off[l - A_LD]), dst_b + stage + (l - A_LD) * 1024, 16, 0, BSTREAM ? 2 : 0);
 #endif
     };
     int fetched = 0;  // slices whose loads have been issued
@@ -620,16 +621,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
 template <typename T, int MI, int NI, int WM, int WN, int NSTAGE>
 int launch_direct(dim3 grid, hipStream_t stream, const GemmParams &p, const DirectSchedule &sched) {
     constexpr int LDS_BYTES = NSTAGE * (32 * MI * WM + 32 * NI * WN) * DIRECT_ROW;
-    auto kernel = gemm_direct_kernel<T, MI, NI, WM, WN, NSTAGE>;
+    auto kernel = p.tuning.stream_b ? gemm_direct_kernel<T, MI, NI, WM, WN, NSTAGE, true> : gemm_direct_kernel<T, MI, NI, WM, WN, NSTAGE, false>;
     // more than 64 KB of dynamic LDS has to be asked for, once per device
-    static bool allowed[64] = {};
+    static bool allowed[2][64] = {};
     int device = 0;
     if (LDS_BYTES > 64 * 1024) {
         int e = (int) hipGetDevice(&device);
         if (e == 0 && (device < 0 || device >= 64)) e = (int) hipErrorInvalidDevice;
-        if (e == 0 && !allowed[device]) {
+        if (e == 0 && !allowed[p.tuning.stream_b][device]) {
             e = (int) hipFuncSetAttribute((const void *) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-            if (e == 0) allowed[device] = true;
+            if (e == 0) allowed[p.tuning.stream_b][device] = true;
         }
         if (e != 0) return e;
     }

@@ -22,6 +22,13 @@ struct GemmTuning {
     bool split_k = true;       // workgroups that share a tile along K, of either kind
     bool tail_split = true;    // the split of just the last, sparse round of tiles inside one launch
     bool dot_products = true;  // one wave per result for products of up to 2^20 multiplications
+    // The right operand is a weight that every evaluation reads once, out of more weights than the caches hold: the
+    // direct kernel loads it with the non-temporal hint, so that its lines do not push the left operand's out. Measured:
+    // a stand-alone stream with the matmul's access pattern 91 -> 87 us; the 512 token LLaMA decoder 564.4 -> 559.9 us
+    // per step (alternating on one GPU); weights that do fit the last-level cache (a loop over one product) 5 to 15 %
+    // SLOWER with it, 4096^3 4 % slower. Set by the planner from the size of the plan's constants and the rows of the
+    // left operand.
+    bool stream_b = false;
 };
 
 struct GemmParams {

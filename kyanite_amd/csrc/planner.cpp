@@ -1871,6 +1871,17 @@ Plan plan_graph(const Graph &graph, size_t batch_size, const PlannerOptions &opt
     }
     plan.zero_offset = cursor;
     size_t shared_base = cursor;
+    if (options.stream_weights_bytes != 0 && plan.mem_usage.dedicated_bytes >= options.stream_weights_bytes) {
+        for (auto &step : planner.steps) {
+            if (step.kind != StepKind::MatMul || step.attention || step.operands.size() < 2) continue;
+            // (the right operands follow the left one: one, one per product of a group, or the two of a gated pair)
+            const size_t rights = step.gemm.pair_op ? 2 : (size_t) std::max(step.gemm.groups, 1);
+            // (a weight that many row tiles of the left operand share is read more than once: not a stream)
+            bool constant = step.operands.size() > rights && (long long) step.gemm.batch * step.gemm.m <= 1024;
+            for (size_t k = 1; k <= rights && constant; k++) constant = step.operands[k].tensor.ptr.kind == BufferKind::Constant;
+            step.gemm.tuning.stream_b = constant;
+        }
+    }
 
     // ---- shared region: first-fit placement of live intervals. A buffer whose last use is step s may share
     // memory with one whose first use is step s + 1, never with one that is touched by step s itself.

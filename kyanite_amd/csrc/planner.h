@@ -102,6 +102,10 @@ struct PlannerOptions {
     // keep input buffers out of the reuse pool, so that inputs written once stay valid over many run_async calls
     bool preserve_inputs = false;
     GemmTuning gemm;                   // launch paths of the matmul kernels
+    // A plan with this many bytes of constants or more reads the constant right operands of its matmuls as streams
+    // (GemmTuning::stream_b): they cannot stay in the last-level cache (256 MB) from one evaluation to the next.
+    // 0: never.
+    size_t stream_weights_bytes = (size_t) 256 << 20;
     bool split_conv_channels = true;   // convolutions with few tiles fold slices of their input channels side by side
     bool plane_conv_any_width = true;  // 3 x 3 convolutions on images without a power-of-two width on the plane kernel
     GeneratorOptions generator;        // what the generated kernels may use (streaming accesses, transposing tiles)

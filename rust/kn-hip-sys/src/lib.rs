@@ -82,6 +82,7 @@ pub struct knhip_executor_options {
     pub dot_products: c_int,
     pub streaming_bytes: u64,
     pub mapped_io_bytes: u64,
+    pub stream_weights_bytes: u64,
 }
 
 /// A strided tensor in device memory that the caller owns (`DeviceTensor`); strides in elements.

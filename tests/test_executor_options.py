@@ -153,6 +153,8 @@ OPTIONS = {
     "tail_split": (sparse_last_round_matmul, 0, lambda ex: "tail_split" in plan_text(ex), lambda ex: "tail_split" not in plan_text(ex)),
     "dot_products": (tiny_matmul, 0, lambda ex: "a wave per result" in plan_text(ex), lambda ex: "a wave per result" not in plan_text(ex)),
     "streaming_bytes": (streamed_elementwise, 1 << 20, lambda ex: "nontemporal" not in sources(ex), lambda ex: "nontemporal" in sources(ex)),
+    # (the default asks for 256 MiB of constants before a weight counts as a stream)
+    "stream_weights_bytes": (aligned_matmul_f16, 1 << 10, lambda ex: "weights streamed" not in plan_text(ex), lambda ex: "weights streamed" in plan_text(ex)),
 }
 
 
