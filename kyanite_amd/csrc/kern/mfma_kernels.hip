@@ -324,8 +324,7 @@ __device__ __forceinline__ void mfma_tile_loop(LA &la, LB &lb, S &s, int k_begin
 
 // Tiles are numbered so that the workgroups that run at the same time (consecutive ids) share rows of tiles:
 // groups of 8 tile rows are walked column by column.
-__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) {
-    const int id = blockIdx.x;
+__device__ __forceinline__ void tile_of_id(int id, int tiles_m, int tiles_n, int *tm, int *tn) {
     const int group_rows = 8;
     const int per_group = group_rows * tiles_n;
     const int g = id / per_group, in_g = id - g * per_group;
@@ -333,6 +332,7 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm,
     *tm = g * group_rows + in_g % rows_here;
     *tn = in_g / rows_here;
 }
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int *tm, int *tn) { tile_of_id(blockIdx.x, tiles_m, tiles_n, tm, tn); }
 
 // TI: MFMA tiles per wave and axis (2 -> 128 x 128 workgroup tile, 1 -> 64 x 64); BK: depth of a K slice
 template <int A_MODE, int B_MODE, int TI, int BK>
@@ -447,8 +447,15 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     const int K = C * KH * KW, ohw = H * W;
     const long long N = (long long) p.batch * ohw;
     const int tiles_m = (p.out_c + BM - 1) / BM, tiles_n = (int) ((N + TN - 1) / TN);
+    // the tiles of a sparse last round are shared by `tail_parts` workgroups each, a slice of the input channels per part
+    int tile_id = blockIdx.x, tail_part = -1;
+    if (p.tail_parts > 1 && tile_id >= p.tail_head) {
+        const int t_id = tile_id - p.tail_head;
+        tile_id = p.tail_head + t_id / p.tail_parts;
+        tail_part = t_id % p.tail_parts;
+    }
     int tm, tn;
-    tile_of_block(tiles_m, tiles_n, &tm, &tn);
+    tile_of_id(tile_id, tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * TN;
     int img0 = 0, oy0 = 0;
     if (ANYW) {
@@ -605,8 +612,12 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     // a launch that splits the input channels: slice blockIdx.y takes its own range of them
-    const int c_begin = p.splits > 1 ? blockIdx.y * p.split_channels : 0;
-    const int c_end = p.splits > 1 ? min(C, c_begin + p.split_channels) : C;
+    int c_begin = p.splits > 1 ? blockIdx.y * p.split_channels : 0;
+    int c_end = p.splits > 1 ? min(C, c_begin + p.split_channels) : C;
+    if (tail_part >= 0) {
+        c_begin = tail_part * p.tail_channels;
+        c_end = min(C, c_begin + p.tail_channels);
+    }
     // the padding is never written again
     for (int i = t; i < PLANE_LDS; i += THREADS) Bs[i] = 0.0f;
     fetch(c_begin);
@@ -654,8 +665,9 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     // Epilogue. Bias and residual are requested for a whole MFMA tile row at once (addresses clamped into the tensor
     // instead of branches around the loads), so their latencies overlap; only the stores are predicated.
     // (the partial results of a split launch get bias, residual and activation from the pass that sums them)
-    ConvStore s = p.splits > 1
-        ? ConvStore{p.workspace + (long long) blockIdx.y * p.out_c * N, nullptr, nullptr, 0, p.out_c, ohw, N, 0, {0, 0}, {false, false}}
+    const int part = tail_part >= 0 ? tail_part : (p.splits > 1 ? (int) blockIdx.y : -1);
+    ConvStore s = part >= 0
+        ? ConvStore{p.workspace + (long long) part * p.out_c * N, nullptr, nullptr, 0, p.out_c, ohw, N, 0, {0, 0}, {false, false}}
         : ConvStore{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
     const int col0 = n0 + wn * 32 * NJ + c32;
     s.prepare(col0, col0 + 32);
@@ -997,6 +1009,39 @@ __global__ __launch_bounds__(256) void conv_reduce_partials_kernel(ConvParams p)
     *(Vec *) (p.output + e) = sum;
 }
 
+// Sums the partial tiles of the shared tiles of a launch with a tail split (tiles of 64 x 64 from `tail_head` on; the
+// partial results lie where a launch that splits all of its tiles would put them, [part][image][channel][position])
+// and applies residual, bias and activation in the order the unsplit store does. One workgroup per tile; VEC
+// neighbouring positions per thread (out_h * out_w a multiple of VEC).
+template <int VEC>
+__global__ __launch_bounds__(256) void conv_sum_tail_kernel(ConvParams p) {
+    const long long ohw = (long long) p.out_h * p.out_w, N = (long long) p.batch * ohw, total = N * p.out_c;
+    const int tiles_m = (p.out_c + 63) / 64, tiles_n = (int) ((N + 63) / 64);
+    int tm, tn;
+    tile_of_id(p.tail_head + (int) blockIdx.x, tiles_m, tiles_n, &tm, &tn);
+    typedef float Vec __attribute__((ext_vector_type(VEC)));
+    constexpr int COLS = 64 / VEC, ROWS = 256 / COLS;  // threads along the positions, channels per pass
+    const int col = (threadIdx.x % COLS) * VEC, row0 = threadIdx.x / COLS;
+    const long long pos = (long long) tn * 64 + col;
+    if (pos >= N) return;
+    const long long img = pos / ohw, within = pos - img * ohw;
+    for (int row = row0; row < 64; row += ROWS) {
+        const int channel = tm * 64 + row;
+        if (channel >= p.out_c) break;
+        const long long e = (img * p.out_c + channel) * ohw + within;
+        Vec sum = *(const Vec *) (p.workspace + e);
+        for (int part = 1; part < p.tail_parts; part++) sum += *(const Vec *) (p.workspace + (long long) part * total + e);
+        if (p.res) sum += *(const Vec *) (p.res + e);
+        if (p.bias) {
+            const float b = p.bias[channel * p.bias_stride];
+            for (int j = 0; j < VEC; j++) sum[j] += b;
+        }
+        if (p.relu)
+            for (int j = 0; j < VEC; j++) sum[j] = fmaxf(sum[j], 0.0f);
+        *(Vec *) (p.output + e) = sum;
+    }
+}
+
 int conv_channel_split(const ConvParams &p) {
     const bool enabled = p.channel_split;
     const long long positions = (long long) p.batch * p.out_h * p.out_w;
@@ -1021,10 +1066,36 @@ int conv_channel_split(const ConvParams &p) {
     return (slices + per_split - 1) / per_split;
 }
 
+long long conv_tail_split(const ConvParams &p, int *parts) {
+    *parts = 1;
+    const long long positions = (long long) p.batch * p.out_h * p.out_w;
+    if (!p.channel_split || positions <= 0 || p.out_c <= 0 || p.kernel_h != 3 || conv_channel_split(p) > 1) return 0;
+    ConvParams shape_only = p;
+    shape_only.input = shape_only.filter = nullptr;
+    PlaneGeom geom;
+    if (!plane_geometry(shape_only, 64, &geom) && !(p.plane_any_width && plane_geometry_any(shape_only, 64, &geom))) return 0;
+    // only where the launch picks tiles of 64 x 64 (the same estimate as in launch_conv_f32)
+    const long long tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64), big = ((positions + 127) / 128) * ((p.out_c + 127) / 128);
+    const bool big_fits = plane_geometry(shape_only, 128, &geom) || (p.plane_any_width && plane_geometry_any(shape_only, 128, &geom));
+    if (big_fits && (double) ((big * 4 + 1023) / 1024) * 4.0 <= (double) ((tiles * 4 + 1023) / 1024) * 1.1) return tiles;
+    // Whole rounds of one tile per compute unit stay whole. Measured on 2 x 64 x 64 images, 320 input channels (us by
+    // output channels): 256 112, 320 153, 384 154 - a compute unit with three tiles takes as long as if all had three.
+    const long long rest = tiles % 256, slices = (p.in_c + CB - 1) / CB;
+    if (tiles < 256 || tiles > 0x7fffffffll / 8 || rest < 16 || rest > 128 || slices < 8) return tiles;
+    const long long most = std::min<long long>({4, 256 / rest, slices / 4});
+    if (most < 2) return tiles;
+    const long long per_part = (slices + most - 1) / most;
+    *parts = (int) ((slices + per_part - 1) / per_part);
+    return tiles - rest;
+}
+
 size_t conv_workspace_bytes(const ConvParams &p) {
     const int splits = conv_channel_split(p);
-    if (splits <= 1) return 0;
-    return (size_t) splits * p.batch * p.out_c * p.out_h * p.out_w * sizeof(float);
+    int tail_parts = 1;
+    if (splits <= 1) conv_tail_split(p, &tail_parts);
+    const int most = std::max(splits, tail_parts);
+    if (most <= 1) return 0;
+    return (size_t) most * p.batch * p.out_c * p.out_h * p.out_w * sizeof(float);
 }
 
 int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
@@ -1076,10 +1147,31 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost;
         if (!best || cost < best_cost) { best = &v; best_cost = cost; any_w = !classic; }
     }
+    // a sparse last round of 64 x 64 tiles: its tiles shared by workgroups that take a slice of the input channels each
+    long long tail_tiles = 0;
+    if (best && best->id == 11 && !split && p.workspace) {
+        int parts = 1;
+        const long long head = conv_tail_split(params, &parts);
+        if (parts > 1) {
+            const int slices = (p.in_c + CB - 1) / CB;
+            p.tail_head = (int) head;
+            p.tail_parts = parts;
+            p.tail_channels = (slices + parts - 1) / parts * CB;
+            tail_tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64) - head;
+        }
+    }
+    auto sum_tail = [&]() {
+        if (tail_tiles == 0) return (int) hipGetLastError();
+        const bool vec = (p.out_h * p.out_w) % 4 == 0 && (uintptr_t) p.output % 16 == 0 && (uintptr_t) p.workspace % 16 == 0 &&
+                         (!p.res || (uintptr_t) p.res % 16 == 0);
+        if (vec) hipLaunchKernelGGL((conv_sum_tail_kernel<4>), dim3((unsigned) tail_tiles), dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((conv_sum_tail_kernel<1>), dim3((unsigned) tail_tiles), dim3(256), 0, stream, p);
+        return (int) hipGetLastError();
+    };
     if (best && any_w) {
         plane_geometry_any(p, best->tn, &geom);
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
-        const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
+        const dim3 grid((unsigned) (tiles + tail_tiles * (p.tail_parts - 1)), (unsigned) p.splits), block(THREADS);
         const bool ragged = p.in_c % plane_slice_channels(p.kernel_h, p.kernel_w) != 0;
         const bool by4 = geom.by4 != 0;
         if (p.kernel_h == 5) {
@@ -1095,12 +1187,12 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true, 1>), grid, block, 0, stream, p, geom);
         else if (by4) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false, 2>), grid, block, 0, stream, p, geom);
         else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false, 1>), grid, block, 0, stream, p, geom);
-        return sum_slices();
+        return tail_tiles ? sum_tail() : sum_slices();
     }
     if (best) {
         plane_geometry(p, best->tn, &geom);
         const long long tiles = ((positions + best->tn - 1) / best->tn) * ((p.out_c + best->bm - 1) / best->bm);
-        const dim3 grid((unsigned) tiles, (unsigned) p.splits), block(THREADS);
+        const dim3 grid((unsigned) (tiles + tail_tiles * (p.tail_parts - 1)), (unsigned) p.splits), block(THREADS);
         const bool ragged = p.in_c % plane_slice_channels(p.kernel_h, p.kernel_w) != 0;
         if (p.kernel_h == 5) {
             hipLaunchKernelGGL((conv_plane_kernel<5, 5, 1, 1, false>), grid, block, 0, stream, p, geom);
@@ -1110,7 +1202,7 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         else if (best->id == 22) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 2, 2, false>), grid, block, 0, stream, p, geom);
         else if (ragged) hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, true>), grid, block, 0, stream, p, geom);
         else hipLaunchKernelGGL((conv_plane_kernel<3, 3, 1, 1, false>), grid, block, 0, stream, p, geom);
-        return sum_slices();
+        return tail_tiles ? sum_tail() : sum_slices();
     }
     const long long K = (long long) p.in_c * p.kernel_h * p.kernel_w;
     const int a_mode = ((uintptr_t) p.filter % 16 == 0 && K % 4 == 0) ? VecK : Scalar;

@@ -11,6 +11,15 @@ const char *step_kind_name(StepKind k) {
     return names[(int) k];
 }
 
+namespace {
+std::string conv_tail_note(const ConvParams &conv) {
+    int parts = 1;
+    const long long head = conv_tail_split(conv, &parts);
+    if (parts <= 1) return std::string();
+    return " [the tiles after " + std::to_string(head) + " in " + std::to_string(parts) + " slices of the input channels]";
+}
+}  // namespace
+
 std::string Step::str() const {
     std::ostringstream ss;
     ss << step_kind_name(kind) << " value=" << debug_value;
@@ -27,7 +36,8 @@ std::string Step::str() const {
     else if (kind == StepKind::Conv)
         ss << " n=" << conv.batch << " c=" << conv.in_c << "->" << conv.out_c << " hw=" << conv.in_h << "x" << conv.in_w << " k="
            << conv.kernel_h << "x" << conv.kernel_w << (conv_has_bias ? " +bias" : "") << (conv_has_res ? " +res" : "")
-           << (conv.relu ? " relu" : "") << (conv_channel_split(conv) > 1 ? " [input channels in " + std::to_string(conv_channel_split(conv)) + " slices]" : std::string());
+           << (conv.relu ? " relu" : "") << (conv_channel_split(conv) > 1 ? " [input channels in " + std::to_string(conv_channel_split(conv)) + " slices]" : std::string())
+           << conv_tail_note(conv);
     else ss << " [" << kernel.strategy << "] grid=" << kernel.grid << "x" << kernel.block;
     ss << " operands:";
     for (auto &op : operands) ss << " " << dtype_name(op.tensor.dtype) << vec_str(op.tensor.shape.shape());

@@ -2035,6 +2035,33 @@ def conv_with_input_channels_in_slices():
 
 
 @case
+def conv_with_a_sparse_last_round_of_tiles():
+    """a tile count that leaves the last round of workgroups sparse: the tiles of that round are shared by workgroups that
+    take a slice of the input channels each, and a small second kernel sums their partial tiles and applies bias,
+    residual and activation. 640 tiles on power-of-two images with all three (two slices); 584 tiles on 9 x 9 boards
+    (81 positions per image: tiles that straddle images, no vectors in the summing kernel); 288 tiles on 48 x 48 images
+    in four slices; and, with the option off, the first one again on whole tiles"""
+    from kyanite_amd import HipExecutor
+    g = Graph()
+    rng = np.random.default_rng(641)
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    images = g.input([2, 320, 64, 64])
+    bias = g.constant([1, 320, 1, 1], rng.standard_normal(320).astype(np.float32))
+    g.output(g.relu(g.add(g.add(g.conv(images, w(320, 320, 3, 3), 1, 1, 1, 1), bias), images)))
+    boards = g.input([230, 64, 9, 9])
+    g.output(g.add(g.conv(boards, w(128, 64, 3, 3), 1, 1, 1, 1), g.constant([1, 128, 1, 1], rng.standard_normal(128).astype(np.float32))))
+    wide = g.input([2, 128, 48, 48])
+    g.output(g.conv(wide, w(256, 128, 3, 3), 1, 1, 1, 1))
+    plan = HipExecutor(0, g, 0, plan_only=True)
+    text = [plan.step_str(i) for i in range(plan.step_count())]
+    assert "the tiles after 512 in 2 slices" in text[0] and "the tiles after 512 in 2 slices" in text[1] and "the tiles after 256 in 4 slices" in text[2], text
+    whole = HipExecutor(0, g, 0, plan_only=True, split_conv_channels=False)
+    assert not any("slices" in whole.step_str(i) for i in range(whole.step_count()))
+    f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    return g, 0, [f(2, 320, 64, 64), f(230, 64, 9, 9), f(2, 128, 48, 48)], None
+
+
+@case
 def products_with_few_rows():
     """a left operand of 1, 8 and 32 rows against constant [k, n] weights, f32 and f16: the weights are laid out again
     as [n, k] and the product runs on the kernel that loads global -> LDS directly (f32: on 32 x 128 tiles), with a
