@@ -535,7 +535,10 @@ void HipExecutor::evaluate(const void *const *inputs, void *const *outputs) {
         for (size_t off = 0; off < bytes; off += kCopyChunkBytes) chunks.push_back({i, off, std::min(kCopyChunkBytes, bytes - off)});
     }
     // an event behind every chunk but the last, so that the host can copy a chunk out while the next ones still move
-    const size_t n_events = chunks.empty() ? 0 : chunks.size() - 1;
+    // (outputs that make one chunk's worth between them wait for the stream once instead)
+    size_t output_bytes = 0;
+    for (auto &ch : chunks) output_bytes += ch.bytes;
+    const size_t n_events = output_bytes > kCopyChunkBytes ? chunks.size() - 1 : 0;
     if (mapped) {
         last_profile_ = std::nullopt;
         if (fused_function_) launch_fused(true);
@@ -563,16 +566,22 @@ void HipExecutor::evaluate(const void *const *inputs, void *const *outputs) {
         // (an acquire load: the outputs are read from page-locked memory right behind it)
         for (int spin = 0; spin < 400000 && !done; spin++) done = __atomic_load_n(fused_done_, __ATOMIC_ACQUIRE) == fused_seq_;
     }
-    if (mapped && !done) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    bool synchronized = done;
+    if (mapped && !done) {
+        hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+        synchronized = true;
+    }
     for (size_t c = 0; c < chunks.size(); c++) {
         const Chunk &ch = chunks[c];
-        if (!mapped) {
-            if (c < n_events) hip_check(hipEventSynchronize(chunk_events_[c]), "hipEventSynchronize");
-            else hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+        if (c < n_events && !mapped) {
+            hip_check(hipEventSynchronize(chunk_events_[c]), "hipEventSynchronize");
+        } else if (!synchronized) {
+            hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+            synchronized = true;
         }
         host_copy((char *) outputs[ch.output] + ch.offset, (char *) pinned_outputs_[ch.output] + ch.offset, ch.bytes);
     }
-    if (chunks.empty() && !mapped) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    if (!synchronized) hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
     for (size_t i = 0; i < plan_.outputs.size(); i++) {
         if (plan_.outputs[i].dtype != DType::Bool) continue;
         const uint8_t *bytes = (const uint8_t *) outputs[i];

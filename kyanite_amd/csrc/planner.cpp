@@ -769,15 +769,9 @@ private:
             if (n.kind == ScalarNode::Binary) n.b = at[n.b];
             at[i] = push_node(n);
         }
-        // (an epilogue that is the normalised value itself leaves `normalised` as the last node only if nothing
-        // follows it: the result of the expression is its last node)
-        if (at.back() != expr.nodes.size() - 1) {
-            // the result is an earlier node: repeat it through a multiplication by one, which changes no bit of a float
-            ScalarNode one = node(ScalarNode::Const);
-            one.constant = DScalar::f32(1.0f);
-            const size_t c = push_node(one);
-            binary(BinaryOp::Mul, at.back(), c);
-        }
+        // (the result of an expression is its last node: the epilogue's, or the normalised value of an epilogue that
+        // is nothing but that value)
+        KN_ASSERT(at.back() == expr.nodes.size() - 1);
         plan_scalar_op(expr, operands, value);
     }
 
