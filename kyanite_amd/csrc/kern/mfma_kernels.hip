@@ -1009,24 +1009,26 @@ __global__ __launch_bounds__(256) void conv_reduce_partials_kernel(ConvParams p)
     *(Vec *) (p.output + e) = sum;
 }
 
-// Sums the partial tiles of the shared tiles of a launch with a tail split (tiles of 64 x 64 from `tail_head` on; the
-// partial results lie where a launch that splits all of its tiles would put them, [part][image][channel][position])
-// and applies residual, bias and activation in the order the unsplit store does. One workgroup per tile; VEC
-// neighbouring positions per thread (out_h * out_w a multiple of VEC).
+// Sums the partial tiles of the shared tiles of a launch with a tail split (tiles from `tail_head` on; the partial
+// results lie where a launch that splits all of its tiles would put them, [part][image][channel][position]) and
+// applies residual, bias and activation in the order the unsplit store does. One workgroup per 64 positions of a
+// tile (blockIdx.y: the second half of a tile of 128); VEC neighbouring positions per thread (out_h * out_w a
+// multiple of VEC).
 template <int VEC>
 __global__ __launch_bounds__(256) void conv_sum_tail_kernel(ConvParams p) {
     const long long ohw = (long long) p.out_h * p.out_w, N = (long long) p.batch * ohw, total = N * p.out_c;
-    const int tiles_m = (p.out_c + 63) / 64, tiles_n = (int) ((N + 63) / 64);
+    const int tile = p.tail_tile;
+    const int tiles_m = (p.out_c + tile - 1) / tile, tiles_n = (int) ((N + tile - 1) / tile);
     int tm, tn;
     tile_of_id(p.tail_head + (int) blockIdx.x, tiles_m, tiles_n, &tm, &tn);
     typedef float Vec __attribute__((ext_vector_type(VEC)));
     constexpr int COLS = 64 / VEC, ROWS = 256 / COLS;  // threads along the positions, channels per pass
     const int col = (threadIdx.x % COLS) * VEC, row0 = threadIdx.x / COLS;
-    const long long pos = (long long) tn * 64 + col;
+    const long long pos = (long long) tn * tile + 64 * blockIdx.y + col;
     if (pos >= N) return;
     const long long img = pos / ohw, within = pos - img * ohw;
-    for (int row = row0; row < 64; row += ROWS) {
-        const int channel = tm * 64 + row;
+    for (int row = row0; row < tile; row += ROWS) {
+        const int channel = tm * tile + row;
         if (channel >= p.out_c) break;
         const long long e = (img * p.out_c + channel) * ohw + within;
         Vec sum = *(const Vec *) (p.workspace + e);
@@ -1066,23 +1068,30 @@ int conv_channel_split(const ConvParams &p) {
     return (slices + per_split - 1) / per_split;
 }
 
-long long conv_tail_split(const ConvParams &p, int *parts) {
+long long conv_tail_split(const ConvParams &p, int *parts, int *tile) {
     *parts = 1;
+    if (tile) *tile = 64;
     const long long positions = (long long) p.batch * p.out_h * p.out_w;
     if (!p.channel_split || positions <= 0 || p.out_c <= 0 || p.kernel_h != 3 || conv_channel_split(p) > 1) return 0;
     ConvParams shape_only = p;
     shape_only.input = shape_only.filter = nullptr;
     PlaneGeom geom;
     if (!plane_geometry(shape_only, 64, &geom) && !(p.plane_any_width && plane_geometry_any(shape_only, 64, &geom))) return 0;
-    // only where the launch picks tiles of 64 x 64 (the same estimate as in launch_conv_f32)
-    const long long tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64), big = ((positions + 127) / 128) * ((p.out_c + 127) / 128);
+    // which tiles the launch picks (the same estimate as in launch_conv_f32)
+    const long long small = ((positions + 63) / 64) * ((p.out_c + 63) / 64), big = ((positions + 127) / 128) * ((p.out_c + 127) / 128);
     const bool big_fits = plane_geometry(shape_only, 128, &geom) || (p.plane_any_width && plane_geometry_any(shape_only, 128, &geom));
-    if (big_fits && (double) ((big * 4 + 1023) / 1024) * 4.0 <= (double) ((tiles * 4 + 1023) / 1024) * 1.1) return tiles;
-    // Whole rounds of one tile per compute unit stay whole. Measured on 2 x 64 x 64 images, 320 input channels (us by
-    // output channels): 256 112, 320 153, 384 154 - a compute unit with three tiles takes as long as if all had three.
-    const long long rest = tiles % 256, slices = (p.in_c + CB - 1) / CB;
-    if (tiles < 256 || tiles > 0x7fffffffll / 8 || rest < 16 || rest > 128 || slices < 8) return tiles;
-    const long long most = std::min<long long>({4, 256 / rest, slices / 4});
+    const bool big_wins = big_fits && (double) ((big * 4 + 1023) / 1024) * 4.0 <= (double) ((small * 4 + 1023) / 1024) * 1.1;
+    const long long tiles = big_wins ? big : small, slices = (p.in_c + CB - 1) / CB;
+    if (tile) *tile = big_wins ? 128 : 64;
+    if (tiles > 0x7fffffffll / 8 || slices < 8) return tiles;
+    // Tiles of 64 x 64: whole rounds of one tile per compute unit stay whole. Measured on 2 x 64 x 64 images, 320 input
+    // channels (us by output channels): 256 112, 320 153, 384 154 - a compute unit with three tiles takes as long as if
+    // all had three. Tiles of 128 x 128: a compute unit holds two, and what a round of 512 leaves over runs as a round
+    // of its own (the tower convolution of a board game network, us per evaluation of 21 of them by batch size:
+    // 1024 3487, 1536 6601, 2048 6912).
+    const long long round = big_wins ? 512 : 256, rest = tiles % round;
+    if (tiles < round || rest < round / 16 || rest > round / 2) return tiles;
+    const long long most = std::min<long long>({4, round / rest, slices / 4});
     if (most < 2) return tiles;
     const long long per_part = (slices + most - 1) / most;
     *parts = (int) ((slices + per_part - 1) / per_part);
@@ -1149,23 +1158,26 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
     }
     // a sparse last round of 64 x 64 tiles: its tiles shared by workgroups that take a slice of the input channels each
     long long tail_tiles = 0;
-    if (best && best->id == 11 && !split && p.workspace) {
-        int parts = 1;
-        const long long head = conv_tail_split(params, &parts);
-        if (parts > 1) {
+    if (best && !split && p.workspace) {
+        int parts = 1, tile = 64;
+        const long long head = conv_tail_split(params, &parts, &tile);
+        // (only if the launch picked the tiles the plan was made for)
+        if (parts > 1 && tile == best->tn) {
             const int slices = (p.in_c + CB - 1) / CB;
             p.tail_head = (int) head;
             p.tail_parts = parts;
             p.tail_channels = (slices + parts - 1) / parts * CB;
-            tail_tiles = ((positions + 63) / 64) * ((p.out_c + 63) / 64) - head;
+            p.tail_tile = tile;
+            tail_tiles = ((positions + tile - 1) / tile) * ((p.out_c + tile - 1) / tile) - head;
         }
     }
     auto sum_tail = [&]() {
         if (tail_tiles == 0) return (int) hipGetLastError();
         const bool vec = (p.out_h * p.out_w) % 4 == 0 && (uintptr_t) p.output % 16 == 0 && (uintptr_t) p.workspace % 16 == 0 &&
                          (!p.res || (uintptr_t) p.res % 16 == 0);
-        if (vec) hipLaunchKernelGGL((conv_sum_tail_kernel<4>), dim3((unsigned) tail_tiles), dim3(256), 0, stream, p);
-        else hipLaunchKernelGGL((conv_sum_tail_kernel<1>), dim3((unsigned) tail_tiles), dim3(256), 0, stream, p);
+        const dim3 tail_grid((unsigned) tail_tiles, (unsigned) (p.tail_tile / 64));
+        if (vec) hipLaunchKernelGGL((conv_sum_tail_kernel<4>), tail_grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((conv_sum_tail_kernel<1>), tail_grid, dim3(256), 0, stream, p);
         return (int) hipGetLastError();
     };
     if (best && any_w) {

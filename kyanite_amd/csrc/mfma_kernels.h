@@ -123,9 +123,9 @@ struct ConvParams {
     float *workspace = nullptr;
     // filled in by the launch: slices of the input channels that are folded side by side, and channels per slice
     int splits = 1, split_channels = 0;
-    // filled in by the launch: the tiles from `tail_head` on are each shared by `tail_parts` workgroups that take
-    // `tail_channels` input channels each (conv_tail_split)
-    int tail_head = 0, tail_parts = 1, tail_channels = 0;
+    // filled in by the launch: the tiles (of `tail_tile` x `tail_tile`) from `tail_head` on are each shared by
+    // `tail_parts` workgroups that take `tail_channels` input channels each (conv_tail_split)
+    int tail_head = 0, tail_parts = 1, tail_channels = 0, tail_tile = 64;
     // launch paths a caller may switch off
     bool channel_split = true;    // slices of the input channels folded side by side when the tiles are few
     bool plane_any_width = true;  // the plane kernel for 3 x 3 convolutions on images without a power-of-two width
@@ -137,11 +137,12 @@ struct ConvParams {
 // activation. A function of the shapes alone, so that the planner can reserve the scratch ahead of time.
 int conv_channel_split(const ConvParams &p);
 // A tile count that leaves the last round of workgroups sparse (640 tiles of 64 x 64 on 256 compute units: two tiles
-// each, and a third on half of them, which the other half waits for): the tiles of that round are each shared by
-// `parts` workgroups that take a slice of the input channels and store f32 partial tiles, summed by a second, small
-// kernel. Returns the number of tiles that stay whole (`parts` is 1 when nothing is split). A function of the shapes
-// alone, like conv_channel_split.
-long long conv_tail_split(const ConvParams &p, int *parts);
+// each, and a third on half of them, which the other half waits for; 768 tiles of 128 x 128, of which a compute unit
+// holds two at a time): the tiles of that round are each shared by `parts` workgroups that take a slice of the input
+// channels and store f32 partial tiles, summed by a second, small kernel. Returns the number of tiles that stay whole
+// (`parts` is 1 when nothing is split) and the edge of the tiles the launch picks (64 or 128). A function of the
+// shapes alone, like conv_channel_split.
+long long conv_tail_split(const ConvParams &p, int *parts, int *tile = nullptr);
 size_t conv_workspace_bytes(const ConvParams &p);
 
 // O[b] = softmax(scale * Q[b] K[b]^T + mask[b]) V[b] with the softmax along the keys; Q is [batch, lq, dk],
