@@ -190,6 +190,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         lp.tall_tile = best_tile >= TILE_TALL;
         lp.mid_tile = best_tile == TILE_MID;
         lp.wide_tile = best_tile == TILE_WIDE;
+        lp.estimated_us = best_us;
         model_split = best_split;
     }
     // f32 under a left operand of up to 32 rows: a pass over the weights in which a 64 row tile would spend its MFMAs
@@ -316,8 +317,18 @@ bool gemm_group_ok(const GemmParams &p, bool f16) {
     if (p.groups < 2 || p.groups > GEMM_MAX_GROUPS || p.addend != nullptr || p.relu) return false;
     auto mag = [](long long x) { return x < 0 ? -x : x; };
     if (mag(p.c_sm) < mag(p.c_sn)) return false;  // the launch would swap the operands
-    // A grouped launch never splits K. Where even all products together leave the chip short of tiles, separate
-    // launches that split K are faster.
+    // A grouped launch never splits K. With the cost model (f16, the kernel that loads global -> LDS directly): one
+    // launch if it is expected to take no longer than the products one by one, each on the tiles and the split of K it
+    // would pick. (The rule below saw a split of K in the plan of all columns together for 384 rows against three
+    // weights of 4096 x 4096 and left three launches of too few tiles each: a 384 token prefill of the two LLaMA
+    // layers took 621 us, more than one of 512 tokens; 576 us as one launch. 256 tokens, which it had as one launch and
+    // a pair, are 3 % slower as one launch of three.)
+    GemmParams one = p;
+    one.groups = 1;
+    const GemmLaunchPlan single = plan_gemm_launch(one, f16), grouped = plan_gemm_launch(p, f16);
+    if (single.estimated_us > 0.0 && grouped.estimated_us > 0.0) return grouped.estimated_us <= p.groups * single.estimated_us;
+    // Otherwise: where even all products together leave the chip short of tiles, separate launches that split K are
+    // faster.
     GemmParams wide = p;
     wide.groups = 1;
     wide.n = p.n * p.groups;

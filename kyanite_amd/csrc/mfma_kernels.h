@@ -94,6 +94,7 @@ struct GemmLaunchPlan {
     int head_tiles, tail_split, tail_k_chunk;
     size_t workspace_bytes;  // f32 scratch: split_k * batch * m * n * 4 when split_k > 1; one tile per sharing workgroup
     size_t counter_bytes;    // one int per shared tile
+    double estimated_us;     // f16 direct kernel: what the cost model expects of the launch (0: no estimate)
 };
 GemmLaunchPlan plan_gemm_launch(const GemmParams &p, bool f16);
 // the launch of a plan with `dot` set (both element types; `mfma_kernels.hip`)
