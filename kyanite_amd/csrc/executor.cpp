@@ -341,6 +341,7 @@ void HipExecutor::realise_launch(size_t index, Launch &l, bool mapped) {
         l.conv.res = step.conv_has_res ? (const float *) l.ptrs[k++] : nullptr;
         l.conv.output = (float *) l.ptrs[k++];
         l.conv.workspace = k < l.ptrs.size() ? (float *) l.ptrs[k++] : nullptr;
+        l.conv.counters = k < l.ptrs.size() ? (int *) l.ptrs[k++] : nullptr;
     }
 }
 

@@ -29,6 +29,7 @@ namespace {
 constexpr int BM = 128, BN = 128, THREADS = 256;
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 enum LoadMode { Scalar = 0, VecOuter = 1, VecK = 2 };
@@ -666,7 +667,53 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
     // instead of branches around the loads), so their latencies overlap; only the stores are predicated.
     // (the partial results of a split launch get bias, residual and activation from the pass that sums them)
     const int part = tail_part >= 0 ? tail_part : (p.splits > 1 ? (int) blockIdx.y : -1);
-    ConvStore s = part >= 0
+    if (part >= 0 && p.counters) {
+        // Summed inside the launch: every workgroup of a tile parks its partial tile, [part][wave][MFMA tile][register / 4]
+        // [lane][register % 4], and counts itself in; the last one to arrive adds the parts up in their order and goes
+        // on to the epilogue. The partial tiles travel between workgroups that may sit on different XCDs, each with an L2
+        // of its own: they are written and read with device scope accesses, which go past those caches. What orders the
+        // exchange: every wave waits for the acknowledgements of its own stores, the barrier collects the waves, and only
+        // then one thread adds to the tile's counter; the workgroup that reads `parts - 1` there is behind all the others'
+        // stores. It puts the counter back to zero for the next launch, which the stream orders behind this one.
+        constexpr int SC1 = 16;  // auxiliary bits of the buffer instructions: device scope
+        const int parts = tail_part >= 0 ? p.tail_parts : p.splits;
+        const int shared_index = tail_part >= 0 ? tile_id - p.tail_head : tile_id;
+        float *tile_slots = p.workspace + (size_t) shared_index * parts * (BM * TN);
+        const __amdgpu_buffer_rsrc_t slots = __builtin_amdgcn_make_buffer_rsrc(tile_slots, 0, parts * (BM * TN) * 4, 0x00020000);
+        const int thread_off = (wave * (MI * NJ * 16 * 64) + lane * 4) * 4;
+#pragma unroll
+        for (int i = 0; i < MI; i++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const floatx4 x = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, x), slots,
+                                                           part * (BM * TN * 4) + thread_off + ((i * NJ + j) * 4 + q) * 1024, 0, SC1);
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // (also: every wave is done with the LDS operands)
+        int *counter = p.counters + shared_index, *arrived = (int *) &As[0][0];
+        if (threadIdx.x == 0) *arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*(volatile int *) arrived != parts - 1) return;
+        for (int from = 0; from < parts; from++) {
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const floatx4 x = __builtin_bit_cast(
+                            floatx4, __builtin_amdgcn_raw_buffer_load_b128(slots, from * (BM * TN * 4) + thread_off + ((i * NJ + j) * 4 + q) * 1024, 0, SC1));
+#pragma unroll
+                        for (int u = 0; u < 4; u++) acc[i][j][4 * q + u] = from == 0 ? x[u] : acc[i][j][4 * q + u] + x[u];
+                    }
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const bool to_scratch = part >= 0 && !p.counters;
+    ConvStore s = to_scratch
         ? ConvStore{p.workspace + (long long) part * p.out_c * N, nullptr, nullptr, 0, p.out_c, ohw, N, 0, {0, 0}, {false, false}}
         : ConvStore{p.output, p.bias, p.res, p.bias_stride, p.out_c, ohw, N, p.relu, {0, 0}, {false, false}};
     const int col0 = n0 + wn * 32 * NJ + c32;
@@ -1098,13 +1145,44 @@ long long conv_tail_split(const ConvParams &p, int *parts, int *tile) {
     return tiles - rest;
 }
 
+namespace {
+// whether the kernel that keeps raw planes in LDS takes this convolution on tiles of 64 x 64 (shapes only)
+bool plane_kernel_small_tiles(const ConvParams &p) {
+    ConvParams shape_only = p;
+    shape_only.input = shape_only.filter = nullptr;
+    PlaneGeom geom;
+    return plane_geometry(shape_only, 64, &geom) || (p.plane_any_width && plane_geometry_any(shape_only, 64, &geom));
+}
+}  // namespace
+
+size_t conv_counter_bytes(const ConvParams &p) {
+    const long long positions = (long long) p.batch * p.out_h * p.out_w;
+    if (positions <= 0 || p.out_c <= 0) return 0;
+    // A split of all tiles: only the plane kernel (on tiles of 64 x 64 then) sums inside the launch, and only up to four
+    // parts: the last workgroup of a tile reads the parts one after the other, which with eight of them takes longer
+    // than the second kernel (the ResNet tower, us per evaluation with the second kernel / summed inside: batch 1
+    // 291 / 306, 8 316 / 343 with eight parts; 32 400 / 387 with four, 64 527 / 488 with two).
+    if (const int splits = conv_channel_split(p); splits > 1)
+        return splits <= 4 && plane_kernel_small_tiles(p) ? (size_t) (((positions + 63) / 64) * ((p.out_c + 63) / 64)) * sizeof(int) : 0;
+    int parts = 1, tile = 64;
+    const long long head = conv_tail_split(p, &parts, &tile);
+    if (parts <= 1) return 0;
+    return (size_t) (((positions + tile - 1) / tile) * ((p.out_c + tile - 1) / tile) - head) * sizeof(int);
+}
+
 size_t conv_workspace_bytes(const ConvParams &p) {
     const int splits = conv_channel_split(p);
     int tail_parts = 1;
     if (splits <= 1) conv_tail_split(p, &tail_parts);
     const int most = std::max(splits, tail_parts);
     if (most <= 1) return 0;
-    return (size_t) most * p.batch * p.out_c * p.out_h * p.out_w * sizeof(float);
+    // [part][image][channel][position] for the kernel that sums the parts; whole tiles per part and tile where the parts
+    // are summed inside the launch
+    const size_t plain = (size_t) most * p.batch * p.out_c * p.out_h * p.out_w * sizeof(float);
+    int tile = 64;
+    if (splits <= 1) conv_tail_split(p, &tail_parts, &tile);
+    const size_t slots = conv_counter_bytes(p) / sizeof(int) * (size_t) most * tile * tile * sizeof(float);
+    return std::max(plain, slots);
 }
 
 int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
@@ -1118,8 +1196,9 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         p.split_channels = (slices + p.splits - 1) / p.splits * CB;
     }
     const bool split = p.splits > 1;
+    bool plane_sums_inside = false;
     auto sum_slices = [&]() {
-        if (!split) return (int) hipGetLastError();
+        if (!split || plane_sums_inside) return (int) hipGetLastError();
         const long long total = (long long) p.batch * p.out_c * p.out_h * p.out_w;
         const bool vec = (p.out_h * p.out_w) % 4 == 0 && (uintptr_t) p.output % 16 == 0 && (!p.res || (uintptr_t) p.res % 16 == 0);
         const long long threads = vec ? total / 4 : total;
@@ -1171,8 +1250,12 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
             tail_tiles = ((positions + tile - 1) / tile) * ((p.out_c + tile - 1) / tile) - head;
         }
     }
+    // (the plane kernel sums inside the launch when it has counters; the patch kernel never does)
+    const bool sums_inside = best != nullptr && p.counters != nullptr;
+    if (!best) p.counters = nullptr;
+    plane_sums_inside = sums_inside;
     auto sum_tail = [&]() {
-        if (tail_tiles == 0) return (int) hipGetLastError();
+        if (tail_tiles == 0 || sums_inside) return (int) hipGetLastError();
         const bool vec = (p.out_h * p.out_w) % 4 == 0 && (uintptr_t) p.output % 16 == 0 && (uintptr_t) p.workspace % 16 == 0 &&
                          (!p.res || (uintptr_t) p.res % 16 == 0);
         const dim3 tail_grid((unsigned) tail_tiles, (unsigned) (p.tail_tile / 64));

@@ -122,6 +122,10 @@ struct ConvParams {
     // f32 scratch of `conv_workspace_bytes` bytes (256 byte aligned) when the launch splits the input channels; may
     // be null otherwise
     float *workspace = nullptr;
+    // `conv_counter_bytes` bytes of zero-filled ints that every launch hands back zero-filled: with them the kernel that
+    // keeps raw planes in LDS sums the slices of a split inside the launch (the last workgroup to arrive at a tile adds
+    // the parts up in their order and stores); without them (null) a second kernel does
+    int *counters = nullptr;
     // filled in by the launch: slices of the input channels that are folded side by side, and channels per slice
     int splits = 1, split_channels = 0;
     // filled in by the launch: the tiles (of `tail_tile` x `tail_tile`) from `tail_head` on are each shared by
@@ -145,6 +149,7 @@ int conv_channel_split(const ConvParams &p);
 // shapes alone, like conv_channel_split.
 long long conv_tail_split(const ConvParams &p, int *parts, int *tile = nullptr);
 size_t conv_workspace_bytes(const ConvParams &p);
+size_t conv_counter_bytes(const ConvParams &p);
 
 // O[b] = softmax(scale * Q[b] K[b]^T + mask[b]) V[b] with the softmax along the keys; Q is [batch, lq, dk],
 // K [batch, lk, dk], V [batch, lk, dv], O [batch, lq, dv], mask [batch, lq, lk], with arbitrary element strides (batch,

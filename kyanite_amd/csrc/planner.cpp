@@ -1580,6 +1580,15 @@ private:
             // partial results of a launch that splits the input channels
             if (const size_t bytes = conv_workspace_bytes(p))
                 step.operands.push_back({alloc_tensor_shared({bytes / 4}, DType::F32), OperandKind::Out});
+            // counters of the tiles whose parts are summed inside the launch: zero, and left at zero by every launch
+            if (const size_t bytes = conv_counter_bytes(p)) {
+                constants.push_back(HostTensor(DType::I32, {bytes / 4}));
+                PlanTensor t;
+                t.ptr = PlanPtr{BufferKind::Constant, constants.size() - 1, 0};
+                t.dtype = DType::I32;
+                t.shape = StridedShape::simple({bytes / 4});
+                step.operands.push_back({t, OperandKind::Out});
+            }
             push(std::move(step), value);
         }
         return R::done(output);
