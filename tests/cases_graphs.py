@@ -2062,6 +2062,29 @@ def conv_with_a_sparse_last_round_of_tiles():
 
 
 @case
+def conv_parts_summed_inside_the_launch():
+    """input channels in two and in four slices on the kernel that keeps raw planes in LDS: the workgroups of a tile park
+    their partial tiles and the last one to arrive sums them and applies bias, residual and activation (no second
+    kernel); twice through the same executor, so that the counters must have come back to zero"""
+    from kyanite_amd import HipExecutor
+    g = Graph()
+    rng = np.random.default_rng(88)
+    w = lambda *shape: g.constant(list(shape), (rng.standard_normal(shape) * 0.05).astype(np.float32))
+    two, four = g.input([64, 128, 8, 8]), g.input([32, 128, 8, 8])
+    bias = g.constant([1, 128, 1, 1], rng.standard_normal(128).astype(np.float32))
+    first = g.relu(g.add(g.add(g.conv(two, w(128, 128, 3, 3), 1, 1, 1, 1), bias), two))
+    g.output(g.relu(g.add(g.conv(first, w(128, 128, 3, 3), 1, 1, 1, 1), bias)))
+    g.output(g.add(g.conv(four, w(72, 128, 3, 3), 1, 1, 1, 1), g.constant([1, 72, 1, 1], rng.standard_normal(72).astype(np.float32))))
+    plan = HipExecutor(0, g, 0, plan_only=True)
+    text = [plan.step_str(i) for i in range(plan.step_count())]
+    assert sum("input channels in 2 slices" in t for t in text) == 2 and sum("input channels in 4 slices" in t for t in text) == 1, text
+    # (the last operand of each is the counters: one per tile)
+    assert all(t.endswith("i32[128]") or t.endswith("i32[64]") for t in text), text
+    f = lambda *shape: rng.standard_normal(shape).astype(np.float32)
+    return g, 0, [f(64, 128, 8, 8), f(32, 128, 8, 8)], None
+
+
+@case
 def products_with_few_rows():
     """a left operand of 1, 8 and 32 rows against constant [k, n] weights, f32 and f16: the weights are laid out again
     as [n, k] and the product runs on the kernel that loads global -> LDS directly (f32: on 32 x 128 tiles), with a
