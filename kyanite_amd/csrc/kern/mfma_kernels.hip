@@ -1106,8 +1106,11 @@ int conv_channel_split(const ConvParams &p) {
     shape_only.input = shape_only.filter = nullptr;
     PlaneGeom geom;
     const long long target = plane_geometry(shape_only, 64, &geom) || plane_geometry_any(shape_only, 64, &geom) ? 1024 : 3072;
-    if (tiles * 4 * 2 > target || k < 512) return 1;
-    const long long most = std::min<long long>({16, target / (tiles * 4), p.in_c / 16});
+    // (the plane kernel also takes two parts when every compute unit has a tile but none has two: the ResNet tower at
+    // batch 128, 256 tiles, 709 -> 687 us per evaluation with the parts summed inside the launch)
+    const bool plane = target == 1024;
+    if ((plane ? tiles * 4 > target : tiles * 4 * 2 > target) || k < 512) return 1;
+    const long long most = std::min<long long>({16, std::max<long long>(plane ? 2 : 1, target / (tiles * 4)), p.in_c / 16});
     if (most < 2) return 1;
     // whole slices of CB channels per split, and no split without channels
     const int slices = (p.in_c + CB - 1) / CB;
