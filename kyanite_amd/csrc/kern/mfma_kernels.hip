@@ -697,18 +697,36 @@ __global__ __launch_bounds__(THREADS) void conv_plane_kernel(ConvParams p, Plane
         if (threadIdx.x == 0) *arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (*(volatile int *) arrived != parts - 1) return;
-        for (int from = 0; from < parts; from++) {
+        // (the parts of a small tile are requested four at a time before the first is added: one round trip for four)
+        constexpr int AHEAD = MI * NJ == 1 ? 4 : 1;
+        for (int from0 = 0; from0 < parts; from0 += AHEAD) {
+            floatx4 x[AHEAD][MI][NJ][4];
 #pragma unroll
-            for (int i = 0; i < MI; i++)
+            for (int a = 0; a < AHEAD; a++)
 #pragma unroll
-                for (int j = 0; j < NJ; j++)
+                for (int i = 0; i < MI; i++)
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        const floatx4 x = __builtin_bit_cast(
-                            floatx4, __builtin_amdgcn_raw_buffer_load_b128(slots, from * (BM * TN * 4) + thread_off + ((i * NJ + j) * 4 + q) * 1024, 0, SC1));
+                    for (int j = 0; j < NJ; j++)
 #pragma unroll
-                        for (int u = 0; u < 4; u++) acc[i][j][4 * q + u] = from == 0 ? x[u] : acc[i][j][4 * q + u] + x[u];
-                    }
+                        for (int q = 0; q < 4; q++) {
+                            // (parts past the last read the last one again; they are not added)
+                            const int from = min(from0 + a, parts - 1);
+                            x[a][i][j][q] = __builtin_bit_cast(
+                                floatx4, __builtin_amdgcn_raw_buffer_load_b128(slots, from * (BM * TN * 4) + thread_off + ((i * NJ + j) * 4 + q) * 1024, 0, SC1));
+                        }
+#pragma unroll
+            for (int a = 0; a < AHEAD; a++)
+                if (from0 + a < parts) {
+#pragma unroll
+                    for (int i = 0; i < MI; i++)
+#pragma unroll
+                        for (int j = 0; j < NJ; j++)
+#pragma unroll
+                            for (int q = 0; q < 4; q++)
+#pragma unroll
+                                for (int u = 0; u < 4; u++)
+                                    acc[i][j][4 * q + u] = from0 + a == 0 ? x[a][i][j][q][u] : acc[i][j][4 * q + u] + x[a][i][j][q][u];
+                }
         }
         if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
