@@ -1148,7 +1148,7 @@ long long conv_tail_split(const ConvParams &p, int *parts, int *tile) {
     // which tiles the launch picks (the same estimate as in launch_conv_f32)
     const long long small = ((positions + 63) / 64) * ((p.out_c + 63) / 64), big = ((positions + 127) / 128) * ((p.out_c + 127) / 128);
     const bool big_fits = plane_geometry(shape_only, 128, &geom) || (p.plane_any_width && plane_geometry_any(shape_only, 128, &geom));
-    const bool big_wins = big_fits && (double) ((big * 4 + 1023) / 1024) * 4.0 <= (double) ((small * 4 + 1023) / 1024) * 1.1;
+    const bool big_wins = big_fits && (double) ((big * 4 + 1023) / 1024) * 4.0 * (big < 256 ? 1.2 : 1.0) <= (double) ((small * 4 + 1023) / 1024) * 1.1;
     const long long tiles = big_wins ? big : small, slices = (p.in_c + CB - 1) / CB;
     if (tile) *tile = big_wins ? 128 : 64;
     if (tiles > 0x7fffffffll / 8 || slices < 8) return tiles;
@@ -1158,6 +1158,12 @@ long long conv_tail_split(const ConvParams &p, int *parts, int *tile) {
     // of its own (the tower convolution of a board game network, us per evaluation of 21 of them by batch size:
     // 1024 3487, 1536 6601, 2048 6912).
     const long long round = big_wins ? 512 : 256, rest = tiles % round;
+    // (tiles of 128 x 128, one per compute unit or fewer: all in two parts, so that a compute unit has two workgroups
+    // to overlap)
+    if (big_wins && tiles >= 128 && tiles <= 256 && slices >= 8) {
+        *parts = 2;
+        return 0;
+    }
     if (tiles < round || rest < round / 16 || rest > round / 2) return tiles;
     const long long most = std::min<long long>({4, round / rest, slices / 4});
     if (most < 2) return tiles;
@@ -1253,7 +1259,10 @@ int launch_conv_f32(const ConvParams &params, ihipStream_t *stream) {
         const bool classic = plane_geometry(p, v.tn, &geom);
         if (!classic && !(any_enabled && plane_geometry_any(p, v.tn, &geom))) continue;
         const long long tiles = ((positions + v.tn - 1) / v.tn) * ((p.out_c + v.bm - 1) / v.bm);
-        const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost;
+        // (fewer big tiles than compute units: some of those idle, the others with a single workgroup that has nobody to
+        // overlap its waits with; a fifth dearer. The ResNet tower at batch 448, us: 2110 on 224 big tiles, 1952 on 896
+        // small ones, the last 128 of them shared)
+        const double cost = (double) ((tiles * 4 + 1023) / 1024) * v.unit_cost * (v.id == 22 && tiles < 256 ? 1.2 : 1.0);
         if (!best || cost < best_cost) { best = &v; best_cost = cost; any_w = !classic; }
     }
     // a sparse last round of 64 x 64 tiles: its tiles shared by workgroups that take a slice of the input channels each
