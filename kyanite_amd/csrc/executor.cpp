@@ -308,11 +308,18 @@ void HipExecutor::realise_launch(size_t index, Launch &l, bool mapped) {
     } else if (step.kind == StepKind::MatMul && step.gemm.pair_op) {
         // a gated pair: left operand, the two right operands, the result
         GemmParams gemm = step.gemm;
-        KN_ASSERT(l.ptrs.size() == 4);
+        KN_ASSERT(l.ptrs.size() >= 4);
         gemm.a = l.ptrs[0];
         gemm.b = l.ptrs[1];
         gemm.b_pair = l.ptrs[2];
         gemm.c = l.ptrs[3];
+        {
+            const GemmLaunchPlan lp = plan_gemm_launch(gemm, step.gemm_f16);
+            size_t next = 4;
+            KN_ASSERT(l.ptrs.size() == next + (lp.workspace_bytes > 0) + (lp.counter_bytes > 0));
+            gemm.workspace = lp.workspace_bytes > 0 ? l.ptrs[next++] : nullptr;
+            gemm.counters = lp.counter_bytes > 0 ? l.ptrs[next++] : nullptr;
+        }
         // the kernel reaches both right operands with 32 bit byte offsets from the lower of the two
         const long long apart = std::llabs((const char *) gemm.b_pair - (const char *) gemm.b);
         if (apart + ((long long) (gemm.n / 2) * gemm.b_sn + gemm.k) * 2 >= 0xffffffffll)

@@ -72,9 +72,9 @@ double estimate_f16_direct_us(const GemmParams &p, int groups, int tile, int spl
     if (rest > 0) {
         const long long per_cu = (rest + COMPUTE_UNITS - 1) / COMPUTE_UNITS;
         const int tail = tail_allowed && parts == 1 && p.batch == 1 ? tail_parts(tiles, capacity, p.k) : 0;
-        // a round split into `tail` parts of K: measured at 0.78 of a whole round for two parts (the parts pass
-        // f32 tiles to each other through memory)
-        us += tail ? round_us(per_cu, slices) * (1.0 / tail + 0.28) : round_us(per_cu, slices);
+        // a round split into `tail` parts of K: measured at 0.78 of a whole round for two parts and at 0.46 for
+        // eight (the parts pass f32 tiles through memory and the last one to arrive reads them all)
+        us += tail ? round_us(per_cu, slices) * (1.0 / tail + 0.26 + 0.01 * tail) : round_us(per_cu, slices);
     }
     if (parts > 1) us += SUM_PASS_US + SUM_PASS_US_PER_MB * (double) p.batch * p.m * p.n * (4.0 * parts + 4.0) / 1e6;
     return us;
@@ -177,7 +177,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
                     const unsigned long long bytes = (unsigned long long) split * p.batch * p.m * p.n * 4ull;
                     if (!split_enabled || groups > 1 || p.pair_op || p.k / split < 256 || bytes > (256ull << 20)) continue;
                 }
-                const double us = estimate_f16_direct_us(p, groups, tile, split, tail_enabled && split_enabled && !p.pair_op);
+                const double us = estimate_f16_direct_us(p, groups, tile, split, tail_enabled && split_enabled);
                 if (best_us == 0.0 || us < best_us) {
                     best_us = us;
                     best_tile = tile;
@@ -217,7 +217,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
     // pass between workgroups with accesses that bypass the L2 caches, which costs more than the second launch
     // of a plain split; so a launch with less than one round of tiles keeps that (512 x 4096 x 11008: 69 us
     // against 82 us).
-    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled && model_split <= 1 && !lp.skinny_tile && !p.pair_op) {
+    if (lp.direct && p.batch == 1 && tail_enabled && split_enabled && model_split <= 1 && !lp.skinny_tile) {
         const long long slots = 256 * (lp.tall_tile || lp.narrow_tile ? 1 : 2);
         const long long full = blocks / slots * slots, rest = blocks - full;
         const int parts = tail_parts(blocks, slots, p.k);

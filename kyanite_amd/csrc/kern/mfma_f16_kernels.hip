@@ -606,6 +606,12 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_direct_kernel(GemmParams p,
                     }
         }
         if (threadIdx.x == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if constexpr (sizeof(T) == 2) {
+            if (p.pair_op) {
+                store_tiles_gated<MI, NI>(p, sum, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
+                return;
+            }
+        }
         store_tiles<T, MI, NI>(p, sum, c_base, bz, m0 + wm * 32 * MI, n0 + wn * 32 * NI);
         return;
     }
@@ -711,7 +717,7 @@ int launch_gemm_f16(const GemmLaunchPlan &lp, ihipStream_t *stream) {
         // a gated pair: only what the plan promised (direct kernel, one product per launch, whole K per workgroup), and
         // both matrices within reach of the 32 bit offsets from the lower of the two
         const long long apart = (const char *) p.b_pair - (const char *) p.b, span = ((long long) (p.n / 2) * p.b_sn + p.k) * 2;
-        if (p.pair_op != GEMM_PAIR_SWIGLU || p.b_pair == nullptr || groups > 1 || p.addend || lp.split_k > 1 || lp.tail_split > 1 || lp.swapped ||
+        if (p.pair_op != GEMM_PAIR_SWIGLU || p.b_pair == nullptr || groups > 1 || p.addend || lp.split_k > 1 || lp.swapped ||
             !lp.direct || p.n % 2 != 0 || (apart < 0 ? -apart : apart) + span >= 0xffffffffll || (uintptr_t) p.b_pair % 16 != 0)
             return (int) hipErrorInvalidValue;
     }

@@ -1236,12 +1236,13 @@ private:
         g.pair_op = GEMM_PAIR_SWIGLU;
         // only on the kernel that loads global -> LDS directly, whole K per workgroup (operands in the arena are aligned)
         const GemmLaunchPlan lp = plan_gemm_launch(g, true);
-        if (!lp.direct || lp.swapped || lp.split_k > 1 || lp.tail_split > 1 || lp.dot) return R::done(std::nullopt);
+        if (!lp.direct || lp.swapped || lp.split_k > 1 || lp.dot) return R::done(std::nullopt);
         // both weights lie within the reach of the kernel's 32 bit offsets wherever the arena puts them
         if (dtype_bytes(DType::F16) * (n * (size_t) std::llabs(g.b_sn) + k) * 2 >= ((size_t) 1 << 31)) return R::done(std::nullopt);
 
         PlanTensor result = alloc_tensor_shared({1, m, n}, DType::F16);
         step.operands = {{l, OperandKind::In}, {wg, OperandKind::In}, {wu, OperandKind::In}, {result, OperandKind::Out}};
+        push_gemm_scratch(step);  // (a sparse last round of tiles is shared between workgroups)
         push(std::move(step), value);
         auto viewed = result.view(info.shape.eval(batch_size));
         KN_ASSERT(viewed.has_value(), "a dense matmul result can always be viewed");
