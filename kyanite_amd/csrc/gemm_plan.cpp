@@ -80,6 +80,35 @@ double estimate_f16_direct_us(const GemmParams &p, int groups, int tile, int spl
     return us;
 }
 
+// In how many parts the f32 kernel that loads global -> LDS directly splits K when its tiles do not fill the chip.
+// f32 has a sixteenth of the MFMA rate of f16, so these launches are bound by the matrix cores of the busiest compute
+// unit: workgroups spread evenly, so that unit works through ceil(workgroups / 256) of them, each over its part of K
+// (time per element of K: the MFMA rate at the 0.76 of the peak that 128 x 128 tiles reach and 0.66 for the tiles of
+// 4096 results). The parts that count are those that put a whole number of workgroups on every unit, not as many
+// workgroups as there are places: 86 tiles in 6 parts are 516 workgroups, and the four beyond 2 x 256 made 3 x 704
+// of K the longest path where 5 parts have 2 x 832 (128 x 11008 x 4096: 141 us). The pass that sums the parts and
+// what the memory has to deliver in any case are the other two terms.
+long long f32_direct_parts(const GemmParams &p, long long blocks, bool tile_of_4096, long long most) {
+    const double us_per_k = tile_of_4096 ? 64.0 * 64 * 2 / (256 * 2400.0) / 0.66 : 128.0 * 128 * 2 / (256 * 2400.0) / 0.76;
+    const double results = (double) p.batch * p.m * p.n;
+    const double memory_us = 4.0 * ((double) p.batch * p.k * (p.m + p.n) + results) / 5.0e6;
+    long long best = 1;
+    double best_us = 0.0;
+    for (long long s = 1; s <= std::min(most, 16ll); s++) {
+        long long chunk = ((p.k + s - 1) / s + 31) / 32 * 32;
+        const long long parts = (p.k + chunk - 1) / chunk;
+        if (parts != s || 4.0 * s * results > (double) (256ull << 20)) continue;
+        const long long per_unit = (blocks * s + COMPUTE_UNITS - 1) / COMPUTE_UNITS;
+        // (a stream of weights runs the faster the more workgroups ask for it, up to two per compute unit:
+        // 8 x 4096 x 11008 in 7 parts 40.3 us, in 16 parts 38.6 us)
+        const double asking = std::min(1.0, 0.8 + 0.2 * (double) (blocks * s) / (2.0 * COMPUTE_UNITS));
+        double us = std::max((double) per_unit * ((double) chunk * us_per_k + 1.5), memory_us / asking);
+        if (s > 1) us += 3.0 + 4.0 * (s + 1) * results / 3.0e6;
+        if (best_us == 0.0 || us < best_us) best_us = us, best = s;
+    }
+    return best;
+}
+
 }  // namespace
 
 GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
@@ -257,6 +286,7 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
         const int min_chunk = few_tiles ? 128 : (f16 ? 512 : 256);  // K elements a split should at least cover
         long long s = (split_target + blocks - 1) / blocks;
         if (s > p.k / min_chunk) s = p.k / min_chunk;
+        if (!f16 && lp.direct) s = f32_direct_parts(p, blocks, lp.small_tile || lp.skinny_tile, p.k / min_chunk);
         if (s > 1) {
             long long chunk = (p.k + s - 1) / s;
             chunk = (chunk + lp.bk - 1) / lp.bk * lp.bk;

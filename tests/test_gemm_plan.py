@@ -242,3 +242,25 @@ def test_f16_tiles_come_from_the_cost_model():
         ex = HipExecutor(0, g, 0, plan_only=True)
         text = [ex.step_str(i) for i in range(ex.step_count()) if "MatMul" in ex.step_str(i)][0]
         assert want in text, (m, n, k, text)
+
+
+def test_f32_parts_of_k_put_whole_layers_of_workgroups_on_the_chip():
+    """f32 products on the kernel that loads global -> LDS directly, with too few tiles for 256 compute units: the
+    parts of K are chosen by the busiest unit, which works through ceil(tiles * parts / 256) workgroups. 86 tiles in
+    6 parts would be 516 workgroups, three on four units and two on all others."""
+    expected = {
+        (32, 11008, 4096): ("direct 32x128 bk32 split_k=5x832", 86),
+        (64, 11008, 4096): ("direct 64x64 bk32 split_k=4x1024", 172),
+        (128, 11008, 4096): ("direct 128x128 bk32 split_k=8x512", 86),
+        (256, 4672, 2048): ("direct 128x128 bk32 split_k=3x704", 74),
+        (8, 4096, 11008): ("direct 32x128 bk32 split_k=16x704", 32),
+        (8, 32000, 1024): ("direct 32x128 bk32]", 250),
+    }
+    for (m, n, k), (text, tiles) in expected.items():
+        g = Graph()
+        g.output(g.mat_mul(g.input([m, k]), g.constant([k, n], np.zeros((k, n), np.float32))))
+        ex = HipExecutor(0, g, 0, plan_only=True)
+        assert text in ex.step_str(0), ex.step_str(0)
+        parts = int(re.search(r"split_k=(\d+)x", ex.step_str(0)).group(1)) if "split_k" in text else 1
+        last_layer = tiles * parts % 256
+        assert last_layer == 0 or last_layer >= 128, (m, n, k, tiles * parts)
