@@ -340,9 +340,9 @@ int knhip_executor_io_info(const knhip_executor *ex, int is_output, size_t index
 
 /* CudaExecutor::evaluate (executor.rs:117-195): dense row-major host buffers in, dense row-major host buffers out.
  * Byte counts are checked against the planned shapes. Every byte is copied once on the host on each side (caller's
- * buffer <-> page-locked staging, straight from and into the caller's buffers); tensors above 8 MiB move in chunks, the
+ * buffer <-> page-locked staging, straight from and into the caller's buffers); tensors above 2 MiB move in chunks of 2 to 8 MiB, the
  * host copy of one chunk overlapping the bus transfer of another, with the host copies spread over up to four threads
- * (three of them owned by the executor, started by the first evaluation that has 4 MiB or more to copy at once). */
+ * (three of them owned by the executor, started by the first evaluation that has 2 MiB or more to copy at once). */
 int knhip_executor_evaluate(knhip_executor *ex, const void *const *inputs, const size_t *input_bytes, size_t input_count,
                             void *const *outputs, const size_t *output_bytes, size_t output_count);
 /* run_async (executor.rs:199-258): launch all steps on the executor's stream, no synchronisation */

@@ -508,12 +508,22 @@ void HipExecutor::run_async() {
 
 void HipExecutor::host_copy(void *dst, const void *src, size_t bytes) {
     // below a few MB a second thread would still be waking up when the first one is done
-    if (bytes < ((size_t) 4 << 20)) {
+    if (bytes < ((size_t) 2 << 20)) {
         std::memcpy(dst, src, bytes);
         return;
     }
     if (!copy_pool_) copy_pool_ = std::make_unique<HostCopyPool>(3);
     copy_pool_->copy(dst, src, bytes);
+}
+
+// The chunk a tensor of `bytes` moves in between page-locked staging and the device: a quarter of it, between
+// `kCopyChunkLeast` and `kCopyChunkBytes`, so that tensors of a few MB already overlap the host's copy with the copy
+// engine's (a 512 token LLaMA evaluation with 4 MB in and out 0.885 -> 0.853 ms, the UNet block with 10.5 MB each
+// way 1.90 -> 1.75 ms, the ResNet tower with 19 MB of policies 4.21 -> 4.13 ms against one chunk of 8 MB).
+size_t HipExecutor::copy_chunk_bytes(size_t bytes) {
+    const size_t grain = (size_t) 256 << 10;
+    const size_t quarter = (bytes / 4 + grain - 1) & ~(grain - 1);
+    return std::min(kCopyChunkBytes, std::max(quarter, kCopyChunkLeast));
 }
 
 void HipExecutor::evaluate(const void *const *inputs, void *const *outputs) {
@@ -526,8 +536,9 @@ void HipExecutor::evaluate(const void *const *inputs, void *const *outputs) {
     for (size_t i = 0; i < plan_.inputs.size(); i++) {
         const size_t bytes = plan_.inputs[i].shape.size() * dtype_bytes(plan_.inputs[i].dtype);
         KN_ASSERT(plan_.inputs[i].shape.has_simple_strides());
-        for (size_t off = 0; off < bytes; off += kCopyChunkBytes) {
-            const size_t n = std::min(kCopyChunkBytes, bytes - off);
+        const size_t chunk = copy_chunk_bytes(bytes);
+        for (size_t off = 0; off < bytes; off += chunk) {
+            const size_t n = std::min(chunk, bytes - off);
             host_copy((char *) pinned_inputs_[i] + off, (const char *) inputs[i] + off, n);
             if (!mapped)
                 hip_check(hipMemcpyAsync((char *) input_ptr(i) + off, (char *) pinned_inputs_[i] + off, n, hipMemcpyHostToDevice, stream_),
@@ -540,13 +551,14 @@ void HipExecutor::evaluate(const void *const *inputs, void *const *outputs) {
     std::vector<Chunk> chunks;
     for (size_t i = 0; i < plan_.outputs.size(); i++) {
         const size_t bytes = plan_.outputs[i].shape.size() * dtype_bytes(plan_.outputs[i].dtype);
-        for (size_t off = 0; off < bytes; off += kCopyChunkBytes) chunks.push_back({i, off, std::min(kCopyChunkBytes, bytes - off)});
+        const size_t chunk = copy_chunk_bytes(bytes);
+        for (size_t off = 0; off < bytes; off += chunk) chunks.push_back({i, off, std::min(chunk, bytes - off)});
     }
     // an event behind every chunk but the last, so that the host can copy a chunk out while the next ones still move
-    // (outputs that make one chunk's worth between them wait for the stream once instead)
+    // (outputs that do not make the smallest chunk between them wait for the stream once instead)
     size_t output_bytes = 0;
     for (auto &ch : chunks) output_bytes += ch.bytes;
-    const size_t n_events = output_bytes > kCopyChunkBytes ? chunks.size() - 1 : 0;
+    const size_t n_events = output_bytes > kCopyChunkLeast ? chunks.size() - 1 : 0;
     if (mapped) {
         last_profile_ = std::nullopt;
         if (fused_function_) launch_fused(true);

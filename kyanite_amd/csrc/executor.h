@@ -49,10 +49,12 @@ public:
 
     // Dense host buffers in, dense host buffers out (executor.rs:117-195; the C ABI has checked counts and sizes).
     // Every byte crosses host memory once on each side: caller -> page-locked staging -> device and back. Tensors of
-    // more than `kCopyChunkBytes` move in chunks, so that the copy engine works on one chunk while the host copies
-    // the next one (inputs) or the one before (outputs), with the host copies of big chunks spread over a few threads.
+    // more than `kCopyChunkLeast` move in chunks (a quarter of the tensor, `kCopyChunkBytes` at most), so that the
+    // copy engine works on one chunk while the host copies the next one (inputs) or the one before (outputs), with
+    // the host copies of chunks spread over a few threads.
     void evaluate(const void *const *inputs, void *const *outputs);
-    static constexpr size_t kCopyChunkBytes = (size_t) 8 << 20;
+    static constexpr size_t kCopyChunkBytes = (size_t) 8 << 20, kCopyChunkLeast = (size_t) 2 << 20;
+    static size_t copy_chunk_bytes(size_t bytes);
     // launch the steps on the executor's stream without any synchronisation (executor.rs:197-258)
     void run_async();
     void synchronize();

@@ -1,4 +1,5 @@
-"""`evaluate` moves tensors of more than 8 MiB in chunks (host copy of one chunk while the copy engine moves another)
+"""`evaluate` moves tensors of more than 2 MiB in chunks of a quarter of the tensor, 2 MiB at least and 8 MiB at most
+(host copy of one chunk while the copy engine moves another)
 and spreads big host copies over threads: results must not depend on where the chunk boundaries fall
 (kn-cuda-eval/src/executor.rs:117-195 is the path; the reference copies every tensor in one piece)."""
 import numpy as np
@@ -7,11 +8,12 @@ import pytest
 from kyanite_amd import DType, Graph, HipExecutor, KnError
 from oracle import cpu_eval_graph
 
-CHUNK = 8 << 20
+CHUNK, LEAST = 8 << 20, 2 << 20
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("elements", [CHUNK // 4 - 1, CHUNK // 4, CHUNK // 4 + 1, 3 * (CHUNK // 4) + 12345, 1])
+@pytest.mark.parametrize("elements", [CHUNK // 4 - 1, CHUNK // 4, CHUNK // 4 + 1, 3 * (CHUNK // 4) + 12345, 1,
+                                      LEAST // 4, LEAST // 4 + 1, LEAST + 77, 4 * CHUNK // 4 + 3, 5 * (CHUNK // 4) + 1])
 def test_tensors_around_the_chunk_size_arrive_whole(elements, hip_device):
     print(f"evaluate with {elements} f32 elements per tensor", flush=True)
     g = Graph()
