@@ -424,15 +424,389 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2
     }
 }
 
+// The same computation for long sequences, where the lines of K and V that the workgroups request bound the launch
+// (32 heads of 2048 queries and keys under a causal mask: 104 us in the kernel above, which fetches every block of
+// keys once per 32 queries). Here a workgroup owns 128 queries: wave w has queries 32 w .. 32 w + 31 of the tile, with
+// a running softmax of its own over ALL blocks of keys, and the four waves fetch every block together, a quarter of
+// its vectors each, into one of two LDS buffers: a block is requested once per 128 queries. One barrier per block:
+// the block is staged into the buffer that nobody has read since the barrier before. A block is fetched when any
+// of the four tiles of queries needs it; a wave whose own tile has it masked out only helps to stage it. The result
+// of a query is complete in its wave, so there is no merge; it goes through LDS to be stored as whole rows.
+template <int DK, int DVT>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_f16_shared_kernel(AttentionParams p) {
+    constexpr int DV = 32 * DVT, KS = DK + 8, VS = (DV + 31) / 64 * 64 + 32;
+    constexpr int KC = DK / 8, VC = DV / 8;                 // 16 byte pieces per row
+    constexpr int THREADS = 64 * WAVES;
+    constexpr int K_VECS = BKEYS * KC / THREADS;            // 128 bit loads of K per lane and block
+    constexpr int V_VECS = BKEYS * VC / THREADS;            // and of V
+    constexpr int Q_VECS = 32 * KC / 64;                    // of the wave's own 32 rows of Q
+    constexpr int O_VECS = 32 * VC / 64;                    // 128 bit stores of the wave's 32 rows of the result
+    constexpr int OS = DV + 8;                              // halves per row of the result in LDS
+    constexpr int STAGE = BKEYS * KS + BKEYS * VS;          // halves per buffer
+    constexpr int WAVE_ROWS = 32 * (KS > OS ? KS : OS);     // halves of a wave's own rows of Q, later of the result
+    constexpr int LDS_HALVES = 2 * STAGE > WAVES * WAVE_ROWS ? 2 * STAGE : WAVES * WAVE_ROWS;
+    static_assert(DK % 64 == 0 && BKEYS * KC % THREADS == 0 && BKEYS * VC % THREADS == 0 && 32 * VC % 64 == 0, "unsupported shape");
+    __shared__ __attribute__((aligned(16))) half_t lds[LDS_HALVES];
+    __shared__ unsigned long long needed_by[WAVES][4];
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 31, h = lane >> 5;
+    // (the order of the tiles under a causal mask: see the kernel above)
+    int tile = blockIdx.x, bz = blockIdx.y;
+    {
+        const int nt = gridDim.x, pairs = nt >> 1;
+        if ((nt & 1) == 0) {
+            int linear = bz * nt + tile;
+            const int half_launch = pairs * (int) gridDim.y;
+            const bool late = linear < half_launch;
+            if (!late) linear -= half_launch;
+            bz = linear / pairs;
+            const int t = linear - bz * pairs;
+            tile = late ? nt - 1 - t : t;
+        }
+    }
+    const int tile32 = tile * WAVES + wave, tiles32 = (p.lq + 31) / 32;
+    const bool wave_has_queries = tile32 < tiles32;
+    const int query = tile32 * 32 + c;
+    const int query_c = min(query, p.lq - 1);
+    const int bz1 = bz / p.batch_inner, bz2 = bz - bz1 * p.batch_inner;
+    const half_t *kp = (const half_t *) p.k + bz1 * p.k_sb + bz2 * p.k_sb2, *vp = (const half_t *) p.v + bz1 * p.v_sb + bz2 * p.v_sb2;
+    const half_t *mp = p.mask ? (const half_t *) p.mask + bz * p.m_sb + (long long) query_c * p.m_sq : nullptr;
+
+    // ---- what the mask does to each block of keys for this wave's queries (lane l of register r: block 64 r + l),
+    // and which blocks any wave of the workgroup needs
+    const int n_blocks = (p.lk + BKEYS - 1) / BKEYS;
+    int class_reg[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int kb = 64 * r + lane;
+        int cls = mp ? 0 : 2;
+        if (p.block_class && wave_has_queries && kb < n_blocks)
+            cls = ((const unsigned char *) p.block_class)[((long long) (p.m_sb ? bz : 0) * tiles32 + tile32) * n_blocks + kb];
+        class_reg[r] = wave_has_queries && kb < n_blocks ? cls : 1;
+        const unsigned long long needs = __ballot(class_reg[r] != 1);
+        if (lane == 0) needed_by[wave][r] = needs;
+    }
+    auto block_class = [&](int i) {
+        const int r = i >> 6;
+        const int reg = r == 0 ? class_reg[0] : r == 1 ? class_reg[1] : r == 2 ? class_reg[2] : class_reg[3];
+        return __builtin_amdgcn_readlane(reg, i & 63);
+    };
+
+    // ---- Q: the wave's 32 rows, whole lines at a time, through the wave's own rows of LDS
+    const char *qb = (const char *) ((const half_t *) p.q + bz1 * p.q_sb + bz2 * p.q_sb2);
+    const unsigned q_row = (unsigned) p.q_sm * 2;
+    halfx8 qreg[Q_VECS];
+#pragma unroll
+    for (int i = 0; i < Q_VECS; i++) {
+        const int e = lane + 64 * i, row = e / KC, part = e % KC;
+        qreg[i] = *(const halfx8 *) (qb + ((unsigned) min(tile32 * 32 + row, p.lq - 1) * q_row + 16 * part));
+    }
+    __syncthreads();  // (needed_by is written)
+    unsigned long long needed[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        unsigned long long any = 0;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) any |= needed_by[w][r];
+        needed[r] = ((unsigned long long) __builtin_amdgcn_readfirstlane((unsigned) (any >> 32)) << 32) | (unsigned) __builtin_amdgcn_readfirstlane((unsigned) any);
+    }
+    auto next_live = [&](int i) {
+        while (i < n_blocks) {
+            const int r = i >> 6;
+            const unsigned long long bits = r == 0 ? needed[0] : r == 1 ? needed[1] : r == 2 ? needed[2] : needed[3];
+            if ((bits >> (i & 63)) & 1) break;
+            i++;
+        }
+        return i;
+    };
+
+    // ---- global -> registers -> LDS, a quarter of a block per wave
+    halfx8 kreg[K_VECS], vreg[V_VECS];
+    const unsigned k_row = (unsigned) p.k_sn * 2, v_row = (unsigned) p.v_sk * 2;
+    unsigned koff[K_VECS], voff[V_VECS];  // in bytes
+#pragma unroll
+    for (int i = 0; i < K_VECS; i++) {
+        const int e = (int) threadIdx.x + THREADS * i;
+        koff[i] = (unsigned) (e / KC) * k_row + 16 * (e % KC);
+    }
+#pragma unroll
+    for (int i = 0; i < V_VECS; i++) {
+        const int e = (int) threadIdx.x + THREADS * i;
+        voff[i] = (unsigned) (e / VC) * v_row + 2 * min(8 * (e % VC), (p.dv - 1) & ~7);  // dims past dv: any valid vector
+    }
+    uintx4 mraw[2];
+    const unsigned moff = (unsigned) (query_c * (int) p.m_sq + 16 * h) * 2;
+    const char *mbase = p.mask ? (const char *) ((const half_t *) p.mask + bz * p.m_sb) : nullptr;
+    auto mask_as_rows = [&](int key0) { return p.mask_vec == 2 && key0 + BKEYS <= p.lk; };
+    auto fetch = [&](int i) {
+        const int key0 = i * BKEYS;
+        const char *kb = (const char *) (kp + (long long) key0 * p.k_sn), *vb = (const char *) (vp + (long long) key0 * p.v_sk);
+        if (key0 + BKEYS <= p.lk) {
+#pragma unroll
+            for (int j = 0; j < K_VECS; j++) kreg[j] = *(const halfx8 *) (kb + koff[j]);
+#pragma unroll
+            for (int j = 0; j < V_VECS; j++) vreg[j] = *(const halfx8 *) (vb + voff[j]);
+        } else {
+            const int last = p.lk - 1 - key0;  // last valid row of the block
+#pragma unroll
+            for (int j = 0; j < K_VECS; j++) {
+                const int key = ((int) threadIdx.x + THREADS * j) / KC;
+                kreg[j] = *(const halfx8 *) (kb + (koff[j] - (unsigned) (key - min(key, last)) * k_row));
+            }
+#pragma unroll
+            for (int j = 0; j < V_VECS; j++) {
+                const int key = ((int) threadIdx.x + THREADS * j) / VC;
+                vreg[j] = *(const halfx8 *) (vb + (voff[j] - (unsigned) (key - min(key, last)) * v_row));
+            }
+        }
+        if (block_class(i) == 0) {
+            if (mask_as_rows(key0)) {
+                const char *mb = mbase + 2 * key0;
+                mraw[0] = *(const uintx4 *) (mb + moff);
+                mraw[1] = *(const uintx4 *) (mb + (moff + 16));
+            } else {
+                halfx4 m[4];
+#pragma unroll
+                for (int a = 0; a < 4; a++)
+#pragma unroll
+                    for (int b = 0; b < 4; b++)
+                        m[a][b] = mp[(long long) min(key0 + 8 * a + 4 * h + b, p.lk - 1) * p.m_sk];
+                mraw[0] = uintx4{__builtin_bit_cast(uint2, m[0]).x, __builtin_bit_cast(uint2, m[0]).y, __builtin_bit_cast(uint2, m[1]).x, __builtin_bit_cast(uint2, m[1]).y};
+                mraw[1] = uintx4{__builtin_bit_cast(uint2, m[2]).x, __builtin_bit_cast(uint2, m[2]).y, __builtin_bit_cast(uint2, m[3]).x, __builtin_bit_cast(uint2, m[3]).y};
+            }
+        }
+    };
+    // (the order of the mask's registers: see the kernel above)
+    auto mask_in_order = [&](int key0, halfx4 (&mv)[4]) {
+        uint2 m[4];
+        if (mask_as_rows(key0)) {
+            const auto s0 = __builtin_amdgcn_permlane32_swap(mraw[0][0], mraw[0][2], false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(mraw[0][1], mraw[0][3], false, false);
+            const auto s2 = __builtin_amdgcn_permlane32_swap(mraw[1][0], mraw[1][2], false, false);
+            const auto s3 = __builtin_amdgcn_permlane32_swap(mraw[1][1], mraw[1][3], false, false);
+            m[0] = uint2{s0[0], s1[0]};
+            m[2] = uint2{s0[1], s1[1]};
+            m[1] = uint2{s2[0], s3[0]};
+            m[3] = uint2{s2[1], s3[1]};
+        } else {
+            m[0] = uint2{mraw[0][0], mraw[0][1]};
+            m[1] = uint2{mraw[0][2], mraw[0][3]};
+            m[2] = uint2{mraw[1][0], mraw[1][1]};
+            m[3] = uint2{mraw[1][2], mraw[1][3]};
+        }
+#pragma unroll
+        for (int a = 0; a < 4; a++) mv[a] = __builtin_bit_cast(halfx4, m[a]);
+    };
+    auto stage = [&](int key0, half_t *buffer) {
+        half_t (*Ks)[KS] = (half_t (*)[KS]) buffer;
+        half_t (*Vs)[VS] = (half_t (*)[VS]) (buffer + BKEYS * KS);
+        const halfx8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+        const bool full = key0 + BKEYS <= p.lk;
+#pragma unroll
+        for (int j = 0; j < K_VECS; j++) {
+            const int e = (int) threadIdx.x + THREADS * j;
+            *(halfx8 *) &Ks[e / KC][8 * (e % KC)] = kreg[j];
+        }
+#pragma unroll
+        for (int j = 0; j < V_VECS; j++) {
+            const int e = (int) threadIdx.x + THREADS * j, key = e / VC;
+            *(halfx8 *) &Vs[key][8 * (e % VC)] = full || key0 + key < p.lk ? vreg[j] : zero;
+        }
+    };
+
+    int i = next_live(0);
+    if (i < n_blocks) fetch(i);
+
+    // ---- Q into LDS, and from there each lane's operand: lane (query c, half h) holds k = 16 t + 8 h .. + 7 for step t
+    halfx8 qf[DK / 16];
+    {
+        half_t (*Qs)[KS] = (half_t (*)[KS]) (lds + wave * WAVE_ROWS);
+#pragma unroll
+        for (int j = 0; j < Q_VECS; j++) {
+            const int e = lane + 64 * j;
+            *(halfx8 *) &Qs[e / KC][8 * (e % KC)] = qreg[j];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < DK / 16; t++) {
+            qf[t] = *(const halfx8 *) &Qs[c][16 * t + 8 * h];
+            if (query >= p.lq) qf[t] = halfx8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+        __syncthreads();  // (the buffers of K and V lie over these rows)
+    }
+
+    floatx16 oacc[DVT];
+#pragma unroll
+    for (int t = 0; t < DVT; t++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) oacc[t][v] = 0.0f;
+    float row_max = -INFINITY, row_sum = 0.0f;
+    const float scale = p.scale;
+    constexpr float LOG2E = 1.44269504088896340736f;
+    // the lane's corner of the transposed reads of V inside a buffer (see the kernel above)
+    const int v_corner = BKEYS * KS + (4 * h + (lane & 15) / 4) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    int parity = 0;
+    while (i < n_blocks) {
+        const int key0 = i * BKEYS, cls = block_class(i), i_next = next_live(i + 1);
+        half_t *buffer = lds + parity * STAGE;
+        parity ^= 1;
+        halfx4 mv[4];
+        bool skip = cls == 1;
+        if (cls == 0) {
+            mask_in_order(key0, mv);
+            unsigned differs = 0;  // from -inf (0xfc00), two values at a time
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                const uint2 bits = __builtin_bit_cast(uint2, mv[a]);
+                differs |= (bits.x ^ 0xfc00fc00u) | (bits.y ^ 0xfc00fc00u);
+            }
+            skip = __all(differs == 0);
+        }
+        stage(key0, buffer);
+        if (i_next < n_blocks) fetch(i_next);
+        i = i_next;
+        __syncthreads();
+        if (skip) continue;
+
+        const half_t (*Ks)[KS] = (const half_t (*)[KS]) buffer;
+        floatx16 st;
+#pragma unroll
+        for (int v = 0; v < 16; v++) st[v] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < DK / 16; t++) {
+            const halfx8 a = *(const halfx8 *) &Ks[c][16 * t + 8 * h];
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[t], st, 0, 0, 0);
+        }
+        // the roundings of matmul -> * scale -> + mask in f16 arithmetic (see the kernel above)
+        halfx2 sh[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            floatx2 two;
+            two[0] = st[2 * j];
+            two[1] = st[2 * j + 1];
+            sh[j] = __builtin_convertvector(two, halfx2);
+        }
+        if (p.has_scale) {
+            halfx2 scale2;
+            scale2[0] = scale2[1] = (half_t) scale;
+#pragma unroll
+            for (int j = 0; j < 8; j++) sh[j] = sh[j] * scale2;
+        }
+        if (cls == 0) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                halfx2 m;
+                m[0] = mv[j >> 1][2 * (j & 1)];
+                m[1] = mv[j >> 1][2 * (j & 1) + 1];
+                sh[j] = sh[j] + m;
+            }
+        }
+        if (key0 + BKEYS > p.lk) {  // the last, partial block of keys
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                if (key0 + 8 * (v >> 2) + 4 * h + (v & 3) >= p.lk) sh[v >> 1][v & 1] = (half_t) -INFINITY;
+        }
+        // the running softmax in f32, its reference following the maximum lazily (see the kernel above)
+        float block_max = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            st[v] = (float) sh[v >> 1][v & 1];
+            block_max = fmaxf(block_max, st[v]);
+        }
+        block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
+        constexpr float SLACK = 8.0f / LOG2E;
+        if (__any(block_max > row_max + SLACK)) {
+            const float new_max = fmaxf(row_max, block_max);
+            const float alpha = __builtin_amdgcn_exp2f((row_max - (new_max == -INFINITY ? 0.0f : new_max)) * LOG2E);
+            row_max = new_max;
+            row_sum *= alpha;
+#pragma unroll
+            for (int t = 0; t < DVT; t++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) oacc[t][v] *= alpha;
+        }
+        const float minus_ref = (row_max == -INFINITY ? 0.0f : -row_max) * LOG2E;
+        float block_sum = 0.0f;
+        halfx8 pv[2];
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(st[v], LOG2E, minus_ref));
+            block_sum += e;
+            pv[v >> 3][v & 7] = (half_t) e;
+        }
+        row_sum += block_sum;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            halfx8 a[DVT];
+#pragma unroll
+            for (int t = 0; t < DVT; t++) {
+                const halfx4 lo = lds_read_transposed(buffer + v_corner + (16 * s) * VS + 32 * t);
+                const halfx4 hi = lds_read_transposed(buffer + v_corner + (16 * s + 8) * VS + 32 * t);
+                a[t] = halfx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            }
+#pragma unroll
+            for (int t = 0; t < DVT; t++) oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[t], pv[s], oacc[t], 0, 0, 0);
+        }
+    }
+
+    // ---- the result: normalised, rounded, through the wave's own rows of LDS into whole rows of O
+    row_sum += __shfl_xor(row_sum, 32);
+    const float inv = 1.0f / row_sum;
+    __syncthreads();  // (every wave is done with the buffers of K and V)
+    half_t (*Os)[OS] = (half_t (*)[OS]) (lds + wave * WAVE_ROWS);
+#pragma unroll
+    for (int t = 0; t < DVT; t++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {  // registers 4 a .. 4 a + 3: dims 32 t + 8 a + 4 h + (0 .. 3)
+            halfx4 out;
+#pragma unroll
+            for (int u = 0; u < 4; u++) out[u] = (half_t) (oacc[t][4 * a + u] * inv);
+            *(halfx4 *) &Os[c][32 * t + 8 * a + 4 * h] = out;
+        }
+    __syncthreads();
+    half_t *ob = (half_t *) p.o + bz1 * p.o_sb + bz2 * p.o_sb2;
+#pragma unroll
+    for (int j = 0; j < O_VECS; j++) {
+        const int e = lane + 64 * j, row = e / VC, d0 = 8 * (e % VC), q = tile32 * 32 + row;
+        if (q >= p.lq || d0 >= p.dv) continue;
+        const halfx8 out = *(const halfx8 *) &Os[row][d0];
+        half_t *op = ob + (long long) q * p.o_sm;
+        if (p.o_sn == 1 && p.o_vec) {
+            *(halfx8 *) (op + d0) = out;
+        } else {
+#pragma unroll
+            for (int u = 0; u < 8; u++) op[(long long) (d0 + u) * p.o_sn] = out[u];
+        }
+    }
+}
+
 template <int DK, int DVT>
 void launch_waves(const AttentionParams &p, hipStream_t stream) {
     hipLaunchKernelGGL((attention_f16_kernel<DK, DVT>), dim3((unsigned) ((p.lq + 31) / 32), (unsigned) p.batch), dim3(64 * WAVES), 0, stream, p);
+}
+
+template <int DK, int DVT>
+void launch_shared(const AttentionParams &p, hipStream_t stream) {
+    hipLaunchKernelGGL((attention_f16_shared_kernel<DK, DVT>), dim3((unsigned) ((p.lq + 127) / 128), (unsigned) p.batch), dim3(64 * WAVES), 0, stream, p);
 }
 
 }  // namespace
 
 bool attention_f16_supported(int dk, int dv) {
     return (dk == 64 || dk == 128) && dv >= 8 && dv <= 128 && dv % 8 == 0;
+}
+
+// The kernel whose workgroups own 128 queries takes four times fewer lines of K and V through the caches, and per
+// block of keys a wave of it does four times the work between two barriers. It wins from two workgroups per compute
+// unit on (causal, width 128, us: 32 heads of 2048 tokens 100.7 -> 75.8, of 4096 295.8 -> 231.2; 64 heads of 1024
+// 64.7 -> 43.5, of 2048 183.9 -> 111.9; 16 x 4096 queries on 77 keys 16.6 -> 9.1) and loses below (32 heads of 1024
+// tokens 35.3 -> 39.8, of 512 14.8 -> 21.8). Its staging needs the width of V in tiles of 32 to be 2 or 4.
+bool attention_f16_shares_keys(const AttentionParams &p) {
+    const int dvt = (p.dv + 31) / 32;
+    if (dvt != 2 && dvt != 4) return false;
+    return (long long) ((p.lq + 127) / 128) * p.batch >= 512;
 }
 
 int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream) {
@@ -460,6 +834,16 @@ int launch_attention_f16(const AttentionParams &p, ihipStream_t *stream) {
     // block classes are indexed by at most 64 blocks per wave
     if (!p.mask || p.lk > 64 * 4 * ATTENTION_F16_BLOCK) q.block_class = nullptr;
     const int dvt = (p.dv + 31) / 32;
+    if (attention_f16_shares_keys(p)) {
+        if (p.dk == 64) {
+            if (dvt == 2) launch_shared<64, 2>(q, stream);
+            else launch_shared<64, 4>(q, stream);
+        } else {
+            if (dvt == 2) launch_shared<128, 2>(q, stream);
+            else launch_shared<128, 4>(q, stream);
+        }
+        return (int) hipGetLastError();
+    }
     if (p.dk == 64) {
         switch (dvt) {
             case 1: launch_waves<64, 1>(q, stream); break;

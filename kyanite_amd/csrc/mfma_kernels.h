@@ -188,6 +188,8 @@ std::vector<unsigned char> attention_f16_block_classes(const void *mask_f16, int
 // widths the fused kernel is built for; other chains run as matmul, softmax, matmul
 bool attention_supported(int dk, int dv);
 bool attention_f16_supported(int dk, int dv);
+// whether the launch takes the kernel whose workgroups own 128 queries and fetch every block of keys once
+bool attention_f16_shares_keys(const AttentionParams &p);
 
 // All return a hipError_t value (0 = success).
 int launch_attention_f32(const AttentionParams &p, ihipStream_t *stream);

@@ -25,7 +25,8 @@ std::string Step::str() const {
     ss << step_kind_name(kind) << " value=" << debug_value;
     if (!debug_id.empty()) ss << " id=\"" << debug_id << "\"";
     if (kind == StepKind::MatMul && attention)
-        ss << " attention " << (gemm_f16 ? "f16" : "f32") << (attention_has_mask ? (attention_has_classes ? " +mask (constant, classified by block)" : " +mask") : "") << " b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv;
+        ss << " attention " << (gemm_f16 ? "f16" : "f32") << (attention_has_mask ? (attention_has_classes ? " +mask (constant, classified by block)" : " +mask") : "") << " b=" << attn.batch << " lq=" << attn.lq << " lk=" << attn.lk << " dk=" << attn.dk << " dv=" << attn.dv
+           << (gemm_f16 && attention_f16_shares_keys(attn) ? " [128 queries share each block of keys]" : "");
     else if (kind == StepKind::MatMul) {
         ss << (gemm_f16 ? " f16" : " f32") << " b=" << gemm.batch << " m=" << gemm.m << " n=" << gemm.n << " k=" << gemm.k
            << (gemm_has_addend ? " +add" : "") << (gemm_has_addend2 ? " +add" : "") << (gemm.relu ? " relu" : "");

@@ -1728,6 +1728,47 @@ def attention_f16_mask_on_the_left_no_scale():
     return _attention_f16_case(133, 2, 40, 72, 128, 96, False, "left")
 
 
+# From 512 workgroups of 128 queries on, the f16 attention runs on the kernel whose four waves own 32 queries each and
+# stage every block of keys together (`attention_f16_shares_keys`).
+
+@case
+def attention_f16_shared_keys_causal():
+    """128 batch entries of 450 queries and keys under a causal mask: the last tile of 128 has 66 queries, so its
+    third wave holds two and its fourth none (it only helps to stage); every wave skips the blocks above its own
+    part of the diagonal while the waves below it still need them"""
+    return _attention_f16_case(140, 128, 450, 450, 64, 64, True, "causal")
+
+
+@case
+def attention_f16_shared_keys_mask_tensor():
+    """a mask tensor whose rows of 77 values are not aligned (read value by value), keys in two whole blocks and one
+    of 13, V of width 40 in two tiles of 32"""
+    return _attention_f16_case(141, 128, 512, 77, 128, 40, True, "full")
+
+
+@case
+def attention_f16_shared_keys_plain_heads():
+    """no mask, no scale, operands that are permuted views, width 128. (Queries a tenth as large, so that the scores
+    stay around 1 without the scale: at 11 a last place of an f16 score is 3 % of its key's weight, and among 8 M
+    results one lands further than 2 % from the oracle, whose dot products add up in another order.)"""
+    g, batch, inputs, _ = _attention_f16_case(142, 128, 512, 130, 128, 128, False, None, "heads")
+    inputs[0] = (inputs[0].astype(np.float32) * 0.1).astype(np.float16)
+    return g, batch, inputs, None
+
+
+@case
+def attention_f16_shared_keys_aligned_mask_rows():
+    """a mask tensor with rows of 96 values (whole, aligned rows: read as vectors), K of width 64 against V of 128"""
+    return _attention_f16_case(143, 128, 512, 96, 64, 128, True, "full")
+
+
+@case
+def attention_f16_shared_keys_many_blocks():
+    """8 queries per batch entry against 2100 keys (66 blocks: the classes of a wave fill more than one register),
+    the causal mask shifted so that only the last, partial block is masked in part"""
+    return _attention_f16_case(144, 512, 8, 2100, 64, 64, True, "causal")
+
+
 @case
 def rotary_of_two_tensors_is_one_launch():
     """two rotary embeddings (two concats of two elementwise halves each) over different inputs and the same cos / sin:
