@@ -1758,8 +1758,9 @@ def attention_f16_shared_keys_plain_heads():
 
 @case
 def attention_f16_shared_keys_aligned_mask_rows():
-    """a mask tensor with rows of 96 values (whole, aligned rows: read as vectors), K of width 64 against V of 128"""
-    return _attention_f16_case(143, 128, 512, 96, 64, 128, True, "full")
+    """a mask tensor with rows of 96 values (whole, aligned rows: read as vectors), K of width 64 against V of 128;
+    40 queries per batch entry: one full wave, one with 8 queries and two that only stage"""
+    return _attention_f16_case(143, 512, 40, 96, 64, 128, True, "full")
 
 
 @case
