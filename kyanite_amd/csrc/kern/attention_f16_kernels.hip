@@ -677,11 +677,15 @@ void attention_f16_shared_kernel(AttentionParams p) {
         floatx16 st;
 #pragma unroll
         for (int v = 0; v < 16; v++) st[v] = 0.0f;
+        // (all of the block's K operands are requested before the first MFMA: one LDS round trip ahead of the chain
+        // instead of one per pair of MFMAs, which is what the compiler makes of the plain loop; 2 % here, and a
+        // loss in the kernel above, whose waves do not wait for each other)
+        halfx8 ka[DK / 16];
 #pragma unroll
-        for (int t = 0; t < DK / 16; t++) {
-            const halfx8 a = *(const halfx8 *) &Ks[c][16 * t + 8 * h];
-            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[t], st, 0, 0, 0);
-        }
+        for (int t = 0; t < DK / 16; t++) ka[t] = *(const halfx8 *) &Ks[c][16 * t + 8 * h];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < DK / 16; t++) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[t], qf[t], st, 0, 0, 0);
         // the roundings of matmul -> * scale -> + mask in f16 arithmetic (see the kernel above)
         halfx2 sh[8];
 #pragma unroll
