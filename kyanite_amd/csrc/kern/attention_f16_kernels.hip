@@ -812,7 +812,8 @@ bool attention_f16_supported(int dk, int dv) {
 // tokens 35.3 -> 39.8, of 512 14.8 -> 21.8). Its staging needs the width of V in tiles of 32 to be 2 or 4.
 bool attention_f16_shares_keys(const AttentionParams &p) {
     const int dvt = (p.dv + 31) / 32;
-    if (dvt != 2 && dvt != 4) return false;
+    // (a wave of it keeps what the mask does to each block of keys in four registers, a lane per block)
+    if ((dvt != 2 && dvt != 4) || p.lk > 256 * ATTENTION_F16_BLOCK) return false;
     return (long long) ((p.lq + 127) / 128) * p.batch >= 512;
 }
 

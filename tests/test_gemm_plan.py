@@ -264,3 +264,21 @@ def test_f32_parts_of_k_put_whole_layers_of_workgroups_on_the_chip():
         parts = int(re.search(r"split_k=(\d+)x", ex.step_str(0)).group(1)) if "split_k" in text else 1
         last_layer = tiles * parts % 256
         assert last_layer == 0 or last_layer >= 128, (m, n, k, tiles * parts)
+
+
+def test_which_f16_attention_kernel_a_launch_takes():
+    """from 512 workgroups of 128 queries on, the kernel whose waves stage every block of keys together; below that,
+    for widths of V that are not 2 or 4 tiles of 32, and past 256 blocks of keys, the kernel whose waves split the
+    keys of 32 queries"""
+    def plan(b, lq, lk, dk, dv):
+        g = Graph()
+        q, k, v = g.input([b, lq, dk], DType.F16), g.input([b, lk, dk], DType.F16), g.input([b, lk, dv], DType.F16)
+        g.output(g.batched_mat_mul(g.softmax(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), 2), v))
+        ex = HipExecutor(0, g, 0, plan_only=True)
+        assert ex.step_count() == 1 and "attention f16" in ex.step_str(0), ex.step_str(0)
+        return "[128 queries share each block of keys]" in ex.step_str(0)
+
+    assert plan(32, 2048, 2048, 128, 128) and plan(64, 1024, 300, 64, 64) and plan(512, 1, 8192, 128, 40)
+    assert not plan(32, 1024, 1024, 128, 128) and not plan(32, 512, 512, 128, 128)
+    assert not plan(64, 1024, 300, 64, 96) and not plan(64, 1024, 300, 64, 24)
+    assert not plan(512, 1, 8193, 128, 128)
