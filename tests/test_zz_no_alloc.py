@@ -75,7 +75,7 @@ def test_products_without_scratch_and_empty_ones(hip_device):
 @pytest.mark.gpu
 def test_more_scratch_than_the_static_array_is_refused(hip_device):
     # rejected from the sizes alone, before anything is launched: the operands are never touched
-    args = matmul_args(DType.F32, 1, 640, 640, 65536, 256, (0, 65536, 1), 256, (0, 1, 65536), 256, (0, 640, 1))
+    args = matmul_args(DType.F32, 1, 1536, 1536, 65536, 256, (0, 65536, 1), 256, (0, 1, 65536), 256, (0, 1536, 1))
     assert batched_mat_mul_workspace_bytes(args) > STATIC_SCRATCH_BYTES
     with pytest.raises(KnError, match="static scratch holds"):
         batched_mat_mul_static(hip_device, HipStream(hip_device), args)
