@@ -3,7 +3,7 @@
     python -m kyanite_amd.op_bench [-d DEVICE] [-n ITERATIONS] [-p] [FAMILY ...]
 
 Families (default: all): `elementwise`, `activations`, `gather`, `reduce`, `rows` (softmax / layernorm), `conv`,
-`matmul`. `-p` plans and
+`matmul`, `attention`. `-p` plans and
 compiles every case without a device and prints its steps instead of running it.
 
 Every case is built like a user's graph (inputs, constants for weights), gets normally distributed inputs (matrix
@@ -156,6 +156,27 @@ def _cases():
         matmul_case(1024, 4672, 2048, dtype)
         matmul_case(512, 11008, 4096, dtype)
         matmul_case(4096, 4096, 4096, dtype)
+
+    def attention_case(heads, lq, lk, width, causal, dtype=f16):
+        elem = 2 if dtype == f16 else 4
+
+        def build(g):
+            q, k, v = g.input([heads, lq, width], dtype), g.input([heads, lk, width], dtype), g.input([heads, lk, width], dtype)
+            scores = g.mul(g.batched_mat_mul(q, g.permute(k, [0, 2, 1])), g.scalar(width ** -0.5, dtype))
+            if causal:
+                mask = np.where(np.tril(np.ones((lq, lk), bool), lk - lq), 0.0, -np.inf).astype(dtype.numpy)
+                scores = g.add(scores, g.constant([1, lq, lk], mask, dtype))
+            g.output(g.batched_mat_mul(g.softmax(scores, 2), v))
+
+        case("attention", f"{dtype.name.lower()} {heads} x {lq} queries x {lk} keys, width {width}" + (", causal" if causal else ""), build,
+             elem * heads * width * 2 * (lq + lk), 4.0 * heads * lq * lk * width * (0.5 if causal else 1.0))
+
+    for tokens in (512, 1024, 2048, 4096):
+        attention_case(32, tokens, tokens, 128, True)
+    attention_case(64, 2048, 2048, 64, True)
+    attention_case(32, 2048, 2048, 128, False)
+    attention_case(16, 4096, 77, 64, False)
+    attention_case(16, 4096, 4096, 40, False, f32)
     return out
 
 
@@ -191,7 +212,7 @@ def main(argv=None):
 
     from . import Graph, HipExecutor
 
-    known = ["elementwise", "activations", "gather", "reduce", "rows", "conv", "matmul"]
+    known = ["elementwise", "activations", "gather", "reduce", "rows", "conv", "matmul", "attention"]
     for family in args.families:
         if family not in known:
             parser.error(f"unknown family {family!r}; choose from {', '.join(known)}")
@@ -205,8 +226,9 @@ def main(argv=None):
         kernels = []
         for i in range(ex.step_count()):
             text = ex.step_str(i)
-            kernels.append(text.split(" value=")[0] + " [" + text.split("[", 1)[1].split("]")[0] + "]" if "[" in text.split(" operands")[0]
-                           else text.split(" value=")[0])
+            head = text.split(" operands")[0]
+            kind = text.split(" value=")[0] + (" attention" if " attention " in head else "")
+            kernels.append(kind + " [" + head.split("[", 1)[1].split("]")[0] + "]" if "[" in head else kind)
         if args.plan_only:
             print(f"{name}\n    " + "\n    ".join(kernels))
             continue

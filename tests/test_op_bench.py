@@ -6,8 +6,9 @@ from kyanite_amd import op_bench
 
 
 def test_plans_without_a_device(capsys):
-    assert op_bench.main(["-p", "reduce", "rows", "elementwise", "gather", "activations"]) == 0
+    assert op_bench.main(["-p", "reduce", "rows", "elementwise", "gather", "activations", "attention"]) == 0
     text = capsys.readouterr().out
+    assert text.count("MatMul attention") == 8 and text.count("[128 queries share each block of keys]") == 5
     assert "fold of 1024 partial results" in text and "columns TX=32 TY=8" in text and "transposed tiles 64x64" in text
     assert "rank=2 vec=8 unroll=4" in text  # embedding rows of halves: 16 bytes per thread
 
