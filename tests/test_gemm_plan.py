@@ -1,8 +1,9 @@
-"""Launch decisions of the matrix multiply (no device needed): which shapes reserve a split-K workspace in the
+"""Launch decisions of the matrix multiply (no device needed but for the last test): which shapes reserve a split-K workspace in the
 arena, and that the workspace is the size the launch will use (split * batch * m * n f32 values)."""
 import re
 
 import numpy as np
+import pytest
 
 from kyanite_amd import DType, Graph, HipExecutor, UnaryOp
 
@@ -282,3 +283,23 @@ def test_which_f16_attention_kernel_a_launch_takes():
     assert not plan(32, 1024, 1024, 128, 128) and not plan(32, 512, 512, 128, 128)
     assert not plan(64, 1024, 300, 64, 96) and not plan(64, 1024, 300, 64, 24)
     assert not plan(512, 1, 8193, 128, 128)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(32, 11008, 4096), (64, 4672, 2048), (100, 4096, 4096), (8, 4096, 11008)])
+def test_f32_products_in_parts_of_k_match_the_oracle(shape, hip_device):
+    """the f32 products whose parts of K the rule above picks (5, 3, 8 and 16 parts), against the oracle"""
+    from oracle import cpu_eval_graph
+    from runner import PARITY_RECORDS, check_outputs
+    m, n, k = shape
+    print(f"f32 product {m} x {n} x {k} in parts of K", flush=True)
+    rng = np.random.default_rng(m + n + k)
+    g = Graph()
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    g.output(g.mat_mul(g.input([m, k]), g.constant([k, n], w)))
+    inputs = [rng.standard_normal((m, k)).astype(np.float32)]
+    ex = HipExecutor(hip_device, g, 0)
+    assert "split_k=" in ex.step_str(0), ex.step_str(0)
+    expected = cpu_eval_graph(g, 0, inputs)
+    for run in range(2):
+        check_outputs(g, 0, inputs, expected, ex.evaluate(inputs), f"f32 product {shape} run {run}", PARITY_RECORDS)
