@@ -1,5 +1,5 @@
-"""Launch decisions of the matrix multiply (no device needed but for the last test): which shapes reserve a split-K workspace in the
-arena, and that the workspace is the size the launch will use (split * batch * m * n f32 values)."""
+"""Launch decisions of the matrix multiply (no device needed but for the last test): which shapes reserve a split-K
+workspace in the arena, and that the workspace is the size the launch will use (split * batch * m * n f32 values)."""
 import re
 
 import numpy as np
