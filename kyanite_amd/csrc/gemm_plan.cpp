@@ -265,6 +265,24 @@ GemmLaunchPlan plan_gemm_launch(const GemmParams &params, bool f16) {
             }
         }
     }
+    // A handful of tiles in a grouped f32 launch (which never splits K over gridDim.z): every tile is shared by
+    // workgroups that take 128 or more of K each and sum inside the launch (head_tiles = 0). Two projections of a
+    // context of 154 rows, 768 -> 320, were two launches that split K 6 ways plus their two summing passes, 25 us; a
+    // workgroup per tile over all of K walks 24 slices at one memory round trip each, 41 us for one of them.
+    if (!f16 && lp.direct && p.batch == 1 && groups > 1 && tail_enabled && split_enabled && few_tiles && !lp.skinny_tile && p.k >= 256 && !p.pair_op) {
+        long long parts = std::min<long long>(p.k / 128, 16);
+        long long chunk = ((p.k + parts - 1) / parts + 31) / 32 * 32;
+        parts = (p.k + chunk - 1) / chunk;
+        if (parts >= 2) {
+            lp.head_tiles = 0;
+            lp.tail_split = (int) parts;
+            lp.tail_k_chunk = (int) chunk;
+            const long long tile = lp.small_tile ? 64 : 128;
+            lp.workspace_bytes = (size_t) (blocks * parts * tile * tile * 4);
+            lp.counter_bytes = (size_t) blocks * 4;
+            return lp;
+        }
+    }
     if (f16 && lp.direct) {
         if (model_split > 1) {
             long long chunk = (p.k + model_split - 1) / model_split;
@@ -359,6 +377,8 @@ bool gemm_group_ok(const GemmParams &p, bool f16) {
     if (single.estimated_us > 0.0 && grouped.estimated_us > 0.0) return grouped.estimated_us <= p.groups * single.estimated_us;
     // Otherwise: where even all products together leave the chip short of tiles, separate launches that split K are
     // faster.
+    // (a handful of f32 tiles: the grouped launch shares every tile between workgroups along K)
+    if (grouped.tail_split > 1 && grouped.head_tiles == 0) return true;
     GemmParams wide = p;
     wide.groups = 1;
     wide.n = p.n * p.groups;

@@ -162,9 +162,13 @@ def test_projections_of_one_input_share_a_launch():
     ex = HipExecutor(0, _projections(3, 256, 64, 128, bias_on=(1,)), 0, plan_only=True)
     texts = sorted(ex.step_str(i).split(" [")[0].split("k=64")[1].strip() for i in range(ex.step_count()))
     assert texts == ["+add", "x2 grouped"]
-    # where even the group leaves the chip short of tiles, the products run apart and split K
+    # where even the group leaves the chip short of tiles, every tile of the one launch is shared along K (f32; 16.4 us
+    # against 24.4 us for the products apart, each with its K split and its summing pass, which is the plan without
+    # the in-launch split)
     ex = HipExecutor(0, _projections(2, 8, 4096, 256), 0, plan_only=True)
-    assert ex.step_count() == 2 and all("grouped" not in ex.step_str(i) for i in range(2))
+    assert ex.step_count() == 1 and "x2 grouped [direct 64x64 bk32 head=0 tail_split=16x256]" in ex.step_str(0), ex.step_str(0)
+    ex = HipExecutor(0, _projections(2, 8, 4096, 256), 0, plan_only=True, tail_split=False)
+    assert ex.step_count() == 2 and all("grouped" not in ex.step_str(i) and "split_k=" in ex.step_str(i) for i in range(2))
 
 
 def test_constant_weights_are_laid_out_again_for_f16_matmuls(monkeypatch):

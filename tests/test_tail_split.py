@@ -3,7 +3,7 @@
 instantiation the launch plan picks: f32 on 64 x 64 and 128 x 128 tiles, f16 on 64 x 64, 128 x 64, 256 x 192 and
 256 x 256 tiles (with the f16 cost model a sparse last round of 128 x 128 or 256 x 128 tiles never comes out cheapest:
 a larger tile that fits one round does), splits of 2, 3, 4 and 8, epilogues (bias, residual, relu), ragged tile rows
-and grouped launches. The GPU multiplies the whole product, twice (the second run finds the counters as the first left them); the
+and grouped launches, and the grouped f32 launches of a handful of tiles, all of which are shared. The GPU multiplies the whole product, twice (the second run finds the counters as the first left them); the
 oracle evaluates the same graph on a sample of the rows of the left operand that reaches every tile row of every
 workgroup tile, and those rows of the GPU result are compared with it."""
 import numpy as np
@@ -28,6 +28,9 @@ CASES = [
     (DType.F16, 300, 2688, 1536, (False, False, False), 3, "x3 grouped [direct 64x64 bk64 head=512 tail_split=3x512"),
     (DType.F16, 300, 11008, 1024, (False, False, False), 3, "x3 grouped [direct 256x192 bk64 head=256 tail_split=2x512"),
     (DType.F16, 1024, 6528, 2048, (False, False, False), 3, "x3 grouped [direct 256x256 bk64 head=256 tail_split=4x512"),
+    # a handful of tiles in a grouped f32 launch: every tile shared (head = 0)
+    (DType.F32, 154, 320, 768, (False, False, False), 2, "x2 grouped [direct 64x64 bk32 head=0 tail_split=6x128"),
+    (DType.F32, 100, 200, 2144, (False, False, False), 3, "x3 grouped [direct 128x128 bk32 head=0 tail_split=14x160"),
 ]
 
 
